@@ -1,0 +1,110 @@
+/*
+ * ref_shim.c - exports a few of the reference's own static functions as a shared library.
+ *
+ * TEST INFRASTRUCTURE ONLY. This translation unit includes the reference's header-only C
+ * sources where they lie (the include path points at the read-only reference checkout); no
+ * reference source is copied into this repository. The library it builds (oracle/_ref/) is
+ * used to (1) write the golden fixtures under tests/golden/, (2) cross-check the oracle, and
+ * (3) serve as the "reference" CPU baseline timed by the benchmark. It is never linked into or
+ * loaded by the shipped library.
+ */
+#include <string.h>
+#include <stdlib.h>
+#include <time.h>
+
+#define GGUF_LOADER_IMPLEMENTATION
+#include "common/gguf_loader.h"
+#define GGML_DEQUANT_IMPLEMENTATION
+#include "common/ggml_dequant.h"
+#define BPE_TOKENIZER_IMPLEMENTATION
+#include "common/bpe_tokenizer.h"
+#define TRANSFORMER_IMPLEMENTATION
+#include "common/transformer.h"
+
+float ref_fp16_to_fp32(uint16_t h) { return ggml_fp16_to_fp32(h); }
+void ref_fp16_table(float *out) { for (uint32_t h = 0; h < 65536u; h++) out[h] = ggml_fp16_to_fp32((uint16_t)h); }
+int ref_dequant_row(uint32_t type, const void *src, float *dst, int n) { return dequant_row(type, src, dst, n); }
+size_t ref_dequant_row_size(uint32_t type, int n) { return dequant_row_size(type, n); }
+size_t ref_tf_row_bytes(uint32_t type, int n_cols) { return tf_row_bytes(type, n_cols); }
+
+static qtensor make_qt(const void *data, uint32_t type, int n_rows, int n_cols) {
+    qtensor t;
+    memset(&t, 0, sizeof(t));
+    t.data = (void *)data;
+    t.type = type;
+    t.n_rows = n_rows;
+    t.n_cols = n_cols;
+    t.n_dims = 2;
+    t.dims[0] = (uint64_t)n_cols;
+    t.dims[1] = (uint64_t)n_rows;
+    return t;
+}
+
+/* tf_qmatvec on a 2-D tensor; f64_accum selects the reference's double-accumulate oracle mode
+ * (which only exists in the worker, so it is reached through a 1-thread pool call). */
+void ref_tf_qmatvec(float *dst, const void *W, uint32_t type, const float *x, int n_rows, int n_cols) {
+    qtensor t = make_qt(W, type, n_rows, n_cols);
+    float *tmp = (float *)malloc((size_t)n_cols * sizeof(float));
+    tf_qmatvec(dst, &t, x, n_rows, tmp);
+    free(tmp);
+}
+
+void ref_tf_qmatvec_f64(float *dst, const void *W, uint32_t type, const float *x, int n_rows, int n_cols) {
+    qtensor t = make_qt(W, type, n_rows, n_cols);
+    float *tmp = (float *)malloc((size_t)n_cols * sizeof(float));
+    tf_matvec_task task = {dst, &t, x, 0, n_rows, tmp};
+    int saved = tf_g_f64_accum;
+    tf_g_f64_accum = 1;
+    tf_qmatvec_worker(&task);
+    tf_g_f64_accum = saved;
+    free(tmp);
+}
+
+void ref_tf_qmatvec_expert(float *dst, const void *W, uint32_t type, int expert, const float *x,
+                           int rows_per_expert, int n_cols) {
+    qtensor t = make_qt(W, type, rows_per_expert, n_cols);
+    float *tmp = (float *)malloc((size_t)n_cols * sizeof(float));
+    tf_qmatvec_expert(dst, &t, expert, x, rows_per_expert, tmp);
+    free(tmp);
+}
+
+void ref_tf_gemm_tokenmajor(float *Y, const void *W, uint32_t type, const float *X, int n_rows,
+                            int n_cols, int N, int out_stride, int X_stride, int n_threads) {
+    qtensor t = make_qt(W, type, n_rows, n_cols);
+    tf_gemm_f16_mt_tokenmajor(Y, &t, X, n_rows, N, out_stride, X_stride, n_threads);
+}
+
+void ref_tf_softmax(float *x, int n) { tf_softmax(x, n); }
+void ref_tf_silu_mul(float *out, const float *gate, const float *up, int n) { tf_silu_mul_avx2(out, gate, up, n); }
+
+/* tf_qmatvec_pool on a stand-in model that only carries what the pool path reads: thread
+ * count, per-thread scratch and the pool itself. Returns seconds per call over `iters` calls. */
+double ref_tf_qmatvec_pool_time(float *dst, const void *W, uint32_t type, const float *x,
+                                int n_rows, int n_cols, int n_threads, int iters) {
+    transformer_model *m = (transformer_model *)calloc(1, sizeof(transformer_model));
+    qtensor t = make_qt(W, type, n_rows, n_cols);
+    if (n_threads < 1) n_threads = 1;
+    m->n_threads = n_threads;
+    m->thread_tmp = (float **)calloc((size_t)n_threads, sizeof(float *));
+    for (int i = 0; i < n_threads; i++) m->thread_tmp[i] = (float *)calloc((size_t)n_cols, sizeof(float));
+    if (n_threads > 1) tf_pool_start(m);
+    tf_qmatvec_pool(m, dst, &t, x, n_rows); /* warm-up */
+    struct timespec a, b;
+    clock_gettime(CLOCK_MONOTONIC, &a);
+    for (int i = 0; i < iters; i++) tf_qmatvec_pool(m, dst, &t, x, n_rows);
+    clock_gettime(CLOCK_MONOTONIC, &b);
+    if (n_threads > 1) tf_pool_shutdown(m);
+    for (int i = 0; i < n_threads; i++) free(m->thread_tmp[i]);
+    free(m->thread_tmp);
+    free(m);
+    return ((double)(b.tv_sec - a.tv_sec) + 1e-9 * (double)(b.tv_nsec - a.tv_nsec)) / (double)(iters > 0 ? iters : 1);
+}
+
+const void *ref_table(const char *name, size_t *bytes) {
+    if (!strcmp(name, "iq2xxs_grid")) { *bytes = sizeof(iq2xxs_grid); return iq2xxs_grid; }
+    if (!strcmp(name, "iq3s_grid")) { *bytes = sizeof(iq3s_grid); return iq3s_grid; }
+    if (!strcmp(name, "iq4nl_values")) { *bytes = sizeof(kvalues_iq4nl); return kvalues_iq4nl; }
+    if (!strcmp(name, "ksigns")) { *bytes = sizeof(ksigns_iq2xs); return ksigns_iq2xs; }
+    *bytes = 0;
+    return NULL;
+}
