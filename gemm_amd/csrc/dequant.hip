@@ -1,0 +1,89 @@
+/*
+ * dequant.hip - block decoders: raw GGML blocks -> fp32, bit-identical to the reference's
+ * scalar decoders (common/ggml_dequant.h:1479-1687, :2793-3058, type switch :3177-3265).
+ *
+ * One thread decodes eight consecutive elements and writes 32 contiguous bytes, so a
+ * wavefront writes 2 KiB of contiguous fp32 per store pair. The kernel is bound by that
+ * write stream (4 B out per 0.26..1.06 B in).
+ */
+#include "qlin_device.h"
+#include "qlin_internal.h"
+
+namespace qlin {
+
+template <uint32_t T, bool VEC>
+__global__ void __launch_bounds__(256)
+dequant_kernel(const uint8_t *__restrict__ W, float *__restrict__ out, int n_rows, int n_cols,
+               size_t row_bytes, int blocks_per_row) {
+    using C = Codec<T>;
+    constexpr int GPB = C::BE / 8; /* 8-element groups per block */
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long groups_per_row = (long long)blocks_per_row * GPB;
+    if (gid >= groups_per_row * n_rows) return;
+    const int row = (int)(gid / groups_per_row);
+    const int g = (int)(gid - (long long)row * groups_per_row);
+    const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+    float y[8];
+    C::decode8(W + (size_t)row * row_bytes + (size_t)blk * C::BB, k0, y);
+    float *o = out + (size_t)row * n_cols + (size_t)blk * C::BE + k0;
+    if (VEC) {
+        reinterpret_cast<float4 *>(o)[0] = make_float4(y[0], y[1], y[2], y[3]);
+        reinterpret_cast<float4 *>(o)[1] = make_float4(y[4], y[5], y[6], y[7]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) o[i] = y[i];
+    }
+}
+
+/* F16 / BF16 / F32 rows (common/ggml_dequant.h:3251-3261) */
+__global__ void __launch_bounds__(256)
+convert_plain_kernel(uint32_t type, const uint8_t *__restrict__ src, float *__restrict__ out, long long n) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    if (type == T_F32) {
+        reinterpret_cast<uint32_t *>(out)[i] = reinterpret_cast<const uint32_t *>(src)[i];
+    } else {
+        const uint32_t h = reinterpret_cast<const uint16_t *>(src)[i];
+        out[i] = (type == T_F16) ? half_bits_exact(h) : __uint_as_float(h << 16);
+    }
+}
+
+template <uint32_t T>
+static hipError_t launch_typed(const void *W, float *out, int n_rows, int n_cols, size_t row_bytes,
+                               hipStream_t stream) {
+    const int bpr = n_cols / Codec<T>::BE;
+    const long long groups = (long long)bpr * (Codec<T>::BE / 8) * n_rows;
+    if (groups == 0) return hipSuccess;
+    const unsigned grid = (unsigned)((groups + 255) / 256);
+    const bool vec = (n_cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
+    if (vec)
+        hipLaunchKernelGGL((dequant_kernel<T, true>), dim3(grid), dim3(256), 0, stream,
+                           (const uint8_t *)W, out, n_rows, n_cols, row_bytes, bpr);
+    else
+        hipLaunchKernelGGL((dequant_kernel<T, false>), dim3(grid), dim3(256), 0, stream,
+                           (const uint8_t *)W, out, n_rows, n_cols, row_bytes, bpr);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, int n_cols,
+                          size_t row_bytes, hipStream_t stream) {
+    switch (type) {
+    case T_Q8_0: return launch_typed<T_Q8_0>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_Q4_K: return launch_typed<T_Q4_K>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_Q5_K: return launch_typed<T_Q5_K>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_Q6_K: return launch_typed<T_Q6_K>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_IQ2_XXS: return launch_typed<T_IQ2_XXS>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_IQ4_NL: return launch_typed<T_IQ4_NL>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_IQ3_S: return launch_typed<T_IQ3_S>(W, out, n_rows, n_cols, row_bytes, stream);
+    case T_F32: case T_F16: case T_BF16: {
+        const long long n = (long long)n_rows * n_cols;
+        if (n == 0) return hipSuccess;
+        hipLaunchKernelGGL(convert_plain_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                           type, (const uint8_t *)W, out, n);
+        return hipGetLastError();
+    }
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace qlin

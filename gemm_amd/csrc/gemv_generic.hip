@@ -1,0 +1,139 @@
+/*
+ * gemv_generic.hip - y = W.x and Y = X.W^T in fp32 for every supported block type.
+ *
+ * The plain path: correct for any shape made of whole blocks, used for types and shapes the
+ * tuned kernels do not take. A wavefront owns R consecutive rows; its lanes stride over
+ * 8-element groups of the row, decode them in registers and FMA them with x (read as two
+ * float4 per group, contiguous across the lanes). fp32 accumulate, wave64 shuffle reduction.
+ * Computes what tf_qmatvec computes (common/transformer.h:1049-1114): the dot of each
+ * decoded row with x; only the summation order differs.
+ */
+#include "qlin_device.h"
+#include "qlin_internal.h"
+
+namespace qlin {
+
+template <uint32_t T, int R>
+__global__ void __launch_bounds__(256)
+gemv_generic_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
+                    int n_rows, int n_cols, size_t row_bytes) {
+    using C = Codec<T>;
+    constexpr int GPB = C::BE / 8;
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int row0 = wave * R;
+    if (row0 >= n_rows) return;
+    const int groups = (n_cols / C::BE) * GPB;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.0f;
+    for (int g = lane; g < groups; g += 64) {
+        const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+        const float4 xa = *reinterpret_cast<const float4 *>(x + (size_t)blk * C::BE + k0);
+        const float4 xb = *reinterpret_cast<const float4 *>(x + (size_t)blk * C::BE + k0 + 4);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (row0 + r < n_rows) {
+                float w[8];
+                C::decode8(W + (size_t)(row0 + r) * row_bytes + (size_t)blk * C::BB, k0, w);
+                acc[r] += w[0] * xa.x + w[1] * xa.y + w[2] * xa.z + w[3] * xa.w +
+                          w[4] * xb.x + w[5] * xb.y + w[6] * xb.z + w[7] * xb.w;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < n_rows) y[row0 + r] = s;
+    }
+}
+
+/* prefill in fp32: a wavefront owns one weight row and TT tokens at a time; the row is
+ * decoded once per token tile. Y is token-major. (Semantics of the reference's generic
+ * prefill path, common/transformer.h:4535-4572.) */
+template <uint32_t T, int TT>
+__global__ void __launch_bounds__(256)
+gemm_f32_generic_kernel(const uint8_t *__restrict__ W, const float *__restrict__ X, float *__restrict__ Y,
+                        int n_rows, int n_cols, int n_tok, int ldx, int ldy, size_t row_bytes) {
+    using C = Codec<T>;
+    constexpr int GPB = C::BE / 8;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int t0 = blockIdx.y * TT;
+    const int groups = (n_cols / C::BE) * GPB;
+    float acc[TT];
+#pragma unroll
+    for (int t = 0; t < TT; t++) acc[t] = 0.0f;
+    for (int g = lane; g < groups; g += 64) {
+        const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+        float w[8];
+        C::decode8(W + (size_t)row * row_bytes + (size_t)blk * C::BB, k0, w);
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            if (t0 + t < n_tok) {
+                const float *xp = X + (size_t)(t0 + t) * ldx + (size_t)blk * C::BE + k0;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[t] += w[i] * xp[i];
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < TT; t++) {
+        const float s = wave_sum(acc[t]);
+        if (lane == 0 && t0 + t < n_tok) Y[(size_t)(t0 + t) * ldy + row] = s;
+    }
+}
+
+template <uint32_t T>
+static hipError_t gemv_typed(const void *W, const float *x, float *y, int n_rows, int n_cols, hipStream_t s) {
+    constexpr int R = 2;
+    const size_t rb = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
+    const int waves = (n_rows + R - 1) / R;
+    hipLaunchKernelGGL((gemv_generic_kernel<T, R>), dim3((waves + 3) / 4), dim3(256), 0, s,
+                       (const uint8_t *)W, x, y, n_rows, n_cols, rb);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, float *y, int n_rows,
+                               int n_cols, hipStream_t s) {
+    if (n_rows == 0) return hipSuccess;
+    switch (type) {
+    case T_Q8_0: return gemv_typed<T_Q8_0>(W, x, y, n_rows, n_cols, s);
+    case T_Q4_K: return gemv_typed<T_Q4_K>(W, x, y, n_rows, n_cols, s);
+    case T_Q5_K: return gemv_typed<T_Q5_K>(W, x, y, n_rows, n_cols, s);
+    case T_Q6_K: return gemv_typed<T_Q6_K>(W, x, y, n_rows, n_cols, s);
+    case T_IQ2_XXS: return gemv_typed<T_IQ2_XXS>(W, x, y, n_rows, n_cols, s);
+    case T_IQ4_NL: return gemv_typed<T_IQ4_NL>(W, x, y, n_rows, n_cols, s);
+    case T_IQ3_S: return gemv_typed<T_IQ3_S>(W, x, y, n_rows, n_cols, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+template <uint32_t T>
+static hipError_t gemm_typed(const void *W, const float *X, float *Y, int n_rows, int n_cols, int n_tok,
+                             int ldx, int ldy, hipStream_t s) {
+    constexpr int TT = 8;
+    const size_t rb = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
+    dim3 grid((n_rows + 3) / 4, (n_tok + TT - 1) / TT);
+    hipLaunchKernelGGL((gemm_f32_generic_kernel<T, TT>), grid, dim3(256), 0, s, (const uint8_t *)W, X, Y,
+                       n_rows, n_cols, n_tok, ldx, ldy, rb);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *Y, int n_rows,
+                           int n_cols, int n_tok, int ldx, int ldy, hipStream_t s) {
+    if (n_rows == 0 || n_tok == 0) return hipSuccess;
+    switch (type) {
+    case T_Q8_0: return gemm_typed<T_Q8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    case T_Q4_K: return gemm_typed<T_Q4_K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    case T_Q5_K: return gemm_typed<T_Q5_K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    case T_Q6_K: return gemm_typed<T_Q6_K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    case T_IQ2_XXS: return gemm_typed<T_IQ2_XXS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    case T_IQ4_NL: return gemm_typed<T_IQ4_NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    case T_IQ3_S: return gemm_typed<T_IQ3_S>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace qlin

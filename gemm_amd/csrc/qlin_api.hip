@@ -1,0 +1,601 @@
+/*
+ * qlin_api.hip - the C ABI of libqlinear (declared in include/qlinear.h).
+ *
+ * This layer owns the device, one stream, the weight registry and the staging buffers of the
+ * host-pointer entry points, checks every argument the kernels rely on (whole blocks,
+ * alignment, sizes) and turns HIP failures into status codes. It contains no arithmetic and
+ * no CPU fallback: if the GPU cannot be used every call fails.
+ */
+#include "../../include/qlinear.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+
+#include "qlin_device.h"
+#include "qlin_internal.h"
+
+namespace {
+
+using namespace qlin;
+
+thread_local std::string t_error;
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    t_error = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                          \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess)                                                                  \
+            return fail(QLIN_ERR_DEVICE, "%s failed: %s", #expr, hipGetErrorString(e_));       \
+    } while (0)
+
+/* grow-only device buffer for staging */
+struct DevBuf {
+    void *p = nullptr;
+    size_t cap = 0;
+    int ensure(size_t n) {
+        if (n <= cap) return QLIN_OK;
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+        size_t want = n + n / 4 + 256;
+        if (hipMalloc(&p, want) != hipSuccess) {
+            p = nullptr;
+            return fail(QLIN_ERR_NOMEM, "hipMalloc of %zu bytes failed", want);
+        }
+        cap = want;
+        return QLIN_OK;
+    }
+    void release() {
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+    }
+};
+
+struct Range { size_t bytes; void *dev; };
+
+struct State {
+    std::mutex mu;
+    bool ready = false;
+    int device = 0;
+    int n_cu = 256;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    std::map<uintptr_t, Range> registry; /* host begin -> range */
+    DevBuf w[3], x, y[3], tmp[4];
+    /* tuning knobs read once from the environment (QLIN_Q4K_RPP, QLIN_Q4K_WAVES); 0 = default */
+    int tune_rpp = 0, tune_waves = 0;
+} g;
+
+int ensure_init_locked(int device) {
+    if (g.ready) return QLIN_OK;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0)
+        return fail(QLIN_ERR_DEVICE, "no HIP device available (this library has no CPU path)");
+    if (device < 0 || device >= count) return fail(QLIN_ERR_ARG, "device %d out of range (%d devices)", device, count);
+    HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    g.n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    HIP_TRY(hipStreamCreate(&g.stream));
+    HIP_TRY(hipEventCreate(&g.ev0));
+    HIP_TRY(hipEventCreate(&g.ev1));
+    if (const char *e = getenv("QLIN_Q4K_RPP")) g.tune_rpp = atoi(e);
+    if (const char *e = getenv("QLIN_Q4K_WAVES")) g.tune_waves = atoi(e);
+    g.device = device;
+    g.ready = true;
+    return QLIN_OK;
+}
+
+bool known_type(uint32_t t) {
+    int be, bb;
+    return type_geometry(t, &be, &bb);
+}
+bool block_type(uint32_t t) {
+    int be, bb;
+    return type_geometry(t, &be, &bb) && be > 1;
+}
+size_t row_size(uint32_t t, int n) {
+    int be, bb;
+    if (!type_geometry(t, &be, &bb) || n < 0) return 0;
+    return (size_t)((n + be - 1) / be) * (size_t)bb;
+}
+bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+/* device pointer mirroring a host pointer inside a registered range, or nullptr */
+const void *lookup_locked(const void *host, size_t need) {
+    if (g.registry.empty()) return nullptr;
+    const uintptr_t h = reinterpret_cast<uintptr_t>(host);
+    auto it = g.registry.upper_bound(h);
+    if (it == g.registry.begin()) return nullptr;
+    --it;
+    if (h < it->first || h + need > it->first + it->second.bytes) return nullptr;
+    return static_cast<const uint8_t *>(it->second.dev) + (h - it->first);
+}
+
+/* device view of host weights: the registered copy, or a staged copy in `buf` */
+int weights_on_device_locked(const void *host, size_t bytes, DevBuf &buf, const void **dev) {
+    if (const void *d = lookup_locked(host, bytes)) {
+        *dev = d;
+        return QLIN_OK;
+    }
+    if (int rc = buf.ensure(bytes)) return rc;
+    HIP_TRY(hipMemcpyAsync(buf.p, host, bytes, hipMemcpyHostToDevice, g.stream));
+    *dev = buf.p;
+    return QLIN_OK;
+}
+
+/* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the plain kernel */
+hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y, int n_rows,
+                         int n_cols, hipStream_t s) {
+    if (n_rows == 0) return hipSuccess;
+    if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && aligned(W, 16) && aligned(x, 16)) {
+        const int n_sb = n_cols / 256;
+        const int n_slices = (n_sb + 15) / 16;
+        /* one pass of 7 or 8 rows per wave when the row count allows ~8 waves per CU */
+        int target = g.tune_waves > 0 ? g.tune_waves : 8;
+        long long groups = (long long)g.n_cu * target / n_slices;
+        int rpw = (int)((n_rows + groups - 1) / groups);
+        int rpp = rpw >= 8 ? 8 : rpw >= 7 ? 7 : rpw >= 4 ? 4 : rpw >= 2 ? 2 : 1;
+        if (g.tune_rpp > 0) rpp = g.tune_rpp;
+        return launch_gemv_q4k(W, x, y, n_rows, n_cols, s, g.n_cu, rpp, target);
+    }
+    return launch_gemv_generic(type, W, x, y, n_rows, n_cols, s);
+}
+
+int check_linear_shape(uint32_t type, int n_rows, int n_cols) {
+    int be, bb;
+    if (!type_geometry(type, &be, &bb) || be == 1)
+        return fail(QLIN_ERR_TYPE, "unsupported weight type %u", type);
+    if (n_rows < 0 || n_cols <= 0) return fail(QLIN_ERR_ARG, "bad shape %d x %d", n_rows, n_cols);
+    if (n_cols % be) return fail(QLIN_ERR_ARG, "n_cols %d is not a whole number of %d-element blocks", n_cols, be);
+    return QLIN_OK;
+}
+
+int matvec_host_locked(float *dst, const void *W, uint32_t type, int n_cols, const float *x, int n_rows,
+                       int slot, bool upload_x) {
+    const size_t rb = row_size(type, n_cols);
+    const void *dW;
+    if (int rc = weights_on_device_locked(W, rb * (size_t)n_rows, g.w[slot], &dW)) return rc;
+    if (upload_x) {
+        if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
+        HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_cols * 4, hipMemcpyHostToDevice, g.stream));
+    }
+    if (int rc = g.y[slot].ensure((size_t)n_rows * 4 + 16)) return rc;
+    HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)g.y[slot].p, n_rows, n_cols, g.stream));
+    HIP_TRY(hipMemcpyAsync(dst, g.y[slot].p, (size_t)n_rows * 4, hipMemcpyDeviceToHost, g.stream));
+    return QLIN_OK;
+}
+
+void void_decoder(uint32_t type, const char *name, const void *src, float *dst, int n) {
+    const int rc = qlin_dequant_row(type, src, dst, n);
+    if (rc != QLIN_OK) {
+        fprintf(stderr, "%s: %s\n", name, qlin_last_error());
+        if (dst && n > 0) memset(dst, 0, (size_t)n * sizeof(float));
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+/* ------------------------------------------------------------------ lifecycle */
+
+int qlin_init(int device) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (g.ready && device != g.device) return fail(QLIN_ERR_ARG, "already initialised on device %d", g.device);
+    return ensure_init_locked(device);
+}
+
+void qlin_shutdown(void) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (!g.ready) return;
+    (void)hipStreamSynchronize(g.stream);
+    for (auto &kv : g.registry) (void)hipFree(kv.second.dev);
+    g.registry.clear();
+    for (auto &b : g.w) b.release();
+    for (auto &b : g.y) b.release();
+    for (auto &b : g.tmp) b.release();
+    g.x.release();
+    (void)hipEventDestroy(g.ev0);
+    (void)hipEventDestroy(g.ev1);
+    (void)hipStreamDestroy(g.stream);
+    g.stream = nullptr;
+    g.ready = false;
+}
+
+const char *qlin_last_error(void) { return t_error.c_str(); }
+
+int qlin_device_info(char *name, size_t cap, int *compute_units, size_t *mem_bytes) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, g.device));
+    if (name && cap) {
+        snprintf(name, cap, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = prop.multiProcessorCount;
+    if (mem_bytes) *mem_bytes = prop.totalGlobalMem;
+    return QLIN_OK;
+}
+
+/* ------------------------------------------------------------------ codec */
+
+size_t qlin_dequant_row_size(uint32_t ggml_type, int n) { return row_size(ggml_type, n); }
+
+int qlin_dequant_rows(uint32_t ggml_type, const void *src, float *dst, int n_rows, int n_cols) {
+    if (!known_type(ggml_type)) return fail(QLIN_ERR_TYPE, "unsupported type %u", ggml_type);
+    if (n_rows < 0 || n_cols < 0) return fail(QLIN_ERR_ARG, "negative size");
+    int be, bb;
+    type_geometry(ggml_type, &be, &bb);
+    const int whole = n_cols / be * be; /* a ragged tail is not decoded */
+    if (n_rows == 0 || whole == 0) return QLIN_OK;
+    if (!src || !dst) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const size_t rb = row_size(ggml_type, n_cols);
+    const void *dW;
+    if (int rc = weights_on_device_locked(src, rb * (size_t)(n_rows - 1) + (size_t)(whole / be) * bb, g.w[0], &dW)) return rc;
+    const size_t out_bytes = (size_t)n_rows * n_cols * 4;
+    if (int rc = g.tmp[0].ensure(out_bytes)) return rc;
+    HIP_TRY(launch_dequant(ggml_type, dW, (float *)g.tmp[0].p, n_rows, n_cols, rb, g.stream));
+    if (whole == n_cols) {
+        HIP_TRY(hipMemcpyAsync(dst, g.tmp[0].p, out_bytes, hipMemcpyDeviceToHost, g.stream));
+    } else { /* leave the undecoded tail of every row untouched in dst */
+        HIP_TRY(hipMemcpy2DAsync(dst, (size_t)n_cols * 4, g.tmp[0].p, (size_t)n_cols * 4, (size_t)whole * 4,
+                                 (size_t)n_rows, hipMemcpyDeviceToHost, g.stream));
+    }
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_dequant_row(uint32_t ggml_type, const void *src, float *dst, int n) {
+    return qlin_dequant_rows(ggml_type, src, dst, 1, n);
+}
+
+void qlin_dequantize_row_q8_0(const void *s, float *d, int n) { void_decoder(T_Q8_0, "qlin_dequantize_row_q8_0", s, d, n); }
+void qlin_dequantize_row_q4_K(const void *s, float *d, int n) { void_decoder(T_Q4_K, "qlin_dequantize_row_q4_K", s, d, n); }
+void qlin_dequantize_row_q5_K(const void *s, float *d, int n) { void_decoder(T_Q5_K, "qlin_dequantize_row_q5_K", s, d, n); }
+void qlin_dequantize_row_q6_K(const void *s, float *d, int n) { void_decoder(T_Q6_K, "qlin_dequantize_row_q6_K", s, d, n); }
+void qlin_dequantize_row_iq2_xxs(const void *s, float *d, int n) { void_decoder(T_IQ2_XXS, "qlin_dequantize_row_iq2_xxs", s, d, n); }
+void qlin_dequantize_row_iq3_s(const void *s, float *d, int n) { void_decoder(T_IQ3_S, "qlin_dequantize_row_iq3_s", s, d, n); }
+void qlin_dequantize_row_iq4_nl(const void *s, float *d, int n) { void_decoder(T_IQ4_NL, "qlin_dequantize_row_iq4_nl", s, d, n); }
+
+/* ------------------------------------------------------------------ weights */
+
+int qlin_weight_register(const void *host_data, size_t n_bytes) {
+    if (!host_data || n_bytes == 0) return fail(QLIN_ERR_ARG, "null or empty weight range");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const uintptr_t h = reinterpret_cast<uintptr_t>(host_data);
+    if (lookup_locked(host_data, 1) || lookup_locked((const uint8_t *)host_data + n_bytes - 1, 1))
+        return fail(QLIN_ERR_ARG, "range overlaps a registered range");
+    auto nxt = g.registry.lower_bound(h);
+    if (nxt != g.registry.end() && nxt->first < h + n_bytes) return fail(QLIN_ERR_ARG, "range overlaps a registered range");
+    void *dev = nullptr;
+    if (hipMalloc(&dev, n_bytes + 256) != hipSuccess) return fail(QLIN_ERR_NOMEM, "hipMalloc of %zu bytes failed", n_bytes);
+    hipError_t e = hipMemcpy(dev, host_data, n_bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return fail(QLIN_ERR_DEVICE, "upload failed: %s", hipGetErrorString(e));
+    }
+    g.registry[h] = Range{n_bytes, dev};
+    return QLIN_OK;
+}
+
+int qlin_weight_unregister(const void *host_data) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    auto it = g.registry.find(reinterpret_cast<uintptr_t>(host_data));
+    if (it == g.registry.end()) return fail(QLIN_ERR_ARG, "pointer was not registered");
+    if (g.ready) (void)hipStreamSynchronize(g.stream);
+    (void)hipFree(it->second.dev);
+    g.registry.erase(it);
+    return QLIN_OK;
+}
+
+const void *qlin_weight_device_ptr(const void *host_ptr) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    return lookup_locked(host_ptr, 1);
+}
+
+/* ------------------------------------------------------------------ linear, host pointers */
+
+int qlin_matvec(float *dst, const void *W, uint32_t type, int n_cols, const float *x, int n_rows) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!dst || !W || !x) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    if (int rc = matvec_host_locked(dst, W, type, n_cols, x, n_rows, 0, true)) return rc;
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2, const void *W2,
+                       uint32_t type2, int n_cols, const float *x, int n_rows) {
+    if (int rc = check_linear_shape(type1, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type2, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!dst1 || !dst2 || !W1 || !W2 || !x) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    if (int rc = matvec_host_locked(dst1, W1, type1, n_cols, x, n_rows, 0, true)) return rc;
+    if (int rc = matvec_host_locked(dst2, W2, type2, n_cols, x, n_rows, 1, false)) return rc;
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k, const void *Wk,
+                    uint32_t type_k, float *v, const void *Wv, uint32_t type_v, int n_kv,
+                    int n_cols, const float *x) {
+    if (int rc = check_linear_shape(type_q, n_q, n_cols)) return rc;
+    if (int rc = check_linear_shape(type_k, n_kv, n_cols)) return rc;
+    if (int rc = check_linear_shape(type_v, n_kv, n_cols)) return rc;
+    if (!x || (n_q && (!q || !Wq)) || (n_kv && (!k || !Wk || !v || !Wv))) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    bool up = true;
+    if (n_q) { if (int rc = matvec_host_locked(q, Wq, type_q, n_cols, x, n_q, 0, up)) return rc; up = false; }
+    if (n_kv) {
+        if (int rc = matvec_host_locked(k, Wk, type_k, n_cols, x, n_kv, 1, up)) return rc;
+        if (int rc = matvec_host_locked(v, Wv, type_v, n_cols, x, n_kv, 2, false)) return rc;
+    }
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_matvec_expert(float *dst, const void *W, uint32_t type, int n_cols, int expert, const float *x,
+                       int rows_per_expert) {
+    if (int rc = check_linear_shape(type, rows_per_expert, n_cols)) return rc;
+    if (expert < 0) return fail(QLIN_ERR_ARG, "negative expert index");
+    if (!W) return fail(QLIN_ERR_ARG, "null pointer");
+    const size_t rb = row_size(type, n_cols);
+    const uint8_t *slice = (const uint8_t *)W + (size_t)expert * (size_t)rows_per_expert * rb;
+    return qlin_matvec(dst, slice, type, n_cols, x, rows_per_expert);
+}
+
+int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, const float *X, int n_rows,
+                         int n_tok, int out_stride, int x_stride) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_tok < 0 || out_stride < n_rows || x_stride < n_cols) return fail(QLIN_ERR_ARG, "bad token count or stride");
+    if (n_rows == 0 || n_tok == 0) return QLIN_OK;
+    if (!Y || !W || !X) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const size_t rb = row_size(type, n_cols);
+    const void *dW;
+    if (int rc = weights_on_device_locked(W, rb * (size_t)n_rows, g.w[0], &dW)) return rc;
+    /* X and Y are staged densely (ldx = n_cols, ldy = n_rows); strides are applied by the copies */
+    if (int rc = g.tmp[0].ensure((size_t)n_tok * n_cols * 4)) return rc;
+    if (int rc = g.tmp[1].ensure((size_t)n_tok * n_rows * 4)) return rc;
+    HIP_TRY(hipMemcpy2DAsync(g.tmp[0].p, (size_t)n_cols * 4, X, (size_t)x_stride * 4, (size_t)n_cols * 4,
+                             (size_t)n_tok, hipMemcpyHostToDevice, g.stream));
+    HIP_TRY(launch_gemm_f32(type, dW, (const float *)g.tmp[0].p, (float *)g.tmp[1].p, n_rows, n_cols, n_tok,
+                            n_cols, n_rows, g.stream));
+    HIP_TRY(hipMemcpy2DAsync(Y, (size_t)out_stride * 4, g.tmp[1].p, (size_t)n_rows * 4, (size_t)n_rows * 4,
+                             (size_t)n_tok, hipMemcpyDeviceToHost, g.stream));
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_moe_ffn_token(float *out, const void *gate_exps, const void *up_exps, const void *down_exps,
+                       uint32_t type, int n_embd, int n_ff, int n_expert, int top_k,
+                       const float *router_logits, const float *x) {
+    if (int rc = check_linear_shape(type, n_ff, n_embd)) return rc;
+    if (int rc = check_linear_shape(type, n_embd, n_ff)) return rc;
+    if (n_expert <= 0 || top_k <= 0 || top_k > n_expert || top_k > 64 || n_expert > 8192)
+        return fail(QLIN_ERR_ARG, "bad expert counts (n_expert %d, top_k %d)", n_expert, top_k);
+    if (!out || !gate_exps || !up_exps || !down_exps || !router_logits || !x) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const size_t rb_in = row_size(type, n_embd), rb_dn = row_size(type, n_ff);
+    const size_t bytes_in = rb_in * (size_t)n_ff * n_expert, bytes_dn = rb_dn * (size_t)n_embd * n_expert;
+    const void *dG, *dU, *dD;
+    if (int rc = weights_on_device_locked(gate_exps, bytes_in, g.w[0], &dG)) return rc;
+    if (int rc = weights_on_device_locked(up_exps, bytes_in, g.w[1], &dU)) return rc;
+    if (int rc = weights_on_device_locked(down_exps, bytes_dn, g.w[2], &dD)) return rc;
+    /* tmp[0]: logits | idx | w ; tmp[1]: gate ; tmp[2]: up ; tmp[3]: down out ; y[0]: accumulated out */
+    const size_t off_idx = ((size_t)n_expert * 4 + 255) & ~(size_t)255;
+    const size_t off_w = off_idx + 256;
+    if (int rc = g.tmp[0].ensure(off_w + 256)) return rc;
+    if (int rc = g.tmp[1].ensure((size_t)n_ff * 4)) return rc;
+    if (int rc = g.tmp[2].ensure((size_t)n_ff * 4)) return rc;
+    if (int rc = g.tmp[3].ensure((size_t)n_embd * 4)) return rc;
+    if (int rc = g.y[0].ensure((size_t)n_embd * 4)) return rc;
+    if (int rc = g.x.ensure((size_t)n_embd * 4)) return rc;
+    uint8_t *t0 = (uint8_t *)g.tmp[0].p;
+    int32_t *d_idx = (int32_t *)(t0 + off_idx);
+    float *d_w = (float *)(t0 + off_w);
+    HIP_TRY(hipMemcpyAsync(t0, router_logits, (size_t)n_expert * 4, hipMemcpyHostToDevice, g.stream));
+    HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_embd * 4, hipMemcpyHostToDevice, g.stream));
+    HIP_TRY(launch_moe_route((const float *)t0, 1, n_expert, top_k, d_idx, d_w, g.stream));
+    int32_t h_idx[64];
+    HIP_TRY(hipMemcpyAsync(h_idx, d_idx, (size_t)top_k * 4, hipMemcpyDeviceToHost, g.stream));
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    for (int k = 0; k < top_k; k++) {
+        const int e = h_idx[k];
+        if (e < 0 || e >= n_expert) return fail(QLIN_ERR_DEVICE, "router produced expert %d", e);
+        const uint8_t *ge = (const uint8_t *)dG + (size_t)e * n_ff * rb_in;
+        const uint8_t *ue = (const uint8_t *)dU + (size_t)e * n_ff * rb_in;
+        const uint8_t *de = (const uint8_t *)dD + (size_t)e * n_embd * rb_dn;
+        HIP_TRY(dispatch_gemv(type, ge, (const float *)g.x.p, (float *)g.tmp[1].p, n_ff, n_embd, g.stream));
+        HIP_TRY(dispatch_gemv(type, ue, (const float *)g.x.p, (float *)g.tmp[2].p, n_ff, n_embd, g.stream));
+        HIP_TRY(launch_silu_mul((float *)g.tmp[1].p, (const float *)g.tmp[1].p, (const float *)g.tmp[2].p, n_ff, g.stream));
+        HIP_TRY(dispatch_gemv(type, de, (const float *)g.tmp[1].p, (float *)g.tmp[3].p, n_embd, n_ff, g.stream));
+        HIP_TRY(launch_axpy_dev_weight((float *)g.y[0].p, (const float *)g.tmp[3].p, d_w, k, n_embd, k == 0, g.stream));
+    }
+    HIP_TRY(hipMemcpyAsync(out, g.y[0].p, (size_t)n_embd * 4, hipMemcpyDeviceToHost, g.stream));
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+/* ------------------------------------------------------------------ device-resident */
+
+void *qlin_dev_alloc(size_t n_bytes) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (ensure_init_locked(0)) return nullptr;
+    void *p = nullptr;
+    if (hipMalloc(&p, n_bytes ? n_bytes : 1) != hipSuccess) {
+        fail(QLIN_ERR_NOMEM, "hipMalloc of %zu bytes failed", n_bytes);
+        return nullptr;
+    }
+    return p;
+}
+
+void qlin_dev_free(void *p) {
+    if (p) (void)hipFree(p);
+}
+
+int qlin_dev_upload(void *dst_dev, const void *src_host, size_t n_bytes) {
+    if (n_bytes == 0) return QLIN_OK;
+    if (!dst_dev || !src_host) return fail(QLIN_ERR_ARG, "null pointer");
+    HIP_TRY(hipMemcpy(dst_dev, src_host, n_bytes, hipMemcpyHostToDevice));
+    return QLIN_OK;
+}
+
+int qlin_dev_download(void *dst_host, const void *src_dev, size_t n_bytes) {
+    if (n_bytes == 0) return QLIN_OK;
+    if (!dst_host || !src_dev) return fail(QLIN_ERR_ARG, "null pointer");
+    HIP_TRY(hipMemcpy(dst_host, src_dev, n_bytes, hipMemcpyDeviceToHost));
+    return QLIN_OK;
+}
+
+int qlin_dev_sync(void *stream) {
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_dequant_dev(uint32_t type, const void *W, float *out, int n_rows, int n_cols, void *stream) {
+    if (!known_type(type)) return fail(QLIN_ERR_TYPE, "unsupported type %u", type);
+    if (n_rows < 0 || n_cols < 0) return fail(QLIN_ERR_ARG, "negative size");
+    if (n_rows == 0 || n_cols == 0) return QLIN_OK;
+    if (!W || !out) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 2) || !aligned(out, 4)) return fail(QLIN_ERR_ARG, "W needs 2-byte, out 4-byte alignment");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(launch_dequant(type, W, out, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_gemv_dev(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, void *stream) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!W || !x || !y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 2) || !aligned(x, 16) || !aligned(y, 4))
+        return fail(QLIN_ERR_ARG, "W needs 2-byte, x 16-byte, y 4-byte alignment");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(dispatch_gemv(type, W, x, y, n_rows, n_cols, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_gemm_f32_dev(uint32_t type, const void *W, const float *X, float *Y, int n_rows, int n_cols,
+                      int n_tok, int ldx, int ldy, void *stream) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_tok < 0 || ldx < n_cols || ldy < n_rows) return fail(QLIN_ERR_ARG, "bad token count or leading dimension");
+    if (n_rows == 0 || n_tok == 0) return QLIN_OK;
+    if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 2) || !aligned(X, 4) || !aligned(Y, 4)) return fail(QLIN_ERR_ARG, "misaligned pointer");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(launch_gemm_f32(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_gemm_bf16_dev(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                       int n_tok, int ldx, int ldy, void *stream) {
+    if (type != T_Q4_K) return fail(QLIN_ERR_TYPE, "bf16 matrix-core GEMM takes Q4_K weights only (got %u)", type);
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_tok < 0 || ldx < n_cols || ldy < n_rows) return fail(QLIN_ERR_ARG, "bad token count or leading dimension");
+    if (n_rows == 0 || n_tok == 0) return QLIN_OK;
+    if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 16) || ldx % 8 || ldy % 4)
+        return fail(QLIN_ERR_ARG, "W, X, Y need 16-byte alignment, ldx %% 8 == 0, ldy %% 4 == 0");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(launch_gemm_q4k_bf16(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_moe_route_dev(const float *router_logits, int n_tok, int n_expert, int top_k, int32_t *expert_idx,
+                       float *expert_w, void *stream) {
+    if (n_tok < 0 || n_expert <= 0 || top_k <= 0 || top_k > n_expert || n_expert > 8192)
+        return fail(QLIN_ERR_ARG, "bad routing shape");
+    if (n_tok == 0) return QLIN_OK;
+    if (!router_logits || !expert_idx || !expert_w) return fail(QLIN_ERR_ARG, "null pointer");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(launch_moe_route(router_logits, n_tok, n_expert, top_k, expert_idx, expert_w, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
+    return moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert);
+}
+
+int qlin_moe_ffn_dev(uint32_t type, const void *gate_exps, const void *up_exps, const void *down_exps,
+                     const uint16_t *X, const int32_t *expert_idx, const float *expert_w, float *out,
+                     int n_tok, int top_k, int n_embd, int n_ff, int n_expert, void *workspace, void *stream) {
+    if (type != T_Q4_K) return fail(QLIN_ERR_TYPE, "grouped MoE FFN takes Q4_K experts only (got %u)", type);
+    if (int rc = check_linear_shape(type, n_ff, n_embd)) return rc;
+    if (int rc = check_linear_shape(type, n_embd, n_ff)) return rc;
+    if (n_tok < 0 || n_expert <= 0 || top_k <= 0 || top_k > n_expert) return fail(QLIN_ERR_ARG, "bad MoE shape");
+    if (n_tok == 0) return QLIN_OK;
+    if (!gate_exps || !up_exps || !down_exps || !X || !expert_idx || !expert_w || !out || !workspace)
+        return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(gate_exps, 16) || !aligned(up_exps, 16) || !aligned(down_exps, 16) || !aligned(X, 16) ||
+        !aligned(out, 16) || !aligned(workspace, 256))
+        return fail(QLIN_ERR_ARG, "misaligned pointer (16 bytes; workspace 256)");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(launch_moe_ffn_q4k(gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out, n_tok, top_k,
+                               n_embd, n_ff, n_expert, workspace, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_timer_begin(void *stream) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    HIP_TRY(hipEventRecord(g.ev0, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_timer_end(void *stream, float *ms) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (!g.ready) return fail(QLIN_ERR_ARG, "qlin_timer_begin was not called");
+    if (!ms) return fail(QLIN_ERR_ARG, "null pointer");
+    HIP_TRY(hipEventRecord(g.ev1, (hipStream_t)stream));
+    HIP_TRY(hipEventSynchronize(g.ev1));
+    HIP_TRY(hipEventElapsedTime(ms, g.ev0, g.ev1));
+    return QLIN_OK;
+}
+
+}  // extern "C"

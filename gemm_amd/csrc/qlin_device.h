@@ -1,0 +1,223 @@
+/*
+ * qlin_device.h - device-side view of the GGML block formats (gfx950).
+ *
+ * Byte layouts follow the packed block structs of common/ggml_dequant.h:30-204. Blocks are
+ * addressed as raw bytes: inside a row only 2-byte alignment holds (block sizes 34, 210, 66,
+ * 110 and 18 are not multiples of 4), so multi-byte fields are assembled from 16-bit loads.
+ */
+#ifndef QLIN_DEVICE_H
+#define QLIN_DEVICE_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "qlin_codebooks.h"
+
+namespace qlin {
+
+enum : uint32_t {
+    T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14,
+    T_IQ2_XXS = 16, T_IQ4_NL = 20, T_IQ3_S = 21, T_BF16 = 30
+};
+
+/* elements and bytes per block (common/ggml_dequant.h:261-294) */
+template <uint32_t T> struct Geom;
+template <> struct Geom<T_Q8_0>    { static constexpr int BE = 32,  BB = 34;  };
+template <> struct Geom<T_Q4_K>    { static constexpr int BE = 256, BB = 144; };
+template <> struct Geom<T_Q5_K>    { static constexpr int BE = 256, BB = 176; };
+template <> struct Geom<T_Q6_K>    { static constexpr int BE = 256, BB = 210; };
+template <> struct Geom<T_IQ2_XXS> { static constexpr int BE = 256, BB = 66;  };
+template <> struct Geom<T_IQ4_NL>  { static constexpr int BE = 32,  BB = 18;  };
+template <> struct Geom<T_IQ3_S>   { static constexpr int BE = 256, BB = 110; };
+
+__host__ __device__ inline bool type_geometry(uint32_t t, int *be, int *bb) {
+    switch (t) {
+    case T_F32: *be = 1; *bb = 4; return true;
+    case T_F16: case T_BF16: *be = 1; *bb = 2; return true;
+    case T_Q8_0: *be = 32; *bb = 34; return true;
+    case T_Q4_K: *be = 256; *bb = 144; return true;
+    case T_Q5_K: *be = 256; *bb = 176; return true;
+    case T_Q6_K: *be = 256; *bb = 210; return true;
+    case T_IQ2_XXS: *be = 256; *bb = 66; return true;
+    case T_IQ4_NL: *be = 32; *bb = 18; return true;
+    case T_IQ3_S: *be = 256; *bb = 110; return true;
+    default: return false;
+    }
+}
+
+__device__ __forceinline__ uint32_t ld_u16(const uint8_t *p) {
+    return *reinterpret_cast<const uint16_t *>(p);
+}
+__device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) { /* 2-byte aligned dword */
+    return ld_u16(p) | (ld_u16(p + 2) << 16);
+}
+
+/* IEEE half -> float, bit-exact for every input like common/ggml_dequant.h:206-229: NaN
+ * payloads pass through unquieted, subnormals become m * 2^-24 (exact, and a normal float,
+ * so the result does not depend on the denormal mode). */
+__device__ __forceinline__ float half_bits_exact(uint32_t h) {
+    const uint32_t sign = (h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 31u;
+    const uint32_t m = h & 1023u;
+    uint32_t bits;
+    if (e == 31u) bits = sign | 0x7F800000u | (m << 13);
+    else if (e != 0u) bits = sign | ((e + 112u) << 23) | (m << 13);
+    else bits = sign | __float_as_uint((float)m * 0x1p-24f);
+    return __uint_as_float(bits);
+}
+
+/* hardware conversion: exact for finite inputs, may quiet a signalling NaN */
+__device__ __forceinline__ float half_bits_fast(uint32_t h) {
+    union { unsigned short u; _Float16 f; } v;
+    v.u = (unsigned short)h;
+    return (float)v.f;
+}
+
+/* sign byte of the 2/3-bit i-quants: 7 stored bits + their parity in bit 7
+ * (table at common/ggml_dequant.h:1765-1774) */
+__device__ __forceinline__ uint32_t iq_sign_byte(uint32_t i7) {
+    return i7 | ((__popc(i7) & 1u) << 7);
+}
+
+/* 6-bit scale and min of sub-block g from the 12 packed bytes of a Q4_K/Q5_K super-block
+ * (get_scale_min_k4, common/ggml_dequant.h:1582-1590) */
+__device__ __forceinline__ void k4_scale_min(const uint8_t *s, int g, uint32_t &sc, uint32_t &mn) {
+    if (g < 4) {
+        sc = s[g] & 63u;
+        mn = s[g + 4] & 63u;
+    } else {
+        sc = (s[g + 4] & 15u) | ((uint32_t)(s[g - 4] >> 6) << 4);
+        mn = ((uint32_t)s[g + 4] >> 4) | ((uint32_t)(s[g] >> 6) << 4);
+    }
+}
+
+/*
+ * decode8<T>(blk, k0, y): elements k0..k0+7 (k0 a multiple of 8) of one block, with exactly
+ * the reference's fp32 operation order, so that results are bit-identical:
+ *   Q8_0     d*q                               common/ggml_dequant.h:1479-1489
+ *   Q4_K/5_K (d*sc)*q - (dmin*m)               :1592-1651   (d*sc, dmin*m, (d*sc)*q are exact
+ *                                              in fp32, so a fused multiply-subtract rounds the
+ *                                              same way as the separate multiply and subtract)
+ *   Q6_K     (d*sc)*q                          :1653-1687
+ *   IQ4_NL   d*codebook[nibble]                :2942-2954
+ *   IQ2_XXS  ((d*(0.5+s))*0.25)*grid*(+-1)     :2793-2816
+ *   IQ3_S    (d*(1+2s))*grid*(+-1)             :3022-3058
+ */
+template <uint32_t T> struct Codec;
+
+template <> struct Codec<T_Q8_0> : Geom<T_Q8_0> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk));
+        const int8_t *q = reinterpret_cast<const int8_t *>(blk + 2 + k0);
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = d * (float)q[i];
+    }
+};
+
+template <> struct Codec<T_Q4_K> : Geom<T_Q4_K> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk));
+        const float dmin = half_bits_exact(ld_u16(blk + 2));
+        const int g = k0 >> 5, l0 = k0 & 31;
+        uint32_t sc, mn;
+        k4_scale_min(blk + 4, g, sc, mn);
+        const float dl = d * (float)sc, ml = dmin * (float)mn;
+        const uint8_t *q = blk + 16 + (g >> 1) * 32 + l0;
+        const int sh = (g & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = dl * (float)((q[i] >> sh) & 15) - ml;
+    }
+};
+
+template <> struct Codec<T_Q5_K> : Geom<T_Q5_K> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk));
+        const float dmin = half_bits_exact(ld_u16(blk + 2));
+        const int g = k0 >> 5, l0 = k0 & 31;
+        uint32_t sc, mn;
+        k4_scale_min(blk + 4, g, sc, mn);
+        const float dl = d * (float)sc, ml = dmin * (float)mn;
+        const uint8_t *qh = blk + 16 + l0;
+        const uint8_t *q = blk + 48 + (g >> 1) * 32 + l0;
+        const int sh = (g & 1) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int v = ((q[i] >> sh) & 15) + (((qh[i] >> g) & 1) << 4);
+            y[i] = dl * (float)v - ml;
+        }
+    }
+};
+
+template <> struct Codec<T_Q6_K> : Geom<T_Q6_K> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk + 208));
+        const int half = k0 >> 7, r = k0 & 127, seg = r >> 5, l0 = r & 31;
+        const uint8_t *ql = blk + 64 * half + 32 * (seg & 1) + l0;
+        const uint8_t *qh = blk + 128 + 32 * half + l0;
+        const int8_t sc = reinterpret_cast<const int8_t *>(blk + 192)[8 * half + 2 * seg + (l0 >> 4)];
+        const float dl = d * (float)sc;
+        const int nsh = (seg >> 1) * 4, hsh = 2 * seg;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int q = (((ql[i] >> nsh) & 15) | (((qh[i] >> hsh) & 3) << 4)) - 32;
+            y[i] = dl * (float)q;
+        }
+    }
+};
+
+template <> struct Codec<T_IQ4_NL> : Geom<T_IQ4_NL> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk));
+        const uint8_t *q = blk + 2 + (k0 & 15);
+        const int sh = (k0 >> 4) * 4;
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = d * (float)qlin_iq4nl_values[(q[i] >> sh) & 15];
+    }
+};
+
+template <> struct Codec<T_IQ2_XXS> : Geom<T_IQ2_XXS> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk));
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint32_t a0 = ld_u32_a2(blk + 2 + 8 * g), a1 = ld_u32_a2(blk + 6 + 8 * g);
+        const float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
+        const uint64_t cell = qlin_iq2xxs_grid[(a0 >> (8 * l)) & 255u];
+        const uint32_t sg = iq_sign_byte((a1 >> (7 * l)) & 127u);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float mag = db * (float)(uint32_t)((cell >> (8 * i)) & 255u);
+            y[i] = mag * (((sg >> i) & 1u) ? -1.0f : 1.0f);
+        }
+    }
+};
+
+template <> struct Codec<T_IQ3_S> : Geom<T_IQ3_S> {
+    __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
+        const float d = half_bits_exact(ld_u16(blk));
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint32_t nib = (blk[106 + (g >> 1)] >> (4 * (g & 1))) & 15u;
+        const float db = d * (float)(1u + 2u * nib);
+        const uint32_t qh = blk[66 + g];
+        const uint32_t i0 = blk[2 + 8 * g + 2 * l] | (((qh >> (2 * l)) & 1u) << 8);
+        const uint32_t i1 = blk[2 + 8 * g + 2 * l + 1] | (((qh >> (2 * l + 1)) & 1u) << 8);
+        const uint32_t c0 = qlin_iq3s_grid[i0], c1 = qlin_iq3s_grid[i1];
+        const uint32_t sb = blk[74 + 4 * g + l];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float m0 = db * (float)((c0 >> (8 * i)) & 255u);
+            const float m1 = db * (float)((c1 >> (8 * i)) & 255u);
+            y[i] = m0 * (((sb >> i) & 1u) ? -1.0f : 1.0f);
+            y[i + 4] = m1 * (((sb >> (i + 4)) & 1u) ? -1.0f : 1.0f);
+        }
+    }
+};
+
+/* wave64 sum: every lane ends up with the total */
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+}  // namespace qlin
+#endif /* QLIN_DEVICE_H */

@@ -1,0 +1,50 @@
+/*
+ * qlin_internal.h - host-side launchers shared between the translation units of libqlinear.
+ * Every launcher validates nothing: the C-ABI layer (qlin_api.hip) checks shapes, alignment
+ * and types before it calls in here. All return the hipError_t of the launch.
+ */
+#ifndef QLIN_INTERNAL_H
+#define QLIN_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace qlin {
+
+/* out[n_rows, n_cols] = decode(W); n_cols may be ragged: only n_cols / block_elems blocks per
+ * row are decoded, row r of W starts at r * row_bytes, row r of out at r * n_cols. */
+hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, int n_cols,
+                          size_t row_bytes, hipStream_t stream);
+
+/* y[n_rows] = W . x, any supported type and any whole-block shape */
+hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, float *y, int n_rows,
+                               int n_cols, hipStream_t stream);
+/* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned.
+ * rows_per_pass in {1,2,4,7,8}; target_waves_per_cu sets how many rows one wave streams. */
+hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, int n_cols,
+                           hipStream_t stream, int n_cu, int rows_per_pass, int target_waves_per_cu);
+
+/* Y[t*ldy + r] = dot(W[r,:], X[t*ldx..]) in fp32 */
+hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *Y, int n_rows,
+                           int n_cols, int n_tok, int ldx, int ldy, hipStream_t stream);
+
+/* Q4_K x bf16 on the matrix cores */
+hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                                int n_tok, int ldx, int ldy, hipStream_t stream);
+
+/* grouped MoE expert FFN on the matrix cores (Q4_K experts, bf16 activations) */
+size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
+hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down, const uint16_t *X,
+                              const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
+                              int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream);
+
+/* MoE pieces */
+hipError_t launch_moe_route(const float *logits, int n_tok, int n_expert, int top_k, int32_t *idx,
+                            float *w, hipStream_t stream);
+hipError_t launch_silu_mul(float *h, const float *gate, const float *up, int n, hipStream_t stream);
+hipError_t launch_axpy_dev_weight(float *out, const float *q, const float *w, int widx, int n,
+                                  int overwrite, hipStream_t stream);
+
+}  // namespace qlin
+#endif

@@ -1,0 +1,200 @@
+"""ctypes binding of libqlinear.so (the C ABI declared in include/qlinear.h).
+
+The library is the product; this module only marshals numpy arrays and device pointers into
+it. There is no fallback: if the shared library is missing or no GPU is usable, calls raise.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libqlinear.so")
+
+OK, ERR_TYPE, ERR_ARG, ERR_DEVICE, ERR_NOMEM = 0, -1, -2, -3, -4
+
+_vp, _fp, _ip, _u16p = C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_int32), C.POINTER(C.c_uint16)
+
+# name -> (restype, argtypes); every symbol include/qlinear.h declares
+SIGNATURES = {
+    "qlin_init": (C.c_int, [C.c_int]),
+    "qlin_shutdown": (None, []),
+    "qlin_last_error": (C.c_char_p, []),
+    "qlin_device_info": (C.c_int, [C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_size_t)]),
+    "qlin_dequant_row_size": (C.c_size_t, [C.c_uint32, C.c_int]),
+    "qlin_dequant_row": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q8_0": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q4_K": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q5_K": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q6_K": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq2_xxs": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq3_s": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq4_nl": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequant_rows": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int]),
+    "qlin_weight_register": (C.c_int, [_vp, C.c_size_t]),
+    "qlin_weight_unregister": (C.c_int, [_vp]),
+    "qlin_weight_device_ptr": (_vp, [_vp]),
+    "qlin_matvec": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
+    "qlin_matvec_fused2": (C.c_int, [_vp, _vp, C.c_uint32, _vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
+    "qlin_matvec_qkv": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, _vp, C.c_uint32, _vp, _vp, C.c_uint32,
+                                  C.c_int, C.c_int, _vp]),
+    "qlin_matvec_expert": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, C.c_int, _vp, C.c_int]),
+    "qlin_gemm_tokenmajor": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "qlin_moe_ffn_token": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp]),
+    "qlin_dev_alloc": (_vp, [C.c_size_t]),
+    "qlin_dev_free": (None, [_vp]),
+    "qlin_dev_upload": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "qlin_dev_download": (C.c_int, [_vp, _vp, C.c_size_t]),
+    "qlin_dev_sync": (C.c_int, [_vp]),
+    "qlin_dequant_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "qlin_gemv_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "qlin_gemm_bf16_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp]),
+    "qlin_gemm_f32_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp]),
+    "qlin_moe_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "qlin_moe_route_dev": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, _vp, _vp, _vp]),
+    "qlin_moe_ffn_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int,
+                                   C.c_int, C.c_int, _vp, _vp]),
+    "qlin_timer_begin": (C.c_int, [_vp]),
+    "qlin_timer_end": (C.c_int, [_vp, _fp]),
+}
+
+_lib = None
+
+
+class QlinError(RuntimeError):
+    def __init__(self, code, text):
+        super().__init__("qlinear error %d: %s" % (code, text))
+        self.code = code
+
+
+def load():
+    """dlopen libqlinear.so and declare every entry point. Raises if the library is absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(LIB_PATH + " is missing: run `python -m gemm_amd.build` (there is no fallback)")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def check(rc):
+    if rc != OK:
+        raise QlinError(rc, load().qlin_last_error().decode(errors="replace"))
+
+
+def _ptr(a):
+    return a.ctypes.data_as(_vp)
+
+
+def device_info():
+    lib = load()
+    name = C.create_string_buffer(256)
+    cu, mem = C.c_int(0), C.c_size_t(0)
+    check(lib.qlin_device_info(name, 256, C.byref(cu), C.byref(mem)))
+    return name.value.decode(), cu.value, mem.value
+
+
+class DevBuf:
+    """A device allocation owned through the library (hipMalloc / hipFree)."""
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        self.ptr = load().qlin_dev_alloc(max(self.nbytes, 1))
+        if not self.ptr:
+            raise QlinError(ERR_NOMEM, load().qlin_last_error().decode())
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        if a.nbytes:
+            check(load().qlin_dev_upload(b.ptr, _ptr(a), a.nbytes))
+        return b
+
+    def to_numpy(self, dtype, shape):
+        out = np.empty(shape, dtype=dtype)
+        assert out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(load().qlin_dev_download(_ptr(out), self.ptr, out.nbytes))
+        return out
+
+    def free(self):
+        if self.ptr:
+            load().qlin_dev_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+# ---------------------------------------------------------------- host-pointer calls (numpy in, numpy out)
+
+def dequant_row(type_id, src, n, dst=None):
+    src = np.ascontiguousarray(src, np.uint8)
+    if dst is None:
+        dst = np.zeros(n, np.float32)
+    rc = load().qlin_dequant_row(type_id, _ptr(src), _ptr(dst), n)
+    return rc, dst
+
+
+def dequant_rows(type_id, src, n_rows, n_cols):
+    src = np.ascontiguousarray(src, np.uint8)
+    dst = np.zeros((n_rows, n_cols), np.float32)
+    check(load().qlin_dequant_rows(type_id, _ptr(src), _ptr(dst), n_rows, n_cols))
+    return dst
+
+
+def matvec(type_id, W, x, n_cols):
+    W = np.ascontiguousarray(W, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.zeros(W.shape[0], np.float32)
+    check(load().qlin_matvec(_ptr(y), _ptr(W), type_id, n_cols, _ptr(x), W.shape[0]))
+    return y
+
+
+def gemm_tokenmajor(type_id, W, X, n_cols):
+    W = np.ascontiguousarray(W, np.uint8)
+    X = np.ascontiguousarray(X, np.float32)
+    Y = np.zeros((X.shape[0], W.shape[0]), np.float32)
+    check(load().qlin_gemm_tokenmajor(_ptr(Y), _ptr(W), type_id, n_cols, _ptr(X), W.shape[0], X.shape[0],
+                                      W.shape[0], X.shape[1]))
+    return Y
+
+
+# ---------------------------------------------------------------- device-resident calls
+
+def gemv_dev(type_id, dW, dx, dy, n_rows, n_cols, stream=None):
+    check(load().qlin_gemv_dev(type_id, dW.ptr, dx.ptr, dy.ptr, n_rows, n_cols, stream))
+
+
+def dequant_dev(type_id, dW, dout, n_rows, n_cols, stream=None):
+    check(load().qlin_dequant_dev(type_id, dW.ptr, dout.ptr, n_rows, n_cols, stream))
+
+
+def gemm_bf16_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, stream=None):
+    check(load().qlin_gemm_bf16_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy, stream))
+
+
+def gemm_f32_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, stream=None):
+    check(load().qlin_gemm_f32_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy, stream))
+
+
+def sync(stream=None):
+    check(load().qlin_dev_sync(stream))
+
+
+def timer_begin(stream=None):
+    check(load().qlin_timer_begin(stream))
+
+
+def timer_end(stream=None):
+    ms = C.c_float(0)
+    check(load().qlin_timer_end(stream, C.byref(ms)))
+    return ms.value

@@ -1,0 +1,160 @@
+/*
+ * qlinear.h - C ABI of the MI355X (gfx950) quantized-linear engine.
+ *
+ * GGML block dequantization and quantized matvec / matmul / MoE expert FFN on one GPU, behind
+ * plain-C entry points (pointers and sizes only). The first two groups below have the shapes
+ * of the reference's own C functions so that a C engine built like common/transformer.h can
+ * call them where it calls its CPU path today; the third group works on device-resident
+ * buffers (no copies per call) for engines that keep activations on the GPU.
+ *
+ * Supported ggml types (ids are enum ggml_dtype, common/gguf_loader.h:45-85):
+ *   Q8_0 = 8, Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16, IQ4_NL = 20, IQ3_S = 21,
+ *   and F32 = 0 / F16 = 1 / BF16 = 30 in the codec group only.
+ *
+ * Every function returns a status (0 = ok, negative = error) unless it mirrors a `void`
+ * reference function, in which case it reports on stderr and zero-fills its output the way
+ * the reference does for an unsupported type (common/transformer.h:451-454, :520-523).
+ * There is no CPU fallback anywhere: without a usable GPU every call fails with
+ * QLIN_ERR_DEVICE.
+ *
+ * Threading: all entry points are serialised on one internal mutex; host-pointer calls run on
+ * the library's own stream and return after the result is in host memory. Device-resident
+ * calls are asynchronous on the stream they are given.
+ */
+#ifndef QLINEAR_H
+#define QLINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define QLIN_OK            0
+#define QLIN_ERR_TYPE     (-1) /* unsupported ggml type; same value dequant_row returns */
+#define QLIN_ERR_ARG      (-2) /* null pointer, negative size, shape the kernels cannot take */
+#define QLIN_ERR_DEVICE   (-3) /* no GPU / HIP failure; text in qlin_last_error() */
+#define QLIN_ERR_NOMEM    (-4)
+
+enum qlin_type {
+    QLIN_TYPE_F32 = 0, QLIN_TYPE_F16 = 1, QLIN_TYPE_Q8_0 = 8, QLIN_TYPE_Q4_K = 12,
+    QLIN_TYPE_Q5_K = 13, QLIN_TYPE_Q6_K = 14, QLIN_TYPE_IQ2_XXS = 16, QLIN_TYPE_IQ4_NL = 20,
+    QLIN_TYPE_IQ3_S = 21, QLIN_TYPE_BF16 = 30
+};
+
+/* ------------------------------------------------------------------ lifecycle */
+
+/* Select the GPU, create the library stream, upload the codebooks. Idempotent. Called
+ * implicitly (device 0) by the first entry point that needs the GPU.
+ * Stands where transformer_load sets a model up (common/transformer.h:225). */
+int  qlin_init(int device);
+void qlin_shutdown(void);
+/* Text of the most recent error on this thread's last failing call ("" if none). */
+const char *qlin_last_error(void);
+/* Device name (truncated to cap-1 chars), compute units, total memory in bytes. */
+int  qlin_device_info(char *name, size_t cap, int *compute_units, size_t *mem_bytes);
+
+/* ------------------------------------------------------------------ codec (host pointers)
+ * Same signatures and meaning as common/ggml_dequant.h:231-294: n = element count, whole
+ * blocks are decoded (n / block_elems of them), a ragged tail is left untouched; src needs
+ * 2-byte alignment at most. Decoding runs on the GPU; results are bit-identical to the
+ * reference's scalar decoders. */
+size_t qlin_dequant_row_size(uint32_t ggml_type, int n);               /* :261-294, 0 if unknown */
+int    qlin_dequant_row(uint32_t ggml_type, const void *src, float *dst, int n); /* :258, :3177 */
+void   qlin_dequantize_row_q8_0(const void *src, float *dst, int n);    /* :233, :1479 */
+void   qlin_dequantize_row_q4_K(const void *src, float *dst, int n);    /* :237, :1592 */
+void   qlin_dequantize_row_q5_K(const void *src, float *dst, int n);    /* :238, :1620 */
+void   qlin_dequantize_row_q6_K(const void *src, float *dst, int n);    /* :239, :1653 */
+void   qlin_dequantize_row_iq2_xxs(const void *src, float *dst, int n); /* :240, :2793 */
+void   qlin_dequantize_row_iq3_s(const void *src, float *dst, int n);   /* :248, :3022 */
+void   qlin_dequantize_row_iq4_nl(const void *src, float *dst, int n);  /* :249, :2942 */
+/* Many rows at once: src holds n_rows rows of qlin_dequant_row_size(type, n_cols) bytes,
+ * dst is [n_rows, n_cols] fp32. Shape of the per-row loop in tf_dequant_row callers
+ * (common/transformer.h:425-460). */
+int    qlin_dequant_rows(uint32_t ggml_type, const void *src, float *dst, int n_rows, int n_cols);
+
+/* ------------------------------------------------------------------ weights
+ * The reference's tensors are borrowed pointers into the GGUF mapping, immutable for the
+ * life of the model (tf_load_tensor, common/transformer.h:363-381). Registering such a
+ * pointer uploads its bytes to HBM once; later host-pointer calls that name the same pointer
+ * (or a pointer inside the registered range, e.g. an expert slice) use the device copy.
+ * Calls with an unregistered pointer still work: the bytes are staged for that call only. */
+int  qlin_weight_register(const void *host_data, size_t n_bytes);
+int  qlin_weight_unregister(const void *host_data);
+/* Device address that mirrors host_ptr, or NULL if host_ptr is in no registered range. */
+const void *qlin_weight_device_ptr(const void *host_ptr);
+
+/* ------------------------------------------------------------------ linear (host pointers)
+ * W: raw ggml blocks, n_rows rows of n_cols elements; x, dst: host fp32. */
+
+/* dst[n_rows] = W . x        tf_qmatvec / tf_qmatvec_pool, common/transformer.h:1049, :1117 */
+int qlin_matvec(float *dst, const void *W, uint32_t ggml_type, int n_cols, const float *x, int n_rows);
+/* two matrices, one x        tf_qmatvec_fused2_pool, common/transformer.h:897 */
+int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2, const void *W2,
+                       uint32_t type2, int n_cols, const float *x, int n_rows);
+/* Q/K/V in one call, each with its own type; K and V share n_kv
+ *                            tf_qmatvec_fused_qkv_pool, common/transformer.h:1021 */
+int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k, const void *Wk,
+                    uint32_t type_k, float *v, const void *Wv, uint32_t type_v, int n_kv,
+                    int n_cols, const float *x);
+/* one expert of a [n_cols, rows_per_expert, n_expert] tensor: rows start at
+ * W + expert * rows_per_expert * row_bytes
+ *                            tf_qmatvec_expert(_pool), common/transformer.h:517, :1136 */
+int qlin_matvec_expert(float *dst, const void *W, uint32_t ggml_type, int n_cols, int expert,
+                       const float *x, int rows_per_expert);
+/* prefill: Y[t*out_stride + r] = dot(W[r,:], X[t*x_stride ...]), r < n_rows, t < n_tok; X fp32.
+ * Computed in fp32 (no bf16 rounding) so that it can stand in for the CPU path exactly.
+ *                            tf_gemm_f16_mt_tokenmajor, common/transformer.h:4487 */
+int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t ggml_type, int n_cols, const float *X,
+                         int n_rows, int n_tok, int out_stride, int x_stride);
+/* one token of the MoE FFN block (common/transformer.h:4045-4131) without the router matvec:
+ * logits[n_expert] -> softmax -> top_k -> renormalise -> sum_k w_k down_k(silu(gate_k x)*up_k x).
+ * out[n_embd] is overwritten (the caller adds it to the residual, :4130). */
+int qlin_moe_ffn_token(float *out, const void *gate_exps, const void *up_exps, const void *down_exps,
+                       uint32_t ggml_type, int n_embd, int n_ff_expert, int n_expert, int top_k,
+                       const float *router_logits, const float *x);
+
+/* ------------------------------------------------------------------ device-resident
+ * All pointers are device addresses; `stream` is a hipStream_t passed as void* (NULL = the
+ * null stream). Calls only enqueue work. No counterpart in the reference's CPU API; the
+ * arithmetic is the same as the group above. */
+void *qlin_dev_alloc(size_t n_bytes);
+void  qlin_dev_free(void *p);
+int   qlin_dev_upload(void *dst_dev, const void *src_host, size_t n_bytes);
+int   qlin_dev_download(void *dst_host, const void *src_dev, size_t n_bytes);
+int   qlin_dev_sync(void *stream);
+
+/* out[n_rows, n_cols] fp32 = decode(W); whole blocks only */
+int qlin_dequant_dev(uint32_t ggml_type, const void *W, float *out, int n_rows, int n_cols, void *stream);
+/* y[n_rows] = W . x, x fp32 */
+int qlin_gemv_dev(uint32_t ggml_type, const void *W, const float *x, float *y, int n_rows,
+                  int n_cols, void *stream);
+/* Y[t*ldy + r] = dot(W[r,:], X[t*ldx ...]); X bf16 (uint16 bit patterns), fp32 accumulate on
+ * the matrix cores, Y fp32 token-major. Q4_K only; n_cols % 256 == 0. */
+int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,
+                       int n_cols, int n_tok, int ldx, int ldy, void *stream);
+/* Same contraction in fp32 (X fp32, no rounding of weights or activations); any supported type. */
+int qlin_gemm_f32_dev(uint32_t ggml_type, const void *W, const float *X, float *Y, int n_rows,
+                      int n_cols, int n_tok, int ldx, int ldy, void *stream);
+/* Grouped MoE expert FFN over n_tok tokens:
+ *   X bf16 [n_tok, n_embd]; expert_idx int32 [n_tok, top_k]; expert_w fp32 [n_tok, top_k];
+ *   gate/up: [n_expert][n_ff][n_embd] blocks, down: [n_expert][n_embd][n_ff] blocks;
+ *   out fp32 [n_tok, n_embd] (overwritten). workspace: qlin_moe_workspace_bytes() bytes. */
+size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
+int qlin_moe_route_dev(const float *router_logits, int n_tok, int n_expert, int top_k,
+                       int32_t *expert_idx, float *expert_w, void *stream);
+int qlin_moe_ffn_dev(uint32_t ggml_type, const void *gate_exps, const void *up_exps,
+                     const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
+                     const float *expert_w, float *out, int n_tok, int top_k, int n_embd,
+                     int n_ff, int n_expert, void *workspace, void *stream);
+
+/* Elapsed milliseconds of work enqueued on `stream` between the two calls, by HIP events
+ * recorded on that stream (the role of elapsed_kernel_ms in rdna4/dequant/bench_dequant.c:764-780). */
+int qlin_timer_begin(void *stream);
+int qlin_timer_end(void *stream, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* QLINEAR_H */
