@@ -26,7 +26,14 @@ def test_matvec_shapes(oracle, tid, name, n_rows, n_cols):
     W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows * 7 + tid)
     x = synth.make_activation(n_cols, seed=n_cols + tid)
     y = qlinear.matvec(tid, W, x, n_cols)
-    assert rel_l2(y, oracle.gemv_f64(tid, W, x, n_cols)) <= TOL, (name, n_rows, n_cols)
+    want = oracle.gemv_f64(tid, W, x, n_cols)
+    if n_rows >= 13:
+        assert rel_l2(y, want) <= TOL, (name, n_rows, n_cols)
+    # a relative-L2 figure over one or a few outputs only measures cancellation in those dot
+    # products, so every output is also held to the fp32 dot-product error bound
+    # |err| <= 1e-6 * sum|w||x| (about 10 ulp of the un-cancelled magnitude)
+    bound = np.abs(oracle.dequant_matrix(tid, W, n_cols)).astype(np.float64) @ np.abs(x).astype(np.float64)
+    assert np.all(np.abs(y.astype(np.float64) - want) <= 1e-6 * bound + 1e-30), (name, n_rows, n_cols)
 
 
 @pytest.mark.parametrize("tid,name", NAMES)
