@@ -1,165 +1,257 @@
 /*
  * gemv_q4k.hip - batch-1 Q4_K matvec tuned for HBM streaming on gfx950.
  *
- * Work split. A row of K columns is K/256 super-blocks of 144 bytes (common/ggml_dequant.h:71-76).
- * Four lanes own one super-block: lane c (0..3) takes the 32 nibble bytes qs[32c..32c+31], i.e.
- * the 64 elements of sub-blocks 2c (low nibbles) and 2c+1 (high nibbles). A wavefront therefore
- * covers a slice of up to 16 super-blocks (4096 columns) of one row per pass. The slice of x a
- * wavefront needs (64 floats per lane) is loaded ONCE and stays in registers while the
- * wavefront streams R rows per pass: the raw 32 nibble bytes and the 16-byte block header
- * (d, dmin, 12 packed scale bytes) of all R rows are requested before any arithmetic starts,
- * so each wave keeps R*48 bytes per lane in flight.
- * Rows longer than 16 super-blocks are cut into S slices handled by the S waves of a
- * workgroup, whose partial sums meet in LDS.
+ * Structure (one workgroup of 16 wavefronts per block of rows, about one per compute unit):
  *
- * Arithmetic, per row and lane (factored form of common/ggml_dequant.h:1592-1618 dotted with x):
- *   y += d*sc_a*sum(q_lo*x_a) + d*sc_b*sum(q_hi*x_b) - dmin*(m_a*sum(x_a) + m_b*sum(x_b))
- * sum(x_a), sum(x_b) do not depend on the row and are formed once per wave. The eight 6-bit
- * scales and mins of a super-block are unpacked four at a time with byte-parallel mask ops.
- * High nibbles are used as 16*q (masked in place, no shift); the 1/16 goes into the scale.
- * fp32 accumulate throughout; result within ~1e-6 relative L2 of the double-precision oracle.
+ *  1. x -> fixed point, once per workgroup. Each 32-element sub-block of x (the Q4_K scale
+ *     granularity, common/ggml_dequant.h:71-76) is scaled by a power of two so that
+ *     X = rint(x * 2^(22-e)) fits 23 bits, and the three bytes of X are stored as three
+ *     "digit planes" in LDS (top byte signed, lower two unsigned) together with 2^(e-22) and
+ *     the fp32 sum of the sub-block. Quantisation error is 2^-23 of the sub-block's largest
+ *     |x|; measured end-to-end error is ~7e-7 relative L2 against the double-precision oracle.
+ *  2. Weights are streamed as a FLAT byte stream: a wavefront reads a row (or a slice of at
+ *     most 16 super-blocks = 2304 bytes of it) with three fully contiguous 16-byte-per-lane
+ *     loads, two rows ahead of the arithmetic, and drops the bytes into a private LDS row
+ *     image. Only this pattern reaches the streaming rate of a plain copy kernel; lane-owned
+ *     strided 16-byte loads cost 40 % more time on this part.
+ *  3. Arithmetic re-reads the row image in the layout it wants: four lanes per super-block,
+ *     lane c takes nibble bytes qs[32c..32c+31] = sub-blocks 2c (low nibbles) and 2c+1 (high
+ *     nibbles). The nibbles are masked into bytes and multiplied with the digit planes by
+ *     4-way integer dot instructions: 48 per row and lane instead of 128 converts and FMAs.
+ *     Per sub-block: S = top*65536 + mid*256 + low, y += d*sc*2^(e-22)*S - dmin*m*sum(x)
+ *     (the factored form of common/ggml_dequant.h:1592-1618 dotted with x; scales unpacked
+ *     four at a time from the 12 packed bytes, get_scale_min_k4, :1582-1590).
+ *  4. Rows longer than 16 super-blocks are cut into S = 2 or 4 slices; slice s of a row is
+ *     handled by a wave with (wave % S) == s, so every wave keeps ONE slice of the digit
+ *     planes in registers for all its rows. Partial sums meet in LDS at the end.
+ *
+ * A non-finite x makes every output NaN (the fixed-point form cannot carry Inf).
  */
 #include "qlin_device.h"
 #include "qlin_internal.h"
 
 namespace qlin {
 
-__device__ __forceinline__ float ub0(uint32_t v) { return (float)(v & 0xFFu); }
-__device__ __forceinline__ float ub1(uint32_t v) { return (float)((v >> 8) & 0xFFu); }
-__device__ __forceinline__ float ub2(uint32_t v) { return (float)((v >> 16) & 0xFFu); }
-__device__ __forceinline__ float ub3(uint32_t v) { return (float)(v >> 24); }
+namespace {
 
-/* Per-lane scale terms for sub-blocks 2c and 2c+1 from the block header.
- * hdr.x = d | dmin << 16 (two halves), hdr.y/z/w = the 12 packed scale bytes.
- * Bytes 0..3 of (y & 0x3F..) are scales 0..3, of (z & 0x3F..) mins 0..3; scales 4..7 are
- * (w & 0x0F..) | ((y >> 2) & 0x30..), mins 4..7 are ((w >> 4) & 0x0F..) | ((z >> 2) & 0x30..)
- * (get_scale_min_k4, common/ggml_dequant.h:1582-1590, four fields per operation). */
-__device__ __forceinline__ void q4k_lane_scales(const uint4 hdr, int c, float &da, float &db16,
-                                                float &ma, float &mb) {
-    const float d = half_bits_fast(hdr.x & 0xFFFFu);
-    const float dmin = half_bits_fast(hdr.x >> 16);
-    const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu;
-    const uint32_t mn_lo = hdr.z & 0x3F3F3F3Fu;
-    const uint32_t sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
-    const uint32_t mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
-    const uint32_t sc4 = (c & 2) ? sc_hi : sc_lo;
-    const uint32_t mn4 = (c & 2) ? mn_hi : mn_lo;
-    const uint32_t sh = (c & 1) * 16;
-    const uint32_t sc2 = sc4 >> sh, mn2 = mn4 >> sh;
-    da = d * ub0(sc2);
-    db16 = d * ub1(sc2) * 0.0625f;
-    ma = dmin * ub0(mn2);
-    mb = dmin * ub1(mn2);
+constexpr int kWaves = 16;          /* wavefronts per workgroup */
+constexpr int kThreads = kWaves * 64;
+constexpr int kChunk = 52;          /* dwords per 64-element x chunk: 3 planes x 16, padded so that
+                                       consecutive lanes' 16-byte reads fall on distinct banks */
+constexpr int kRowImage = 3072;     /* bytes per LDS row image: 2304 + room for the full-wave tail store */
+constexpr int kMaxRowsPerWg = 128;
+
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+/* sum over the 64 lanes with cross-lane data-path moves (no LDS round trips); uniform result */
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_mov<0xB1>(v);  /* quad_perm [1,0,3,2] */
+    v += dpp_mov<0x4E>(v);  /* quad_perm [2,3,0,1] */
+    v += dpp_mov<0x141>(v); /* row_half_mirror */
+    v += dpp_mov<0x140>(v); /* row_mirror: every lane of a 16-lane row now holds the row total */
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
-template <int R>
-__global__ void __launch_bounds__(256)
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
+__device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_udot4(a, b, c, false); }
+
+struct RowRegs { uint4 a, b, c; };
+
+}  // namespace
+
+__global__ void __launch_bounds__(kThreads)
 gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
-                int n_rows, int n_sb, int slice_sb, int n_slices, int rows_per_wave) {
-    __shared__ float partial[4][8];
-    const int lane = threadIdx.x & 63;
-    const int wv = threadIdx.x >> 6;
-    const int waves_per_wg = blockDim.x >> 6;
-    const int slice = (n_slices == 1) ? 0 : wv;
-    const int rowset = (n_slices == 1) ? blockIdx.x * waves_per_wg + wv : blockIdx.x;
+                int n_rows, int n_sb, int n_slices, int slice_sb, int rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    /* LDS map: planes [n_sb*4][kChunk] dwords | meta [n_sb*4] float4 | row images [16][2][kRowImage] |
+     * partial sums [rows_per_wg * n_slices] floats */
+    uint32_t *planes = reinterpret_cast<uint32_t *>(lds);
+    float4 *meta = reinterpret_cast<float4 *>(planes + n_sb * 4 * kChunk);
+    uint8_t *images = reinterpret_cast<uint8_t *>(meta + n_sb * 4);
+    float *partial = reinterpret_cast<float *>(images + kWaves * 2 * kRowImage);
+
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int c = lane & 3;
+    const int slice = wv % n_slices;
     const int sb0 = slice * slice_sb;
     int sb_cnt = n_sb - sb0;
     if (sb_cnt > slice_sb) sb_cnt = slice_sb;
-    const int c = lane & 3;
     const bool active = (lane >> 2) < sb_cnt;
-    const int sb = sb0 + (active ? (lane >> 2) : 0); /* idle lanes re-read block sb0, scaled by 0 */
+    const int sb_local = active ? (lane >> 2) : 0;
     const size_t row_bytes = (size_t)n_sb * 144;
+    const int last_chunk = sb_cnt * 9 - 1; /* last 16-byte chunk of this wave's slice of a row */
 
-    /* this lane's 64 x values: xa = elements of sub-block 2c, xb = of sub-block 2c+1 */
-    float xa[32], xb[32];
+    const int row0 = blockIdx.x * rows_per_wg; /* first real row of this workgroup */
+    int rows_here = n_rows - row0;
+    if (rows_here > rows_per_wg) rows_here = rows_per_wg;
+    const int n_vrows = rows_here * n_slices; /* (row, slice) pairs of this workgroup */
+
+    /* this wave's virtual rows: wv, wv + 16, ... ; virtual row j = (row j / S, slice j % S), and
+     * 16 % S == 0 keeps the slice of a wave fixed */
+    const uint8_t *slice_base = W + (size_t)row0 * row_bytes + (size_t)sb0 * 144;
+    const int i0 = lane < last_chunk ? lane : last_chunk;
+    const int i1 = 64 + lane < last_chunk ? 64 + lane : last_chunk;
+    const int i2 = 128 + (lane & 15) < last_chunk ? 128 + (lane & 15) : last_chunk;
+    auto fetch = [&](int j) {
+        if (j >= n_vrows) j = wv < n_vrows ? wv : 0; /* stay in bounds; the value is never used */
+        const uint4 *q = reinterpret_cast<const uint4 *>(slice_base + (size_t)(j / n_slices) * row_bytes);
+        /* streamed once: non-temporal, so that x and the codebooks are not pushed out of L2 */
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 *qv = reinterpret_cast<const u32x4 *>(q);
+        const u32x4 va = __builtin_nontemporal_load(qv + i0), vb = __builtin_nontemporal_load(qv + i1),
+                    vc = __builtin_nontemporal_load(qv + i2);
+        RowRegs t;
+        t.a = make_uint4(va.x, va.y, va.z, va.w);
+        t.b = make_uint4(vb.x, vb.y, vb.z, vb.w);
+        t.c = make_uint4(vc.x, vc.y, vc.z, vc.w);
+        return t;
+    };
+    /* weights first: two rows in flight per wave while x is being prepared */
+    RowRegs p0 = fetch(wv), p1 = fetch(wv + kWaves);
+
+    /* ---- x -> digit planes (whole workgroup, 4 elements per thread and step) */
     {
-        const float4 *xp = reinterpret_cast<const float4 *>(x + (size_t)sb * 256 + 64 * c);
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float4 v = xp[i], u = xp[8 + i];
-            xa[4 * i] = v.x; xa[4 * i + 1] = v.y; xa[4 * i + 2] = v.z; xa[4 * i + 3] = v.w;
-            xb[4 * i] = u.x; xb[4 * i + 1] = u.y; xb[4 * i + 2] = u.z; xb[4 * i + 3] = u.w;
+        const int n4 = n_sb * 64;
+        const float4 *xg = reinterpret_cast<const float4 *>(x);
+        for (int idx = threadIdx.x; idx < n4; idx += kThreads) {
+            const float4 v = xg[idx];
+            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+            float sum = (v.x + v.y) + (v.z + v.w);
+            /* 8 consecutive threads share one 32-element sub-block */
+            amax = fmaxf(amax, dpp_mov<0xB1>(amax));
+            amax = fmaxf(amax, dpp_mov<0x4E>(amax));
+            amax = fmaxf(amax, dpp_mov<0x141>(amax));
+            sum += dpp_mov<0xB1>(sum);
+            sum += dpp_mov<0x4E>(sum);
+            sum += dpp_mov<0x141>(sum);
+            int e = (int)(__float_as_uint(amax) >> 23) - 126; /* amax in [2^(e-1), 2^e) */
+            if (e < -100) e = -100;                            /* zero and tiny blocks */
+            const float scale = __uint_as_float((uint32_t)(127 + 22 - e) << 23);
+            float inv = __uint_as_float((uint32_t)(127 - 22 + e) << 23);
+            if (!(amax <= 3.0e38f)) inv = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
+            const uint32_t X0 = (uint32_t)__float2int_rn(v.x * scale), X1 = (uint32_t)__float2int_rn(v.y * scale);
+            const uint32_t X2 = (uint32_t)__float2int_rn(v.z * scale), X3 = (uint32_t)__float2int_rn(v.w * scale);
+            /* byte transpose: plane k = byte k of X0..X3 (selector 0-3: second operand, 4-7: first) */
+            const uint32_t lo01 = __builtin_amdgcn_perm(X1, X0, 0x05010400u); /* X0.b0 X1.b0 X0.b1 X1.b1 */
+            const uint32_t lo23 = __builtin_amdgcn_perm(X3, X2, 0x05010400u);
+            const uint32_t hi01 = __builtin_amdgcn_perm(X1, X0, 0x07030602u); /* X0.b2 X1.b2 X0.b3 X1.b3 */
+            const uint32_t hi23 = __builtin_amdgcn_perm(X3, X2, 0x07030602u);
+            const uint32_t pl_low = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); /* bytes 0 of X0..X3 */
+            const uint32_t pl_mid = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u); /* bytes 1 */
+            const uint32_t pl_top = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u); /* bytes 2 */
+            const int sub = idx >> 3, j = idx & 7;
+            const int chunk = sub >> 1, is_b = sub & 1;
+            uint32_t *dst = planes + chunk * kChunk + is_b * 8 + j;
+            dst[0] = pl_top;
+            dst[16] = pl_mid;
+            dst[32] = pl_low;
+            if (j == 0) {
+                float *m = reinterpret_cast<float *>(meta + chunk);
+                m[is_b] = inv;
+                m[2 + is_b] = sum;
+            }
         }
     }
-    float sxa = 0.0f, sxb = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 32; i++) { sxa += xa[i]; sxb += xb[i]; }
+    __syncthreads();
 
-    const int row_begin = rowset * rows_per_wave;
-    for (int p = 0; p < rows_per_wave; p += R) {
-        uint4 hdr[R], q0[R], q1[R];
+    /* this lane's x: 16 dwords per plane (8 for sub-block 2c, 8 for 2c+1) */
+    uint32_t xt[16], xm[16], xl[16];
+    {
+        const uint4 *pp = reinterpret_cast<const uint4 *>(planes + ((sb0 + sb_local) * 4 + c) * kChunk);
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            int row = row_begin + p + r;
-            if (row >= n_rows) row = n_rows - 1; /* keep the load in bounds; result discarded */
-            const uint8_t *blk = W + (size_t)row * row_bytes + (size_t)sb * 144;
-            hdr[r] = *reinterpret_cast<const uint4 *>(blk);
-            q0[r] = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c);
-            q1[r] = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * c);
+        for (int i = 0; i < 4; i++) {
+            const uint4 t = pp[i], m = pp[4 + i], l = pp[8 + i];
+            xt[4 * i] = t.x; xt[4 * i + 1] = t.y; xt[4 * i + 2] = t.z; xt[4 * i + 3] = t.w;
+            xm[4 * i] = m.x; xm[4 * i + 1] = m.y; xm[4 * i + 2] = m.z; xm[4 * i + 3] = m.w;
+            xl[4 * i] = l.x; xl[4 * i + 1] = l.y; xl[4 * i + 2] = l.z; xl[4 * i + 3] = l.w;
         }
+    }
+    const float4 mt = meta[(sb0 + sb_local) * 4 + c];
+    const float inv_a = mt.x, inv_b = mt.y, sum_a = mt.z, sum_b = mt.w;
+
+    uint8_t *my_images = images + wv * (2 * kRowImage);
+    auto process = [&](RowRegs &p, int j, int slot) {
+        uint8_t *img = my_images + slot * kRowImage;
+        *reinterpret_cast<uint4 *>(img + 16 * lane) = p.a;
+        *reinterpret_cast<uint4 *>(img + 1024 + 16 * lane) = p.b;
+        *reinterpret_cast<uint4 *>(img + 2048 + 16 * lane) = p.c; /* lanes >= 16 land in the pad */
+        p = fetch(j + 2 * kWaves);
+        const uint8_t *blk = img + sb_local * 144;
+        const uint4 h = *reinterpret_cast<const uint4 *>(blk);
+        const uint4 qa = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c);
+        const uint4 qb = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * c);
+        const float d = half_bits_fast(h.x & 0xFFFFu), dmin = half_bits_fast(h.x >> 16);
+        /* bytes of sc_lo: scales 0..3, mn_lo: mins 0..3, sc_hi: scales 4..7, mn_hi: mins 4..7 */
+        const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
+        const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+        const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+        const uint32_t sc2 = ((c & 2) ? sc_hi : sc_lo) >> ((c & 1) * 16);
+        const uint32_t mn2 = ((c & 2) ? mn_hi : mn_lo) >> ((c & 1) * 16);
+        const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+        int at = 0, bt = 0;
+        uint32_t am = 0, al = 0, bm = 0, bl = 0;
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            float da, db16, ma, mb;
-            q4k_lane_scales(hdr[r], c, da, db16, ma, mb);
-            const uint32_t w[8] = {q0[r].x, q0[r].y, q0[r].z, q0[r].w, q1[r].x, q1[r].y, q1[r].z, q1[r].w};
-            float sa = 0.0f, sb_ = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                const uint32_t lo = w[i] & 0x0F0F0F0Fu;
-                const uint32_t hi = w[i] & 0xF0F0F0F0u;
-                sa += ub0(lo) * xa[4 * i] + ub1(lo) * xa[4 * i + 1] + ub2(lo) * xa[4 * i + 2] + ub3(lo) * xa[4 * i + 3];
-                sb_ += ub0(hi) * xb[4 * i] + ub1(hi) * xb[4 * i + 1] + ub2(hi) * xb[4 * i + 2] + ub3(hi) * xb[4 * i + 3];
-            }
-            float v = active ? (da * sa + db16 * sb_ - (ma * sxa + mb * sxb)) : 0.0f;
-            v = wave_sum(v);
-            const int row = row_begin + p + r;
-            if (n_slices == 1) {
-                if (lane == 0 && row < n_rows && p + r < rows_per_wave) y[row] = v;
-            } else {
-                if (lane == 0) partial[wv][r] = v;
-            }
+        for (int i = 0; i < 8; i++) {
+            const uint32_t lo = w[i] & 0x0F0F0F0Fu, hi = (w[i] >> 4) & 0x0F0F0F0Fu;
+            at = sdot4(lo, xt[i], at);
+            am = udot4(lo, xm[i], am);
+            al = udot4(lo, xl[i], al);
+            bt = sdot4(hi, xt[8 + i], bt);
+            bm = udot4(hi, xm[8 + i], bm);
+            bl = udot4(hi, xl[8 + i], bl);
         }
-        if (n_slices > 1) {
-            __syncthreads();
-            if (threadIdx.x < R) {
-                const int row = row_begin + p + threadIdx.x;
-                float s = 0.0f;
-                for (int k = 0; k < n_slices; k++) s += partial[k][threadIdx.x];
-                if (row < n_rows && p + (int)threadIdx.x < rows_per_wave) y[row] = s;
-            }
-            __syncthreads();
-        }
+        /* |top| <= 32*15*64, mid/low <= 32*15*255: the low part fits an int exactly */
+        const float fa = fmaf((float)at, 65536.0f, (float)((am << 8) + al)) * inv_a;
+        const float fb = fmaf((float)bt, 65536.0f, (float)((bm << 8) + bl)) * inv_b;
+        const float da = d * (float)(sc2 & 0xFFu), db = d * (float)((sc2 >> 8) & 0xFFu);
+        const float ma = dmin * (float)(mn2 & 0xFFu), mb = dmin * (float)((mn2 >> 8) & 0xFFu);
+        float v = active ? (da * fa + db * fb - (ma * sum_a + mb * sum_b)) : 0.0f;
+        v = wave_sum_dpp(v);
+        if (lane == 0 && j < n_vrows) partial[j] = v;
+    };
+
+    for (int j = wv; j < n_vrows; j += 2 * kWaves) {
+        process(p0, j, 0);
+        process(p1, j + kWaves, 1);
+    }
+    __syncthreads();
+
+    /* combine the slices of each row */
+    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+        float s = 0.0f;
+        for (int k = 0; k < n_slices; k++) s += partial[r * n_slices + k];
+        y[row0 + r] = s;
     }
 }
 
-/* Launch geometry: slices of at most 16 super-blocks; rows per wave chosen so that the grid
- * fills the 256 compute units evenly with about `target_waves_per_cu` waves each. */
+/* Launch geometry: one 16-wave workgroup per block of rows, sized so that the grid covers the
+ * compute units once (more workgroups only when a block would exceed kMaxRowsPerWg rows). */
 hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, int n_cols,
-                           hipStream_t stream, int n_cu, int rows_per_pass, int target_waves_per_cu) {
+                           hipStream_t stream, int n_cu) {
+    static bool lds_raised = false;
     const int n_sb = n_cols / 256;
-    const int n_slices = (n_sb + 15) / 16;
-    if (n_slices > 4) return hipErrorInvalidValue;
+    if (n_sb > 64 || n_sb < 1) return hipErrorInvalidValue;
+    const int n_slices = n_sb <= 16 ? 1 : n_sb <= 32 ? 2 : 4;
     const int slice_sb = (n_sb + n_slices - 1) / n_slices;
-    const int waves_per_wg = (n_slices == 1) ? 4 : n_slices;
-    /* row sets = groups of rows handled by one wave (or one workgroup of slice-waves) */
-    const int wave_groups_target = n_cu * target_waves_per_cu / n_slices;
-    int rpw = (n_rows + wave_groups_target - 1) / wave_groups_target;
-    if (rpw < 1) rpw = 1;
-    const int rowsets = (n_rows + rpw - 1) / rpw;
-    const int grid = (n_slices == 1) ? (rowsets + waves_per_wg - 1) / waves_per_wg : rowsets;
-    const dim3 block(64 * waves_per_wg);
-#define QLIN_Q4K_LAUNCH(RR)                                                                     \
-    hipLaunchKernelGGL((gemv_q4k_kernel<RR>), dim3(grid), block, 0, stream, (const uint8_t *)W, \
-                       x, y, n_rows, n_sb, slice_sb, n_slices, rpw)
-    switch (rows_per_pass) {
-    case 1: QLIN_Q4K_LAUNCH(1); break;
-    case 2: QLIN_Q4K_LAUNCH(2); break;
-    case 4: QLIN_Q4K_LAUNCH(4); break;
-    case 7: QLIN_Q4K_LAUNCH(7); break;
-    case 8: QLIN_Q4K_LAUNCH(8); break;
-    default: return hipErrorInvalidValue;
+    int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
+    if (rows_per_wg < 1) rows_per_wg = 1;
+    if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
+    const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
+    const size_t lds_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 +
+                             (size_t)kWaves * 2 * kRowImage + (size_t)rows_per_wg * n_slices * 4;
+    if (lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+    if (!lds_raised) {
+        hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_kernel,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        lds_raised = true;
     }
-#undef QLIN_Q4K_LAUNCH
+    hipLaunchKernelGGL(gemv_q4k_kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, (const uint8_t *)W, x, y,
+                       n_rows, n_sb, n_slices, slice_sb, rows_per_wg);
     return hipGetLastError();
 }
 

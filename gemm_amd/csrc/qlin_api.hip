@@ -79,8 +79,6 @@ struct State {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::map<uintptr_t, Range> registry; /* host begin -> range */
     DevBuf w[3], x, y[3], tmp[4];
-    /* tuning knobs read once from the environment (QLIN_Q4K_RPP, QLIN_Q4K_WAVES); 0 = default */
-    int tune_rpp = 0, tune_waves = 0;
 } g;
 
 int ensure_init_locked(int device) {
@@ -96,8 +94,6 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipStreamCreate(&g.stream));
     HIP_TRY(hipEventCreate(&g.ev0));
     HIP_TRY(hipEventCreate(&g.ev1));
-    if (const char *e = getenv("QLIN_Q4K_RPP")) g.tune_rpp = atoi(e);
-    if (const char *e = getenv("QLIN_Q4K_WAVES")) g.tune_waves = atoi(e);
     g.device = device;
     g.ready = true;
     return QLIN_OK;
@@ -146,15 +142,7 @@ hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y,
                          int n_cols, hipStream_t s) {
     if (n_rows == 0) return hipSuccess;
     if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && aligned(W, 16) && aligned(x, 16)) {
-        const int n_sb = n_cols / 256;
-        const int n_slices = (n_sb + 15) / 16;
-        /* one pass of 7 or 8 rows per wave when the row count allows ~8 waves per CU */
-        int target = g.tune_waves > 0 ? g.tune_waves : 8;
-        long long groups = (long long)g.n_cu * target / n_slices;
-        int rpw = (int)((n_rows + groups - 1) / groups);
-        int rpp = rpw >= 8 ? 8 : rpw >= 7 ? 7 : rpw >= 4 ? 4 : rpw >= 2 ? 2 : 1;
-        if (g.tune_rpp > 0) rpp = g.tune_rpp;
-        return launch_gemv_q4k(W, x, y, n_rows, n_cols, s, g.n_cu, rpp, target);
+        return launch_gemv_q4k(W, x, y, n_rows, n_cols, s, g.n_cu);
     }
     return launch_gemv_generic(type, W, x, y, n_rows, n_cols, s);
 }

@@ -20,10 +20,9 @@ hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, 
 /* y[n_rows] = W . x, any supported type and any whole-block shape */
 hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, float *y, int n_rows,
                                int n_cols, hipStream_t stream);
-/* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned.
- * rows_per_pass in {1,2,4,7,8}; target_waves_per_cu sets how many rows one wave streams. */
+/* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, int n_cols,
-                           hipStream_t stream, int n_cu, int rows_per_pass, int target_waves_per_cu);
+                           hipStream_t stream, int n_cu);
 
 /* Y[t*ldy + r] = dot(W[r,:], X[t*ldx..]) in fp32 */
 hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *Y, int n_rows,
