@@ -519,8 +519,8 @@ int qlin_gemm_bf16_dev(uint32_t type, const void *W, const uint16_t *X, float *Y
     if (n_tok < 0 || ldx < n_cols || ldy < n_rows) return fail(QLIN_ERR_ARG, "bad token count or leading dimension");
     if (n_rows == 0 || n_tok == 0) return QLIN_OK;
     if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
-    if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 16) || ldx % 8 || ldy % 4)
-        return fail(QLIN_ERR_ARG, "W, X, Y need 16-byte alignment, ldx %% 8 == 0, ldy %% 4 == 0");
+    if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
+        return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
     {
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
