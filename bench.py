@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one Q4_K matvec y = W.x with W 14336 x 4096 (the decode-shape weight the headline
+metric is quoted on), x fp32, all inputs resident in HBM before the clock starts. Successive
+steps walk through enough distinct copies of W (> 256 MB in total) that no step finds its
+weights in the 256 MB last-level cache, so the figure is an HBM figure. The timed region is
+bracketed by stream synchronisation and timed with HIP events recorded on the stream the
+kernels are launched on.
+
+Prints ONE JSON line. `value` is algorithmic bytes per step (weight bytes + x + y,
+33 103 872 B) divided by the time per step. `roofline` restates that against the 8 TB/s HBM
+peak; `cpu_baseline` is the reference's own CPU matvec (tf_qmatvec_pool compiled from its
+sources, or this repository's C restatement when that library is absent) timed on this host
+for a bounded sample; `extra` carries the prefill GEMM (second half of the metric) and the
+other benchmark shapes.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from gemm_amd import qlinear, synth  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
+BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
+Q4K = synth.GGML_Q4_K
+
+# HBM bytes moved per Q4_K 14336x4096 matvec launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by what the same counters read for a device-to-device copy of known size
+# (profiles/gemv_q4k_14336x4096_pmc.md). None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def gemv_bytes(type_id, n_rows, n_cols):
+    return n_rows * synth.row_bytes(type_id, n_cols) + 4 * n_cols + 4 * n_rows
+
+
+def time_gemv(type_id, n_rows, n_cols, steps, warmup, min_total_bytes=320 << 20, max_copies=24):
+    """-> (ms per step, number of weight copies)"""
+    W = synth.make_weights(type_id, n_rows, n_cols, seed=20260 + type_id)
+    x = synth.make_activation(n_cols, seed=7)
+    copies = max(2, min(max_copies, -(-min_total_bytes // W.nbytes)))
+    dWs = [qlinear.DevBuf.from_numpy(W) for _ in range(copies)]
+    dx = qlinear.DevBuf.from_numpy(x)
+    dy = qlinear.DevBuf(n_rows * 4)
+    for i in range(warmup):
+        qlinear.gemv_dev(type_id, dWs[i % copies], dx, dy, n_rows, n_cols)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for i in range(steps):
+        qlinear.gemv_dev(type_id, dWs[i % copies], dx, dy, n_rows, n_cols)
+    ms = qlinear.timer_end()  # records the end event on the stream and waits for it
+    qlinear.sync()
+    for d in dWs:
+        d.free()
+    return ms / steps, copies
+
+
+def time_gemm(n_tok, n_rows, n_cols, steps, warmup):
+    W = synth.make_weights(Q4K, n_rows, n_cols, seed=31)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=32, tokens=n_tok))
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xb)
+    dY = qlinear.DevBuf(n_tok * n_rows * 4)
+    for _ in range(warmup):
+        qlinear.gemm_bf16_dev(Q4K, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        qlinear.gemm_bf16_dev(Q4K, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows)
+    ms = qlinear.timer_end()
+    for d in (dW, dX, dY):
+        d.free()
+    return ms / steps
+
+
+def cpu_baseline(n_rows, n_cols, budget_s=12.0):
+    """The reference CPU matvec on this host, all cores the process may use; bounded sample."""
+    from oracle import pyoracle  # the only use of the oracle package here: the reported CPU baseline
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = max(1, min(cores, 64))
+    W = synth.make_weights(Q4K, n_rows, n_cols, seed=20260 + Q4K)
+    x = synth.make_activation(n_cols, seed=7)
+    nbytes = gemv_bytes(Q4K, n_rows, n_cols)
+    if pyoracle.Reference.available():
+        ref, kind = pyoracle.Reference(), "reference"
+        run = lambda nt, it: ref.qmatvec_pool_time(Q4K, W, x, n_cols, nt, it)  # noqa: E731
+    else:
+        orc, kind = pyoracle.Oracle(), "port"
+        run = lambda nt, it: orc.gemv_f32_time(Q4K, W, x, n_cols, nt, it)  # noqa: E731
+    t1 = run(1, 2)                                    # one thread, to size the sample
+    iters1 = max(2, int(budget_s * 0.4 / max(t1, 1e-6)))
+    t1 = run(1, iters1)
+    tn = run(cores, 3)
+    itersn = max(3, int(budget_s * 0.6 / max(tn, 1e-6)))
+    tn = run(cores, itersn)
+    return {
+        "value": round(nbytes / tn / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": kind,
+        "sample": "Q4_K 14336x4096 matvec, %d calls on %d threads (%.2f ms/call) after %d calls on 1 thread "
+                  "(%.2f ms/call, %.3f GB/s)" % (itersn, cores, tn * 1e3, iters1, t1 * 1e3, nbytes / t1 / 1e9),
+    }
+
+
+def probe(args):
+    """Helper for counter collection (see profiles/): run only the named device work."""
+    if args.probe == "copy":
+        hip = ctypes.CDLL("libamdhip64.so")
+        n = 256 << 20
+        a, b = qlinear.DevBuf(n), qlinear.DevBuf(n)
+        hip.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
+        for _ in range(4):
+            assert hip.hipMemcpy(b.ptr, a.ptr, n, 3) == 0  # hipMemcpyDeviceToDevice
+        qlinear.sync()
+        print(json.dumps({"probe": "copy", "bytes_each": n, "copies": 4}))
+    elif args.probe == "gemv":
+        ms, copies = time_gemv(Q4K, 14336, 4096, args.steps, args.warmup)
+        print(json.dumps({"probe": "gemv", "ms_per_step": ms, "copies": copies}))
+    elif args.probe == "gemm":
+        ms = time_gemm(512, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemm"], help="device work only, for rocprofv3 runs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
+              "weight rows with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        return 2
+    if args.probe:
+        probe(args)
+        return 0
+
+    name, n_cu, mem = qlinear.device_info()
+    n_rows, n_cols = 14336, 4096
+    nbytes = gemv_bytes(Q4K, n_rows, n_cols)
+    t0 = time.time()
+    ms, copies = time_gemv(Q4K, n_rows, n_cols, args.steps, args.warmup)
+    gbps = nbytes / (ms * 1e-3) / 1e9
+
+    extra = {}
+    if not args.no_extra:
+        shapes = [("q4_K", Q4K, 4096, 4096), ("q4_K", Q4K, 4096, 14336), ("q8_0", synth.GGML_Q8_0, 4096, 4096),
+                  ("q5_K", synth.GGML_Q5_K, 4096, 4096), ("iq4_nl", synth.GGML_IQ4_NL, 14336, 4096),
+                  ("iq2_xxs", synth.GGML_IQ2_XXS, 4096, 14336), ("iq3_s", synth.GGML_IQ3_S, 4096, 14336),
+                  ("q6_K", synth.GGML_Q6_K, 151936, 4096)]
+        gemv = {}
+        for tname, tid, r, c in shapes:
+            st = max(20, args.steps // 8)
+            m, _ = time_gemv(tid, r, c, st, 4, max_copies=24 if r < 100000 else 2)
+            b = gemv_bytes(tid, r, c)
+            gemv["%s_%dx%d" % (tname, r, c)] = {"us": round(m * 1e3, 2), "GB/s": round(b / (m * 1e-3) / 1e9, 1)}
+        extra["gemv_other_shapes"] = gemv
+        gemm = {}
+        for M in (128, 512, 2048):
+            m = time_gemm(M, 14336, 4096, max(5, args.steps // 40), 2)
+            fl = 2.0 * M * 14336 * 4096
+            gemm["M=%d" % M] = {"us": round(m * 1e3, 1), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}
+        extra["q4k_prefill_gemm_14336x4096_bf16"] = gemm
+        tf = gemm["M=512"]["TFLOP/s"]
+        extra["q4k_prefill_gemm_roofline"] = {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS,
+                                              "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),
+                                              "traffic": None}
+
+    out = {
+        "metric": "Q4_K GEMV GB/s (% HBM peak); Q4_K prefill GEMM TFLOP/s at M=512",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "Q4_K GEMV 14336x4096, batch 1, x fp32 (BASELINE configs[1])",
+                   "bytes_per_step": nbytes, "weight_copies_rotated": copies, "device": name.strip(),
+                   "compute_units": n_cu},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(n_rows, n_cols)
+    if extra:
+        out["extra"] = extra
+    out["wall_s"] = round(time.time() - t0, 1)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -11,17 +11,20 @@
  * about 1.7e-3 relative L2 against an exact-weight reference (budget 2e-3); truncation would
  * not fit.
  *
- * Tiling. A workgroup owns BM = 64*WM tokens x BN = 128 weight rows and walks K in steps of
- * 64 = one pair of Q4_K sub-blocks (the low and high nibbles of 32 quant bytes). Its waves
- * form a WM x 2 grid of 64x64 sub-tiles (2x2 MFMA tiles of 32x32, 64 accumulator registers).
- * Per step every thread
- *   - decodes 16 weights (8 nibble bytes of one row) into registers and stores them as bf16
- *     into the LDS B tile,
- *   - copies 4 x 16 bytes of activations into the LDS A tile,
- * and after one barrier the waves run 4 k-steps x 4 MFMAs from LDS. Global loads for step
- * i+2 are issued into a second register set before the MFMAs of step i (two LDS buffers, two
- * register sets). LDS rows are padded from 128 to 144 bytes so that the 32 rows read by one
- * MFMA operand fetch fall on distinct bank groups.
+ * Tiling. A workgroup (512 threads) owns BM = 256 tokens x BN = 128 weight rows and walks K in
+ * tiles of 64 = one pair of Q4_K sub-blocks (the low and high nibbles of 32 quant bytes). Its 8
+ * waves form a 4 x 2 grid of 64x64 sub-tiles (2x2 MFMA tiles of 32x32, 64 accumulator
+ * registers). Per tile every thread decodes 16 weights (8 nibble bytes of one row) to bf16 and
+ * copies 4 x 16 bytes of activations into an LDS ring of three stages; the MFMA operands of a
+ * tile are fetched from LDS half a tile ahead of the MFMAs that use them, the decode of tile
+ * i+2 is issued in the shadow of the MFMAs of tile i, and global loads run four tiles ahead
+ * (two register sets). One barrier per tile.
+ *
+ * Measured on MI355X at M=512, N=14336, K=4096: 78 us, 0.77 PFLOP/s. Taking pieces out of the
+ * loop shows what is left to win: MFMAs + barriers alone 41 us (the matrix pipe idles about
+ * 500 cycles around every barrier), + operand fetches 53 us, + decode and LDS stores 78 us: the
+ * three pipes (matrix, LDS, vector ALU) each need about 1000 cycles per tile and overlap only
+ * partly with two waves per SIMD that are re-aligned by a barrier every tile.
  *
  * Both MFMA operands are read from LDS with the same [row][k] indexing, so the result does
  * not depend on which k a given lane/element position feeds inside the instruction.
@@ -39,7 +42,16 @@ typedef float float2v __attribute__((ext_vector_type(2)));
 
 constexpr int kBN = 128;        /* weight rows per workgroup */
 constexpr int kBK = 64;         /* k per step */
-constexpr int kLdsRow = 144;    /* bytes per LDS tile row: 64 bf16 + 16 bytes of padding */
+constexpr int kRow = 136;       /* average bytes per LDS tile row: pairs of 128-byte rows + 16 bytes */
+constexpr int kStages = 3;      /* LDS ring depth */
+
+/* byte offset of 16-byte chunk `chunk` (0..7) of tile row `row`: rows are stored in pairs of
+ * 2 x 128 bytes followed by 16 bytes of padding. With 64 banks of 4 bytes, the 16-byte slot of
+ * (row, chunk) is ((row>>1) + 8*(row&1) + chunk) mod 16, so the 16 rows that one LDS cycle
+ * serves for an MFMA operand fetch (16 lanes x 16 bytes, consecutive rows, same chunk) use 16
+ * distinct slots, and a row written as 8 consecutive chunks stays clear of its pair row.
+ * (Padding every row to 144 bytes would do the same but three ring stages would not fit.) */
+__device__ __forceinline__ int swz(int row, int chunk) { return (row >> 1) * 272 + (row & 1) * 128 + (chunk << 4); }
 
 struct StepRegs {
     uint4 x[4];   /* 4 x 8 bf16 of activations */
@@ -78,11 +90,11 @@ __global__ void __launch_bounds__(128 * WM)
 gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y,
                      int n_rows, int n_sb, int n_tok, int ldx, int ldy, int m_tiles) {
     constexpr int BM = 64 * WM, NT = 128 * WM;
-    constexpr int PP = 512 / NT; /* (row, part) pairs of the B tile per thread */
-    static_assert(PP == 1, "one weight-row part per thread: 512 threads");
+    static_assert(NT == 512, "one weight-row part per thread: 512 threads");
+    constexpr int kATile = BM * kRow, kBTile = kBN * kRow;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    uint8_t *As = lds;                          /* [2][BM][kLdsRow] */
-    uint8_t *Bs = lds + 2 * BM * kLdsRow;       /* [2][kBN][kLdsRow] */
+    uint8_t *As = lds;                      /* [kStages][BM][kRow]  */
+    uint8_t *Bs = lds + kStages * kATile;   /* [kStages][kBN][kRow] */
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = wv >> 1, wn = wv & 1;
@@ -101,38 +113,31 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     int w_row = tile_n * kBN + br;
     if (w_row >= n_rows) w_row = n_rows - 1;
     const uint8_t *w_ptr = W + (size_t)w_row * row_bytes;
-    /* A-tile role: chunk q = tid + j*NT -> token row q/8, 16-byte column q%8 */
+    /* A-tile role: chunks (token row ar + 64j, 16-byte column ac), j = 0..3 */
+    const int ar = tid >> 3, ac = tid & 7;
     const int n_steps = n_sb * 4;
 
-    auto fetch = [&](int step) {
-        StepRegs r;
+    /* register set of one tile in flight from global memory; named members only (a set that
+     * lives across the tile loop stays in registers only when nothing indexes it) */
+    struct StepRegs { uint4 x0, x1, x2, x3, hdr; uint2 qs; };
+    auto x_chunk = [&](int j, int step) {
+        /* token rows past the end re-read row 0: their products land in accumulator rows that
+         * are never stored */
+        const int m = tile_m * BM + ar + 64 * j;
+        return *reinterpret_cast<const uint4 *>(X + (size_t)(m < n_tok ? m : 0) * ldx + (size_t)step * kBK + 8 * ac);
+    };
+    auto fetch = [&](StepRegs &r, int step) {
         if (step >= n_steps) step = n_steps - 1; /* harmless re-read past the end */
         const int sb = step >> 2, c = step & 3;
         const uint8_t *blk = w_ptr + (size_t)sb * 144;
         r.hdr = *reinterpret_cast<const uint4 *>(blk);
         r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * bp);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int q = tid + j * NT;
-            const int m = tile_m * BM + (q >> 3);
-            const uint16_t *xp = X + (size_t)(m < n_tok ? m : 0) * ldx + (size_t)step * kBK + 8 * (q & 7);
-            uint4 v = *reinterpret_cast<const uint4 *>(xp);
-            if (m >= n_tok) v = make_uint4(0, 0, 0, 0);
-            r.x[j] = v;
-        }
-        return r;
+        r.x0 = x_chunk(0, step); r.x1 = x_chunk(1, step); r.x2 = x_chunk(2, step); r.x3 = x_chunk(3, step);
     };
 
     const float unit = 1.0f / fp8_pair_lo(1u).x;
-
-    auto stage = [&](const StepRegs &r, int step, int buf) {
-        /* activations */
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int q = tid + j * NT;
-            *reinterpret_cast<uint4 *>(As + (size_t)buf * BM * kLdsRow + (q >> 3) * kLdsRow + 16 * (q & 7)) = r.x[j];
-        }
-        /* weights: sub-blocks 2c (low nibbles) and 2c+1 (high nibbles) */
+    /* the two halves of the work that puts one tile into LDS stage `st` */
+    auto stage_weights = [&](const StepRegs &r, int step, int st) {
         const int c = step & 3;
         const uint4 h = r.hdr;
         const float d = half_bits_fast(h.x & 0xFFFFu) * unit, dmin = half_bits_fast(h.x >> 16);
@@ -143,64 +148,135 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
         const uint32_t mn2 = ((c & 2) ? mn_hi : mn_lo) >> ((c & 1) * 16);
         const float dl_a = d * (float)(sc2 & 0xFFu), dl_b = d * (float)((sc2 >> 8) & 0xFFu);
         const float ml_a = dmin * (float)(mn2 & 0xFFu), ml_b = dmin * (float)((mn2 >> 8) & 0xFFu);
-        const uint32_t lo0 = r.qs.x & 0x0F0F0F0Fu, lo1 = r.qs.y & 0x0F0F0F0Fu;
-        const uint32_t hi0 = (r.qs.x >> 4) & 0x0F0F0F0Fu, hi1 = (r.qs.y >> 4) & 0x0F0F0F0Fu;
-        uint8_t *brow = Bs + (size_t)buf * kBN * kLdsRow + br * kLdsRow;
-        *reinterpret_cast<uint4 *>(brow + 16 * bp) = decode8(lo0, lo1, dl_a, ml_a);
-        *reinterpret_cast<uint4 *>(brow + 64 + 16 * bp) = decode8(hi0, hi1, dl_b, ml_b);
+        uint8_t *bt = Bs + st * kBTile;
+        /* sub-block 2c (low nibbles) -> k 0..31 = chunks 0..3, sub-block 2c+1 -> chunks 4..7 */
+        *reinterpret_cast<uint4 *>(bt + swz(br, bp)) = decode8(r.qs.x & 0x0F0F0F0Fu, r.qs.y & 0x0F0F0F0Fu, dl_a, ml_a);
+        *reinterpret_cast<uint4 *>(bt + swz(br, 4 + bp)) =
+            decode8((r.qs.x >> 4) & 0x0F0F0F0Fu, (r.qs.y >> 4) & 0x0F0F0F0Fu, dl_b, ml_b);
+    };
+    auto stage_acts = [&](const StepRegs &r, int st) {
+        uint8_t *at = As + st * kATile;
+        *reinterpret_cast<uint4 *>(at + swz(ar, ac)) = r.x0;
+        *reinterpret_cast<uint4 *>(at + swz(ar + 64, ac)) = r.x1;
+        *reinterpret_cast<uint4 *>(at + swz(ar + 128, ac)) = r.x2;
+        *reinterpret_cast<uint4 *>(at + swz(ar + 192, ac)) = r.x3;
     };
 
-    floatx16 acc[2][2];
+    floatx16 acc00, acc01, acc10, acc11;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    for (int v = 0; v < 16; v++) { acc00[v] = 0.0f; acc01[v] = 0.0f; acc10[v] = 0.0f; acc11[v] = 0.0f; }
 
-    const int frag_row = lane & 31, frag_k = (lane >> 5) * 16; /* byte offset of this lane's 8 k */
-    auto compute = [&](int buf) {
-        const uint8_t *a_base = As + (size_t)buf * BM * kLdsRow + (wm * 64 + frag_row) * kLdsRow + frag_k;
-        const uint8_t *b_base = Bs + (size_t)buf * kBN * kLdsRow + (wn * 64 + frag_row) * kLdsRow + frag_k;
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-            const bf16x8 a0 = *reinterpret_cast<const bf16x8 *>(a_base + 32 * s);
-            const bf16x8 a1 = *reinterpret_cast<const bf16x8 *>(a_base + 32 * kLdsRow + 32 * s);
-            const bf16x8 b0 = *reinterpret_cast<const bf16x8 *>(b_base + 32 * s);
-            const bf16x8 b1 = *reinterpret_cast<const bf16x8 *>(b_base + 32 * kLdsRow + 32 * s);
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
-        }
+    /* operand fragments of two k-steps (half a tile): 2 x (2 A + 2 B) x 8 bf16 */
+    struct Frags { bf16x8 a0, a1, b0, b1, c0, c1, d0, d1; };
+    const int frag_row = lane & 31, kg = lane >> 5;
+    const int a_row = wm * 64 + frag_row, b_row = wn * 64 + frag_row;
+    auto load_frags = [&](Frags &f, int st, int half) {
+        const uint8_t *at = As + st * kATile, *bt = Bs + st * kBTile;
+        const int ch0 = 4 * half + kg, ch1 = ch0 + 2; /* logical chunks of k-steps 2*half, 2*half+1 */
+        f.a0 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row, ch0));
+        f.a1 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row + 32, ch0));
+        f.b0 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row, ch0));
+        f.b1 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row + 32, ch0));
+        f.c0 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row, ch1));
+        f.c1 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row + 32, ch1));
+        f.d0 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row, ch1));
+        f.d1 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row + 32, ch1));
+    };
+    auto mma_half = [&](const Frags &f) {
+        acc00 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a0, f.b0, acc00, 0, 0, 0);
+        acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a0, f.b1, acc01, 0, 0, 0);
+        acc10 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a1, f.b0, acc10, 0, 0, 0);
+        acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a1, f.b1, acc11, 0, 0, 0);
+        acc00 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c0, f.d0, acc00, 0, 0, 0);
+        acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c0, f.d1, acc01, 0, 0, 0);
+        acc10 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c1, f.d0, acc10, 0, 0, 0);
+        acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c1, f.d1, acc11, 0, 0, 0);
     };
 
-    StepRegs r0 = fetch(0), r1 = fetch(1);
+    /* ask the instruction scheduler for "one MFMA, then a few vector-ALU instructions" eight
+     * times over, so that the decode arithmetic is issued in the shadow of the MFMAs of the same
+     * wave instead of in front of them */
+#define QLIN_INTERLEAVE_8(VALU_PER_MFMA)                                  \
+    _Pragma("unroll") for (int q_ = 0; q_ < 8; q_++) {                    \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
+        __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);    \
+    }
+
+    /* Pipeline, per tile i (LDS stage i % 3), all in one basic block between two barriers:
+     *   matrix pipe : 16 MFMAs on tile i from fragment registers
+     *   LDS reads   : second half of tile i, then first half of tile i+1 (half a tile ahead)
+     *   vector ALU  : decode tile i+2 from registers into stage (i+2) % 3
+     *   global loads: tile i+4 into the registers just freed
+     * Stage (i+2) % 3 held tile i-1, whose last fragments were read before the barrier that
+     * opens tile i; tile i+1 was completed before that same barrier. */
+    StepRegs r0, r1;
+    fetch(r0, 0);
+    fetch(r1, 1);
+    stage_weights(r0, 0, 0);
+    stage_acts(r0, 0);
+    fetch(r0, 2);
+    stage_weights(r1, 1, 1);
+    stage_acts(r1, 1);
+    fetch(r1, 3);
+    __syncthreads();
+    Frags f0, f1;
+    load_frags(f0, 0, 0);
+    int st = 0; /* stage of the current tile */
     for (int step = 0; step < n_steps; step += 2) {
-        stage(r0, step, 0);
+        /* even tile: registers r0 hold tile step+2 */
+        {
+            const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
+            load_frags(f1, st, 1);
+            __builtin_amdgcn_sched_barrier(0); /* keep the operand fetch ahead of the MFMAs it hides behind */
+            stage_weights(r0, step + 2, st2);
+            mma_half(f0);
+            QLIN_INTERLEAVE_8(8)
+            __builtin_amdgcn_sched_barrier(0);
+            load_frags(f0, st1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            stage_acts(r0, st2);
+            fetch(r0, step + 4);
+            mma_half(f1);
+            QLIN_INTERLEAVE_8(5)
+            __builtin_amdgcn_sched_barrier(0);
+            st = st1;
+        }
         __syncthreads();
-        r0 = fetch(step + 2);
-        compute(0);
-        stage(r1, step + 1, 1);
+        /* odd tile: registers r1 hold tile step+3 */
+        {
+            const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
+            load_frags(f1, st, 1);
+            __builtin_amdgcn_sched_barrier(0); /* keep the operand fetch ahead of the MFMAs it hides behind */
+            stage_weights(r1, step + 3, st2);
+            mma_half(f0);
+            QLIN_INTERLEAVE_8(8)
+            __builtin_amdgcn_sched_barrier(0);
+            load_frags(f0, st1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            stage_acts(r1, st2);
+            fetch(r1, step + 5);
+            mma_half(f1);
+            QLIN_INTERLEAVE_8(5)
+            __builtin_amdgcn_sched_barrier(0);
+            st = st1;
+        }
         __syncthreads();
-        r1 = fetch(step + 3);
-        compute(1);
     }
 
     /* C layout of the 32x32 MFMA: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4,
      * column l%32. Columns are weight rows, contiguous in the token-major output. */
+    auto store_tile = [&](const floatx16 &acc, int mi, int ni) {
+        const int n = tile_n * kBN + wn * 64 + ni * 32 + (lane & 31);
 #pragma unroll
-    for (int mi = 0; mi < 2; mi++) {
-#pragma unroll
-        for (int ni = 0; ni < 2; ni++) {
-            const int n = tile_n * kBN + wn * 64 + ni * 32 + (lane & 31);
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = tile_m * BM + wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (m < n_tok && n < n_rows) Y[(size_t)m * ldy + n] = acc[mi][ni][v];
-            }
+        for (int v = 0; v < 16; v++) {
+            const int m = tile_m * BM + wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+            if (m < n_tok && n < n_rows) Y[(size_t)m * ldy + n] = acc[v];
         }
-    }
+    };
+    store_tile(acc00, 0, 0);
+    store_tile(acc01, 0, 1);
+    store_tile(acc10, 1, 0);
+    store_tile(acc11, 1, 1);
 }
 
 hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
@@ -213,7 +289,7 @@ hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int 
     /* ids are dealt to 8 XCDs; pad the n-tile count to a multiple of 8 (surplus groups exit) */
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const int grid = n_tiles_pad * m_tiles;
-    const size_t lds_bytes = (size_t)2 * (BM + kBN) * kLdsRow;
+    const size_t lds_bytes = (size_t)kStages * (BM + kBN) * kRow;
     if (!lds_raised) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_q4k_bf16_kernel<WM>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
