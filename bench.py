@@ -83,6 +83,41 @@ def time_gemm(n_tok, n_rows, n_cols, steps, warmup):
     return ms / steps
 
 
+def time_moe(steps, warmup, n_expert=128, n_embd=2048, n_ff=768, top_k=8, n_tok=64, copies=2):
+    """Grouped MoE expert FFN: -> (ms per step, algorithmic bytes per step, flops per step)"""
+    sets = []
+    for c in range(copies):
+        sets.append([qlinear.DevBuf.from_numpy(synth.make_weights(Q4K, n_expert * r, k, seed=900 + 3 * c + i))
+                     for i, (r, k) in enumerate(((n_ff, n_embd), (n_ff, n_embd), (n_embd, n_ff)))])
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=41, tokens=n_tok))
+    dX = qlinear.DevBuf.from_numpy(Xb)
+    dl = qlinear.DevBuf.from_numpy(synth.make_router_logits(n_tok, n_expert, seed=42))
+    di, dw = qlinear.DevBuf(n_tok * top_k * 4), qlinear.DevBuf(n_tok * top_k * 4)
+    dout = qlinear.DevBuf(n_tok * n_embd * 4)
+    dws = qlinear.DevBuf(qlinear.moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert))
+    qlinear.moe_route_dev(dl, n_tok, n_expert, top_k, di, dw)
+    qlinear.sync()
+    routed = len(np.unique(di.to_numpy(np.int32, (n_tok, top_k))))
+
+    def step(i):
+        g, u, d = sets[i % copies]
+        qlinear.moe_ffn_dev(Q4K, g, u, d, dX, di, dw, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
+
+    for i in range(warmup):
+        step(i)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for i in range(steps):
+        step(i)
+    ms = qlinear.timer_end()
+    expert_bytes = 2 * n_ff * synth.row_bytes(Q4K, n_embd) + n_embd * synth.row_bytes(Q4K, n_ff)
+    nbytes = routed * expert_bytes + n_tok * n_embd * 2 + n_tok * n_embd * 4 + n_tok * top_k * 8
+    flops = 2.0 * n_tok * top_k * 3 * n_ff * n_embd
+    for b in [x for st in sets for x in st] + [dX, dl, di, dw, dout, dws]:
+        b.free()
+    return ms / steps, nbytes, flops, routed
+
+
 def cpu_baseline(n_rows, n_cols, budget_s=12.0):
     """The reference CPU matvec on this host, all cores the process may use; bounded sample."""
     from oracle import pyoracle  # the only use of the oracle package here: the reported CPU baseline
@@ -124,6 +159,9 @@ def probe(args):
     elif args.probe == "gemv":
         ms, copies = time_gemv(Q4K, 14336, 4096, args.steps, args.warmup)
         print(json.dumps({"probe": "gemv", "ms_per_step": ms, "copies": copies}))
+    elif args.probe == "moe":
+        m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
+        print(json.dumps({"probe": "moe", "ms_per_step": m, "bytes": b, "routed": routed}))
     elif args.probe == "gemm":
         ms = time_gemm(512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
@@ -136,7 +174,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemm"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemm", "moe"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
@@ -176,6 +214,11 @@ def main():
         extra["q4k_prefill_gemm_roofline"] = {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS,
                                               "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),
                                               "traffic": None}
+
+        m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
+        extra["q4k_moe_ffn_128x(768x2048)_64tok_top8"] = {
+            "us": round(m * 1e3, 1), "routed_experts": routed, "bytes": b, "GB/s": round(b / (m * 1e-3) / 1e9, 1),
+            "hbm_frac": round(b / (m * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}
 
     out = {
         "metric": "Q4_K GEMV GB/s (% HBM peak); Q4_K prefill GEMM TFLOP/s at M=512",

@@ -1,0 +1,389 @@
+/*
+ * moe_ffn_q4k.hip - grouped MoE expert FFN for Q4_K experts and bf16 activations:
+ *
+ *     out[t] = sum_k w[t,k] * down_e( silu(gate_e x_t) * (up_e x_t) ),  e = idx[t,k]
+ *
+ * the batched form of the per-token loop of common/transformer.h:4093-4128. With a few dozen
+ * tokens spread over a hundred experts every expert sees a handful of tokens, so the job is
+ * to stream each routed expert's blocks from HBM exactly once; the arithmetic is small.
+ *
+ * Four launches:
+ *   1. group:   counting sort of the (token, k) pairs by expert (one workgroup).
+ *   2. gate_up: one wavefront per (expert, 32 rows of gate and of up). For every 32-element
+ *               sub-block it issues v_mfma_f32_16x16x32_bf16 with
+ *                   A = 16 of the expert's tokens x 32 activations (bf16, as given),
+ *                   B = 32 raw 4-bit codes x 16 rows, the codes 0..15 converted to bf16
+ *                       (exact), two per instruction, by the scaled fp8 conversion,
+ *               which yields S = sum_k q*x per (token, row) without any rounding of the
+ *               weights; the block scales go on in fp32: acc += (d*sc)*S - (dmin*m)*SX, where
+ *               SX = sum_k x comes from one more MFMA against a B of ones and lands in the
+ *               same lanes as S. silu(g)*u is then split into a bf16 head and a bf16 tail
+ *               (h = hi + lo up to 2^-17 relative), so the second GEMM sees h to ~fp32.
+ *   3. down:    same scheme over K = n_ff with A = hi and A = lo accumulated in one
+ *               accumulator; writes w[t,k] * result per pair.
+ *   4. combine: out[t] = the token's top_k partial rows added in k order (deterministic).
+ *
+ * Lane layout of the 16x16x32 MFMA (A: tokens i, B: rows j): lane l feeds A[i = l%16]
+ * [k = 8*(l/16) .. +7] and B[k = 8*(l/16) .. +7][j = l%16]; it receives C[i = 4*(l/16)+v][j = l%16],
+ * v = 0..3. So a lane owns one weight row (one scale pair per sub-block) and four tokens.
+ * Sub-block 2c of a super-block is the low nibbles of qs[32c..32c+31], 2c+1 the high nibbles
+ * (common/ggml_dequant.h:1592-1618): one 8-byte load per lane serves two MFMAs.
+ */
+#include "qlin_device.h"
+#include "qlin_internal.h"
+
+namespace qlin {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr int kQ4KBlock = 144;
+
+struct Workspace {
+    int32_t *offsets;  /* [n_expert + 1] first slot of each expert */
+    int32_t *order;    /* [n_pairs] slot -> pair (t*top_k + k), grouped by expert */
+    int32_t *slot_of;  /* [n_pairs] pair -> slot, -1 for an expert index out of range */
+    uint16_t *h_hi;    /* [n_pairs, n_ff] bf16 head of silu(g)*u, by slot */
+    uint16_t *h_lo;    /* [n_pairs, n_ff] bf16 tail */
+    float *part;       /* [n_pairs, n_embd] w * down(h), by slot */
+    size_t bytes;
+};
+
+size_t round256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
+    const size_t n_pairs = (size_t)n_tok * top_k;
+    char *p = (char *)base;
+    size_t off = 0;
+    Workspace w;
+    w.offsets = (int32_t *)(p + off); off += round256(((size_t)n_expert + 1) * 4);
+    w.order = (int32_t *)(p + off);   off += round256(n_pairs * 4);
+    w.slot_of = (int32_t *)(p + off); off += round256(n_pairs * 4);
+    w.h_hi = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
+    w.h_lo = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
+    w.part = (float *)(p + off);      off += round256(n_pairs * n_embd * 4);
+    w.bytes = off;
+    return w;
+}
+
+/* ---- 1. counting sort of pairs by expert; cnt[] and cur[] live in LDS ---- */
+__global__ void __launch_bounds__(1024)
+moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int32_t *__restrict__ offsets,
+                 int32_t *__restrict__ order, int32_t *__restrict__ slot_of) {
+    extern __shared__ int32_t lds[]; /* cnt[n_expert], cur[n_expert] */
+    int32_t *cnt = lds, *cur = lds + n_expert;
+    for (int e = threadIdx.x; e < n_expert; e += blockDim.x) cnt[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = idx[p];
+        if (e >= 0 && e < n_expert) atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int e = 0; e < n_expert; e++) {
+            offsets[e] = run;
+            cur[e] = run;
+            run += cnt[e];
+        }
+        offsets[n_expert] = run;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = idx[p];
+        int slot = -1;
+        if (e >= 0 && e < n_expert) {
+            slot = atomicAdd(&cur[e], 1);
+            order[slot] = p;
+        }
+        slot_of[p] = slot;
+    }
+}
+
+/* ---- shared pieces of the two matrix kernels ---- */
+
+/* the sixteen 6-bit fields of a super-block as bytes: sc_lo = scales of sub-blocks 0..3,
+ * sc_hi = 4..7, likewise the mins (get_scale_min_k4, common/ggml_dequant.h:1582-1590) */
+struct Scales {
+    float d, dmin;
+    uint32_t sc_lo, sc_hi, mn_lo, mn_hi;
+};
+
+__device__ __forceinline__ Scales unpack_header(u32x4 h) {
+    Scales s;
+    s.d = half_bits_fast(h.x & 0xFFFFu);
+    s.dmin = half_bits_fast(h.x >> 16);
+    const uint32_t y = h.y, z = h.z, w = h.w;
+    s.sc_lo = y & 0x3F3F3F3Fu;
+    s.mn_lo = z & 0x3F3F3F3Fu;
+    s.sc_hi = (w & 0x0F0F0F0Fu) | ((y >> 2) & 0x30303030u);
+    s.mn_hi = ((w >> 4) & 0x0F0F0F0Fu) | ((z >> 2) & 0x30303030u);
+    return s;
+}
+
+template <int SUB>
+__device__ __forceinline__ void sub_scales(const Scales &s, float &dsc, float &dm) {
+    const uint32_t sc = (SUB < 4) ? s.sc_lo : s.sc_hi;
+    const uint32_t mn = (SUB < 4) ? s.mn_lo : s.mn_hi;
+    constexpr int sh = 8 * (SUB & 3);
+    dsc = s.d * (float)((sc >> sh) & 0xFFu);
+    dm = s.dmin * (float)((mn >> sh) & 0xFFu);
+}
+
+/* 8 bytes 0x0q -> 8 bf16 holding q exactly: an E4M3 byte 0x0q is q * 2^-9, the scale 2^9 undoes that */
+__device__ __forceinline__ bf16x8 codes_to_bf16(uint32_t a, uint32_t b) {
+    const bf16x2 p0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(a, 512.0f, false);
+    const bf16x2 p1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(a, 512.0f, true);
+    const bf16x2 p2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b, 512.0f, false);
+    const bf16x2 p3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b, 512.0f, true);
+    bf16x8 r;
+    r[0] = p0[0]; r[1] = p0[1]; r[2] = p1[0]; r[3] = p1[1];
+    r[4] = p2[0]; r[5] = p2[1]; r[6] = p3[0]; r[7] = p3[1];
+    return r;
+}
+
+__device__ __forceinline__ bf16x8 ones_bf16() {
+    const u32x4 v = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+__device__ __forceinline__ f32x4 mma(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ bf16x8 load_a(const uint16_t *p, bool live) {
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (live) v = *(const u32x4 *)p;
+    return __builtin_bit_cast(bf16x8, v);
+}
+
+/* acc[v] += dsc0*S0[v] - dm0*X0[v] + dsc1*S1[v] - dm1*X1[v] */
+__device__ __forceinline__ void apply_scales(f32x4 &acc, f32x4 S0, f32x4 S1, f32x4 X0, f32x4 X1, float dsc0,
+                                             float dm0, float dsc1, float dm1) {
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        float a = acc[v];
+        a = fmaf(dsc0, S0[v], a);
+        a = fmaf(-dm0, X0[v], a);
+        a = fmaf(dsc1, S1[v], a);
+        a = fmaf(-dm1, X1[v], a);
+        acc[v] = a;
+    }
+}
+
+/* one 64-element slice c of a super-block for one weight row pointer `blk` (start of the super-block):
+ * the lane's 8 bytes give its 8 codes of sub-block 2c (low nibbles) and of 2c+1 (high nibbles) */
+template <int C>
+__device__ __forceinline__ void slice_codes(const uint8_t *blk, int kg, bf16x8 &b_lo, bf16x8 &b_hi) {
+    const u32x2 q = *(const u32x2 *)(blk + 16 + 32 * C + 8 * kg);
+    b_lo = codes_to_bf16(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu);
+    b_hi = codes_to_bf16((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu);
+}
+
+/* ---- 2. gate and up for 32 rows of one expert, all of its tokens ---- */
+template <int C>
+__device__ __forceinline__ void gate_up_slice(const uint8_t *g0, const uint8_t *g1, const uint8_t *u0,
+                                              const uint8_t *u1, const Scales &sg0, const Scales &sg1,
+                                              const Scales &su0, const Scales &su1, const uint16_t *xk, bool live,
+                                              int kg, f32x4 &ag0, f32x4 &ag1, f32x4 &au0, f32x4 &au1) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bf16x8 a0 = load_a(xk + 64 * C + 8 * kg, live);
+    const bf16x8 a1 = load_a(xk + 64 * C + 32 + 8 * kg, live);
+    const f32x4 X0 = mma(a0, ones_bf16(), zero);
+    const f32x4 X1 = mma(a1, ones_bf16(), zero);
+    bf16x8 lo, hi;
+    float dsc0, dm0, dsc1, dm1;
+
+    slice_codes<C>(g0, kg, lo, hi);
+    sub_scales<2 * C>(sg0, dsc0, dm0);
+    sub_scales<2 * C + 1>(sg0, dsc1, dm1);
+    apply_scales(ag0, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
+
+    slice_codes<C>(g1, kg, lo, hi);
+    sub_scales<2 * C>(sg1, dsc0, dm0);
+    sub_scales<2 * C + 1>(sg1, dsc1, dm1);
+    apply_scales(ag1, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
+
+    slice_codes<C>(u0, kg, lo, hi);
+    sub_scales<2 * C>(su0, dsc0, dm0);
+    sub_scales<2 * C + 1>(su0, dsc1, dm1);
+    apply_scales(au0, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
+
+    slice_codes<C>(u1, kg, lo, hi);
+    sub_scales<2 * C>(su1, dsc0, dm0);
+    sub_scales<2 * C + 1>(su1, dsc1, dm1);
+    apply_scales(au1, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
+}
+
+__device__ __forceinline__ void store_h(uint16_t *h_hi, uint16_t *h_lo, size_t at, float g, float u) {
+    const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
+    const __bf16 hi = (__bf16)h;
+    const __bf16 lo = (__bf16)(h - (float)hi);
+    h_hi[at] = __builtin_bit_cast(uint16_t, hi);
+    h_lo[at] = __builtin_bit_cast(uint16_t, lo);
+}
+
+__global__ void __launch_bounds__(256)
+moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
+                   const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
+                   const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
+                   int n_embd, int n_ff, int top_k) {
+    const int e = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
+    if (row0 >= n_ff) return;
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int j = lane & 15, kg = lane >> 4;
+    const int n_sb = n_embd >> 8;
+    const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
+    const size_t ebase = (size_t)e * n_ff * row_bytes;
+    const uint8_t *g0 = gate + ebase + (size_t)(row0 + j) * row_bytes;
+    const uint8_t *g1 = g0 + 16 * row_bytes;
+    const uint8_t *u0 = up + ebase + (size_t)(row0 + j) * row_bytes;
+    const uint8_t *u1 = u0 + 16 * row_bytes;
+
+    for (int t0 = 0; t0 < cnt; t0 += 16) {
+        const bool live = t0 + j < cnt; /* as an A lane, j is the token slot */
+        const int tok = live ? order[first + t0 + j] / top_k : 0;
+        const uint16_t *xrow = X + (size_t)tok * n_embd;
+        f32x4 ag0 = {0, 0, 0, 0}, ag1 = {0, 0, 0, 0}, au0 = {0, 0, 0, 0}, au1 = {0, 0, 0, 0};
+        for (int sb = 0; sb < n_sb; sb++) {
+            const size_t o = (size_t)sb * kQ4KBlock;
+            const Scales sg0 = unpack_header(*(const u32x4 *)(g0 + o));
+            const Scales sg1 = unpack_header(*(const u32x4 *)(g1 + o));
+            const Scales su0 = unpack_header(*(const u32x4 *)(u0 + o));
+            const Scales su1 = unpack_header(*(const u32x4 *)(u1 + o));
+            const uint16_t *xk = xrow + sb * 256;
+            gate_up_slice<0>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
+            gate_up_slice<1>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
+            gate_up_slice<2>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
+            gate_up_slice<3>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
+        }
+        /* as a C lane: row j, token slots 4*kg + v */
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int ts = t0 + 4 * kg + v;
+            if (ts < cnt) {
+                const size_t at = (size_t)(first + ts) * n_ff + row0 + j;
+                store_h(h_hi, h_lo, at, ag0[v], au0[v]);
+                store_h(h_hi, h_lo, at + 16, ag1[v], au1[v]);
+            }
+        }
+    }
+}
+
+/* ---- 3. down for 32 rows of one expert ---- */
+template <int C>
+__device__ __forceinline__ void down_slice(const uint8_t *d0, const uint8_t *d1, const Scales &s0, const Scales &s1,
+                                           const uint16_t *hk, const uint16_t *lk, bool live, int kg, f32x4 &a0,
+                                           f32x4 &a1) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bf16x8 h0 = load_a(hk + 64 * C + 8 * kg, live), l0 = load_a(lk + 64 * C + 8 * kg, live);
+    const bf16x8 h1 = load_a(hk + 64 * C + 32 + 8 * kg, live), l1 = load_a(lk + 64 * C + 32 + 8 * kg, live);
+    const f32x4 X0 = mma(l0, ones_bf16(), mma(h0, ones_bf16(), zero));
+    const f32x4 X1 = mma(l1, ones_bf16(), mma(h1, ones_bf16(), zero));
+    bf16x8 lo, hi;
+    float dsc0, dm0, dsc1, dm1;
+
+    slice_codes<C>(d0, kg, lo, hi);
+    sub_scales<2 * C>(s0, dsc0, dm0);
+    sub_scales<2 * C + 1>(s0, dsc1, dm1);
+    apply_scales(a0, mma(l0, lo, mma(h0, lo, zero)), mma(l1, hi, mma(h1, hi, zero)), X0, X1, dsc0, dm0, dsc1, dm1);
+
+    slice_codes<C>(d1, kg, lo, hi);
+    sub_scales<2 * C>(s1, dsc0, dm0);
+    sub_scales<2 * C + 1>(s1, dsc1, dm1);
+    apply_scales(a1, mma(l0, lo, mma(h0, lo, zero)), mma(l1, hi, mma(h1, hi, zero)), X0, X1, dsc0, dm0, dsc1, dm1);
+}
+
+__global__ void __launch_bounds__(256)
+moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
+                const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
+                const int32_t *__restrict__ order, const float *__restrict__ expert_w, float *__restrict__ part,
+                int n_embd, int n_ff) {
+    const int e = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
+    if (row0 >= n_embd) return;
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int j = lane & 15, kg = lane >> 4;
+    const int n_sb = n_ff >> 8;
+    const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
+    const uint8_t *d0 = down + (size_t)e * n_embd * row_bytes + (size_t)(row0 + j) * row_bytes;
+    const uint8_t *d1 = d0 + 16 * row_bytes;
+
+    for (int t0 = 0; t0 < cnt; t0 += 16) {
+        const bool live = t0 + j < cnt;
+        const size_t arow = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
+        f32x4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
+        for (int sb = 0; sb < n_sb; sb++) {
+            const size_t o = (size_t)sb * kQ4KBlock;
+            const Scales s0 = unpack_header(*(const u32x4 *)(d0 + o));
+            const Scales s1 = unpack_header(*(const u32x4 *)(d1 + o));
+            const uint16_t *hk = h_hi + arow + sb * 256, *lk = h_lo + arow + sb * 256;
+            down_slice<0>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
+            down_slice<1>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
+            down_slice<2>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
+            down_slice<3>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const int ts = t0 + 4 * kg + v;
+            if (ts < cnt) {
+                const float w = expert_w[order[first + ts]];
+                const size_t at = (size_t)(first + ts) * n_embd + row0 + j;
+                part[at] = w * a0[v];      /* w * q, as out[i] += w*q does (:4116-4127) */
+                part[at + 16] = w * a1[v];
+            }
+        }
+    }
+}
+
+/* ---- 4. out[t] = sum over k, in k order ---- */
+__global__ void __launch_bounds__(256)
+moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of, float *__restrict__ out,
+                   int n_embd, int top_k) {
+    const int t = blockIdx.x;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (c >= n_embd) return;
+    float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int k = 0; k < top_k; k++) {
+        const int slot = slot_of[t * top_k + k];
+        if (slot < 0) continue;
+        const float4 p = *(const float4 *)(part + (size_t)slot * n_embd + c);
+        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+    }
+    *(float4 *)(out + (size_t)t * n_embd + c) = s;
+}
+
+}  // namespace
+
+size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
+    return carve(nullptr, n_tok, top_k, n_embd, n_ff, n_expert).bytes;
+}
+
+hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down, const uint16_t *X,
+                              const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
+                              int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream) {
+    const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
+    const int n_pairs = n_tok * top_k;
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)n_expert * 2 * sizeof(int32_t), stream, idx,
+                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of);
+    hipLaunchKernelGGL(moe_gate_up_kernel, dim3((n_ff / 32 + 3) / 4, n_expert), dim3(256), 0, stream,
+                       (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
+                       n_ff, top_k);
+    hipLaunchKernelGGL(moe_down_kernel, dim3((n_embd / 32 + 3) / 4, n_expert), dim3(256), 0, stream,
+                       (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.order, w, ws.part, n_embd, n_ff);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 255) / 256), dim3(256), 0, stream, ws.part,
+                       ws.slot_of, out, n_embd, top_k);
+    return hipGetLastError();
+}
+
+}  // namespace qlin

@@ -554,6 +554,9 @@ int qlin_moe_ffn_dev(uint32_t type, const void *gate_exps, const void *up_exps, 
     if (int rc = check_linear_shape(type, n_ff, n_embd)) return rc;
     if (int rc = check_linear_shape(type, n_embd, n_ff)) return rc;
     if (n_tok < 0 || n_expert <= 0 || top_k <= 0 || top_k > n_expert) return fail(QLIN_ERR_ARG, "bad MoE shape");
+    if (n_expert > 4096) return fail(QLIN_ERR_ARG, "grouped MoE FFN handles at most 4096 experts (got %d)", n_expert);
+    if ((long long)n_tok * top_k > (1 << 24))
+        return fail(QLIN_ERR_ARG, "grouped MoE FFN handles at most 2^24 (token, expert) pairs per call");
     if (n_tok == 0) return QLIN_OK;
     if (!gate_exps || !up_exps || !down_exps || !X || !expert_idx || !expert_w || !out || !workspace)
         return fail(QLIN_ERR_ARG, "null pointer");

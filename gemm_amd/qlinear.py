@@ -186,6 +186,20 @@ def gemm_f32_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, stream=No
     check(load().qlin_gemm_f32_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy, stream))
 
 
+def moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert):
+    return load().qlin_moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert)
+
+
+def moe_route_dev(dlogits, n_tok, n_expert, top_k, didx, dw, stream=None):
+    check(load().qlin_moe_route_dev(dlogits.ptr, n_tok, n_expert, top_k, didx.ptr, dw.ptr, stream))
+
+
+def moe_ffn_dev(type_id, dgate, dup, ddown, dX, didx, dw, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws,
+                stream=None):
+    check(load().qlin_moe_ffn_dev(type_id, dgate.ptr, dup.ptr, ddown.ptr, dX.ptr, didx.ptr, dw.ptr, dout.ptr,
+                                  n_tok, top_k, n_embd, n_ff, n_expert, dws.ptr, stream))
+
+
 def sync(stream=None):
     check(load().qlin_dev_sync(stream))
 

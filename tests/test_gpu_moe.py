@@ -1,0 +1,165 @@
+"""GPU parity of the grouped MoE expert FFN (Q4_K experts, bf16 activations), through the C ABI.
+
+The reference computes, per token, sum_k w_k * down_e(silu(gate_e x) * up_e x) with fp32 matvecs
+over decoded rows (common/transformer.h:4093-4128). The checks here use
+  * the CPU oracle's per-token function with double accumulation on the same bf16-rounded x and
+    the same (idx, w), and
+  * for the full-size case, a numpy float64 restatement over oracle-decoded expert matrices.
+Contract: relative L2 <= 2e-3. The kernel keeps the weights exact and carries the intermediate
+activation as a bf16 head + tail, so it is held to 2e-5 here.
+"""
+import numpy as np
+import pytest
+
+from gemm_amd import qlinear, synth
+from tests.conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+Q4K = synth.GGML_Q4_K
+CONTRACT, DESIGNED = 2e-3, 2e-5
+
+
+def make_experts(n_expert, n_embd, n_ff, seed):
+    gate = synth.make_weights(Q4K, n_expert * n_ff, n_embd, seed=seed)
+    up = synth.make_weights(Q4K, n_expert * n_ff, n_embd, seed=seed + 1)
+    down = synth.make_weights(Q4K, n_expert * n_embd, n_ff, seed=seed + 2)
+    return gate, up, down
+
+
+def run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, fill=-7.0):
+    n_tok, top_k = idx.shape
+    bufs = [qlinear.DevBuf.from_numpy(a) for a in (gate, up, down, Xb, idx.astype(np.int32), w.astype(np.float32))]
+    out0 = np.full((max(n_tok, 1), n_embd), fill, np.float32)
+    dout = qlinear.DevBuf.from_numpy(out0)
+    nws = qlinear.moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert)
+    dws = qlinear.DevBuf(max(nws, 256))
+    qlinear.moe_ffn_dev(Q4K, *bufs, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
+    qlinear.sync()
+    out = dout.to_numpy(np.float32, out0.shape)[:n_tok]
+    for b in bufs + [dout, dws]:
+        b.free()
+    return out
+
+
+def route(oracle, logits, top_k):
+    idx = np.zeros((logits.shape[0], top_k), np.int32)
+    w = np.zeros((logits.shape[0], top_k), np.float32)
+    for t in range(logits.shape[0]):
+        idx[t], w[t] = oracle.moe_route(logits[t], top_k)
+    return idx, w
+
+
+def oracle_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff):
+    X = synth.bf16_bits_to_f32(Xb)
+    return np.stack([oracle.moe_ffn_token(Q4K, gate, up, down, n_embd, n_ff, X[t], idx[t], w[t], f64=True)
+                     for t in range(X.shape[0])])
+
+
+def numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff):
+    """float64 restatement grouped by expert: decode each routed expert once."""
+    X = synth.bf16_bits_to_f32(Xb).astype(np.float64)
+    out = np.zeros((X.shape[0], n_embd), np.float64)
+    gb, db = synth.row_bytes(Q4K, n_embd), synth.row_bytes(Q4K, n_ff)
+    for e in np.unique(idx):
+        if e < 0:
+            continue
+        G = oracle.dequant_matrix(Q4K, gate[e * n_ff:(e + 1) * n_ff].reshape(n_ff, gb), n_embd).astype(np.float64)
+        U = oracle.dequant_matrix(Q4K, up[e * n_ff:(e + 1) * n_ff].reshape(n_ff, gb), n_embd).astype(np.float64)
+        D = oracle.dequant_matrix(Q4K, down[e * n_embd:(e + 1) * n_embd].reshape(n_embd, db), n_ff).astype(np.float64)
+        toks, ks = np.nonzero(idx == e)
+        g, u = X[toks] @ G.T, X[toks] @ U.T
+        with np.errstate(over="ignore"):  # exp(-g) -> inf gives h -> 0, as in fp32
+            h = g / (1.0 + np.exp(-g)) * u
+        out[toks] += w[toks, ks].astype(np.float64)[:, None] * (h @ D.T)
+    return out
+
+
+@pytest.mark.parametrize("n_tok", [1, 5, 40, 100])
+def test_grouped_ffn_small(oracle, n_tok):
+    n_expert, n_embd, n_ff, k = 16, 512, 256, 4
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=300)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=310 + n_tok, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=320 + n_tok), k)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+    want = oracle_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff)
+    err = rel_l2(got, want)
+    assert err <= DESIGNED, err
+    assert err <= CONTRACT
+    # per-token as well: no token may hide behind the others
+    for t in range(n_tok):
+        assert rel_l2(got[t], want[t]) <= 10 * DESIGNED, t
+    assert rel_l2(numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff), want) <= 1e-6
+
+
+def test_grouped_ffn_all_tokens_one_expert(oracle):
+    """37 tokens on one expert: three passes of 16 token slots, the last one ragged."""
+    n_expert, n_embd, n_ff, k, n_tok = 8, 256, 256, 2, 37
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=400)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=401, tokens=n_tok))
+    idx = np.tile(np.array([[5, 2]], np.int32), (n_tok, 1))
+    w = np.tile(np.array([[0.75, 0.25]], np.float32), (n_tok, 1))
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+    want = oracle_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff)
+    assert rel_l2(got, want) <= DESIGNED
+
+
+def test_grouped_ffn_linearity_and_bad_index(oracle):
+    """A pair whose expert index is out of range contributes nothing; weights enter linearly."""
+    n_expert, n_embd, n_ff, k, n_tok = 8, 256, 256, 3, 9
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=500)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=501, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=502), k)
+    full = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+    idx2 = idx.copy()
+    idx2[:, 1] = np.where(np.arange(n_tok) % 2 == 0, -1, n_expert + 3)
+    w0 = w.copy()
+    w0[:, 1] = 0.0
+    dropped = run_ffn(gate, up, down, Xb, idx2, w, n_embd, n_ff, n_expert)
+    zeroed = run_ffn(gate, up, down, Xb, idx, w0, n_embd, n_ff, n_expert)
+    assert np.array_equal(dropped, zeroed + 0.0) or rel_l2(dropped, zeroed) <= 1e-7
+    assert rel_l2(run_ffn(gate, up, down, Xb, idx, 2.0 * w, n_embd, n_ff, n_expert), 2.0 * full) <= 1e-7
+    assert np.array_equal(run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert), full)  # deterministic
+
+
+def test_grouped_ffn_zero_tokens():
+    n_expert, n_embd, n_ff, k = 4, 256, 256, 2
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=600)
+    out = run_ffn(gate, up, down, np.zeros((1, n_embd), np.uint16), np.zeros((0, k), np.int32),
+                  np.zeros((0, k), np.float32), n_embd, n_ff, n_expert)
+    assert out.shape == (0, n_embd)
+
+
+def test_grouped_ffn_rejects_other_types_and_shapes():
+    lib = qlinear.load()
+    d = qlinear.DevBuf(4096)
+    p = d.ptr
+    assert lib.qlin_moe_ffn_dev(synth.GGML_Q8_0, p, p, p, p, p, p, p, 1, 1, 256, 256, 2, p, None) == qlinear.ERR_TYPE
+    assert lib.qlin_moe_ffn_dev(Q4K, p, p, p, p, p, p, p, 1, 1, 250, 256, 2, p, None) == qlinear.ERR_ARG
+    assert lib.qlin_moe_ffn_dev(Q4K, p, p, p, p, p, p, p, 1, 3, 256, 256, 2, p, None) == qlinear.ERR_ARG
+    assert lib.qlin_moe_ffn_dev(Q4K, p, p, p, p, p, p, p, 1, 1, 256, 256, 2, None, None) == qlinear.ERR_ARG
+    d.free()
+
+
+def test_grouped_ffn_full_size(oracle):
+    """128 experts of gate/up 768x2048 and down 2048x768, 64 tokens, top-8 (the MoE benchmark shape)."""
+    n_expert, n_embd, n_ff, k, n_tok = 128, 2048, 768, 8, 64
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=700)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=701, tokens=n_tok))
+    logits = synth.make_router_logits(n_tok, n_expert, seed=702)
+    # route on the device, as a caller would, and check it against the oracle's routing
+    dl = qlinear.DevBuf.from_numpy(logits)
+    di, dw = qlinear.DevBuf(n_tok * k * 4), qlinear.DevBuf(n_tok * k * 4)
+    qlinear.moe_route_dev(dl, n_tok, n_expert, k, di, dw)
+    qlinear.sync()
+    idx, w = di.to_numpy(np.int32, (n_tok, k)), dw.to_numpy(np.float32, (n_tok, k))
+    oi, ow = route(oracle, logits, k)
+    assert np.array_equal(np.sort(idx, axis=1), np.sort(oi, axis=1))
+    assert np.allclose(np.sort(w, axis=1), np.sort(ow, axis=1), rtol=1e-5)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff)
+    err = rel_l2(got, want)
+    assert err <= DESIGNED, err
+    for t in (0, 17, 63):  # the per-token oracle on a few tokens ties the numpy restatement to it
+        one = oracle.moe_ffn_token(Q4K, gate, up, down, n_embd, n_ff, synth.bf16_bits_to_f32(Xb[t]), idx[t], w[t], f64=True)
+        assert rel_l2(want[t], one) <= 1e-6
+        assert rel_l2(got[t], one) <= 10 * DESIGNED
