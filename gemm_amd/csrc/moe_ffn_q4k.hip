@@ -176,50 +176,100 @@ __device__ __forceinline__ void apply_scales(f32x4 &acc, f32x4 S0, f32x4 S1, f32
     }
 }
 
-/* one 64-element slice c of a super-block for one weight row pointer `blk` (start of the super-block):
- * the lane's 8 bytes give its 8 codes of sub-block 2c (low nibbles) and of 2c+1 (high nibbles) */
-template <int C>
-__device__ __forceinline__ void slice_codes(const uint8_t *blk, int kg, bf16x8 &b_lo, bf16x8 &b_hi) {
-    const u32x2 q = *(const u32x2 *)(blk + 16 + 32 * C + 8 * kg);
-    b_lo = codes_to_bf16(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu);
-    b_hi = codes_to_bf16((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu);
+/* Raw registers of one super-block step of a wavefront: for each of its NW weight streams (a
+ * stream = 16 rows of one matrix, one row per lane group) the 16 header bytes and the lane's
+ * 4 x 8 code bytes; for each of its NA activation operands the lane's eight 16-byte pieces.
+ * Two of these are kept in flight: the loads of step sb+1 are issued before the arithmetic of
+ * step sb, which is what hides the HBM latency at one or two wavefronts per SIMD. */
+template <int NW, int NA>
+struct Step {
+    u32x4 hdr[NW];
+    u32x2 q[NW][4];
+    u32x4 a[NA][8]; /* [operand][2*c + half]: elements 64c + 32*half + 8*kg .. +7 of the super-block */
+};
+
+template <int NW, int NA>
+__device__ __forceinline__ void load_step(Step<NW, NA> &s, const uint8_t *const (&wrow)[NW],
+                                          const uint16_t *const (&arow)[NA], int sb, int kg, bool live) {
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+        const uint8_t *blk = wrow[w] + (size_t)sb * kQ4KBlock;
+        s.hdr[w] = *(const u32x4 *)blk;
+#pragma unroll
+        for (int c = 0; c < 4; c++) s.q[w][c] = *(const u32x2 *)(blk + 16 + 32 * c + 8 * kg);
+    }
+#pragma unroll
+    for (int v = 0; v < NA; v++) {
+        const uint16_t *xk = arow[v] + sb * 256 + 8 * kg;
+#pragma unroll
+        for (int p = 0; p < 8; p++) {
+            u32x4 t = {0u, 0u, 0u, 0u};
+            if (live) t = *(const u32x4 *)(xk + 32 * p);
+            s.a[v][p] = t;
+        }
+    }
+}
+
+template <int C, int NW, int NA>
+__device__ __forceinline__ void slice_math(const Step<NW, NA> &s, const Scales (&sc)[NW], f32x4 (&acc)[NW]) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    bf16x8 a0[NA], a1[NA];
+    f32x4 X0 = zero, X1 = zero;
+#pragma unroll
+    for (int v = 0; v < NA; v++) {
+        a0[v] = __builtin_bit_cast(bf16x8, s.a[v][2 * C]);
+        a1[v] = __builtin_bit_cast(bf16x8, s.a[v][2 * C + 1]);
+        X0 = mma(a0[v], ones_bf16(), X0);
+        X1 = mma(a1[v], ones_bf16(), X1);
+    }
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+        /* the lane's 8 bytes hold its 8 codes of sub-block 2c (low nibbles) and of 2c+1 (high nibbles) */
+        const u32x2 q = s.q[w][C];
+        const bf16x8 lo = codes_to_bf16(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu);
+        const bf16x8 hi = codes_to_bf16((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu);
+        f32x4 S0 = zero, S1 = zero;
+#pragma unroll
+        for (int v = 0; v < NA; v++) {
+            S0 = mma(a0[v], lo, S0);
+            S1 = mma(a1[v], hi, S1);
+        }
+        float dsc0, dm0, dsc1, dm1;
+        sub_scales<2 * C>(sc[w], dsc0, dm0);
+        sub_scales<2 * C + 1>(sc[w], dsc1, dm1);
+        apply_scales(acc[w], S0, S1, X0, X1, dsc0, dm0, dsc1, dm1);
+    }
+}
+
+template <int NW, int NA>
+__device__ __forceinline__ void step_math(const Step<NW, NA> &s, f32x4 (&acc)[NW]) {
+    Scales sc[NW];
+#pragma unroll
+    for (int w = 0; w < NW; w++) sc[w] = unpack_header(s.hdr[w]);
+    slice_math<0>(s, sc, acc);
+    slice_math<1>(s, sc, acc);
+    slice_math<2>(s, sc, acc);
+    slice_math<3>(s, sc, acc);
+}
+
+/* all super-blocks of the rows in wrow[] against the activations in arow[], two steps in flight */
+template <int NW, int NA>
+__device__ __forceinline__ void stream_rows(const uint8_t *const (&wrow)[NW], const uint16_t *const (&arow)[NA],
+                                            int n_sb, int kg, bool live, f32x4 (&acc)[NW]) {
+    Step<NW, NA> ping, pong;
+    load_step(ping, wrow, arow, 0, kg, live);
+    for (int sb = 0; sb < n_sb; sb += 2) {
+        const bool has1 = sb + 1 < n_sb, has2 = sb + 2 < n_sb;
+        if (has1) load_step(pong, wrow, arow, sb + 1, kg, live);
+        step_math(ping, acc);
+        if (has1) {
+            if (has2) load_step(ping, wrow, arow, sb + 2, kg, live);
+            step_math(pong, acc);
+        }
+    }
 }
 
 /* ---- 2. gate and up for 32 rows of one expert, all of its tokens ---- */
-template <int C>
-__device__ __forceinline__ void gate_up_slice(const uint8_t *g0, const uint8_t *g1, const uint8_t *u0,
-                                              const uint8_t *u1, const Scales &sg0, const Scales &sg1,
-                                              const Scales &su0, const Scales &su1, const uint16_t *xk, bool live,
-                                              int kg, f32x4 &ag0, f32x4 &ag1, f32x4 &au0, f32x4 &au1) {
-    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bf16x8 a0 = load_a(xk + 64 * C + 8 * kg, live);
-    const bf16x8 a1 = load_a(xk + 64 * C + 32 + 8 * kg, live);
-    const f32x4 X0 = mma(a0, ones_bf16(), zero);
-    const f32x4 X1 = mma(a1, ones_bf16(), zero);
-    bf16x8 lo, hi;
-    float dsc0, dm0, dsc1, dm1;
-
-    slice_codes<C>(g0, kg, lo, hi);
-    sub_scales<2 * C>(sg0, dsc0, dm0);
-    sub_scales<2 * C + 1>(sg0, dsc1, dm1);
-    apply_scales(ag0, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
-
-    slice_codes<C>(g1, kg, lo, hi);
-    sub_scales<2 * C>(sg1, dsc0, dm0);
-    sub_scales<2 * C + 1>(sg1, dsc1, dm1);
-    apply_scales(ag1, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
-
-    slice_codes<C>(u0, kg, lo, hi);
-    sub_scales<2 * C>(su0, dsc0, dm0);
-    sub_scales<2 * C + 1>(su0, dsc1, dm1);
-    apply_scales(au0, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
-
-    slice_codes<C>(u1, kg, lo, hi);
-    sub_scales<2 * C>(su1, dsc0, dm0);
-    sub_scales<2 * C + 1>(su1, dsc1, dm1);
-    apply_scales(au1, mma(a0, lo, zero), mma(a1, hi, zero), X0, X1, dsc0, dm0, dsc1, dm1);
-}
-
 __device__ __forceinline__ void store_h(uint16_t *h_hi, uint16_t *h_lo, size_t at, float g, float u) {
     const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
     const __bf16 hi = (__bf16)h;
@@ -228,7 +278,10 @@ __device__ __forceinline__ void store_h(uint16_t *h_hi, uint16_t *h_lo, size_t a
     h_lo[at] = __builtin_bit_cast(uint16_t, lo);
 }
 
-__global__ void __launch_bounds__(256)
+#ifndef MOE_WAVES
+#define MOE_WAVES 2
+#endif
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
 moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
                    const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
                    const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
@@ -242,67 +295,31 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
     const int j = lane & 15, kg = lane >> 4;
     const int n_sb = n_embd >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
-    const size_t ebase = (size_t)e * n_ff * row_bytes;
-    const uint8_t *g0 = gate + ebase + (size_t)(row0 + j) * row_bytes;
-    const uint8_t *g1 = g0 + 16 * row_bytes;
-    const uint8_t *u0 = up + ebase + (size_t)(row0 + j) * row_bytes;
-    const uint8_t *u1 = u0 + 16 * row_bytes;
+    const size_t ebase = ((size_t)e * n_ff + row0 + j) * row_bytes;
+    const uint8_t *const wrow[4] = {gate + ebase, gate + ebase + 16 * row_bytes, up + ebase,
+                                    up + ebase + 16 * row_bytes};
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt; /* as an A lane, j is the token slot */
         const int tok = live ? order[first + t0 + j] / top_k : 0;
-        const uint16_t *xrow = X + (size_t)tok * n_embd;
-        f32x4 ag0 = {0, 0, 0, 0}, ag1 = {0, 0, 0, 0}, au0 = {0, 0, 0, 0}, au1 = {0, 0, 0, 0};
-        for (int sb = 0; sb < n_sb; sb++) {
-            const size_t o = (size_t)sb * kQ4KBlock;
-            const Scales sg0 = unpack_header(*(const u32x4 *)(g0 + o));
-            const Scales sg1 = unpack_header(*(const u32x4 *)(g1 + o));
-            const Scales su0 = unpack_header(*(const u32x4 *)(u0 + o));
-            const Scales su1 = unpack_header(*(const u32x4 *)(u1 + o));
-            const uint16_t *xk = xrow + sb * 256;
-            gate_up_slice<0>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
-            gate_up_slice<1>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
-            gate_up_slice<2>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
-            gate_up_slice<3>(g0 + o, g1 + o, u0 + o, u1 + o, sg0, sg1, su0, su1, xk, live, kg, ag0, ag1, au0, au1);
-        }
+        const uint16_t *const arow[1] = {X + (size_t)tok * n_embd};
+        f32x4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+        stream_rows<4, 1>(wrow, arow, n_sb, kg, live, acc);
         /* as a C lane: row j, token slots 4*kg + v */
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int ts = t0 + 4 * kg + v;
             if (ts < cnt) {
                 const size_t at = (size_t)(first + ts) * n_ff + row0 + j;
-                store_h(h_hi, h_lo, at, ag0[v], au0[v]);
-                store_h(h_hi, h_lo, at + 16, ag1[v], au1[v]);
+                store_h(h_hi, h_lo, at, acc[0][v], acc[2][v]);
+                store_h(h_hi, h_lo, at + 16, acc[1][v], acc[3][v]);
             }
         }
     }
 }
 
 /* ---- 3. down for 32 rows of one expert ---- */
-template <int C>
-__device__ __forceinline__ void down_slice(const uint8_t *d0, const uint8_t *d1, const Scales &s0, const Scales &s1,
-                                           const uint16_t *hk, const uint16_t *lk, bool live, int kg, f32x4 &a0,
-                                           f32x4 &a1) {
-    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
-    const bf16x8 h0 = load_a(hk + 64 * C + 8 * kg, live), l0 = load_a(lk + 64 * C + 8 * kg, live);
-    const bf16x8 h1 = load_a(hk + 64 * C + 32 + 8 * kg, live), l1 = load_a(lk + 64 * C + 32 + 8 * kg, live);
-    const f32x4 X0 = mma(l0, ones_bf16(), mma(h0, ones_bf16(), zero));
-    const f32x4 X1 = mma(l1, ones_bf16(), mma(h1, ones_bf16(), zero));
-    bf16x8 lo, hi;
-    float dsc0, dm0, dsc1, dm1;
-
-    slice_codes<C>(d0, kg, lo, hi);
-    sub_scales<2 * C>(s0, dsc0, dm0);
-    sub_scales<2 * C + 1>(s0, dsc1, dm1);
-    apply_scales(a0, mma(l0, lo, mma(h0, lo, zero)), mma(l1, hi, mma(h1, hi, zero)), X0, X1, dsc0, dm0, dsc1, dm1);
-
-    slice_codes<C>(d1, kg, lo, hi);
-    sub_scales<2 * C>(s1, dsc0, dm0);
-    sub_scales<2 * C + 1>(s1, dsc1, dm1);
-    apply_scales(a1, mma(l0, lo, mma(h0, lo, zero)), mma(l1, hi, mma(h1, hi, zero)), X0, X1, dsc0, dm0, dsc1, dm1);
-}
-
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                 const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
                 const int32_t *__restrict__ order, const float *__restrict__ expert_w, float *__restrict__ part,
@@ -316,31 +333,23 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
     const int j = lane & 15, kg = lane >> 4;
     const int n_sb = n_ff >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
-    const uint8_t *d0 = down + (size_t)e * n_embd * row_bytes + (size_t)(row0 + j) * row_bytes;
-    const uint8_t *d1 = d0 + 16 * row_bytes;
+    const uint8_t *d0 = down + ((size_t)e * n_embd + row0 + j) * row_bytes;
+    const uint8_t *const wrow[2] = {d0, d0 + 16 * row_bytes};
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt;
-        const size_t arow = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
-        f32x4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
-        for (int sb = 0; sb < n_sb; sb++) {
-            const size_t o = (size_t)sb * kQ4KBlock;
-            const Scales s0 = unpack_header(*(const u32x4 *)(d0 + o));
-            const Scales s1 = unpack_header(*(const u32x4 *)(d1 + o));
-            const uint16_t *hk = h_hi + arow + sb * 256, *lk = h_lo + arow + sb * 256;
-            down_slice<0>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
-            down_slice<1>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
-            down_slice<2>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
-            down_slice<3>(d0 + o, d1 + o, s0, s1, hk, lk, live, kg, a0, a1);
-        }
+        const size_t at_a = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
+        const uint16_t *const arow[2] = {h_hi + at_a, h_lo + at_a};
+        f32x4 acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+        stream_rows<2, 2>(wrow, arow, n_sb, kg, live, acc);
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const int ts = t0 + 4 * kg + v;
             if (ts < cnt) {
                 const float w = expert_w[order[first + ts]];
                 const size_t at = (size_t)(first + ts) * n_embd + row0 + j;
-                part[at] = w * a0[v];      /* w * q, as out[i] += w*q does (:4116-4127) */
-                part[at + 16] = w * a1[v];
+                part[at] = w * acc[0][v];      /* w * q, as out[i] += w*q does (:4116-4127) */
+                part[at + 16] = w * acc[1][v];
             }
         }
     }

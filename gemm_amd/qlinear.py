@@ -9,7 +9,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libqlinear.so")
+# QLINEAR_LIB names another build of the same library (e.g. an experimental one); default: the in-tree build
+LIB_PATH = os.environ.get("QLINEAR_LIB") or os.path.join(_HERE, "libqlinear.so")
 
 OK, ERR_TYPE, ERR_ARG, ERR_DEVICE, ERR_NOMEM = 0, -1, -2, -3, -4
 
