@@ -83,6 +83,24 @@ def time_gemm(n_tok, n_rows, n_cols, steps, warmup):
     return ms / steps
 
 
+def time_host_boundary(n_rows, n_cols, calls=200):
+    """qlin_matvec through host pointers: W registered (resident in HBM), x uploaded and y downloaded
+    on every call. -> ms per call"""
+    lib = qlinear.load()
+    W = synth.make_weights(Q4K, n_rows, n_cols, seed=77)
+    x = synth.make_activation(n_cols, seed=78)
+    y = np.zeros(n_rows, np.float32)
+    qlinear.check(lib.qlin_weight_register(W.ctypes.data, W.nbytes))
+    for _ in range(5):
+        qlinear.check(lib.qlin_matvec(y.ctypes.data, W.ctypes.data, Q4K, n_cols, x.ctypes.data, n_rows))
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        qlinear.check(lib.qlin_matvec(y.ctypes.data, W.ctypes.data, Q4K, n_cols, x.ctypes.data, n_rows))
+    dt = (time.perf_counter() - t0) / calls
+    qlinear.check(lib.qlin_weight_unregister(W.ctypes.data))
+    return dt * 1e3
+
+
 def time_moe(steps, warmup, n_expert=128, n_embd=2048, n_ff=768, top_k=8, n_tok=64, copies=2):
     """Grouped MoE expert FFN: -> (ms per step, algorithmic bytes per step, flops per step)"""
     sets = []
@@ -215,6 +233,9 @@ def main():
                                               "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),
                                               "traffic": None}
 
+        hb = time_host_boundary(n_rows, n_cols)
+        extra["host_pointer_matvec_14336x4096"] = {"us": round(hb * 1e3, 1), "GB/s": round(nbytes / (hb * 1e-3) / 1e9, 1),
+                                                  "note": "W registered; x H2D and y D2H every call"}
         m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
         extra["q4k_moe_ffn_128x(768x2048)_64tok_top8"] = {
             "us": round(m * 1e3, 1), "routed_experts": routed, "bytes": b, "GB/s": round(b / (m * 1e-3) / 1e9, 1),

@@ -14,6 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libqlinear.so")
+TF_LIB = os.path.join(HERE, "libqlinear_tf.so")
 SOURCES = ["qlin_api.hip", "dequant.hip", "gemv_generic.hip", "gemv_q4k.hip", "gemm_q4k_mfma.hip", "moe.hip", "moe_ffn_q4k.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -42,7 +43,29 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", LIB, os.path.getsize(LIB), "bytes")
+    build_host(verbose)
     return LIB
+
+
+def build_host(verbose=True):
+    """The plain-C layer with the reference's call shapes (libqlinear_tf.so) and its C test program."""
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    common = ["gcc", "-O2", "-std=c11", "-Wall", "-Wextra", "-fPIC", "-I", inc]
+    link = ["-L", HERE, "-lqlinear", "-Wl,-rpath,$ORIGIN"]
+    r = subprocess.run(common + ["-shared", "-o", TF_LIB, os.path.join(HERE, "host", "qlinear_tf.c")] + link,
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("gcc failed on qlinear_tf.c:\n" + r.stderr)
+    tests_c = os.path.join(os.path.dirname(HERE), "tests", "c")
+    exe = os.path.join(tests_c, "test_tf_mirror")
+    r = subprocess.run(common + ["-o", exe, os.path.join(tests_c, "test_tf_mirror.c"), "-L", HERE, "-lqlinear_tf",
+                                 "-lqlinear", "-lm", "-Wl,-rpath,$ORIGIN/../../gemm_amd"], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("gcc failed on test_tf_mirror.c:\n" + r.stderr)
+    if r.stderr.strip():
+        sys.stderr.write(r.stderr)
+    if verbose:
+        print("built", TF_LIB, "and", exe)
 
 
 if __name__ == "__main__":

@@ -49,3 +49,22 @@ def test_row_size_matches_reference_manifest(lib, manifest):
     for t, per_n in manifest["row_size"].items():
         for n, want in per_n.items():
             assert lib.qlin_dequant_row_size(int(t), int(n)) == want, (t, n)
+
+
+def test_reference_shaped_layer_exports_its_header():
+    """libqlinear_tf.so (plain C over the ABI) exports every function include/qlinear_tf.h declares."""
+    import ctypes
+    from gemm_amd import build
+    if not os.path.exists(build.TF_LIB):
+        build.build_host(verbose=False)
+    text = open(os.path.join(ROOT, "include", "qlinear_tf.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    text = re.sub(r"^#.*$", "", text, flags=re.M)
+    names = sorted(set(re.findall(r"\b(qtf_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) >= 13
+    tf = ctypes.CDLL(build.TF_LIB)
+    for name in names:
+        assert hasattr(tf, name), name
+    tf.qtf_row_bytes.restype = ctypes.c_size_t
+    assert tf.qtf_row_bytes(12, 4096) == 2304
+    assert tf.qtf_is_supported_weight_type(14) == 1 and tf.qtf_is_supported_weight_type(3) == 0
