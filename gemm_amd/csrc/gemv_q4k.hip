@@ -9,11 +9,17 @@
  *     "digit planes" in LDS (top byte signed, lower two unsigned) together with 2^(e-22) and
  *     the fp32 sum of the sub-block. Quantisation error is 2^-23 of the sub-block's largest
  *     |x|; measured end-to-end error is ~7e-7 relative L2 against the double-precision oracle.
- *  2. Weights are streamed as a FLAT byte stream: a wavefront reads a row (or a slice of at
- *     most 16 super-blocks = 2304 bytes of it) with three fully contiguous 16-byte-per-lane
- *     loads, two rows ahead of the arithmetic, and drops the bytes into a private LDS row
- *     image. Only this pattern reaches the streaming rate of a plain copy kernel; lane-owned
- *     strided 16-byte loads cost 40 % more time on this part.
+ *  2. Weights are streamed as a FLAT byte stream: a wavefront moves a row (or a slice of at
+ *     most 16 super-blocks = 2304 bytes of it) with up to three fully contiguous
+ *     16-byte-per-lane loads that write straight into a private LDS row image
+ *     (global_load_lds_dwordx4: no registers are held while the data is in flight). Only the
+ *     flat pattern reaches the streaming rate of a plain copy kernel; lane-owned strided
+ *     16-byte loads cost 40 % more time on this part. One row per wavefront in flight (16
+ *     per compute unit, 9.4 MB over the chip) already runs HBM at the rate it gives a burst of
+ *     this size; deeper rings (the code takes up to four images) measured slower, because
+ *     they only lengthen the queue in front of the x loads and of each wave's last row.
+ *     The x loads of all 16 waves are issued before any row load (a barrier separates them),
+ *     so the x preparation overlaps the first rows instead of waiting behind them.
  *  3. Arithmetic re-reads the row image in the layout it wants: four lanes per super-block,
  *     lane c takes nibble bytes qs[32c..32c+31] = sub-blocks 2c (low nibbles) and 2c+1 (high
  *     nibbles). The nibbles are masked into bytes and multiplied with the digit planes by
@@ -34,11 +40,19 @@ namespace qlin {
 
 namespace {
 
-constexpr int kWaves = 16;          /* wavefronts per workgroup */
+#ifndef Q4K_WAVES
+#define Q4K_WAVES 16
+#endif
+constexpr int kWaves = Q4K_WAVES;   /* wavefronts per workgroup: 16 or 8 (a multiple of 4, the most slices) */
 constexpr int kThreads = kWaves * 64;
+constexpr int kXPre = 4096 / kThreads; /* x loads per thread (4 elements each), all issued ahead of the rows: covers K <= 16384 */
 constexpr int kChunk = 52;          /* dwords per 64-element x chunk: 3 planes x 16, padded so that
                                        consecutive lanes' 16-byte reads fall on distinct banks */
-constexpr int kRowImage = 3072;     /* bytes per LDS row image: 2304 + room for the full-wave tail store */
+constexpr int kRowImage = 2304;     /* bytes per LDS row image: 16 super-blocks */
+#ifndef Q4K_MAX_DEPTH
+#define Q4K_MAX_DEPTH 1
+#endif
+constexpr int kMaxDepth = Q4K_MAX_DEPTH; /* row images per wavefront */
 constexpr int kMaxRowsPerWg = 128;
 
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
@@ -59,20 +73,38 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 __device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_udot4(a, b, c, false); }
 
-struct RowRegs { uint4 a, b, c; };
+/* wait until at most n vector-memory operations of this wavefront are outstanding (they retire
+ * in order, so the oldest ones are then complete); n is wave-uniform, at most 12 */
+__device__ __forceinline__ void wait_vm_at_most(int n) {
+    switch (n) {
+    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
+    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
+    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
+    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
+    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+    case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
+    default: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+    }
+}
 
 }  // namespace
 
 __global__ void __launch_bounds__(kThreads)
 gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
-                int n_rows, int n_sb, int n_slices, int slice_sb, int rows_per_wg) {
+                int n_rows, int n_sb, int n_slices, int slice_sb, int rows_per_wg, int depth) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    /* LDS map: planes [n_sb*4][kChunk] dwords | meta [n_sb*4] float4 | row images [16][2][kRowImage] |
+    /* LDS map: planes [n_sb*4][kChunk] dwords | meta [n_sb*4] float4 | row images [16][depth][kRowImage] |
      * partial sums [rows_per_wg * n_slices] floats */
     uint32_t *planes = reinterpret_cast<uint32_t *>(lds);
     float4 *meta = reinterpret_cast<float4 *>(planes + n_sb * 4 * kChunk);
     uint8_t *images = reinterpret_cast<uint8_t *>(meta + n_sb * 4);
-    float *partial = reinterpret_cast<float *>(images + kWaves * 2 * kRowImage);
+    float *partial = reinterpret_cast<float *>(images + kWaves * depth * kRowImage);
 
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int c = lane & 3;
@@ -83,7 +115,8 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     const bool active = (lane >> 2) < sb_cnt;
     const int sb_local = active ? (lane >> 2) : 0;
     const size_t row_bytes = (size_t)n_sb * 144;
-    const int last_chunk = sb_cnt * 9 - 1; /* last 16-byte chunk of this wave's slice of a row */
+    const int n_chunks = sb_cnt * 9;                  /* 16-byte chunks in this wave's slice of a row */
+    const int loads_per_row = (n_chunks + 63) >> 6;   /* wave-uniform: 1, 2 or 3 */
 
     const int row0 = blockIdx.x * rows_per_wg; /* first real row of this workgroup */
     int rows_here = n_rows - row0;
@@ -91,34 +124,63 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     const int n_vrows = rows_here * n_slices; /* (row, slice) pairs of this workgroup */
 
     /* this wave's virtual rows: wv, wv + 16, ... ; virtual row j = (row j / S, slice j % S), and
-     * 16 % S == 0 keeps the slice of a wave fixed */
+     * 16 % S == 0 keeps the slice of a wave fixed. my_rows of them, numbered i = 0.. */
+    const int my_rows = wv < n_vrows ? (n_vrows - wv + kWaves - 1) / kWaves : 0;
     const uint8_t *slice_base = W + (size_t)row0 * row_bytes + (size_t)sb0 * 144;
-    const int i0 = lane < last_chunk ? lane : last_chunk;
-    const int i1 = 64 + lane < last_chunk ? 64 + lane : last_chunk;
-    const int i2 = 128 + (lane & 15) < last_chunk ? 128 + (lane & 15) : last_chunk;
-    auto fetch = [&](int j) {
-        if (j >= n_vrows) j = wv < n_vrows ? wv : 0; /* stay in bounds; the value is never used */
-        const uint4 *q = reinterpret_cast<const uint4 *>(slice_base + (size_t)(j / n_slices) * row_bytes);
-        /* streamed once: non-temporal, so that x and the codebooks are not pushed out of L2 */
-        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-        const u32x4 *qv = reinterpret_cast<const u32x4 *>(q);
-        const u32x4 va = __builtin_nontemporal_load(qv + i0), vb = __builtin_nontemporal_load(qv + i1),
-                    vc = __builtin_nontemporal_load(qv + i2);
-        RowRegs t;
-        t.a = make_uint4(va.x, va.y, va.z, va.w);
-        t.b = make_uint4(vb.x, vb.y, vb.z, vb.w);
-        t.c = make_uint4(vc.x, vc.y, vc.z, vc.w);
-        return t;
+    uint8_t *my_images = images + wv * (depth * kRowImage);
+    const uint32_t my_images_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)my_images;
+    /* Row i of this wave -> image slot i % depth; exactly loads_per_row instructions are issued.
+     * Each is a 16-byte-per-lane load whose data goes to LDS at M0 + 16*lane instead of to
+     * registers. They are written as instructions: for the builtin form the compiler, which
+     * cannot tell the images apart, waits for every outstanding one before any LDS access, and
+     * that would serialise the ring. The waits this kernel needs are placed by hand
+     * (wait_vm_at_most before an image is read, lgkmcnt(0) before its slot is refilled).
+     * Nothing else in this kernel uses M0. */
+    auto issue = [&](int i) {
+        const int j = wv + i * kWaves;
+        const uint4 *g = reinterpret_cast<const uint4 *>(slice_base + (size_t)(j / n_slices) * row_bytes);
+        const uint32_t img = __builtin_amdgcn_readfirstlane(my_images_lds + (uint32_t)((i % depth) * kRowImage));
+#define QLIN_LOAD_TO_LDS(chunk0)                                                                          \
+        if ((chunk0) + lane < n_chunks)                                                                   \
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"                 \
+                         : : "v"(g + (chunk0) + lane), "s"(img + 16u * (chunk0)) : "memory")
+        QLIN_LOAD_TO_LDS(0);
+        QLIN_LOAD_TO_LDS(64);
+        QLIN_LOAD_TO_LDS(128);
+#undef QLIN_LOAD_TO_LDS
     };
-    /* weights first: two rows in flight per wave while x is being prepared */
-    RowRegs p0 = fetch(wv), p1 = fetch(wv + kWaves);
 
-    /* ---- x -> digit planes (whole workgroup, 4 elements per thread and step) */
-    {
-        const int n4 = n_sb * 64;
-        const float4 *xg = reinterpret_cast<const float4 *>(x);
-        for (int idx = threadIdx.x; idx < n4; idx += kThreads) {
-            const float4 v = xg[idx];
+    /* x is requested first, so that it does not queue behind the weight stream; then up to `depth`
+     * rows per wave are put in flight while x is being prepared.
+     * The first x load is written as an instruction, not as a C++ load: the compiler would sink a
+     * C++ load next to its use, below the weight loads, and since loads retire in order the x
+     * preparation would then wait for the rows. The memory clobbers keep the row loads between
+     * the two statements, so "at most that many outstanding" means that x has arrived. */
+    const int n4 = n_sb * 64;
+    const float4 *xg = reinterpret_cast<const float4 *>(x);
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    f32x4 xv[kXPre];
+#pragma unroll
+    for (int u = 0; u < kXPre; u++) {
+        xv[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (u * kThreads < n4) { /* uniform */
+            const int idx = u * kThreads + threadIdx.x;
+            const float4 *xp = xg + (idx < n4 ? idx : 0);
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(xv[u]) : "v"(xp) : "memory");
+        }
+    }
+    /* every wave's x request enters the memory pipeline before any wave's row requests */
+    asm volatile("s_barrier" ::: "memory");
+    int issued = 0;
+    for (; issued < depth && issued < my_rows; issued++) issue(issued);
+    wait_vm_at_most(issued * loads_per_row);
+#pragma unroll
+    for (int u = 0; u < kXPre; u++) asm volatile("" : "+v"(xv[u]) : : "memory");
+
+    /* ---- x -> digit planes (whole workgroup, 4 elements per thread and step); no loads in here,
+     * so nothing in it waits for the weights */
+    auto quantize = [&](int idx, const float4 v) {
+            const bool mine = idx < n4;
             float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
             float sum = (v.x + v.y) + (v.z + v.w);
             /* 8 consecutive threads share one 32-element sub-block */
@@ -146,16 +208,20 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
             const int sub = idx >> 3, j = idx & 7;
             const int chunk = sub >> 1, is_b = sub & 1;
             uint32_t *dst = planes + chunk * kChunk + is_b * 8 + j;
-            dst[0] = pl_top;
-            dst[16] = pl_mid;
-            dst[32] = pl_low;
-            if (j == 0) {
+            if (mine) {
+                dst[0] = pl_top;
+                dst[16] = pl_mid;
+                dst[32] = pl_low;
+            }
+            if (mine && j == 0) {
                 float *m = reinterpret_cast<float *>(meta + chunk);
                 m[is_b] = inv;
                 m[2 + is_b] = sum;
             }
-        }
-    }
+    };
+#pragma unroll
+    for (int u = 0; u < kXPre; u++)
+        if (u * kThreads < n4) quantize(u * kThreads + threadIdx.x, make_float4(xv[u].x, xv[u].y, xv[u].z, xv[u].w));
     __syncthreads();
 
     /* this lane's x: 16 dwords per plane (8 for sub-block 2c, 8 for 2c+1) */
@@ -173,17 +239,19 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     const float4 mt = meta[(sb0 + sb_local) * 4 + c];
     const float inv_a = mt.x, inv_b = mt.y, sum_a = mt.z, sum_b = mt.w;
 
-    uint8_t *my_images = images + wv * (2 * kRowImage);
-    auto process = [&](RowRegs &p, int j, int slot) {
-        uint8_t *img = my_images + slot * kRowImage;
-        *reinterpret_cast<uint4 *>(img + 16 * lane) = p.a;
-        *reinterpret_cast<uint4 *>(img + 1024 + 16 * lane) = p.b;
-        *reinterpret_cast<uint4 *>(img + 2048 + 16 * lane) = p.c; /* lanes >= 16 land in the pad */
-        p = fetch(j + 2 * kWaves);
-        const uint8_t *blk = img + sb_local * 144;
+    for (int i = 0; i < my_rows; i++) {
+        /* rows i .. issued-1 are in flight; row i is the oldest */
+        wait_vm_at_most((issued - i - 1) * loads_per_row);
+        const uint8_t *blk = my_images + (i % depth) * kRowImage + sb_local * 144;
         const uint4 h = *reinterpret_cast<const uint4 *>(blk);
         const uint4 qa = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c);
         const uint4 qb = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * c);
+        /* the image may be overwritten once these reads have returned */
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (issued < my_rows) {
+            issue(issued);
+            issued++;
+        }
         const float d = half_bits_fast(h.x & 0xFFFFu), dmin = half_bits_fast(h.x >> 16);
         /* bytes of sc_lo: scales 0..3, mn_lo: mins 0..3, sc_hi: scales 4..7, mn_hi: mins 4..7 */
         const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
@@ -195,14 +263,14 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
         int at = 0, bt = 0;
         uint32_t am = 0, al = 0, bm = 0, bl = 0;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t lo = w[i] & 0x0F0F0F0Fu, hi = (w[i] >> 4) & 0x0F0F0F0Fu;
-            at = sdot4(lo, xt[i], at);
-            am = udot4(lo, xm[i], am);
-            al = udot4(lo, xl[i], al);
-            bt = sdot4(hi, xt[8 + i], bt);
-            bm = udot4(hi, xm[8 + i], bm);
-            bl = udot4(hi, xl[8 + i], bl);
+        for (int k = 0; k < 8; k++) {
+            const uint32_t lo = w[k] & 0x0F0F0F0Fu, hi = (w[k] >> 4) & 0x0F0F0F0Fu;
+            at = sdot4(lo, xt[k], at);
+            am = udot4(lo, xm[k], am);
+            al = udot4(lo, xl[k], al);
+            bt = sdot4(hi, xt[8 + k], bt);
+            bm = udot4(hi, xm[8 + k], bm);
+            bl = udot4(hi, xl[8 + k], bl);
         }
         /* |top| <= 32*15*64, mid/low <= 32*15*255: the low part fits an int exactly */
         const float fa = fmaf((float)at, 65536.0f, (float)((am << 8) + al)) * inv_a;
@@ -211,12 +279,7 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
         const float ma = dmin * (float)(mn2 & 0xFFu), mb = dmin * (float)((mn2 >> 8) & 0xFFu);
         float v = active ? (da * fa + db * fb - (ma * sum_a + mb * sum_b)) : 0.0f;
         v = wave_sum_dpp(v);
-        if (lane == 0 && j < n_vrows) partial[j] = v;
-    };
-
-    for (int j = wv; j < n_vrows; j += 2 * kWaves) {
-        process(p0, j, 0);
-        process(p1, j + kWaves, 1);
+        if (lane == 0) partial[wv + i * kWaves] = v;
     }
     __syncthreads();
 
@@ -226,6 +289,7 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
         for (int k = 0; k < n_slices; k++) s += partial[r * n_slices + k];
         y[row0 + r] = s;
     }
+
 }
 
 /* Launch geometry: one 16-wave workgroup per block of rows, sized so that the grid covers the
@@ -241,9 +305,11 @@ hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, 
     if (rows_per_wg < 1) rows_per_wg = 1;
     if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
-    const size_t lds_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 +
-                             (size_t)kWaves * 2 * kRowImage + (size_t)rows_per_wg * n_slices * 4;
-    if (lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+    const size_t fixed_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 + (size_t)rows_per_wg * n_slices * 4;
+    if (fixed_bytes + (size_t)kWaves * kRowImage > 160 * 1024) return hipErrorInvalidValue;
+    int depth = (int)((160 * 1024 - fixed_bytes) / ((size_t)kWaves * kRowImage));
+    if (depth > kMaxDepth) depth = kMaxDepth;
+    const size_t lds_bytes = fixed_bytes + (size_t)kWaves * depth * kRowImage;
     if (!lds_raised) {
         hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_kernel,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -251,7 +317,7 @@ hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, 
         lds_raised = true;
     }
     hipLaunchKernelGGL(gemv_q4k_kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, (const uint8_t *)W, x, y,
-                       n_rows, n_sb, n_slices, slice_sb, rows_per_wg);
+                       n_rows, n_sb, n_slices, slice_sb, rows_per_wg, depth);
     return hipGetLastError();
 }
 
