@@ -177,6 +177,10 @@ def probe(args):
     elif args.probe == "gemv":
         ms, copies = time_gemv(Q4K, 14336, 4096, args.steps, args.warmup)
         print(json.dumps({"probe": "gemv", "ms_per_step": ms, "copies": copies}))
+    elif args.probe in ("gemv_q8_0", "gemv_q6_K"):
+        tid, r, c = (synth.GGML_Q8_0, 4096, 4096) if args.probe == "gemv_q8_0" else (synth.GGML_Q6_K, 151936, 4096)
+        ms, copies = time_gemv(tid, r, c, max(10, args.steps // 8), 3, max_copies=24 if r < 100000 else 2)
+        print(json.dumps({"probe": args.probe, "ms_per_step": ms, "copies": copies}))
     elif args.probe == "moe":
         m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
         print(json.dumps({"probe": "moe", "ms_per_step": m, "bytes": b, "routed": routed}))
@@ -192,7 +196,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemm", "moe"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemm", "moe"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "

@@ -45,7 +45,6 @@ namespace {
 #endif
 constexpr int kWaves = Q4K_WAVES;   /* wavefronts per workgroup: 16 or 8 (a multiple of 4, the most slices) */
 constexpr int kThreads = kWaves * 64;
-constexpr int kXPre = 4096 / kThreads; /* x loads per thread (4 elements each), all issued ahead of the rows: covers K <= 16384 */
 constexpr int kChunk = 52;          /* dwords per 64-element x chunk: 3 planes x 16, padded so that
                                        consecutive lanes' 16-byte reads fall on distinct banks */
 constexpr int kRowImage = 2304;     /* bytes per LDS row image: 16 super-blocks */
@@ -73,26 +72,6 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 __device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_udot4(a, b, c, false); }
 
-/* wait until at most n vector-memory operations of this wavefront are outstanding (they retire
- * in order, so the oldest ones are then complete); n is wave-uniform, at most 12 */
-__device__ __forceinline__ void wait_vm_at_most(int n) {
-    switch (n) {
-    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    case 1: asm volatile("s_waitcnt vmcnt(1)" ::: "memory"); break;
-    case 2: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-    case 3: asm volatile("s_waitcnt vmcnt(3)" ::: "memory"); break;
-    case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-    case 5: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
-    case 6: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-    case 7: asm volatile("s_waitcnt vmcnt(7)" ::: "memory"); break;
-    case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-    case 9: asm volatile("s_waitcnt vmcnt(9)" ::: "memory"); break;
-    case 10: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-    case 11: asm volatile("s_waitcnt vmcnt(11)" ::: "memory"); break;
-    default: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-    }
-}
-
 }  // namespace
 
 __global__ void __launch_bounds__(kThreads)
@@ -100,11 +79,12 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
                 int n_rows, int n_sb, int n_slices, int slice_sb, int rows_per_wg, int depth) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     /* LDS map: planes [n_sb*4][kChunk] dwords | meta [n_sb*4] float4 | row images [16][depth][kRowImage] |
-     * partial sums [rows_per_wg * n_slices] floats */
+     * partial sums [rows_per_wg * n_slices] floats (padded to 16 bytes) | raw x [n_sb*256] floats */
     uint32_t *planes = reinterpret_cast<uint32_t *>(lds);
     float4 *meta = reinterpret_cast<float4 *>(planes + n_sb * 4 * kChunk);
     uint8_t *images = reinterpret_cast<uint8_t *>(meta + n_sb * 4);
     float *partial = reinterpret_cast<float *>(images + kWaves * depth * kRowImage);
+    const float4 *xraw = reinterpret_cast<const float4 *>(partial + ((rows_per_wg * n_slices + 3) & ~3));
 
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int c = lane & 3;
@@ -150,32 +130,24 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
 #undef QLIN_LOAD_TO_LDS
     };
 
-    /* x is requested first, so that it does not queue behind the weight stream; then up to `depth`
-     * rows per wave are put in flight while x is being prepared.
-     * The first x load is written as an instruction, not as a C++ load: the compiler would sink a
-     * C++ load next to its use, below the weight loads, and since loads retire in order the x
-     * preparation would then wait for the rows. The memory clobbers keep the row loads between
-     * the two statements, so "at most that many outstanding" means that x has arrived. */
+    /* x is requested first, so that it does not queue behind the weight stream: like the rows it
+     * goes straight to LDS (a raw fp32 copy, 1 KB per instruction and wave), so no register holds
+     * data that is still in flight. A barrier makes every wave's x request precede every row
+     * request; then up to `depth` rows per wave are put in flight while x is being prepared.
+     * Loads retire in order, so "at most the row loads outstanding" means that this wave's part
+     * of x has landed; each thread then prepares exactly the elements its own wave fetched. */
     const int n4 = n_sb * 64;
     const float4 *xg = reinterpret_cast<const float4 *>(x);
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-    f32x4 xv[kXPre];
-#pragma unroll
-    for (int u = 0; u < kXPre; u++) {
-        xv[u] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        if (u * kThreads < n4) { /* uniform */
-            const int idx = u * kThreads + threadIdx.x;
-            const float4 *xp = xg + (idx < n4 ? idx : 0);
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(xv[u]) : "v"(xp) : "memory");
-        }
+    const uint32_t xraw_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)xraw;
+    for (int base = wv * 64; base < n4; base += kThreads) { /* uniform per wave */
+        const uint32_t m0v = __builtin_amdgcn_readfirstlane(xraw_lds + 16u * (uint32_t)base);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     : : "v"(xg + base + lane), "s"(m0v) : "memory");
     }
-    /* every wave's x request enters the memory pipeline before any wave's row requests */
     asm volatile("s_barrier" ::: "memory");
     int issued = 0;
     for (; issued < depth && issued < my_rows; issued++) issue(issued);
     wait_vm_at_most(issued * loads_per_row);
-#pragma unroll
-    for (int u = 0; u < kXPre; u++) asm volatile("" : "+v"(xv[u]) : : "memory");
 
     /* ---- x -> digit planes (whole workgroup, 4 elements per thread and step); no loads in here,
      * so nothing in it waits for the weights */
@@ -219,9 +191,7 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
                 m[2 + is_b] = sum;
             }
     };
-#pragma unroll
-    for (int u = 0; u < kXPre; u++)
-        if (u * kThreads < n4) quantize(u * kThreads + threadIdx.x, make_float4(xv[u].x, xv[u].y, xv[u].z, xv[u].w));
+    for (int idx = threadIdx.x; idx < n4; idx += kThreads) quantize(idx, xraw[idx]);
     __syncthreads();
 
     /* this lane's x: 16 dwords per plane (8 for sub-block 2c, 8 for 2c+1) */
@@ -305,7 +275,8 @@ hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, 
     if (rows_per_wg < 1) rows_per_wg = 1;
     if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
-    const size_t fixed_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 + (size_t)rows_per_wg * n_slices * 4;
+    const size_t fixed_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 +
+                               (size_t)((rows_per_wg * n_slices + 3) & ~3) * 4 + (size_t)n_sb * 256 * 4;
     if (fixed_bytes + (size_t)kWaves * kRowImage > 160 * 1024) return hipErrorInvalidValue;
     int depth = (int)((160 * 1024 - fixed_bytes) / ((size_t)kWaves * kRowImage));
     if (depth > kMaxDepth) depth = kMaxDepth;

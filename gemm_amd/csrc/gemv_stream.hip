@@ -1,0 +1,344 @@
+/*
+ * gemv_stream.hip - batch-1 matvec y = W.x for every supported block type, organised for HBM
+ * streaming (what tf_qmatvec computes, common/transformer.h:1049-1114; the summation order
+ * differs).
+ *
+ * One workgroup per block of rows, about one per compute unit. x is copied once per workgroup
+ * into LDS as fp32. Every wavefront then walks its rows: a row travels from HBM into a private
+ * LDS image as one flat byte stream (fully contiguous 16-byte-per-lane loads that write LDS
+ * directly, global_load_lds_dwordx4), the next row is requested while the current one is
+ * decoded. A lane takes eight consecutive elements per step: the codes are unpacked four bytes
+ * at a time with byte-parallel masks, converted byte-to-float and FMA'd with x; the block scale
+ * goes on once per eight elements, and constant offsets (-128 of Q8_0, -32 of Q6_K, the mins of
+ * Q5_K) are applied to the precomputed sum of the eight x instead of to every element:
+ *     sum (s*q_i - o) x_i = s * sum q_i x_i - o * sum x_i.
+ * The i-quant grids sit in LDS; their sign bits are OR'ed into the converted magnitudes. Results
+ * differ from the decoders' only in rounding (the matvec tolerance is 1e-5, it is not bit-exact
+ * work); fp32 accumulate, one wave reduction per row.
+ *
+ * Shape rules (the launcher returns false and the caller falls back to the plain kernel
+ * otherwise): whole blocks, n_cols <= 16384, row bytes a multiple of 16 and at most 8 KB, W and
+ * x 16-byte aligned.
+ */
+#include "qlin_device.h"
+#include "qlin_internal.h"
+
+namespace qlin {
+
+namespace {
+
+
+/* ---- eight elements of one block against eight x, per type ---- */
+
+__device__ __forceinline__ float ub0(uint32_t v) { float f; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ub1(uint32_t v) { float f; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ub2(uint32_t v) { float f; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ub3(uint32_t v) { float f; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v)); return f; }
+
+/* acc + sum of (unsigned byte i of b) * x_i */
+__device__ __forceinline__ float dot_u4(uint32_t b, const float4 x, float acc) {
+    acc = fmaf(ub0(b), x.x, acc);
+    acc = fmaf(ub1(b), x.y, acc);
+    acc = fmaf(ub2(b), x.z, acc);
+    return fmaf(ub3(b), x.w, acc);
+}
+/* same with sign bit i of `signs` (bits 0..3) applied to term i; magnitudes are non-negative, so
+ * the sign can simply be OR'ed into the converted float */
+__device__ __forceinline__ float dot_u4_signed(uint32_t b, uint32_t signs, const float4 x, float acc) {
+    const uint32_t t = signs << 28; /* bit 3 -> bit 31 */
+    acc = fmaf(__uint_as_float(__float_as_uint(ub0(b)) | ((t << 3) & 0x80000000u)), x.x, acc);
+    acc = fmaf(__uint_as_float(__float_as_uint(ub1(b)) | ((t << 2) & 0x80000000u)), x.y, acc);
+    acc = fmaf(__uint_as_float(__float_as_uint(ub2(b)) | ((t << 1) & 0x80000000u)), x.z, acc);
+    return fmaf(__uint_as_float(__float_as_uint(ub3(b)) | (t & 0x80000000u)), x.w, acc);
+}
+/* 8 (4) bytes at byte offset `off` (even) of a 16-byte aligned LDS image. Misaligned LDS reads
+ * stall the LDS pipeline on this part (they were 3/4 of its busy time in the first version of
+ * this kernel), so the bytes are fetched as aligned dwords and funnel-shifted into place. May
+ * touch up to 4 bytes past the last one asked for. */
+__device__ __forceinline__ uint2 ld8_at(const uint8_t *img, int off) {
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(img + (off & ~3));
+    const uint32_t sh = (uint32_t)(off & 2) * 8u;
+    const uint32_t w0 = q[0], w1 = q[1], w2 = q[2];
+    return make_uint2(__builtin_amdgcn_alignbit(w1, w0, sh), __builtin_amdgcn_alignbit(w2, w1, sh));
+}
+__device__ __forceinline__ uint32_t ld4_at(const uint8_t *img, int off) {
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(img + (off & ~3));
+    return __builtin_amdgcn_alignbit(q[1], q[0], (uint32_t)(off & 2) * 8u);
+}
+
+struct Tables {
+    const uint64_t *grid2; /* iq2xxs grid in LDS */
+    const uint32_t *grid3; /* iq3s grid in LDS */
+    uint32_t nl0, nl1, nl2, nl3; /* the 16 iq4nl values + 128, as bytes */
+};
+
+/* default: the bit-exact decoder (Q4_K reaches this kernel only when the tuned one declines) */
+template <uint32_t T> struct Lean {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float, const Tables &) {
+        const uint8_t *blk = img + boff;
+        float w[8];
+        Codec<T>::decode8(blk, k0, w);
+        return w[0] * xa.x + w[1] * xa.y + w[2] * xa.z + w[3] * xa.w + w[4] * xb.x + w[5] * xb.y + w[6] * xb.z +
+               w[7] * xb.w;
+    }
+};
+
+/* Q8_0 (common/ggml_dequant.h:1479-1489): d * q, q int8 = (q ^ 0x80 as unsigned) - 128 */
+template <> struct Lean<T_Q8_0> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const float d = half_bits_fast(ld_u16(blk));
+        const uint2 q = ld8_at(img, boff + 2 + k0);
+        const float s = dot_u4(q.y ^ 0x80808080u, xb, dot_u4(q.x ^ 0x80808080u, xa, 0.0f));
+        return d * fmaf(-128.0f, xs8, s);
+    }
+};
+
+/* Q5_K (:1620-1651): (d*sc)*(nibble + 16*highbit) - dmin*m */
+template <> struct Lean<T_Q5_K> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const uint4 h = *reinterpret_cast<const uint4 *>(blk);
+        const int g = k0 >> 5, l0 = k0 & 31;
+        /* get_scale_min_k4 (:1582-1590), four fields at a time */
+        const uint32_t scw = g < 4 ? (h.y & 0x3F3F3F3Fu) : ((h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u));
+        const uint32_t mnw = g < 4 ? (h.z & 0x3F3F3F3Fu) : (((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u));
+        const int sh8 = 8 * (g & 3);
+        const float dl = half_bits_fast(h.x & 0xFFFFu) * (float)((scw >> sh8) & 0xFFu);
+        const float ml = half_bits_fast(h.x >> 16) * (float)((mnw >> sh8) & 0xFFu);
+        const uint2 q = *reinterpret_cast<const uint2 *>(blk + 48 + (g >> 1) * 32 + l0);
+        const uint2 qh = *reinterpret_cast<const uint2 *>(blk + 16 + l0);
+        const int sh = (g & 1) * 4;
+        const uint32_t v0 = ((q.x >> sh) & 0x0F0F0F0Fu) | (((qh.x >> g) & 0x01010101u) << 4);
+        const uint32_t v1 = ((q.y >> sh) & 0x0F0F0F0Fu) | (((qh.y >> g) & 0x01010101u) << 4);
+        const float s = dot_u4(v1, xb, dot_u4(v0, xa, 0.0f));
+        return fmaf(dl, s, -ml * xs8);
+    }
+};
+
+/* Q6_K (:1653-1687): (d*sc)*(q - 32), q = low nibble | two high bits << 4 */
+template <> struct Lean<T_Q6_K> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const int half = k0 >> 7, r = k0 & 127, seg = r >> 5, l0 = r & 31;
+        const uint2 ql = ld8_at(img, boff + 64 * half + 32 * (seg & 1) + l0);
+        const uint2 qh = ld8_at(img, boff + 128 + 32 * half + l0);
+        const int nsh = (seg >> 1) * 4, hsh = 2 * seg;
+        const uint32_t v0 = ((ql.x >> nsh) & 0x0F0F0F0Fu) | (((qh.x >> hsh) & 0x03030303u) << 4);
+        const uint32_t v1 = ((ql.y >> nsh) & 0x0F0F0F0Fu) | (((qh.y >> hsh) & 0x03030303u) << 4);
+        const float sc = (float)reinterpret_cast<const int8_t *>(blk + 192)[8 * half + 2 * seg + (l0 >> 4)];
+        const float dl = half_bits_fast(ld_u16(blk + 208)) * sc;
+        const float s = dot_u4(v1, xb, dot_u4(v0, xa, 0.0f));
+        return dl * fmaf(-32.0f, xs8, s);
+    }
+};
+
+/* IQ4_NL (:2942-2954): d * table[nibble]; the 16-entry table lookup is two byte permutes (entries
+ * 0-7 and 8-15) and a select on bit 3 of the nibble; table entries are stored + 128 */
+template <> struct Lean<T_IQ4_NL> {
+    __device__ static uint32_t look4(uint32_t n, const Tables &t) {
+        const uint32_t sel = n & 0x07070707u;
+        const uint32_t lo = __builtin_amdgcn_perm(t.nl1, t.nl0, sel), hi = __builtin_amdgcn_perm(t.nl3, t.nl2, sel);
+        const uint32_t m = ((n >> 3) & 0x01010101u) * 0xFFu;
+        return (hi & m) | (lo & ~m);
+    }
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const float d = half_bits_fast(ld_u16(blk));
+        const uint2 q = ld8_at(img, boff + 2 + (k0 & 15));
+        const int sh = (k0 >> 4) * 4;
+        const uint32_t v0 = look4((q.x >> sh) & 0x0F0F0F0Fu, t), v1 = look4((q.y >> sh) & 0x0F0F0F0Fu, t);
+        const float s = dot_u4(v1, xb, dot_u4(v0, xa, 0.0f));
+        return d * fmaf(-128.0f, xs8, s);
+    }
+};
+
+/* IQ2_XXS (:2793-2816): d*(0.5+s)*0.25 * grid byte * sign */
+template <> struct Lean<T_IQ2_XXS> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const float d = half_bits_fast(ld_u16(blk));
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint2 a = ld8_at(img, boff + 2 + 8 * g);
+        const uint32_t a0 = a.x, a1 = a.y;
+        const float db = d * (0.5f + (float)(a1 >> 28)) * 0.25f;
+        const uint2 cell = *reinterpret_cast<const uint2 *>(t.grid2 + ((a0 >> (8 * l)) & 255u));
+        const uint32_t sg = iq_sign_byte((a1 >> (7 * l)) & 127u);
+        const float s = dot_u4_signed(cell.y, sg >> 4, xb, dot_u4_signed(cell.x, sg & 15u, xa, 0.0f));
+        return db * s;
+    }
+};
+
+/* IQ3_S (:3022-3058): d*(1+2s) * grid byte * sign; two 4-byte grid entries per eight elements */
+template <> struct Lean<T_IQ3_S> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const float d = half_bits_fast(ld_u16(blk));
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint32_t nib = (blk[106 + (g >> 1)] >> (4 * (g & 1))) & 15u;
+        const float db = d * (float)(1u + 2u * nib);
+        const uint32_t qh = blk[66 + g];
+        const uint32_t pair = ld_u16(blk + 2 + 8 * g + 2 * l);
+        const uint32_t i0 = (pair & 255u) | (((qh >> (2 * l)) & 1u) << 8);
+        const uint32_t i1 = (pair >> 8) | (((qh >> (2 * l + 1)) & 1u) << 8);
+        const uint32_t sb = blk[74 + 4 * g + l];
+        const float s = dot_u4_signed(t.grid3[i1], sb >> 4, xb, dot_u4_signed(t.grid3[i0], sb & 15u, xa, 0.0f));
+        return db * s;
+    }
+};
+
+template <uint32_t T> constexpr bool kNeedsGrid2 = (T == T_IQ2_XXS);
+template <uint32_t T> constexpr bool kNeedsGrid3 = (T == T_IQ3_S);
+
+
+template <uint32_t T>
+__global__ void __launch_bounds__(1024)
+gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
+                   int n_rows, int n_cols, int row_bytes, int image_bytes, int depth, int rows_per_wg) {
+    using C = Codec<T>;
+    constexpr int GPB = C::BE / 8;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    /* LDS map: x [n_cols] | sums of eight x [n_cols/8] | i-quant grid, 2 KB, where the type has one |
+     * row images [waves][depth][image_bytes] */
+    float *xs = reinterpret_cast<float *>(lds);
+    float *xs8 = xs + n_cols;
+    uint8_t *grid = reinterpret_cast<uint8_t *>(xs8 + (n_cols >> 3));
+    uint8_t *images = grid + ((kNeedsGrid2<T> || kNeedsGrid3<T>) ? 2048 : 0);
+
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n_waves = blockDim.x >> 6, n_threads = blockDim.x;
+    const int row0 = blockIdx.x * rows_per_wg;
+    int rows_here = n_rows - row0;
+    if (rows_here > rows_per_wg) rows_here = rows_per_wg;
+    const int my_rows = wv < rows_here ? (rows_here - wv + n_waves - 1) / n_waves : 0;
+    const int n_chunks = row_bytes >> 4;
+    const int loads_per_row = (n_chunks + 63) >> 6;
+
+    uint8_t *my_images = images + (size_t)wv * depth * image_bytes;
+    const uint32_t my_images_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)my_images;
+    const uint8_t *wg_base = W + (size_t)row0 * row_bytes;
+    /* Row i of this wave -> image i % depth. The loads are written as instructions: the data goes
+     * to LDS at M0 + 16*lane, no register is held while it is in flight, and the compiler (which
+     * would wait for every outstanding one of them before any LDS access) does not see them; the
+     * waits are placed by hand below. Nothing else in this kernel uses M0. */
+    auto issue = [&](int i) {
+        const uint4 *g = reinterpret_cast<const uint4 *>(wg_base + (size_t)(wv + i * n_waves) * row_bytes);
+        const uint32_t img = my_images_lds + (uint32_t)((i % depth) * image_bytes);
+        for (int c0 = 0; c0 < n_chunks; c0 += 64) {
+            const uint32_t m0v = __builtin_amdgcn_readfirstlane(img + 16u * (uint32_t)c0);
+            if (c0 + lane < n_chunks)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                             : : "v"(g + c0 + lane), "s"(m0v) : "memory");
+        }
+    };
+
+    /* x first: it goes to LDS the same way, 1 KB per instruction and wave, so no register holds
+     * data that is still in flight. A barrier makes every wave's x request precede every row
+     * request, then the first rows are requested. */
+    const int n4 = n_cols >> 2;
+    const float4 *xg = reinterpret_cast<const float4 *>(x);
+    const uint32_t xs_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)xs;
+    for (int base = wv * 64; base < n4; base += n_threads) { /* uniform per wave */
+        const uint32_t m0v = __builtin_amdgcn_readfirstlane(xs_lds + 16u * (uint32_t)base);
+        if (base + lane < n4)
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                         : : "v"(xg + base + lane), "s"(m0v) : "memory");
+    }
+    asm volatile("s_barrier" ::: "memory");
+    int issued = 0;
+    for (; issued < depth && issued < my_rows; issued++) issue(issued);
+    /* loads retire in order: at most the row loads outstanding means this wave's part of x has landed */
+    wait_vm_at_most(issued * loads_per_row);
+    Tables tab;
+    tab.grid2 = reinterpret_cast<const uint64_t *>(grid);
+    tab.grid3 = reinterpret_cast<const uint32_t *>(grid);
+    tab.nl0 = tab.nl1 = tab.nl2 = tab.nl3 = 0;
+    if (T == T_IQ4_NL) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(qlin_iq4nl_values);
+        tab.nl0 = v.x ^ 0x80808080u; tab.nl1 = v.y ^ 0x80808080u; tab.nl2 = v.z ^ 0x80808080u; tab.nl3 = v.w ^ 0x80808080u;
+    }
+    if (kNeedsGrid2<T>)
+        for (int t = threadIdx.x; t < 512; t += n_threads)
+            reinterpret_cast<uint32_t *>(grid)[t] = reinterpret_cast<const uint32_t *>(qlin_iq2xxs_grid)[t];
+    if (kNeedsGrid3<T>)
+        for (int t = threadIdx.x; t < 512; t += n_threads) reinterpret_cast<uint32_t *>(grid)[t] = qlin_iq3s_grid[t];
+    __syncthreads();
+    for (int t = threadIdx.x; t < (n_cols >> 3); t += n_threads) {
+        const float4 a = *reinterpret_cast<const float4 *>(xs + 8 * t), b = *reinterpret_cast<const float4 *>(xs + 8 * t + 4);
+        xs8[t] = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+    }
+    __syncthreads();
+
+    const int groups = (n_cols / C::BE) * GPB;
+    for (int i = 0; i < my_rows; i++) {
+        /* rows i .. issued-1 are in flight, row i the oldest */
+        wait_vm_at_most((issued - i - 1) * loads_per_row);
+        const uint8_t *img = my_images + (size_t)(i % depth) * image_bytes;
+        float acc = 0.0f;
+        for (int g = lane; g < groups; g += 64) {
+            const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+            const float4 xa = *reinterpret_cast<const float4 *>(xs + blk * C::BE + k0);
+            const float4 xb = *reinterpret_cast<const float4 *>(xs + blk * C::BE + k0 + 4);
+            acc += Lean<T>::dot8(img, blk * C::BB, k0, xa, xb, xs8[g], tab);
+        }
+        /* the image may be refilled once its reads have returned */
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (issued < my_rows) {
+            issue(issued);
+            issued++;
+        }
+        const float s = wave_sum(acc);
+        if (lane == 0) y[row0 + wv + i * n_waves] = s;
+    }
+}
+
+template <uint32_t T>
+bool stream_typed(const void *W, const float *x, float *y, int n_rows, int n_cols, int n_cu, hipStream_t stream,
+                  hipError_t *err) {
+    const size_t row_bytes = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
+    if (n_cols > 16384 || (n_cols & 31) || (row_bytes & 15) || row_bytes > 8192) return false;
+    if (((uintptr_t)W & 15) || ((uintptr_t)x & 15)) return false;
+    const size_t x_bytes = (size_t)n_cols * 4 + (size_t)(n_cols >> 3) * 4 + ((kNeedsGrid2<T> || kNeedsGrid3<T>) ? 2048 : 0);
+    const size_t lds_cap = 160 * 1024 - 16;
+    /* 16 waves with two images each if that fits, else one image, else 8 waves */
+    int waves = 16, depth = 2;
+    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) depth = 1;
+    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) { waves = 8; depth = 2; }
+    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) depth = 1;
+    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) return false;
+    if ((size_t)((row_bytes >> 4) + 63) / 64 * depth > 15) return false; /* the hand-placed waits count to 15 */
+    int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
+    if (rows_per_wg < 1) rows_per_wg = 1;
+    const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
+    const size_t lds_bytes = x_bytes + (size_t)waves * depth * row_bytes + 16; /* + slack for ld8_at */
+    static bool raised = false;
+    if (!raised) {
+        *err = hipFuncSetAttribute((const void *)gemv_stream_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   160 * 1024);
+        if (*err != hipSuccess) return true;
+        raised = true;
+    }
+    hipLaunchKernelGGL((gemv_stream_kernel<T>), dim3(grid), dim3(waves * 64), lds_bytes, stream, (const uint8_t *)W,
+                       x, y, n_rows, n_cols, (int)row_bytes, (int)row_bytes, depth, rows_per_wg);
+    *err = hipGetLastError();
+    return true;
+}
+
+}  // namespace
+
+bool launch_gemv_stream(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, int n_cu,
+                        hipStream_t stream, hipError_t *err) {
+    *err = hipSuccess;
+    switch (type) {
+    case T_Q8_0: return stream_typed<T_Q8_0>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    case T_Q4_K: return stream_typed<T_Q4_K>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    case T_Q5_K: return stream_typed<T_Q5_K>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    case T_Q6_K: return stream_typed<T_Q6_K>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    case T_IQ2_XXS: return stream_typed<T_IQ2_XXS>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    case T_IQ4_NL: return stream_typed<T_IQ4_NL>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    case T_IQ3_S: return stream_typed<T_IQ3_S>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    default: return false;
+    }
+}
+
+}  // namespace qlin

@@ -137,13 +137,16 @@ int weights_on_device_locked(const void *host, size_t bytes, DevBuf &buf, const 
     return QLIN_OK;
 }
 
-/* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the plain kernel */
+/* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the streaming kernel,
+ * else (ragged or oversized shapes, unaligned pointers) the plain kernel */
 hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y, int n_rows,
                          int n_cols, hipStream_t s) {
     if (n_rows == 0) return hipSuccess;
     if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && aligned(W, 16) && aligned(x, 16)) {
         return launch_gemv_q4k(W, x, y, n_rows, n_cols, s, g.n_cu);
     }
+    hipError_t err;
+    if (launch_gemv_stream(type, W, x, y, n_rows, n_cols, g.n_cu, s, &err)) return err;
     return launch_gemv_generic(type, W, x, y, n_rows, n_cols, s);
 }
 

@@ -20,6 +20,10 @@ hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, 
 /* y[n_rows] = W . x, any supported type and any whole-block shape */
 hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, float *y, int n_rows,
                                int n_cols, hipStream_t stream);
+/* streaming matvec for every type; returns false if the shape rules of gemv_stream.hip do not
+ * hold (nothing was launched), else true with the launch status in *err */
+bool launch_gemv_stream(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, int n_cu,
+                        hipStream_t stream, hipError_t *err);
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, int n_cols,
                            hipStream_t stream, int n_cu);
