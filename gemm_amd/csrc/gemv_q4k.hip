@@ -86,7 +86,8 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     float *partial = reinterpret_cast<float *>(images + kWaves * depth * kRowImage);
     const float4 *xraw = reinterpret_cast<const float4 *>(partial + ((rows_per_wg * n_slices + 3) & ~3));
 
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* wave-uniform, and the compiler is told so */
     const int c = lane & 3;
     const int slice = wv % n_slices;
     const int sb0 = slice * slice_sb;

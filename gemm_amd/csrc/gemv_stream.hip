@@ -205,7 +205,8 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
     uint8_t *grid = reinterpret_cast<uint8_t *>(xs8 + (n_cols >> 3));
     uint8_t *images = grid + ((kNeedsGrid2<T> || kNeedsGrid3<T>) ? 2048 : 0);
 
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* wave-uniform, and the compiler is told so */
     const int n_waves = blockDim.x >> 6, n_threads = blockDim.x;
     const int row0 = blockIdx.x * rows_per_wg;
     int rows_here = n_rows - row0;
@@ -269,17 +270,20 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
     }
     __syncthreads();
 
-    const int groups = (n_cols / C::BE) * GPB;
+    static_assert(64 % GPB == 0, "a wave covers whole blocks");
+    const int n_blocks = n_cols / C::BE;
+    const int k0 = (lane % GPB) * 8, blk_first = lane / GPB;
     for (int i = 0; i < my_rows; i++) {
         /* rows i .. issued-1 are in flight, row i the oldest */
         wait_vm_at_most((issued - i - 1) * loads_per_row);
         const uint8_t *img = my_images + (size_t)(i % depth) * image_bytes;
         float acc = 0.0f;
-        for (int g = lane; g < groups; g += 64) {
-            const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+        /* 64 is a multiple of the groups per block, so a lane keeps its position k0 inside the
+         * block for the whole row and everything derived from k0 is loop-invariant */
+        for (int blk = blk_first; blk < n_blocks; blk += 64 / GPB) {
             const float4 xa = *reinterpret_cast<const float4 *>(xs + blk * C::BE + k0);
             const float4 xb = *reinterpret_cast<const float4 *>(xs + blk * C::BE + k0 + 4);
-            acc += Lean<T>::dot8(img, blk * C::BB, k0, xa, xb, xs8[g], tab);
+            acc += Lean<T>::dot8(img, blk * C::BB, k0, xa, xb, xs8[blk * GPB + (k0 >> 3)], tab);
         }
         /* the image may be refilled once its reads have returned */
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
