@@ -176,28 +176,15 @@ __device__ __forceinline__ void apply_scales(f32x4 &acc, f32x4 S0, f32x4 S1, f32
     }
 }
 
-/* Raw registers of one super-block step of a wavefront: for each of its NW weight streams (a
- * stream = 16 rows of one matrix, one row per lane group) the 16 header bytes and the lane's
- * 4 x 8 code bytes; for each of its NA activation operands the lane's eight 16-byte pieces.
- * Two of these are kept in flight: the loads of step sb+1 are issued before the arithmetic of
- * step sb, which is what hides the HBM latency at one or two wavefronts per SIMD. */
-template <int NW, int NA>
-struct Step {
-    u32x4 hdr[NW];
-    u32x2 q[NW][4];
-    u32x4 a[NA][8]; /* [operand][2*c + half]: elements 64c + 32*half + 8*kg .. +7 of the super-block */
+/* The lane's activation operands of one super-block: for each of the NA operands eight 16-byte
+ * pieces, [2*c + half] = elements 64c + 32*half + 8*kg .. +7 of the super-block */
+template <int NA>
+struct Acts {
+    u32x4 a[NA][8];
 };
 
-template <int NW, int NA>
-__device__ __forceinline__ void load_step(Step<NW, NA> &s, const uint8_t *const (&wrow)[NW],
-                                          const uint16_t *const (&arow)[NA], int sb, int kg, bool live) {
-#pragma unroll
-    for (int w = 0; w < NW; w++) {
-        const uint8_t *blk = wrow[w] + (size_t)sb * kQ4KBlock;
-        s.hdr[w] = *(const u32x4 *)blk;
-#pragma unroll
-        for (int c = 0; c < 4; c++) s.q[w][c] = *(const u32x2 *)(blk + 16 + 32 * c + 8 * kg);
-    }
+template <int NA>
+__device__ __forceinline__ void load_acts(Acts<NA> &s, const uint16_t *const (&arow)[NA], int sb, int kg, bool live) {
 #pragma unroll
     for (int v = 0; v < NA; v++) {
         const uint16_t *xk = arow[v] + sb * 256 + 8 * kg;
@@ -210,8 +197,37 @@ __device__ __forceinline__ void load_step(Step<NW, NA> &s, const uint8_t *const 
     }
 }
 
+/* One super-block of NW * 16 rows goes from global memory to a wave-private LDS image
+ * [NW * 16 rows][144 bytes] as a flat stream of 16-byte chunks: chunk t = 64 i + lane of
+ * instruction i is chunk t % 9 of image row t / 9, so nine consecutive lanes read one row piece of
+ * 144 contiguous bytes. (Reading the pieces in the layout the matrix instruction wants, 8 bytes per
+ * lane from 16 rows at once, costs one cache access per lane: 63 accesses per load instruction
+ * measured, and the kernels were bound by exactly that.) The loads write LDS directly
+ * (global_load_lds_dwordx4); they are written as instructions and waited for by hand because the
+ * compiler would otherwise serialise every LDS access behind all of them. Image row R is row
+ * R % rows_per_matrix of matrix R / rows_per_matrix (gate then up; one matrix for down).
+ * Nothing else in these kernels uses M0. */
+template <int NW>
+__device__ __forceinline__ void image_from_global(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
+                                                  int rows_per_matrix, size_t row_bytes, int sb, int lane) {
+    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
+    constexpr int kChunks = NW * 16 * 9;
+#pragma unroll
+    for (int i = 0; i < (kChunks + 63) / 64; i++) {
+        const int t = 64 * i + lane;
+        const int R = t / 9, c9 = t - 9 * R;
+        const uint8_t *src = (R < rows_per_matrix ? m0_rows + (size_t)R * row_bytes
+                                                  : m1_rows + (size_t)(R - rows_per_matrix) * row_bytes) +
+                             (size_t)sb * kQ4KBlock + 16 * c9;
+        const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
+        if (t < kChunks)
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0v) : "memory");
+    }
+}
+
 template <int C, int NW, int NA>
-__device__ __forceinline__ void slice_math(const Step<NW, NA> &s, const Scales (&sc)[NW], f32x4 (&acc)[NW]) {
+__device__ __forceinline__ void slice_math(const uint8_t *img_row, const Acts<NA> &s, const Scales (&sc)[NW],
+                                           f32x4 (&acc)[NW]) {
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
     bf16x8 a0[NA], a1[NA];
     f32x4 X0 = zero, X1 = zero;
@@ -225,7 +241,7 @@ __device__ __forceinline__ void slice_math(const Step<NW, NA> &s, const Scales (
 #pragma unroll
     for (int w = 0; w < NW; w++) {
         /* the lane's 8 bytes hold its 8 codes of sub-block 2c (low nibbles) and of 2c+1 (high nibbles) */
-        const u32x2 q = s.q[w][C];
+        const u32x2 q = *(const u32x2 *)(img_row + w * 16 * kQ4KBlock + 16 + 32 * C);
         const bf16x8 lo = codes_to_bf16(q.x & 0x0F0F0F0Fu, q.y & 0x0F0F0F0Fu);
         const bf16x8 hi = codes_to_bf16((q.x >> 4) & 0x0F0F0F0Fu, (q.y >> 4) & 0x0F0F0F0Fu);
         f32x4 S0 = zero, S1 = zero;
@@ -241,117 +257,151 @@ __device__ __forceinline__ void slice_math(const Step<NW, NA> &s, const Scales (
     }
 }
 
+/* img_row: the lane's row j of stream 0 in the image, plus 8 * kg (its code bytes inside a slice) */
 template <int NW, int NA>
-__device__ __forceinline__ void step_math(const Step<NW, NA> &s, f32x4 (&acc)[NW]) {
+__device__ __forceinline__ void step_math(const uint8_t *img, int j, int kg, const Acts<NA> &s, f32x4 (&acc)[NW]) {
     Scales sc[NW];
 #pragma unroll
-    for (int w = 0; w < NW; w++) sc[w] = unpack_header(s.hdr[w]);
-    slice_math<0>(s, sc, acc);
-    slice_math<1>(s, sc, acc);
-    slice_math<2>(s, sc, acc);
-    slice_math<3>(s, sc, acc);
+    for (int w = 0; w < NW; w++) sc[w] = unpack_header(*(const u32x4 *)(img + (w * 16 + j) * kQ4KBlock));
+    const uint8_t *img_row = img + j * kQ4KBlock + 8 * kg;
+    slice_math<0>(img_row, s, sc, acc);
+    slice_math<1>(img_row, s, sc, acc);
+    slice_math<2>(img_row, s, sc, acc);
+    slice_math<3>(img_row, s, sc, acc);
 }
 
-/* all super-blocks of the rows in wrow[] against the activations in arow[], two steps in flight */
+/* A workgroup owns (expert, 32 rows); its waves split K: wave w takes super-blocks w, w + waves, ...
+ * (exactly one each up to K = 256 * waves), so every wave issues all of its loads at once and the
+ * chip has thousands of independent requests in flight instead of a few waves walking K. The
+ * partial sums of the waves meet in LDS: red[wave][stream][lane][4]. After the call and a barrier,
+ * element (stream s, lane l, v) of the tile is the sum over waves of
+ * red[(w * NW + s) * 256 + l * 4 + v], taken in wave order. */
 template <int NW, int NA>
-__device__ __forceinline__ void stream_rows(const uint8_t *const (&wrow)[NW], const uint16_t *const (&arow)[NA],
-                                            int n_sb, int kg, bool live, f32x4 (&acc)[NW]) {
-    Step<NW, NA> ping, pong;
-    load_step(ping, wrow, arow, 0, kg, live);
-    for (int sb = 0; sb < n_sb; sb += 2) {
-        const bool has1 = sb + 1 < n_sb, has2 = sb + 2 < n_sb;
-        if (has1) load_step(pong, wrow, arow, sb + 1, kg, live);
-        step_math(ping, acc);
-        if (has1) {
-            if (has2) load_step(ping, wrow, arow, sb + 2, kg, live);
-            step_math(pong, acc);
+__device__ __forceinline__ void ksplit_tile(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
+                                            int rows_per_matrix, size_t row_bytes,
+                                            const uint16_t *const (&arow)[NA], int n_sb, int wv, int n_waves,
+                                            int lane, bool live, bool image_ready, float *red) {
+    const int j = lane & 15, kg = lane >> 4;
+    f32x4 acc[NW];
+#pragma unroll
+    for (int w = 0; w < NW; w++) acc[w] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int sb = wv; sb < n_sb; sb += n_waves) {
+        Acts<NA> s;
+        if (!image_ready) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous image have returned */
+            image_from_global<NW>(img, m0_rows, m1_rows, rows_per_matrix, row_bytes, sb, lane);
         }
+        load_acts(s, arow, sb, kg, live);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* image (and activations) have landed */
+        step_math<NW, NA>(img, j, kg, s, acc);
     }
+#pragma unroll
+    for (int w = 0; w < NW; w++) *reinterpret_cast<f32x4 *>(red + ((wv * NW + w) * 64 + lane) * 4) = acc[w];
+}
+
+/* thread -> element of the 32-row x 16-slot result tile, ordered so that consecutive threads hold
+ * consecutive rows of one token slot: idx = ((v * 4 + kg) * 2 + r) * 16 + j */
+struct TileElem { int r, lane, v, slot, row; };
+__device__ __forceinline__ TileElem tile_elem(int idx) {
+    TileElem t;
+    const int j = idx & 15, kg = (idx >> 5) & 3;
+    t.r = (idx >> 4) & 1;
+    t.v = idx >> 7;
+    t.lane = kg * 16 + j;
+    t.slot = 4 * kg + t.v;       /* token slot inside the 16-slot tile */
+    t.row = 16 * t.r + j;        /* row inside the 32-row group */
+    return t;
 }
 
 /* ---- 2. gate and up for 32 rows of one expert, all of its tokens ---- */
-__device__ __forceinline__ void store_h(uint16_t *h_hi, uint16_t *h_lo, size_t at, float g, float u) {
-    const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
-    const __bf16 hi = (__bf16)h;
-    const __bf16 lo = (__bf16)(h - (float)hi);
-    h_hi[at] = __builtin_bit_cast(uint16_t, hi);
-    h_lo[at] = __builtin_bit_cast(uint16_t, lo);
-}
-
 #ifndef MOE_WAVES
 #define MOE_WAVES 2
 #endif
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
 moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
                    const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
                    const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
                    int n_embd, int n_ff, int top_k) {
+    extern __shared__ __attribute__((aligned(16))) float red[];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63;
-    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
-    if (row0 >= n_ff) return;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * 32;
     const int first = offsets[e], cnt = offsets[e + 1] - first;
     if (cnt == 0) return;
-    const int j = lane & 15, kg = lane >> 4;
+    const int j = lane & 15;
     const int n_sb = n_embd >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
-    const size_t ebase = ((size_t)e * n_ff + row0 + j) * row_bytes;
-    const uint8_t *const wrow[4] = {gate + ebase, gate + ebase + 16 * row_bytes, up + ebase,
-                                    up + ebase + 16 * row_bytes};
+    const size_t ebase = ((size_t)e * n_ff + row0) * row_bytes;
+    /* LDS: red [waves][4][64][4] floats | images [waves][64 rows][144 bytes] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 1024) + wv * (64 * kQ4KBlock);
+    const bool one_sb = n_sb <= n_waves; /* then a wave's image is fetched once for all token tiles */
+    if (one_sb && wv < n_sb) image_from_global<4>(img, gate + ebase, up + ebase, 32, row_bytes, wv, lane);
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt; /* as an A lane, j is the token slot */
         const int tok = live ? order[first + t0 + j] / top_k : 0;
         const uint16_t *const arow[1] = {X + (size_t)tok * n_embd};
-        f32x4 acc[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
-        stream_rows<4, 1>(wrow, arow, n_sb, kg, live, acc);
-        /* as a C lane: row j, token slots 4*kg + v */
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int ts = t0 + 4 * kg + v;
-            if (ts < cnt) {
-                const size_t at = (size_t)(first + ts) * n_ff + row0 + j;
-                store_h(h_hi, h_lo, at, acc[0][v], acc[2][v]);
-                store_h(h_hi, h_lo, at + 16, acc[1][v], acc[3][v]);
+        ksplit_tile<4, 1>(img, gate + ebase, up + ebase, 32, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 512; idx += blockDim.x) {
+            const TileElem t = tile_elem(idx);
+            float g = 0.0f, u = 0.0f;
+            for (int w = 0; w < n_waves; w++) {
+                g += red[((w * 4 + t.r) * 64 + t.lane) * 4 + t.v];
+                u += red[((w * 4 + 2 + t.r) * 64 + t.lane) * 4 + t.v];
+            }
+            if (t0 + t.slot < cnt) {
+                const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
+                const __bf16 hi = (__bf16)h;
+                const __bf16 lo = (__bf16)(h - (float)hi);
+                const size_t at = (size_t)(first + t0 + t.slot) * n_ff + row0 + t.row;
+                h_hi[at] = __builtin_bit_cast(uint16_t, hi);
+                h_lo[at] = __builtin_bit_cast(uint16_t, lo);
             }
         }
+        __syncthreads();
     }
 }
 
 /* ---- 3. down for 32 rows of one expert ---- */
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                 const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
                 const int32_t *__restrict__ order, const float *__restrict__ expert_w, float *__restrict__ part,
                 int n_embd, int n_ff) {
+    extern __shared__ __attribute__((aligned(16))) float red[];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63;
-    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
-    if (row0 >= n_embd) return;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * 32;
     const int first = offsets[e], cnt = offsets[e + 1] - first;
     if (cnt == 0) return;
-    const int j = lane & 15, kg = lane >> 4;
+    const int j = lane & 15;
     const int n_sb = n_ff >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
-    const uint8_t *d0 = down + ((size_t)e * n_embd + row0 + j) * row_bytes;
-    const uint8_t *const wrow[2] = {d0, d0 + 16 * row_bytes};
+    const uint8_t *d0 = down + ((size_t)e * n_embd + row0) * row_bytes;
+    /* LDS: red [waves][2][64][4] floats | images [waves][32 rows][144 bytes] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 512) + wv * (32 * kQ4KBlock);
+    const bool one_sb = n_sb <= n_waves;
+    if (one_sb && wv < n_sb) image_from_global<2>(img, d0, d0, 32, row_bytes, wv, lane);
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt;
         const size_t at_a = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
         const uint16_t *const arow[2] = {h_hi + at_a, h_lo + at_a};
-        f32x4 acc[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
-        stream_rows<2, 2>(wrow, arow, n_sb, kg, live, acc);
-#pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int ts = t0 + 4 * kg + v;
-            if (ts < cnt) {
-                const float w = expert_w[order[first + ts]];
-                const size_t at = (size_t)(first + ts) * n_embd + row0 + j;
-                part[at] = w * acc[0][v];      /* w * q, as out[i] += w*q does (:4116-4127) */
-                part[at + 16] = w * acc[1][v];
+        ksplit_tile<2, 2>(img, d0, d0, 32, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 512; idx += blockDim.x) {
+            const TileElem t = tile_elem(idx);
+            float d = 0.0f;
+            for (int w = 0; w < n_waves; w++) d += red[((w * 2 + t.r) * 64 + t.lane) * 4 + t.v];
+            if (t0 + t.slot < cnt) {
+                const float w = expert_w[order[first + t0 + t.slot]];
+                part[(size_t)(first + t0 + t.slot) * n_embd + row0 + t.row] = w * d; /* w * q, as out[i] += w*q does (:4116-4127) */
             }
         }
+        __syncthreads();
     }
 }
 
@@ -385,10 +435,18 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
     const int n_pairs = n_tok * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)n_expert * 2 * sizeof(int32_t), stream, idx,
                        n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of);
-    hipLaunchKernelGGL(moe_gate_up_kernel, dim3((n_ff / 32 + 3) / 4, n_expert), dim3(256), 0, stream,
+    static bool lds_raised = false;
+    if (!lds_raised) {
+        hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e1 != hipSuccess) return e1;
+        lds_raised = true;
+    }
+    /* waves per workgroup = super-blocks of K, at most 8 */
+    const int gu_waves = n_embd / 256 < 8 ? n_embd / 256 : 8, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
+    hipLaunchKernelGGL(moe_gate_up_kernel, dim3(n_ff / 32, n_expert), dim3(64 * gu_waves), (size_t)gu_waves * (4 * 1024 + 64 * kQ4KBlock), stream,
                        (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
                        n_ff, top_k);
-    hipLaunchKernelGGL(moe_down_kernel, dim3((n_embd / 32 + 3) / 4, n_expert), dim3(256), 0, stream,
+    hipLaunchKernelGGL(moe_down_kernel, dim3(n_embd / 32, n_expert), dim3(64 * dn_waves), (size_t)dn_waves * (2 * 1024 + 32 * kQ4KBlock), stream,
                        (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.order, w, ws.part, n_embd, n_ff);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 255) / 256), dim3(256), 0, stream, ws.part,
                        ws.slot_of, out, n_embd, top_k);
