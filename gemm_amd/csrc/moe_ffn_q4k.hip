@@ -299,57 +299,64 @@ __device__ __forceinline__ void ksplit_tile(uint8_t *img, const uint8_t *m0_rows
     for (int w = 0; w < NW; w++) *reinterpret_cast<f32x4 *>(red + ((wv * NW + w) * 64 + lane) * 4) = acc[w];
 }
 
-/* thread -> element of the 32-row x 16-slot result tile, ordered so that consecutive threads hold
- * consecutive rows of one token slot: idx = ((v * 4 + kg) * 2 + r) * 16 + j */
+/* thread -> element of the (16 * RT)-row x 16-slot result tile, ordered so that consecutive
+ * threads hold consecutive rows of one token slot: idx = ((v * 4 + kg) * RT + r) * 16 + j */
 struct TileElem { int r, lane, v, slot, row; };
+template <int RT>
 __device__ __forceinline__ TileElem tile_elem(int idx) {
     TileElem t;
-    const int j = idx & 15, kg = (idx >> 5) & 3;
-    t.r = (idx >> 4) & 1;
-    t.v = idx >> 7;
+    const int j = idx & 15, q = idx >> 4;
+    t.r = q % RT;
+    const int kg = (q / RT) & 3;
+    t.v = q / (4 * RT);
     t.lane = kg * 16 + j;
     t.slot = 4 * kg + t.v;       /* token slot inside the 16-slot tile */
-    t.row = 16 * t.r + j;        /* row inside the 32-row group */
+    t.row = 16 * t.r + j;        /* row inside the group */
     return t;
 }
 
-/* ---- 2. gate and up for 32 rows of one expert, all of its tokens ---- */
+/* ---- 2. gate and up for RT * 16 rows of one expert, all of its tokens ---- */
 #ifndef MOE_WAVES
 #define MOE_WAVES 2
 #endif
+#ifndef MOE_GU_RT
+#define MOE_GU_RT 1
+#endif
+template <int RT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
 moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
                    const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
                    const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
                    int n_embd, int n_ff, int top_k) {
+    constexpr int NW = 2 * RT, kRows = 16 * RT; /* streams: RT gate tiles, then RT up tiles */
     extern __shared__ __attribute__((aligned(16))) float red[];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
-    const int row0 = blockIdx.x * 32;
+    const int row0 = blockIdx.x * kRows;
     const int first = offsets[e], cnt = offsets[e + 1] - first;
     if (cnt == 0) return;
     const int j = lane & 15;
     const int n_sb = n_embd >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
     const size_t ebase = ((size_t)e * n_ff + row0) * row_bytes;
-    /* LDS: red [waves][4][64][4] floats | images [waves][64 rows][144 bytes] */
-    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 1024) + wv * (64 * kQ4KBlock);
+    /* LDS: red [waves][NW][64][4] floats | images [waves][NW * 16 rows][144 bytes] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * NW * 256) + wv * (NW * 16 * kQ4KBlock);
     const bool one_sb = n_sb <= n_waves; /* then a wave's image is fetched once for all token tiles */
-    if (one_sb && wv < n_sb) image_from_global<4>(img, gate + ebase, up + ebase, 32, row_bytes, wv, lane);
+    if (one_sb && wv < n_sb) image_from_global<NW>(img, gate + ebase, up + ebase, kRows, row_bytes, wv, lane);
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt; /* as an A lane, j is the token slot */
         const int tok = live ? order[first + t0 + j] / top_k : 0;
         const uint16_t *const arow[1] = {X + (size_t)tok * n_embd};
-        ksplit_tile<4, 1>(img, gate + ebase, up + ebase, 32, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
+        ksplit_tile<NW, 1>(img, gate + ebase, up + ebase, kRows, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 512; idx += blockDim.x) {
-            const TileElem t = tile_elem(idx);
+        for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
+            const TileElem t = tile_elem<RT>(idx);
             float g = 0.0f, u = 0.0f;
             for (int w = 0; w < n_waves; w++) {
-                g += red[((w * 4 + t.r) * 64 + t.lane) * 4 + t.v];
-                u += red[((w * 4 + 2 + t.r) * 64 + t.lane) * 4 + t.v];
+                g += red[((w * NW + t.r) * 64 + t.lane) * 4 + t.v];
+                u += red[((w * NW + RT + t.r) * 64 + t.lane) * 4 + t.v];
             }
             if (t0 + t.slot < cnt) {
                 const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
@@ -393,7 +400,7 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
         ksplit_tile<2, 2>(img, d0, d0, 32, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
         __syncthreads();
         for (int idx = threadIdx.x; idx < 512; idx += blockDim.x) {
-            const TileElem t = tile_elem(idx);
+            const TileElem t = tile_elem<2>(idx);
             float d = 0.0f;
             for (int w = 0; w < n_waves; w++) d += red[((w * 2 + t.r) * 64 + t.lane) * 4 + t.v];
             if (t0 + t.slot < cnt) {
@@ -437,13 +444,16 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
                        n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of);
     static bool lds_raised = false;
     if (!lds_raised) {
-        hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<MOE_GU_RT>,
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e1 != hipSuccess) return e1;
         lds_raised = true;
     }
     /* waves per workgroup = super-blocks of K, at most 8 */
     const int gu_waves = n_embd / 256 < 8 ? n_embd / 256 : 8, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
-    hipLaunchKernelGGL(moe_gate_up_kernel, dim3(n_ff / 32, n_expert), dim3(64 * gu_waves), (size_t)gu_waves * (4 * 1024 + 64 * kQ4KBlock), stream,
+    constexpr int RT = MOE_GU_RT;
+    hipLaunchKernelGGL(moe_gate_up_kernel<RT>, dim3(n_ff / (16 * RT), n_expert), dim3(64 * gu_waves),
+                       (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock), stream,
                        (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
                        n_ff, top_k);
     hipLaunchKernelGGL(moe_down_kernel, dim3(n_embd / 32, n_expert), dim3(64 * dn_waves), (size_t)dn_waves * (2 * 1024 + 32 * kQ4KBlock), stream,
