@@ -68,13 +68,9 @@ static hipError_t launch_typed(const void *W, float *out, int n_rows, int n_cols
 hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, int n_cols,
                           size_t row_bytes, hipStream_t stream) {
     switch (type) {
-    case T_Q8_0: return launch_typed<T_Q8_0>(W, out, n_rows, n_cols, row_bytes, stream);
-    case T_Q4_K: return launch_typed<T_Q4_K>(W, out, n_rows, n_cols, row_bytes, stream);
-    case T_Q5_K: return launch_typed<T_Q5_K>(W, out, n_rows, n_cols, row_bytes, stream);
-    case T_Q6_K: return launch_typed<T_Q6_K>(W, out, n_rows, n_cols, row_bytes, stream);
-    case T_IQ2_XXS: return launch_typed<T_IQ2_XXS>(W, out, n_rows, n_cols, row_bytes, stream);
-    case T_IQ4_NL: return launch_typed<T_IQ4_NL>(W, out, n_rows, n_cols, row_bytes, stream);
-    case T_IQ3_S: return launch_typed<T_IQ3_S>(W, out, n_rows, n_cols, row_bytes, stream);
+#define QLIN_CASE(TT) case TT: return launch_typed<TT>(W, out, n_rows, n_cols, row_bytes, stream);
+    QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+#undef QLIN_CASE
     case T_F32: case T_F16: case T_BF16: {
         const long long n = (long long)n_rows * n_cols;
         if (n == 0) return hipSuccess;

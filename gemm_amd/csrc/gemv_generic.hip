@@ -99,13 +99,9 @@ hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, flo
                                int n_cols, hipStream_t s) {
     if (n_rows == 0) return hipSuccess;
     switch (type) {
-    case T_Q8_0: return gemv_typed<T_Q8_0>(W, x, y, n_rows, n_cols, s);
-    case T_Q4_K: return gemv_typed<T_Q4_K>(W, x, y, n_rows, n_cols, s);
-    case T_Q5_K: return gemv_typed<T_Q5_K>(W, x, y, n_rows, n_cols, s);
-    case T_Q6_K: return gemv_typed<T_Q6_K>(W, x, y, n_rows, n_cols, s);
-    case T_IQ2_XXS: return gemv_typed<T_IQ2_XXS>(W, x, y, n_rows, n_cols, s);
-    case T_IQ4_NL: return gemv_typed<T_IQ4_NL>(W, x, y, n_rows, n_cols, s);
-    case T_IQ3_S: return gemv_typed<T_IQ3_S>(W, x, y, n_rows, n_cols, s);
+#define QLIN_CASE(TT) case TT: return gemv_typed<TT>(W, x, y, n_rows, n_cols, s);
+    QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+#undef QLIN_CASE
     default: return hipErrorInvalidValue;
     }
 }
@@ -125,13 +121,9 @@ hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *
                            int n_cols, int n_tok, int ldx, int ldy, hipStream_t s) {
     if (n_rows == 0 || n_tok == 0) return hipSuccess;
     switch (type) {
-    case T_Q8_0: return gemm_typed<T_Q8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
-    case T_Q4_K: return gemm_typed<T_Q4_K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
-    case T_Q5_K: return gemm_typed<T_Q5_K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
-    case T_Q6_K: return gemm_typed<T_Q6_K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
-    case T_IQ2_XXS: return gemm_typed<T_IQ2_XXS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
-    case T_IQ4_NL: return gemm_typed<T_IQ4_NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
-    case T_IQ3_S: return gemm_typed<T_IQ3_S>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+#define QLIN_CASE(TT) case TT: return gemm_typed<TT>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
+    QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+#undef QLIN_CASE
     default: return hipErrorInvalidValue;
     }
 }

@@ -334,13 +334,9 @@ bool launch_gemv_stream(uint32_t type, const void *W, const float *x, float *y, 
                         hipStream_t stream, hipError_t *err) {
     *err = hipSuccess;
     switch (type) {
-    case T_Q8_0: return stream_typed<T_Q8_0>(W, x, y, n_rows, n_cols, n_cu, stream, err);
-    case T_Q4_K: return stream_typed<T_Q4_K>(W, x, y, n_rows, n_cols, n_cu, stream, err);
-    case T_Q5_K: return stream_typed<T_Q5_K>(W, x, y, n_rows, n_cols, n_cu, stream, err);
-    case T_Q6_K: return stream_typed<T_Q6_K>(W, x, y, n_rows, n_cols, n_cu, stream, err);
-    case T_IQ2_XXS: return stream_typed<T_IQ2_XXS>(W, x, y, n_rows, n_cols, n_cu, stream, err);
-    case T_IQ4_NL: return stream_typed<T_IQ4_NL>(W, x, y, n_rows, n_cols, n_cu, stream, err);
-    case T_IQ3_S: return stream_typed<T_IQ3_S>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+#define QLIN_CASE(TT) case TT: return stream_typed<TT>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+    QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+#undef QLIN_CASE
     default: return false;
     }
 }

@@ -267,6 +267,24 @@ void qlin_dequantize_row_q6_K(const void *s, float *d, int n) { void_decoder(T_Q
 void qlin_dequantize_row_iq2_xxs(const void *s, float *d, int n) { void_decoder(T_IQ2_XXS, "qlin_dequantize_row_iq2_xxs", s, d, n); }
 void qlin_dequantize_row_iq3_s(const void *s, float *d, int n) { void_decoder(T_IQ3_S, "qlin_dequantize_row_iq3_s", s, d, n); }
 void qlin_dequantize_row_iq4_nl(const void *s, float *d, int n) { void_decoder(T_IQ4_NL, "qlin_dequantize_row_iq4_nl", s, d, n); }
+void qlin_dequantize_row_q4_0(const void *s, float *d, int n) { void_decoder(T_Q4_0, "qlin_dequantize_row_q4_0", s, d, n); }
+void qlin_dequantize_row_q4_1(const void *s, float *d, int n) { void_decoder(T_Q4_1, "qlin_dequantize_row_q4_1", s, d, n); }
+void qlin_dequantize_row_q5_0(const void *s, float *d, int n) { void_decoder(T_Q5_0, "qlin_dequantize_row_q5_0", s, d, n); }
+void qlin_dequantize_row_q5_1(const void *s, float *d, int n) { void_decoder(T_Q5_1, "qlin_dequantize_row_q5_1", s, d, n); }
+void qlin_dequantize_row_q2_K(const void *s, float *d, int n) { void_decoder(T_Q2_K, "qlin_dequantize_row_q2_K", s, d, n); }
+void qlin_dequantize_row_q3_K(const void *s, float *d, int n) { void_decoder(T_Q3_K, "qlin_dequantize_row_q3_K", s, d, n); }
+void qlin_dequantize_row_q1_0(const void *s, float *d, int n) { void_decoder(T_Q1_0, "qlin_dequantize_row_q1_0", s, d, n); }
+void qlin_dequantize_row_mxfp4(const void *s, float *d, int n) { void_decoder(T_MXFP4, "qlin_dequantize_row_mxfp4", s, d, n); }
+void qlin_dequantize_row_nvfp4(const void *s, float *d, int n) { void_decoder(T_NVFP4, "qlin_dequantize_row_nvfp4", s, d, n); }
+void qlin_dequantize_row_iq2_xs(const void *s, float *d, int n) { void_decoder(T_IQ2_XS, "qlin_dequantize_row_iq2_xs", s, d, n); }
+void qlin_dequantize_row_iq2_s(const void *s, float *d, int n) { void_decoder(T_IQ2_S, "qlin_dequantize_row_iq2_s", s, d, n); }
+void qlin_dequantize_row_iq3_xxs(const void *s, float *d, int n) { void_decoder(T_IQ3_XXS, "qlin_dequantize_row_iq3_xxs", s, d, n); }
+void qlin_dequantize_row_iq4_xs(const void *s, float *d, int n) { void_decoder(T_IQ4_XS, "qlin_dequantize_row_iq4_xs", s, d, n); }
+void qlin_dequantize_row_iq1_s(const void *s, float *d, int n) { void_decoder(T_IQ1_S, "qlin_dequantize_row_iq1_s", s, d, n); }
+void qlin_dequantize_row_iq1_m(const void *s, float *d, int n) { void_decoder(T_IQ1_M, "qlin_dequantize_row_iq1_m", s, d, n); }
+void qlin_dequantize_row_tq1_0(const void *s, float *d, int n) { void_decoder(T_TQ1_0, "qlin_dequantize_row_tq1_0", s, d, n); }
+void qlin_dequantize_row_tq2_0(const void *s, float *d, int n) { void_decoder(T_TQ2_0, "qlin_dequantize_row_tq2_0", s, d, n); }
+void qlin_dequantize_row_bf16(const void *s, float *d, int n) { void_decoder(T_BF16, "qlin_dequantize_row_bf16", s, d, n); }
 
 /* ------------------------------------------------------------------ weights */
 

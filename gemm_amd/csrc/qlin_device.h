@@ -3,7 +3,8 @@
  *
  * Byte layouts follow the packed block structs of common/ggml_dequant.h:30-204. Blocks are
  * addressed as raw bytes: inside a row only 2-byte alignment holds (block sizes 34, 210, 66,
- * 110 and 18 are not multiples of 4), so multi-byte fields are assembled from 16-bit loads.
+ * 110 and 18 are not multiples of 4), so multi-byte fields are assembled from 16-bit loads
+ * (the 17-byte MXFP4 block has byte fields only).
  */
 #ifndef QLIN_DEVICE_H
 #define QLIN_DEVICE_H
@@ -12,13 +13,23 @@
 #include <stdint.h>
 
 #include "qlin_codebooks.h"
+#include "qlin_codebooks_ext.h"
 
 namespace qlin {
 
 enum : uint32_t {
     T_F32 = 0, T_F16 = 1, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14,
-    T_IQ2_XXS = 16, T_IQ4_NL = 20, T_IQ3_S = 21, T_BF16 = 30
+    T_IQ2_XXS = 16, T_IQ4_NL = 20, T_IQ3_S = 21, T_BF16 = 30,
+    T_Q4_0 = 2, T_Q4_1 = 3, T_Q5_0 = 6, T_Q5_1 = 7, T_Q2_K = 10, T_Q3_K = 11, T_IQ2_XS = 17,
+    T_IQ3_XXS = 18, T_IQ1_S = 19, T_IQ2_S = 22, T_IQ4_XS = 23, T_IQ1_M = 29, T_TQ1_0 = 34,
+    T_TQ2_0 = 35, T_MXFP4 = 39, T_NVFP4 = 40, T_Q1_0 = 41
 };
+
+/* every block format with a decoder, for the type switches: X(type id) */
+#define QLIN_FOR_EACH_BLOCK_TYPE(X)                                                              \
+    X(T_Q8_0) X(T_Q4_K) X(T_Q5_K) X(T_Q6_K) X(T_IQ2_XXS) X(T_IQ4_NL) X(T_IQ3_S) X(T_Q4_0)       \
+    X(T_Q4_1) X(T_Q5_0) X(T_Q5_1) X(T_Q2_K) X(T_Q3_K) X(T_IQ2_XS) X(T_IQ3_XXS) X(T_IQ1_S)      \
+    X(T_IQ2_S) X(T_IQ4_XS) X(T_IQ1_M) X(T_TQ1_0) X(T_TQ2_0) X(T_MXFP4) X(T_NVFP4) X(T_Q1_0)
 
 /* elements and bytes per block (common/ggml_dequant.h:261-294) */
 template <uint32_t T> struct Geom;
@@ -41,6 +52,23 @@ __host__ __device__ inline bool type_geometry(uint32_t t, int *be, int *bb) {
     case T_IQ2_XXS: *be = 256; *bb = 66; return true;
     case T_IQ4_NL: *be = 32; *bb = 18; return true;
     case T_IQ3_S: *be = 256; *bb = 110; return true;
+    case T_Q4_0: *be = 32; *bb = 18; return true;
+    case T_Q4_1: *be = 32; *bb = 20; return true;
+    case T_Q5_0: *be = 32; *bb = 22; return true;
+    case T_Q5_1: *be = 32; *bb = 24; return true;
+    case T_Q2_K: *be = 256; *bb = 84; return true;
+    case T_Q3_K: *be = 256; *bb = 110; return true;
+    case T_IQ2_XS: *be = 256; *bb = 74; return true;
+    case T_IQ3_XXS: *be = 256; *bb = 98; return true;
+    case T_IQ1_S: *be = 256; *bb = 50; return true;
+    case T_IQ2_S: *be = 256; *bb = 82; return true;
+    case T_IQ4_XS: *be = 256; *bb = 136; return true;
+    case T_IQ1_M: *be = 256; *bb = 56; return true;
+    case T_TQ1_0: *be = 256; *bb = 54; return true;
+    case T_TQ2_0: *be = 256; *bb = 66; return true;
+    case T_MXFP4: *be = 32; *bb = 17; return true;
+    case T_NVFP4: *be = 64; *bb = 36; return true;
+    case T_Q1_0: *be = 128; *bb = 18; return true;
     default: return false;
     }
 }
@@ -211,6 +239,10 @@ template <> struct Codec<T_IQ3_S> : Geom<T_IQ3_S> {
         }
     }
 };
+
+}  // namespace qlin
+#include "qlin_codecs_ext.h"
+namespace qlin {
 
 /* wait until at most n vector-memory operations of this wavefront are outstanding (they retire
  * in order, so the oldest ones are then complete); n is wave-uniform, 0..15 (more waits for 15) */

@@ -19,9 +19,25 @@ static void complain(const char *where) {
     fprintf(stderr, "qlinear: %s failed: %s\n", where, qlin_last_error());
 }
 
-size_t qtf_row_bytes(uint32_t type, int n_cols) { return qlin_dequant_row_size(type, n_cols); }
+/* the weight types the reference's model path takes (common/transformer.h:462-487): sixteen
+ * block formats and the three plain ones; the decoders know more formats than this */
+int qtf_is_supported_weight_type(uint32_t type) {
+    switch (type) {
+    case QLIN_TYPE_Q2_K: case QLIN_TYPE_Q3_K: case QLIN_TYPE_Q4_0: case QLIN_TYPE_Q8_0:
+    case QLIN_TYPE_Q4_K: case QLIN_TYPE_Q5_K: case QLIN_TYPE_Q6_K: case QLIN_TYPE_IQ2_XXS:
+    case QLIN_TYPE_IQ2_XS: case QLIN_TYPE_IQ3_XXS: case QLIN_TYPE_IQ1_S: case QLIN_TYPE_IQ4_NL:
+    case QLIN_TYPE_IQ3_S: case QLIN_TYPE_IQ2_S: case QLIN_TYPE_IQ4_XS: case QLIN_TYPE_IQ1_M:
+    case QLIN_TYPE_F32: case QLIN_TYPE_F16: case QLIN_TYPE_BF16:
+        return 1;
+    default:
+        return 0;
+    }
+}
 
-int qtf_is_supported_weight_type(uint32_t type) { return qlin_dequant_row_size(type, 256) != 0; }
+/* 0 for a type outside that list, like the reference (common/transformer.h:489-514) */
+size_t qtf_row_bytes(uint32_t type, int n_cols) {
+    return qtf_is_supported_weight_type(type) ? qlin_dequant_row_size(type, n_cols) : 0;
+}
 
 static size_t tensor_bytes(const qtensor *t) {
     return (size_t)t->n_rows * qtf_row_bytes(t->type, t->n_cols);

@@ -31,6 +31,24 @@ SIGNATURES = {
     "qlin_dequantize_row_iq2_xxs": (None, [_vp, _vp, C.c_int]),
     "qlin_dequantize_row_iq3_s": (None, [_vp, _vp, C.c_int]),
     "qlin_dequantize_row_iq4_nl": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q4_0": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q4_1": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q5_0": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q5_1": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q2_K": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q3_K": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_q1_0": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_mxfp4": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_nvfp4": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq2_xs": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq2_s": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq3_xxs": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq4_xs": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq1_s": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_iq1_m": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_tq1_0": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_tq2_0": (None, [_vp, _vp, C.c_int]),
+    "qlin_dequantize_row_bf16": (None, [_vp, _vp, C.c_int]),
     "qlin_dequant_rows": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int]),
     "qlin_weight_register": (C.c_int, [_vp, C.c_size_t]),
     "qlin_weight_unregister": (C.c_int, [_vp]),

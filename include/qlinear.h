@@ -40,7 +40,12 @@ extern "C" {
 enum qlin_type {
     QLIN_TYPE_F32 = 0, QLIN_TYPE_F16 = 1, QLIN_TYPE_Q8_0 = 8, QLIN_TYPE_Q4_K = 12,
     QLIN_TYPE_Q5_K = 13, QLIN_TYPE_Q6_K = 14, QLIN_TYPE_IQ2_XXS = 16, QLIN_TYPE_IQ4_NL = 20,
-    QLIN_TYPE_IQ3_S = 21, QLIN_TYPE_BF16 = 30
+    QLIN_TYPE_IQ3_S = 21, QLIN_TYPE_BF16 = 30,
+    QLIN_TYPE_Q4_0 = 2, QLIN_TYPE_Q4_1 = 3, QLIN_TYPE_Q5_0 = 6, QLIN_TYPE_Q5_1 = 7,
+    QLIN_TYPE_Q2_K = 10, QLIN_TYPE_Q3_K = 11, QLIN_TYPE_IQ2_XS = 17, QLIN_TYPE_IQ3_XXS = 18,
+    QLIN_TYPE_IQ1_S = 19, QLIN_TYPE_IQ2_S = 22, QLIN_TYPE_IQ4_XS = 23, QLIN_TYPE_IQ1_M = 29,
+    QLIN_TYPE_TQ1_0 = 34, QLIN_TYPE_TQ2_0 = 35, QLIN_TYPE_MXFP4 = 39, QLIN_TYPE_NVFP4 = 40,
+    QLIN_TYPE_Q1_0 = 41
 };
 
 /* ------------------------------------------------------------------ lifecycle */
@@ -69,6 +74,24 @@ void   qlin_dequantize_row_q6_K(const void *src, float *dst, int n);    /* :239,
 void   qlin_dequantize_row_iq2_xxs(const void *src, float *dst, int n); /* :240, :2793 */
 void   qlin_dequantize_row_iq3_s(const void *src, float *dst, int n);   /* :248, :3022 */
 void   qlin_dequantize_row_iq4_nl(const void *src, float *dst, int n);  /* :249, :2942 */
+void   qlin_dequantize_row_q4_0(const void *src, float *dst, int n); /* :241, :2850 */
+void   qlin_dequantize_row_q4_1(const void *src, float *dst, int n); /* :242, :2864 */
+void   qlin_dequantize_row_q5_0(const void *src, float *dst, int n); /* :243, :2879 */
+void   qlin_dequantize_row_q5_1(const void *src, float *dst, int n); /* :244, :2897 */
+void   qlin_dequantize_row_q2_K(const void *src, float *dst, int n); /* :231, :1505 */
+void   qlin_dequantize_row_q3_K(const void *src, float *dst, int n); /* :232, :1536 */
+void   qlin_dequantize_row_q1_0(const void *src, float *dst, int n); /* :234, :1491 */
+void   qlin_dequantize_row_mxfp4(const void *src, float *dst, int n); /* :235, :2818 */
+void   qlin_dequantize_row_nvfp4(const void *src, float *dst, int n); /* :236, :2832 */
+void   qlin_dequantize_row_iq2_xs(const void *src, float *dst, int n); /* :245, :2975 */
+void   qlin_dequantize_row_iq2_s(const void *src, float *dst, int n); /* :246, :2996 */
+void   qlin_dequantize_row_iq3_xxs(const void *src, float *dst, int n); /* :247, :2916 */
+void   qlin_dequantize_row_iq4_xs(const void *src, float *dst, int n); /* :250, :2956 */
+void   qlin_dequantize_row_iq1_s(const void *src, float *dst, int n); /* :251, :3062 */
+void   qlin_dequantize_row_iq1_m(const void *src, float *dst, int n); /* :252, :3084 */
+void   qlin_dequantize_row_tq1_0(const void *src, float *dst, int n); /* :253, :3127 */
+void   qlin_dequantize_row_tq2_0(const void *src, float *dst, int n); /* :254, :3161 */
+void   qlin_dequantize_row_bf16(const void *src, float *dst, int n); /* :255, :1689 */
 /* Many rows at once: src holds n_rows rows of qlin_dequant_row_size(type, n_cols) bytes,
  * dst is [n_rows, n_cols] fp32. Shape of the per-row loop in tf_dequant_row callers
  * (common/transformer.h:425-460). */

@@ -16,7 +16,10 @@ _REF_SO = os.path.join(_HERE, "_ref", "libref.so")
 # enum ggml_dtype values (common/gguf_loader.h:45-85)
 F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, IQ2_XXS, IQ4_NL, IQ3_S, BF16 = 0, 1, 8, 12, 13, 14, 16, 20, 21, 30
 BLOCK_TYPES = {"q8_0": Q8_0, "q4_K": Q4_K, "q5_K": Q5_K, "q6_K": Q6_K,
-               "iq2_xxs": IQ2_XXS, "iq4_nl": IQ4_NL, "iq3_s": IQ3_S}
+               "iq2_xxs": IQ2_XXS, "iq4_nl": IQ4_NL, "iq3_s": IQ3_S,
+               "q4_0": 2, "q4_1": 3, "q5_0": 6, "q5_1": 7, "q2_K": 10, "q3_K": 11, "iq2_xs": 17,
+               "iq3_xxs": 18, "iq1_s": 19, "iq2_s": 22, "iq4_xs": 23, "iq1_m": 29, "tq1_0": 34,
+               "tq2_0": 35, "mxfp4": 39, "nvfp4": 40, "q1_0": 41}
 
 _vp, _fp, _ip = C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_int)
 
@@ -220,6 +223,9 @@ class Reference:
 
     def row_size(self, type_id, n):
         return int(self.lib.ref_dequant_row_size(type_id, n))
+
+    def tf_row_bytes(self, type_id, n_cols):
+        return int(self.lib.ref_tf_row_bytes(type_id, n_cols))
 
     def dequant_row(self, type_id, src, n):
         src, ps = _u8(src)

@@ -72,6 +72,12 @@ static const qo_type_info k_types[] = {
     {QO_TYPE_Q8_0, 32, 34},    {QO_TYPE_Q4_K, 256, 144}, {QO_TYPE_Q5_K, 256, 176},
     {QO_TYPE_Q6_K, 256, 210},  {QO_TYPE_IQ2_XXS, 256, 66}, {QO_TYPE_IQ4_NL, 32, 18},
     {QO_TYPE_IQ3_S, 256, 110},
+    {QO_TYPE_Q4_0, 32, 18},    {QO_TYPE_Q4_1, 32, 20},   {QO_TYPE_Q5_0, 32, 22},
+    {QO_TYPE_Q5_1, 32, 24},    {QO_TYPE_Q2_K, 256, 84},  {QO_TYPE_Q3_K, 256, 110},
+    {QO_TYPE_IQ2_XS, 256, 74}, {QO_TYPE_IQ3_XXS, 256, 98}, {QO_TYPE_IQ1_S, 256, 50},
+    {QO_TYPE_IQ2_S, 256, 82},  {QO_TYPE_IQ4_XS, 256, 136}, {QO_TYPE_IQ1_M, 256, 56},
+    {QO_TYPE_TQ1_0, 256, 54},  {QO_TYPE_TQ2_0, 256, 66}, {QO_TYPE_MXFP4, 32, 17},
+    {QO_TYPE_NVFP4, 64, 36},   {QO_TYPE_Q1_0, 128, 18},
 };
 static const qo_type_info *find_type(uint32_t type) {
     for (size_t i = 0; i < sizeof(k_types) / sizeof(k_types[0]); i++)
@@ -107,8 +113,7 @@ const void *qo_table(const char *name, size_t *bytes) {
         *bytes = 128;
         return g_sign_table;
     }
-    *bytes = 0;
-    return NULL;
+    return qo_table_ext(name, bytes);
 }
 
 /* ------------------------------------------------------------------ decoders
@@ -289,6 +294,23 @@ int qo_dequant_row(uint32_t type, const void *src, float *dst, int n) {
     case QO_TYPE_IQ2_XXS: qo_dequantize_row_iq2_xxs(src, dst, n); return 0;
     case QO_TYPE_IQ4_NL: qo_dequantize_row_iq4_nl(src, dst, n); return 0;
     case QO_TYPE_IQ3_S: qo_dequantize_row_iq3_s(src, dst, n); return 0;
+    case QO_TYPE_Q4_0: qo_dequantize_row_q4_0(src, dst, n); return 0;
+    case QO_TYPE_Q4_1: qo_dequantize_row_q4_1(src, dst, n); return 0;
+    case QO_TYPE_Q5_0: qo_dequantize_row_q5_0(src, dst, n); return 0;
+    case QO_TYPE_Q5_1: qo_dequantize_row_q5_1(src, dst, n); return 0;
+    case QO_TYPE_Q2_K: qo_dequantize_row_q2_K(src, dst, n); return 0;
+    case QO_TYPE_Q3_K: qo_dequantize_row_q3_K(src, dst, n); return 0;
+    case QO_TYPE_Q1_0: qo_dequantize_row_q1_0(src, dst, n); return 0;
+    case QO_TYPE_MXFP4: qo_dequantize_row_mxfp4(src, dst, n); return 0;
+    case QO_TYPE_NVFP4: qo_dequantize_row_nvfp4(src, dst, n); return 0;
+    case QO_TYPE_IQ3_XXS: qo_dequantize_row_iq3_xxs(src, dst, n); return 0;
+    case QO_TYPE_IQ4_XS: qo_dequantize_row_iq4_xs(src, dst, n); return 0;
+    case QO_TYPE_IQ2_XS: qo_dequantize_row_iq2_xs(src, dst, n); return 0;
+    case QO_TYPE_IQ2_S: qo_dequantize_row_iq2_s(src, dst, n); return 0;
+    case QO_TYPE_IQ1_S: qo_dequantize_row_iq1_s(src, dst, n); return 0;
+    case QO_TYPE_IQ1_M: qo_dequantize_row_iq1_m(src, dst, n); return 0;
+    case QO_TYPE_TQ1_0: qo_dequantize_row_tq1_0(src, dst, n); return 0;
+    case QO_TYPE_TQ2_0: qo_dequantize_row_tq2_0(src, dst, n); return 0;
     case QO_TYPE_F32: memcpy(dst, src, (size_t)n * 4); return 0;
     case QO_TYPE_F16: {
         const uint8_t *p = (const uint8_t *)src;

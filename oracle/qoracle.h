@@ -8,7 +8,8 @@
  * It restates, in plain C, the algorithm of the reference's CPU path:
  *   codec      common/ggml_dequant.h:206-229 (fp16), :261-294 (row size), :1479-1489 (Q8_0),
  *              :1582-1687 (Q4_K/Q5_K/Q6_K), :2793-2816 (IQ2_XXS), :2942-2954 (IQ4_NL),
- *              :3022-3058 (IQ3_S), :3177-3265 (type switch)
+ *              :3022-3058 (IQ3_S), :3177-3265 (type switch); the other seventeen block
+ *              formats of that switch are in qoracle_ext.c, cited per function there
  *   matvec     common/transformer.h:651-660 (double-accumulate oracle mode),
  *              :1049-1114 (fp32 path: dequantize row to scratch, 4x8-lane FMA dot),
  *              common/ggml_dequant.h:953-998 (Q8_0 fused dequant-dot), :1117-1133 of
@@ -33,7 +34,12 @@ extern "C" {
 enum {
     QO_TYPE_F32 = 0, QO_TYPE_F16 = 1, QO_TYPE_Q8_0 = 8, QO_TYPE_Q4_K = 12, QO_TYPE_Q5_K = 13,
     QO_TYPE_Q6_K = 14, QO_TYPE_IQ2_XXS = 16, QO_TYPE_IQ4_NL = 20, QO_TYPE_IQ3_S = 21,
-    QO_TYPE_BF16 = 30
+    QO_TYPE_BF16 = 30,
+    /* the further block formats of the type switch (decoders in qoracle_ext.c) */
+    QO_TYPE_Q4_0 = 2, QO_TYPE_Q4_1 = 3, QO_TYPE_Q5_0 = 6, QO_TYPE_Q5_1 = 7, QO_TYPE_Q2_K = 10,
+    QO_TYPE_Q3_K = 11, QO_TYPE_IQ2_XS = 17, QO_TYPE_IQ3_XXS = 18, QO_TYPE_IQ1_S = 19,
+    QO_TYPE_IQ2_S = 22, QO_TYPE_IQ4_XS = 23, QO_TYPE_IQ1_M = 29, QO_TYPE_TQ1_0 = 34,
+    QO_TYPE_TQ2_0 = 35, QO_TYPE_MXFP4 = 39, QO_TYPE_NVFP4 = 40, QO_TYPE_Q1_0 = 41
 };
 
 /* ---- codec ---- */
@@ -53,6 +59,30 @@ void qo_dequantize_row_q6_K(const void *src, float *dst, int n);
 void qo_dequantize_row_iq2_xxs(const void *src, float *dst, int n);
 void qo_dequantize_row_iq4_nl(const void *src, float *dst, int n);
 void qo_dequantize_row_iq3_s(const void *src, float *dst, int n);
+/* further formats (common/ggml_dequant.h:1491-1580 q1_0/q2_K/q3_K, :2818-2914 mxfp4/nvfp4/q4_0/
+ * q4_1/q5_0/q5_1, :2916-3020 iq3_xxs/iq4_xs/iq2_xs/iq2_s, :3062-3175 iq1_s/iq1_m/tq1_0/tq2_0) */
+void qo_dequantize_row_q4_0(const void *src, float *dst, int n);
+void qo_dequantize_row_q4_1(const void *src, float *dst, int n);
+void qo_dequantize_row_q5_0(const void *src, float *dst, int n);
+void qo_dequantize_row_q5_1(const void *src, float *dst, int n);
+void qo_dequantize_row_q2_K(const void *src, float *dst, int n);
+void qo_dequantize_row_q3_K(const void *src, float *dst, int n);
+void qo_dequantize_row_q1_0(const void *src, float *dst, int n);
+void qo_dequantize_row_mxfp4(const void *src, float *dst, int n);
+void qo_dequantize_row_nvfp4(const void *src, float *dst, int n);
+void qo_dequantize_row_iq3_xxs(const void *src, float *dst, int n);
+void qo_dequantize_row_iq4_xs(const void *src, float *dst, int n);
+void qo_dequantize_row_iq2_xs(const void *src, float *dst, int n);
+void qo_dequantize_row_iq2_s(const void *src, float *dst, int n);
+void qo_dequantize_row_iq1_s(const void *src, float *dst, int n);
+void qo_dequantize_row_iq1_m(const void *src, float *dst, int n);
+void qo_dequantize_row_tq1_0(const void *src, float *dst, int n);
+void qo_dequantize_row_tq2_0(const void *src, float *dst, int n);
+/* scale bytes of MXFP4 (E8M0, halved) and NVFP4 (unsigned E4M3, halved) */
+float qo_e8m0_half_to_fp32(uint8_t e);
+float qo_ue4m3_half_to_fp32(uint8_t x);
+/* 6-bit scale i (0..15) of a Q3_K block's 12 packed scale bytes, before the -32 offset */
+int  qo_q3k_scale(const uint8_t packed[12], int i);
 /* 0 on success, -1 for an unsupported type (dst untouched) */
 int  qo_dequant_row(uint32_t type, const void *src, float *dst, int n);
 
@@ -63,6 +93,7 @@ void qo_k4_pack_scales(const uint8_t sc[8], const uint8_t mn[8], uint8_t packed[
 
 /* raw access to the codebooks, for checksum tests */
 const void *qo_table(const char *name, size_t *bytes);
+const void *qo_table_ext(const char *name, size_t *bytes);
 
 /* ---- matvec y[n_rows] = W . x ---- */
 /* dequantize each row to fp32, dot in double, round once to fp32 */

@@ -105,6 +105,11 @@ const void *ref_table(const char *name, size_t *bytes) {
     if (!strcmp(name, "iq3s_grid")) { *bytes = sizeof(iq3s_grid); return iq3s_grid; }
     if (!strcmp(name, "iq4nl_values")) { *bytes = sizeof(kvalues_iq4nl); return kvalues_iq4nl; }
     if (!strcmp(name, "ksigns")) { *bytes = sizeof(ksigns_iq2xs); return ksigns_iq2xs; }
+    if (!strcmp(name, "mxfp4_values")) { *bytes = sizeof(kvalues_mxfp4); return kvalues_mxfp4; }
+    if (!strcmp(name, "iq3xxs_grid")) { *bytes = sizeof(iq3xxs_grid); return iq3xxs_grid; }
+    if (!strcmp(name, "iq2xs_grid")) { *bytes = sizeof(iq2xs_grid); return iq2xs_grid; }
+    if (!strcmp(name, "iq2s_grid")) { *bytes = sizeof(iq2s_grid); return iq2s_grid; }
+    if (!strcmp(name, "iq1s_grid")) { *bytes = sizeof(iq1s_grid); return iq1s_grid; }
     *bytes = 0;
     return NULL;
 }

@@ -30,7 +30,7 @@ static qtensor make_tensor(uint32_t type, int n_rows, int n_cols) {
     const size_t rb = tf_row_bytes(type, n_cols);
     uint8_t *p = (uint8_t *)malloc(rb * (size_t)n_rows);
     for (size_t i = 0; i < rb * (size_t)n_rows; i++) p[i] = (uint8_t)rnd();
-    const int bb = type == 8 ? 34 : type == 12 ? 144 : 210;
+    const int bb = type == 8 ? 34 : type == 12 ? 144 : type == 17 ? 74 : 210;
     for (size_t off = 0; off + bb <= rb * (size_t)n_rows; off += bb) {
         const uint16_t h = (uint16_t)(0x1C00 + (rnd() & 0x3FF)); /* 2^-8 .. 2^-7 */
         if (type == 14) memcpy(p + off + 208, &h, 2);
@@ -70,8 +70,12 @@ int main(void) {
 
     qtensor a = make_tensor(12, 256, K), b = make_tensor(12, 256, K), c8 = make_tensor(8, 96, K),
             c6 = make_tensor(14, 96, K);
-    if (tf_is_supported_weight_type(12) != 1 || tf_is_supported_weight_type(2) != 0) { printf("type check FAIL\n"); failures++; }
-    if (tf_row_bytes(12, 4096) != 2304 || tf_row_bytes(99, 4096) != 0) { printf("row bytes FAIL\n"); failures++; }
+    /* 17 = IQ2_XS is a model weight type; 3 = Q4_1 has a decoder but is not one (common/transformer.h:462-487) */
+    if (tf_is_supported_weight_type(12) != 1 || tf_is_supported_weight_type(17) != 1 || tf_is_supported_weight_type(3) != 0) { printf("type check FAIL\n"); failures++; }
+    if (tf_row_bytes(12, 4096) != 2304 || tf_row_bytes(17, 4096) != 1184 || tf_row_bytes(3, 4096) != 0 || tf_row_bytes(99, 4096) != 0) { printf("row bytes FAIL\n"); failures++; }
+    qtensor c17 = make_tensor(17, 96, K);
+    tf_qmatvec(y, &c17, x, 96, NULL);
+    check_rows("tf_qmatvec iq2_xs", &c17, 0, 96, x, y);
 
     tf_qmatvec(y, &a, x, 256, NULL);
     check_rows("tf_qmatvec q4_K", &a, 0, 256, x, y);
@@ -100,7 +104,7 @@ int main(void) {
 
     /* failure behaviour: unsupported type -> message on stderr, zero-filled output, no crash */
     qtensor bad = a;
-    bad.type = 2; /* Q4_0: not one of the seven formats */
+    bad.type = 9; /* Q8_1: an activation format, no weight decoder */
     for (int i = 0; i < 256; i++) y[i] = 1.0f;
     tf_qmatvec(y, &bad, x, 256, NULL);
     int zeros = 1;

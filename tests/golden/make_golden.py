@@ -33,6 +33,15 @@ def sha(a):
     return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
 
 
+def canonical_nan(bits):
+    """fp32 bit patterns with every NaN replaced by 0x7FC00000: where two NaN scales meet (d and
+    dmin of one block), which payload survives depends on the compiler's operand order, not on
+    the format, so sweep hashes are taken over canonical NaNs."""
+    bits = np.array(bits, dtype=np.uint32, copy=True)
+    bits[(bits & 0x7FFFFFFF) > 0x7F800000] = 0x7FC00000
+    return bits
+
+
 def main():
     ref = Reference()
     manifest = {"generator": "tests/golden/make_golden.py", "source": "reference C compiled via oracle/ref_shim.c"}
@@ -45,7 +54,8 @@ def main():
 
     # codebooks
     manifest["tables_sha256"] = {n: hashlib.sha256(ref.table(n)).hexdigest()
-                                 for n in ("iq2xxs_grid", "iq3s_grid", "iq4nl_values", "ksigns")}
+                                 for n in ("iq2xxs_grid", "iq3s_grid", "iq4nl_values", "ksigns", "mxfp4_values",
+                                           "iq3xxs_grid", "iq2xs_grid", "iq2s_grid", "iq1s_grid")}
 
     codec, sweep = {}, {}
     for tid, name in synth.TYPE_NAMES.items():
@@ -67,10 +77,12 @@ def main():
         for r in range(SWEEP_ROWS):
             dec[r] = ref.dequant_row(tid, big[r], SWEEP_COLS)[1].view(np.uint32)
         sweep[name] = {"seed": 3000 + tid, "rows": SWEEP_ROWS, "cols": SWEEP_COLS, "wild": True,
-                       "input_sha256": sha(big), "output_sha256": sha(dec)}
+                       "input_sha256": sha(big), "output_sha256": sha(canonical_nan(dec))}
     manifest["codec_sweep"] = sweep
     manifest["row_size"] = {str(t): {str(n): ref.row_size(t, n) for n in (0, 1, 31, 32, 33, 255, 256, 257, 4096, 14336)}
                             for t in list(synth.TYPE_NAMES) + [0, 1, 30, 9, 15, 99]}
+    # what the model path accepts, and its own row-size function (0 outside that list)
+    manifest["tf_row_bytes_4096"] = {str(t): ref.tf_row_bytes(t, 4096) for t in list(range(0, 44)) + [99]}
     rc, _ = ref.dequant_row(99, np.zeros(64, np.uint8), 32)
     manifest["dequant_row_unknown_type_rc"] = rc
     np.savez_compressed(os.path.join(OUT, "codec_golden.npz"), **codec)
@@ -80,7 +92,7 @@ def main():
     x = synth.make_activation(LIN_COLS, seed=77)
     X = synth.make_activation(LIN_COLS, seed=78, tokens=5)
     lin["x"], lin["X"] = x, X
-    for tid, name in synth.TYPE_NAMES.items():
+    for tid, name in synth.LINEAR_TYPES.items():  # the types the reference's model path accepts
         W = synth.make_weights(tid, LIN_ROWS, LIN_COLS, seed=4000 + tid)
         lin[name + "_W"] = W
         lin[name + "_y_f32"] = ref.qmatvec(tid, W, x, LIN_COLS)

@@ -9,10 +9,11 @@ from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu
 NAMES = list(synth.TYPE_NAMES.items())
+LINEAR = list(synth.LINEAR_TYPES.items())  # the types the reference golden outputs exist for
 TOL = 1e-5
 
 
-@pytest.mark.parametrize("tid,name", NAMES)
+@pytest.mark.parametrize("tid,name", LINEAR)
 def test_matvec_matches_reference_golden(linear_golden, tid, name):
     W, x = linear_golden[name + "_W"], linear_golden["x"]
     y = qlinear.matvec(tid, W, x, x.shape[0])
@@ -109,7 +110,7 @@ def test_fused_entry_points(oracle, linear_golden):
     assert rel_l2(v, linear_golden["q8_0_y_f64"][:16]) <= TOL
 
 
-@pytest.mark.parametrize("tid,name", NAMES)
+@pytest.mark.parametrize("tid,name", LINEAR)
 def test_expert_slice_and_prefill_match_reference_golden(linear_golden, tid, name):
     lib = qlinear.load()
     W, x, X = linear_golden[name + "_W"], linear_golden["x"], linear_golden["X"]
