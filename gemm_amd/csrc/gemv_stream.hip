@@ -51,25 +51,25 @@ __device__ __forceinline__ float dot_u4_signed(uint32_t b, uint32_t signs, const
     acc = fmaf(__uint_as_float(__float_as_uint(ub2(b)) | ((t << 1) & 0x80000000u)), x.z, acc);
     return fmaf(__uint_as_float(__float_as_uint(ub3(b)) | (t & 0x80000000u)), x.w, acc);
 }
-/* 8 (4) bytes at byte offset `off` (even) of a 16-byte aligned LDS image. Misaligned LDS reads
+/* 8 (4) bytes at any byte offset `off` of a 16-byte aligned LDS image. Misaligned LDS reads
  * stall the LDS pipeline on this part (they were 3/4 of its busy time in the first version of
  * this kernel), so the bytes are fetched as aligned dwords and funnel-shifted into place. May
  * touch up to 4 bytes past the last one asked for. */
 __device__ __forceinline__ uint2 ld8_at(const uint8_t *img, int off) {
     const uint32_t *q = reinterpret_cast<const uint32_t *>(img + (off & ~3));
-    const uint32_t sh = (uint32_t)(off & 2) * 8u;
+    const uint32_t sh = (uint32_t)(off & 3) * 8u;
     const uint32_t w0 = q[0], w1 = q[1], w2 = q[2];
     return make_uint2(__builtin_amdgcn_alignbit(w1, w0, sh), __builtin_amdgcn_alignbit(w2, w1, sh));
 }
 __device__ __forceinline__ uint32_t ld4_at(const uint8_t *img, int off) {
     const uint32_t *q = reinterpret_cast<const uint32_t *>(img + (off & ~3));
-    return __builtin_amdgcn_alignbit(q[1], q[0], (uint32_t)(off & 2) * 8u);
+    return __builtin_amdgcn_alignbit(q[1], q[0], (uint32_t)(off & 3) * 8u);
 }
 
 struct Tables {
     const uint64_t *grid2; /* iq2xxs grid in LDS */
     const uint32_t *grid3; /* iq3s grid in LDS */
-    uint32_t nl0, nl1, nl2, nl3; /* the 16 iq4nl values + 128, as bytes */
+    uint32_t nl0, nl1, nl2, nl3; /* the 16 values of a 4-bit codebook (iq4nl or E2M1) + 128, as bytes */
 };
 
 /* default: the bit-exact decoder (Q4_K reaches this kernel only when the tuned one declines) */
@@ -187,8 +187,237 @@ template <> struct Lean<T_IQ3_S> {
     }
 };
 
-template <uint32_t T> constexpr bool kNeedsGrid2 = (T == T_IQ2_XXS);
-template <uint32_t T> constexpr bool kNeedsGrid3 = (T == T_IQ3_S);
+
+/* bits 0..3 of v spread to bit 0 of bytes 0..3 (the shifted copies of the multiply do not overlap) */
+__device__ __forceinline__ uint32_t spread4(uint32_t v) { return ((v & 15u) * 0x00204081u) & 0x01010101u; }
+
+/* Q4_0 (:2850-2862): d * (nibble - 8) */
+template <> struct Lean<T_Q4_0> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const float d = half_bits_fast(ld_u16(img + boff));
+        const uint2 q = ld8_at(img, boff + 2 + (k0 & 15));
+        const int sh = (k0 >> 4) * 4;
+        const float s = dot_u4((q.y >> sh) & 0x0F0F0F0Fu, xb, dot_u4((q.x >> sh) & 0x0F0F0F0Fu, xa, 0.0f));
+        return d * fmaf(-8.0f, xs8, s);
+    }
+};
+
+/* Q4_1 (:2864-2877): d * nibble + m */
+template <> struct Lean<T_Q4_1> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint32_t h = *reinterpret_cast<const uint32_t *>(img + boff); /* 20-byte blocks: dword aligned */
+        const uint2 q = ld8_at(img, boff + 4 + (k0 & 15));
+        const int sh = (k0 >> 4) * 4;
+        const float s = dot_u4((q.y >> sh) & 0x0F0F0F0Fu, xb, dot_u4((q.x >> sh) & 0x0F0F0F0Fu, xa, 0.0f));
+        return fmaf(half_bits_fast(h & 0xFFFFu), s, half_bits_fast(h >> 16) * xs8);
+    }
+};
+
+/* Q5_0 (:2879-2895): d * (nibble + 16*bit - 16); the eight fifth bits of a group are one byte of qh */
+template <> struct Lean<T_Q5_0> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const float d = half_bits_fast(ld_u16(blk));
+        const uint32_t hb = blk[2 + (k0 >> 3)];
+        const uint2 q = ld8_at(img, boff + 6 + (k0 & 15));
+        const int sh = (k0 >> 4) * 4;
+        const uint32_t v0 = ((q.x >> sh) & 0x0F0F0F0Fu) | (spread4(hb) << 4);
+        const uint32_t v1 = ((q.y >> sh) & 0x0F0F0F0Fu) | (spread4(hb >> 4) << 4);
+        return d * fmaf(-16.0f, xs8, dot_u4(v1, xb, dot_u4(v0, xa, 0.0f)));
+    }
+};
+
+/* Q5_1 (:2897-2914): d * (nibble + 16*bit) + m */
+template <> struct Lean<T_Q5_1> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const uint32_t h = *reinterpret_cast<const uint32_t *>(blk); /* 24-byte blocks: dword aligned */
+        const uint32_t hb = blk[4 + (k0 >> 3)];
+        const uint2 q = *reinterpret_cast<const uint2 *>(blk + 8 + (k0 & 15));
+        const int sh = (k0 >> 4) * 4;
+        const uint32_t v0 = ((q.x >> sh) & 0x0F0F0F0Fu) | (spread4(hb) << 4);
+        const uint32_t v1 = ((q.y >> sh) & 0x0F0F0F0Fu) | (spread4(hb >> 4) << 4);
+        return fmaf(half_bits_fast(h & 0xFFFFu), dot_u4(v1, xb, dot_u4(v0, xa, 0.0f)), half_bits_fast(h >> 16) * xs8);
+    }
+};
+
+/* Q2_K (:1505-1534): (d*(sc&15)) * q2 - dmin*(sc>>4); 84-byte blocks are dword aligned */
+template <> struct Lean<T_Q2_K> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const uint32_t h = *reinterpret_cast<const uint32_t *>(blk + 80);
+        const int half = k0 >> 7, j = (k0 >> 5) & 3, sub = (k0 >> 4) & 1, l0 = k0 & 15;
+        const uint32_t sc = blk[8 * half + 2 * j + sub];
+        const uint2 q = ld8_at(img, boff + 16 + 32 * half + 16 * sub + l0);
+        const float s = dot_u4((q.y >> (2 * j)) & 0x03030303u, xb, dot_u4((q.x >> (2 * j)) & 0x03030303u, xa, 0.0f));
+        return fmaf(half_bits_fast(h & 0xFFFFu) * (float)(sc & 15u), s, -(half_bits_fast(h >> 16) * (float)(sc >> 4)) * xs8);
+    }
+};
+
+/* Q3_K (:1536-1580): (d*(sc-32)) * (q2 + 4*hbit - 4) */
+template <> struct Lean<T_Q3_K> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const int half = k0 >> 7, j = (k0 >> 5) & 3, sub = (k0 >> 4) & 1, l0 = k0 & 15;
+        const int is = 8 * half + 2 * j + sub;
+        const uint8_t *sp = blk + 96;
+        const int lo4 = is < 8 ? (sp[is] & 15) : (sp[is - 8] >> 4);
+        const int hi2 = (sp[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+        const float dl = half_bits_fast(ld_u16(blk + 108)) * (float)((lo4 | (hi2 << 4)) - 32);
+        const uint2 q = ld8_at(img, boff + 32 + 32 * half + 16 * sub + l0);
+        const uint2 hm = ld8_at(img, boff + 16 * sub + l0);
+        const int hsh = 4 * half + j;
+        const uint32_t v0 = ((q.x >> (2 * j)) & 0x03030303u) | (((hm.x >> hsh) & 0x01010101u) << 2);
+        const uint32_t v1 = ((q.y >> (2 * j)) & 0x03030303u) | (((hm.y >> hsh) & 0x01010101u) << 2);
+        return dl * fmaf(-4.0f, xs8, dot_u4(v1, xb, dot_u4(v0, xa, 0.0f)));
+    }
+};
+
+/* IQ4_XS (:2956-2973): (d*(ls-32)) * table[nibble]; 136-byte blocks are dword aligned */
+template <> struct Lean<T_IQ4_XS> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const uint2 h = *reinterpret_cast<const uint2 *>(blk); /* d, scales_h | scales_l */
+        const int g = k0 >> 5, r = k0 & 31;
+        const int ls = (int)(((h.y >> (4 * g)) & 15u) | ((((h.x >> 16) >> (2 * g)) & 3u) << 4));
+        const float dl = half_bits_fast(h.x & 0xFFFFu) * (float)(ls - 32);
+        const uint2 q = *reinterpret_cast<const uint2 *>(blk + 8 + 16 * g + (r & 15));
+        const int sh = (r >> 4) * 4;
+        const uint32_t v0 = Lean<T_IQ4_NL>::look4((q.x >> sh) & 0x0F0F0F0Fu, t), v1 = Lean<T_IQ4_NL>::look4((q.y >> sh) & 0x0F0F0F0Fu, t);
+        return dl * fmaf(-128.0f, xs8, dot_u4(v1, xb, dot_u4(v0, xa, 0.0f)));
+    }
+};
+
+/* IQ2_XS (:2975-2994): d*(0.5+nibble)*0.25 * grid byte * sign */
+template <> struct Lean<T_IQ2_XS> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const float db = half_bits_fast(ld_u16(blk)) * (0.5f + (float)((blk[66 + g] >> (4 * (l >> 1))) & 15)) * 0.25f;
+        const uint32_t w = ld_u16(blk + 2 + 2 * (4 * g + l));
+        const uint2 cell = *reinterpret_cast<const uint2 *>(t.grid2 + (w & 511u));
+        const uint32_t sg = iq_sign_byte(w >> 9);
+        return db * dot_u4_signed(cell.y, sg >> 4, xb, dot_u4_signed(cell.x, sg & 15u, xa, 0.0f));
+    }
+};
+
+/* IQ2_S (:2996-3020): as IQ2_XS with a 10-bit grid index and the sign byte stored as is */
+template <> struct Lean<T_IQ2_S> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const float db = half_bits_fast(ld_u16(blk)) * (0.5f + (float)((blk[74 + g] >> (4 * (l >> 1))) & 15)) * 0.25f;
+        const uint32_t idx = blk[2 + 4 * g + l] | ((((uint32_t)blk[66 + g] >> (2 * l)) & 3u) << 8);
+        const uint2 cell = *reinterpret_cast<const uint2 *>(t.grid2 + idx);
+        const uint32_t sg = blk[34 + 4 * g + l];
+        return db * dot_u4_signed(cell.y, sg >> 4, xb, dot_u4_signed(cell.x, sg & 15u, xa, 0.0f));
+    }
+};
+
+/* IQ3_XXS (:2916-2940): d*(0.5+s)*0.5 * grid byte * sign, two 4-byte grid entries per eight elements */
+template <> struct Lean<T_IQ3_XXS> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint32_t w = ld4_at(img, boff + 66 + 4 * g);
+        const float db = half_bits_fast(ld_u16(blk)) * (0.5f + (float)(w >> 28)) * 0.5f;
+        const uint32_t sg = iq_sign_byte((w >> (7 * l)) & 127u);
+        const uint32_t pair = ld_u16(blk + 2 + 8 * g + 2 * l);
+        return db * dot_u4_signed(t.grid3[pair >> 8], sg >> 4, xb, dot_u4_signed(t.grid3[pair & 255u], sg & 15u, xa, 0.0f));
+    }
+};
+
+/* IQ1_S (:3062-3082): (d*(2s+1)) * (t + delta); the grid is staged as t+1 in {0,1,2}, so
+ * sum (t + delta) x = sum (t+1) x + (delta - 1) sum x */
+template <> struct Lean<T_IQ1_S> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint32_t h = ld_u16(blk + 34 + 2 * g);
+        const float dl = half_bits_fast(ld_u16(blk)) * (float)(2 * (int)((h >> 12) & 7u) + 1);
+        const float dm1 = (h & 0x8000u) ? -1.125f : -0.875f;
+        const uint2 cell = *reinterpret_cast<const uint2 *>(t.grid2 + (blk[2 + 4 * g + l] | (((h >> (3 * l)) & 7u) << 8)));
+        return dl * fmaf(dm1, xs8, dot_u4(cell.y, xb, dot_u4(cell.x, xa, 0.0f)));
+    }
+};
+
+/* IQ1_M (:3084-3125): as IQ1_S with the super-scale in the top nibbles of the four scale words
+ * and per-eight index extension and shift sign in the nibbles of qh; 56-byte blocks are 8-byte aligned */
+template <> struct Lean<T_IQ1_M> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &t) {
+        const uint8_t *blk = img + boff;
+        const uint2 sw = *reinterpret_cast<const uint2 *>(blk + 48);
+        const uint32_t dbits = ((sw.x >> 12) & 0x000Fu) | ((sw.x >> 24) & 0x00F0u) | ((sw.y >> 4) & 0x0F00u) | ((sw.y >> 16) & 0xF000u);
+        const int g = k0 >> 5, l = (k0 & 31) >> 3;
+        const uint32_t word = ((g & 4) ? sw.y : sw.x) >> (16 * ((g >> 1) & 1));
+        const float dl = half_bits_fast(dbits) * (float)(2 * (int)((word >> (6 * (g & 1) + 3 * (l >> 1))) & 7u) + 1);
+        const uint32_t nib = ((uint32_t)blk[32 + 2 * g + (l >> 1)] >> (4 * (l & 1))) & 15u;
+        const float dm1 = (nib & 8u) ? -1.125f : -0.875f;
+        const uint2 cell = *reinterpret_cast<const uint2 *>(t.grid2 + (blk[4 * g + l] | ((nib & 7u) << 8)));
+        return dl * fmaf(dm1, xs8, dot_u4(cell.y, xb, dot_u4(cell.x, xa, 0.0f)));
+    }
+};
+
+/* TQ2_0 (:3161-3175): d * (q2 - 1) */
+template <> struct Lean<T_TQ2_0> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const float d = half_bits_fast(ld_u16(img + boff + 64));
+        const uint2 q = ld8_at(img, boff + 32 * (k0 >> 7) + (k0 & 31));
+        const int sh = 2 * ((k0 >> 5) & 3);
+        return d * (dot_u4((q.y >> sh) & 0x03030303u, xb, dot_u4((q.x >> sh) & 0x03030303u, xa, 0.0f)) - xs8);
+    }
+};
+
+/* Q1_0 (:1491-1503): +d where the bit is set, -d where it is clear: d * (2 * sum_{set} x - sum x) */
+template <> struct Lean<T_Q1_0> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
+        const uint8_t *blk = img + boff;
+        const float d = half_bits_fast(ld_u16(blk));
+        const uint32_t bits = blk[2 + (k0 >> 3)];
+        return d * fmaf(2.0f, dot_u4(spread4(bits >> 4), xb, dot_u4(spread4(bits), xa, 0.0f)), -xs8);
+    }
+};
+
+/* MXFP4 (:2818-2830): 2^(e-128) * E2M1x2[nibble], the 16 values looked up like IQ4_NL's (stored + 128) */
+template <> struct Lean<T_MXFP4> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &t) {
+        const float d = e8m0_half(img[boff]);
+        const uint2 q = ld8_at(img, boff + 1 + (k0 & 15));
+        const int sh = (k0 >> 4) * 4;
+        const uint32_t v0 = Lean<T_IQ4_NL>::look4((q.x >> sh) & 0x0F0F0F0Fu, t), v1 = Lean<T_IQ4_NL>::look4((q.y >> sh) & 0x0F0F0F0Fu, t);
+        return d * fmaf(-128.0f, xs8, dot_u4(v1, xb, dot_u4(v0, xa, 0.0f)));
+    }
+};
+
+/* NVFP4 (:2832-2848): ue4m3 scale per 16 elements, same value table */
+template <> struct Lean<T_NVFP4> {
+    __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &t) {
+        const int sb = k0 >> 4;
+        const float d = ue4m3_half(img[boff + sb]);
+        const uint2 q = ld8_at(img, boff + 4 + 8 * sb);
+        const int sh = ((k0 >> 3) & 1) * 4;
+        const uint32_t v0 = Lean<T_IQ4_NL>::look4((q.x >> sh) & 0x0F0F0F0Fu, t), v1 = Lean<T_IQ4_NL>::look4((q.y >> sh) & 0x0F0F0F0Fu, t);
+        return d * fmaf(-128.0f, xs8, dot_u4(v1, xb, dot_u4(v0, xa, 0.0f)));
+    }
+};
+
+/* codebook a type's dot8 reads from LDS: its source in device memory and its size; the ternary
+ * grid of IQ1_S/IQ1_M is staged with 1 added to every byte */
+template <uint32_t T> struct Grid { static constexpr int kBytes = 0; static constexpr bool kPlusOne = false; __device__ static const uint32_t *src() { return nullptr; } };
+#define QLIN_GRID(TT, TABLE, PLUS)                                                                \
+    template <> struct Grid<TT> {                                                                 \
+        static constexpr int kBytes = (int)sizeof(TABLE);                                          \
+        static constexpr bool kPlusOne = PLUS;                                                     \
+        __device__ static const uint32_t *src() { return reinterpret_cast<const uint32_t *>(TABLE); } \
+    };
+QLIN_GRID(T_IQ2_XXS, qlin_iq2xxs_grid, false)
+QLIN_GRID(T_IQ3_S, qlin_iq3s_grid, false)
+QLIN_GRID(T_IQ2_XS, qlin_iq2xs_grid, false)
+QLIN_GRID(T_IQ2_S, qlin_iq2s_grid, false)
+QLIN_GRID(T_IQ3_XXS, qlin_iq3xxs_grid, false)
+QLIN_GRID(T_IQ1_S, qlin_iq1s_grid, true)
+QLIN_GRID(T_IQ1_M, qlin_iq1s_grid, true)
+#undef QLIN_GRID
 
 
 template <uint32_t T>
@@ -198,12 +427,12 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
     using C = Codec<T>;
     constexpr int GPB = C::BE / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    /* LDS map: x [n_cols] | sums of eight x [n_cols/8] | i-quant grid, 2 KB, where the type has one |
+    /* LDS map: x [n_cols] | sums of eight x [n_cols/8] | i-quant grid (1..16 KB) where the type has one |
      * row images [waves][depth][image_bytes] */
     float *xs = reinterpret_cast<float *>(lds);
     float *xs8 = xs + n_cols;
     uint8_t *grid = reinterpret_cast<uint8_t *>(xs8 + (n_cols >> 3));
-    uint8_t *images = grid + ((kNeedsGrid2<T> || kNeedsGrid3<T>) ? 2048 : 0);
+    uint8_t *images = grid + Grid<T>::kBytes;
 
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* wave-uniform, and the compiler is told so */
@@ -254,15 +483,17 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
     tab.grid2 = reinterpret_cast<const uint64_t *>(grid);
     tab.grid3 = reinterpret_cast<const uint32_t *>(grid);
     tab.nl0 = tab.nl1 = tab.nl2 = tab.nl3 = 0;
-    if (T == T_IQ4_NL) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(qlin_iq4nl_values);
+    if (T == T_IQ4_NL || T == T_IQ4_XS || T == T_MXFP4 || T == T_NVFP4) {
+        const uint4 v = *reinterpret_cast<const uint4 *>((T == T_MXFP4 || T == T_NVFP4) ? qlin_mxfp4_values : qlin_iq4nl_values);
         tab.nl0 = v.x ^ 0x80808080u; tab.nl1 = v.y ^ 0x80808080u; tab.nl2 = v.z ^ 0x80808080u; tab.nl3 = v.w ^ 0x80808080u;
     }
-    if (kNeedsGrid2<T>)
-        for (int t = threadIdx.x; t < 512; t += n_threads)
-            reinterpret_cast<uint32_t *>(grid)[t] = reinterpret_cast<const uint32_t *>(qlin_iq2xxs_grid)[t];
-    if (kNeedsGrid3<T>)
-        for (int t = threadIdx.x; t < 512; t += n_threads) reinterpret_cast<uint32_t *>(grid)[t] = qlin_iq3s_grid[t];
+    if (Grid<T>::kBytes > 0)
+        for (int t = threadIdx.x; t < Grid<T>::kBytes / 4; t += n_threads) {
+            uint32_t v = Grid<T>::src()[t];
+            if (Grid<T>::kPlusOne) /* bytes 0xFF, 0, 1 -> 0, 1, 2: add 1 per byte, no carry between bytes */
+                v = ((v & 0x7F7F7F7Fu) + 0x01010101u) ^ (v & 0x80808080u);
+            reinterpret_cast<uint32_t *>(grid)[t] = v;
+        }
     __syncthreads();
     for (int t = threadIdx.x; t < (n_cols >> 3); t += n_threads) {
         const float4 a = *reinterpret_cast<const float4 *>(xs + 8 * t), b = *reinterpret_cast<const float4 *>(xs + 8 * t + 4);
@@ -302,7 +533,7 @@ bool stream_typed(const void *W, const float *x, float *y, int n_rows, int n_col
     const size_t row_bytes = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
     if (n_cols > 16384 || (n_cols & 31) || (row_bytes & 15) || row_bytes > 8192) return false;
     if (((uintptr_t)W & 15) || ((uintptr_t)x & 15)) return false;
-    const size_t x_bytes = (size_t)n_cols * 4 + (size_t)(n_cols >> 3) * 4 + ((kNeedsGrid2<T> || kNeedsGrid3<T>) ? 2048 : 0);
+    const size_t x_bytes = (size_t)n_cols * 4 + (size_t)(n_cols >> 3) * 4 + (size_t)Grid<T>::kBytes;
     const size_t lds_cap = 160 * 1024 - 16;
     /* 16 waves with two images each if that fits, else one image, else 8 waves */
     int waves = 16, depth = 2;
