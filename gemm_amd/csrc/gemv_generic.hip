@@ -13,16 +13,33 @@
 
 namespace qlin {
 
-template <uint32_t T, int R>
+template <uint32_t T>
 __global__ void __launch_bounds__(256)
-gemv_generic_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
-                    int n_rows, int n_cols, size_t row_bytes) {
+gemv_generic_kernel(const JobView job, const float *__restrict__ x, int n_cols, size_t row_bytes) {
     using C = Codec<T>;
     constexpr int GPB = C::BE / 8;
+    constexpr int R = 2;
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    const int row0 = wave * R;
-    if (row0 >= n_rows) return;
+    /* the wave's two rows: consecutive rows of the concatenated matrices, or (mode 2) row `wave` of
+     * the first and of the second matrix */
+    const bool paired = job.mode == 2;
+    const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
+    const uint8_t *Wr[R];
+    float *yr[R];
+    int rr[R];
+    bool live[R];
+    if (paired) {
+        if (wave >= n_rows) return;
+        Wr[0] = job.W0; Wr[1] = job.W1; yr[0] = yr[1] = job.y0; rr[0] = rr[1] = wave; live[0] = live[1] = true;
+    } else {
+        if (wave * R >= n_rows) return;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            live[r] = wave * R + r < n_rows;
+            job_locate(job, live[r] ? wave * R + r : 0, Wr[r], yr[r], rr[r]);
+        }
+    }
     const int groups = (n_cols / C::BE) * GPB;
     float acc[R];
 #pragma unroll
@@ -33,18 +50,24 @@ gemv_generic_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, 
         const float4 xb = *reinterpret_cast<const float4 *>(x + (size_t)blk * C::BE + k0 + 4);
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            if (row0 + r < n_rows) {
+            if (live[r]) {
                 float w[8];
-                C::decode8(W + (size_t)(row0 + r) * row_bytes + (size_t)blk * C::BB, k0, w);
+                C::decode8(Wr[r] + (size_t)rr[r] * row_bytes + (size_t)blk * C::BB, k0, w);
                 acc[r] += w[0] * xa.x + w[1] * xa.y + w[2] * xa.z + w[3] * xa.w +
                           w[4] * xb.x + w[5] * xb.y + w[6] * xb.z + w[7] * xb.w;
             }
         }
     }
+    float s[R];
 #pragma unroll
-    for (int r = 0; r < R; r++) {
-        const float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < n_rows) y[row0 + r] = s;
+    for (int r = 0; r < R; r++) s[r] = wave_sum(acc[r]);
+    if (lane != 0) return;
+    if (paired) {
+        yr[0][rr[0]] = silu_times(s[0], s[1]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (live[r]) yr[r][rr[r]] = job.mode == 1 ? yr[r][rr[r]] + s[r] : s[r];
     }
 }
 
@@ -86,20 +109,18 @@ gemm_f32_generic_kernel(const uint8_t *__restrict__ W, const float *__restrict__
 }
 
 template <uint32_t T>
-static hipError_t gemv_typed(const void *W, const float *x, float *y, int n_rows, int n_cols, hipStream_t s) {
-    constexpr int R = 2;
+static hipError_t gemv_typed(const GemvJob &job, const float *x, int n_cols, hipStream_t s) {
     const size_t rb = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
-    const int waves = (n_rows + R - 1) / R;
-    hipLaunchKernelGGL((gemv_generic_kernel<T, R>), dim3((waves + 3) / 4), dim3(256), 0, s,
-                       (const uint8_t *)W, x, y, n_rows, n_cols, rb);
+    const int waves = job.mode == kSiluMul ? job.n_rows[0] : (job.total_rows() + 1) / 2;
+    if (waves == 0) return hipSuccess;
+    const JobView view = job_view(job);
+    hipLaunchKernelGGL((gemv_generic_kernel<T>), dim3((waves + 3) / 4), dim3(256), 0, s, view, x, n_cols, rb);
     return hipGetLastError();
 }
 
-hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, float *y, int n_rows,
-                               int n_cols, hipStream_t s) {
-    if (n_rows == 0) return hipSuccess;
+hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t s) {
     switch (type) {
-#define QLIN_CASE(TT) case TT: return gemv_typed<TT>(W, x, y, n_rows, n_cols, s);
+#define QLIN_CASE(TT) case TT: return gemv_typed<TT>(job, x, n_cols, s);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
 #undef QLIN_CASE
     default: return hipErrorInvalidValue;

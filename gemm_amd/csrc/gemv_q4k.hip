@@ -75,8 +75,8 @@ __device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { 
 }  // namespace
 
 __global__ void __launch_bounds__(kThreads)
-gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
-                int n_rows, int n_sb, int n_slices, int slice_sb, int rows_per_wg, int depth) {
+gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int n_slices, int slice_sb,
+                int rows_per_wg, int depth) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     /* LDS map: planes [n_sb*4][kChunk] dwords | meta [n_sb*4] float4 | row images [16][depth][kRowImage] |
      * partial sums [rows_per_wg * n_slices] floats (padded to 16 bytes) | raw x [n_sb*256] floats */
@@ -84,7 +84,11 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     float4 *meta = reinterpret_cast<float4 *>(planes + n_sb * 4 * kChunk);
     uint8_t *images = reinterpret_cast<uint8_t *>(meta + n_sb * 4);
     float *partial = reinterpret_cast<float *>(images + kWaves * depth * kRowImage);
-    const float4 *xraw = reinterpret_cast<const float4 *>(partial + ((rows_per_wg * n_slices + 3) & ~3));
+    /* a workgroup owns rows_per_wg rows: of the concatenated matrices, or, where two results are
+     * combined (mode 2), the same rows of both matrices (local rows: first matrix, then second) */
+    const bool paired = job.mode == 2;
+    const int n_mats_here = paired ? 2 : 1;
+    const float4 *xraw = reinterpret_cast<const float4 *>(partial + ((rows_per_wg * n_mats_here * n_slices + 3) & ~3));
 
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* wave-uniform, and the compiler is told so */
@@ -99,15 +103,27 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     const int n_chunks = sb_cnt * 9;                  /* 16-byte chunks in this wave's slice of a row */
     const int loads_per_row = (n_chunks + 63) >> 6;   /* wave-uniform: 1, 2 or 3 */
 
-    const int row0 = blockIdx.x * rows_per_wg; /* first real row of this workgroup */
+    const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
+    const int row0 = blockIdx.x * rows_per_wg; /* first row of this workgroup */
     int rows_here = n_rows - row0;
     if (rows_here > rows_per_wg) rows_here = rows_per_wg;
-    const int n_vrows = rows_here * n_slices; /* (row, slice) pairs of this workgroup */
+    const int n_lrows = rows_here * n_mats_here;  /* local rows */
+    const int n_vrows = n_lrows * n_slices;       /* (local row, slice) pairs of this workgroup */
 
     /* this wave's virtual rows: wv, wv + 16, ... ; virtual row j = (row j / S, slice j % S), and
      * 16 % S == 0 keeps the slice of a wave fixed. my_rows of them, numbered i = 0.. */
     const int my_rows = wv < n_vrows ? (n_vrows - wv + kWaves - 1) / kWaves : 0;
-    const uint8_t *slice_base = W + (size_t)row0 * row_bytes + (size_t)sb0 * 144;
+    /* where local row lr lives: matrix and row */
+    auto locate = [&](int lr, const uint8_t *&Wm, float *&ym, int &r) {
+        if (paired) {
+            const bool second = lr >= rows_here;
+            Wm = second ? job.W1 : job.W0;
+            ym = job.y0;
+            r = row0 + (second ? lr - rows_here : lr);
+        } else {
+            job_locate(job, row0 + lr, Wm, ym, r);
+        }
+    };
     uint8_t *my_images = images + wv * (depth * kRowImage);
     const uint32_t my_images_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)my_images;
     /* Row i of this wave -> image slot i % depth; exactly loads_per_row instructions are issued.
@@ -119,7 +135,11 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
      * Nothing else in this kernel uses M0. */
     auto issue = [&](int i) {
         const int j = wv + i * kWaves;
-        const uint4 *g = reinterpret_cast<const uint4 *>(slice_base + (size_t)(j / n_slices) * row_bytes);
+        const uint8_t *Wm;
+        float *ym;
+        int r;
+        locate(j / n_slices, Wm, ym, r);
+        const uint4 *g = reinterpret_cast<const uint4 *>(Wm + (size_t)r * row_bytes + (size_t)sb0 * 144);
         const uint32_t img = __builtin_amdgcn_readfirstlane(my_images_lds + (uint32_t)((i % depth) * kRowImage));
 #define QLIN_LOAD_TO_LDS(chunk0)                                                                          \
         if ((chunk0) + lane < n_chunks)                                                                   \
@@ -254,30 +274,45 @@ gemv_q4k_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, floa
     }
     __syncthreads();
 
-    /* combine the slices of each row */
-    for (int r = threadIdx.x; r < rows_here; r += kThreads) {
+    /* combine the slices of each row and store */
+    auto row_total = [&](int lr) {
         float s = 0.0f;
-        for (int k = 0; k < n_slices; k++) s += partial[r * n_slices + k];
-        y[row0 + r] = s;
+        for (int k = 0; k < n_slices; k++) s += partial[lr * n_slices + k];
+        return s;
+    };
+    if (paired) {
+        for (int lr = threadIdx.x; lr < rows_here; lr += kThreads)
+            job.y0[row0 + lr] = silu_times(row_total(lr), row_total(rows_here + lr));
+    } else {
+        for (int lr = threadIdx.x; lr < n_lrows; lr += kThreads) {
+            const uint8_t *Wm;
+            float *ym;
+            int r;
+            locate(lr, Wm, ym, r);
+            const float s = row_total(lr);
+            ym[r] = job.mode == 1 ? ym[r] + s : s;
+        }
     }
 
 }
 
 /* Launch geometry: one 16-wave workgroup per block of rows, sized so that the grid covers the
  * compute units once (more workgroups only when a block would exceed kMaxRowsPerWg rows). */
-hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, int n_cols,
-                           hipStream_t stream, int n_cu) {
+hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu) {
     static bool lds_raised = false;
     const int n_sb = n_cols / 256;
     if (n_sb > 64 || n_sb < 1) return hipErrorInvalidValue;
     const int n_slices = n_sb <= 16 ? 1 : n_sb <= 32 ? 2 : 4;
     const int slice_sb = (n_sb + n_slices - 1) / n_slices;
+    const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
+    const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
+    if (n_rows == 0) return hipSuccess;
     int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
     if (rows_per_wg < 1) rows_per_wg = 1;
-    if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
+    if (rows_per_wg * n_mats_here > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / n_mats_here;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t fixed_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 +
-                               (size_t)((rows_per_wg * n_slices + 3) & ~3) * 4 + (size_t)n_sb * 256 * 4;
+                               (size_t)((rows_per_wg * n_mats_here * n_slices + 3) & ~3) * 4 + (size_t)n_sb * 256 * 4;
     if (fixed_bytes + (size_t)kWaves * kRowImage > 160 * 1024) return hipErrorInvalidValue;
     int depth = (int)((160 * 1024 - fixed_bytes) / ((size_t)kWaves * kRowImage));
     if (depth > kMaxDepth) depth = kMaxDepth;
@@ -288,8 +323,9 @@ hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, 
         if (e != hipSuccess) return e;
         lds_raised = true;
     }
-    hipLaunchKernelGGL(gemv_q4k_kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, (const uint8_t *)W, x, y,
-                       n_rows, n_sb, n_slices, slice_sb, rows_per_wg, depth);
+    const JobView view = job_view(job);
+    hipLaunchKernelGGL(gemv_q4k_kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, view, x, n_sb, n_slices,
+                       slice_sb, rows_per_wg, depth);
     return hipGetLastError();
 }
 

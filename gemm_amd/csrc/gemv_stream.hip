@@ -422,8 +422,8 @@ QLIN_GRID(T_IQ1_M, qlin_iq1s_grid, true)
 
 template <uint32_t T>
 __global__ void __launch_bounds__(1024)
-gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, float *__restrict__ y,
-                   int n_rows, int n_cols, int row_bytes, int image_bytes, int depth, int rows_per_wg) {
+gemv_stream_kernel(const JobView job, const float *__restrict__ x, int n_cols, int row_bytes, int image_bytes,
+                   int depth, int rows_per_wg) {
     using C = Codec<T>;
     constexpr int GPB = C::BE / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -437,22 +437,38 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* wave-uniform, and the compiler is told so */
     const int n_waves = blockDim.x >> 6, n_threads = blockDim.x;
+    /* a workgroup owns rows_per_wg rows of the concatenated matrices; where two results are
+     * combined (mode 2) a wave takes row r of the first matrix, then row r of the second */
+    const bool paired = job.mode == 2;
+    const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
     const int row0 = blockIdx.x * rows_per_wg;
     int rows_here = n_rows - row0;
     if (rows_here > rows_per_wg) rows_here = rows_per_wg;
-    const int my_rows = wv < rows_here ? (rows_here - wv + n_waves - 1) / n_waves : 0;
+    const int my_rows = (wv < rows_here ? (rows_here - wv + n_waves - 1) / n_waves : 0) * (paired ? 2 : 1);
+    auto locate = [&](int i, const uint8_t *&Wm, float *&ym, int &r) {
+        if (paired) {
+            Wm = (i & 1) ? job.W1 : job.W0;
+            ym = job.y0;
+            r = row0 + wv + (i >> 1) * n_waves;
+        } else {
+            job_locate(job, row0 + wv + i * n_waves, Wm, ym, r);
+        }
+    };
     const int n_chunks = row_bytes >> 4;
     const int loads_per_row = (n_chunks + 63) >> 6;
 
     uint8_t *my_images = images + (size_t)wv * depth * image_bytes;
     const uint32_t my_images_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)my_images;
-    const uint8_t *wg_base = W + (size_t)row0 * row_bytes;
     /* Row i of this wave -> image i % depth. The loads are written as instructions: the data goes
      * to LDS at M0 + 16*lane, no register is held while it is in flight, and the compiler (which
      * would wait for every outstanding one of them before any LDS access) does not see them; the
      * waits are placed by hand below. Nothing else in this kernel uses M0. */
     auto issue = [&](int i) {
-        const uint4 *g = reinterpret_cast<const uint4 *>(wg_base + (size_t)(wv + i * n_waves) * row_bytes);
+        const uint8_t *Wm;
+        float *ym;
+        int r;
+        locate(i, Wm, ym, r);
+        const uint4 *g = reinterpret_cast<const uint4 *>(Wm + (size_t)r * row_bytes);
         const uint32_t img = my_images_lds + (uint32_t)((i % depth) * image_bytes);
         for (int c0 = 0; c0 < n_chunks; c0 += 64) {
             const uint32_t m0v = __builtin_amdgcn_readfirstlane(img + 16u * (uint32_t)c0);
@@ -504,6 +520,7 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
     static_assert(64 % GPB == 0, "a wave covers whole blocks");
     const int n_blocks = n_cols / C::BE;
     const int k0 = (lane % GPB) * 8, blk_first = lane / GPB;
+    float gate_value = 0.0f;
     for (int i = 0; i < my_rows; i++) {
         /* rows i .. issued-1 are in flight, row i the oldest */
         wait_vm_at_most((issued - i - 1) * loads_per_row);
@@ -523,16 +540,33 @@ gemv_stream_kernel(const uint8_t *__restrict__ W, const float *__restrict__ x, f
             issued++;
         }
         const float s = wave_sum(acc);
-        if (lane == 0) y[row0 + wv + i * n_waves] = s;
+        const uint8_t *Wm;
+        float *ym;
+        int r;
+        locate(i, Wm, ym, r);
+        if (paired) {
+            if (i & 1) {
+                if (lane == 0) ym[r] = silu_times(gate_value, s);
+            } else {
+                gate_value = s;
+            }
+        } else if (lane == 0) {
+            /* the add is sent as a memory-side atomic: a read of y here would make the wave wait for
+             * the row loads it has in flight */
+            if (job.mode == 1) unsafeAtomicAdd(ym + r, s);
+            else ym[r] = s;
+        }
     }
 }
 
 template <uint32_t T>
-bool stream_typed(const void *W, const float *x, float *y, int n_rows, int n_cols, int n_cu, hipStream_t stream,
-                  hipError_t *err) {
+bool stream_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err) {
     const size_t row_bytes = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
     if (n_cols > 16384 || (n_cols & 31) || (row_bytes & 15) || row_bytes > 8192) return false;
-    if (((uintptr_t)W & 15) || ((uintptr_t)x & 15)) return false;
+    for (int m = 0; m < job.n_mat; m++)
+        if ((uintptr_t)job.W[m] & 15) return false;
+    if ((uintptr_t)x & 15) return false;
+    const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     const size_t x_bytes = (size_t)n_cols * 4 + (size_t)(n_cols >> 3) * 4 + (size_t)Grid<T>::kBytes;
     const size_t lds_cap = 160 * 1024 - 16;
     /* 16 waves with two images each if that fits, else one image, else 8 waves */
@@ -553,19 +587,20 @@ bool stream_typed(const void *W, const float *x, float *y, int n_rows, int n_col
         if (*err != hipSuccess) return true;
         raised = true;
     }
-    hipLaunchKernelGGL((gemv_stream_kernel<T>), dim3(grid), dim3(waves * 64), lds_bytes, stream, (const uint8_t *)W,
-                       x, y, n_rows, n_cols, (int)row_bytes, (int)row_bytes, depth, rows_per_wg);
+    const JobView view = job_view(job);
+    hipLaunchKernelGGL((gemv_stream_kernel<T>), dim3(grid), dim3(waves * 64), lds_bytes, stream, view, x, n_cols,
+                       (int)row_bytes, (int)row_bytes, depth, rows_per_wg);
     *err = hipGetLastError();
     return true;
 }
 
 }  // namespace
 
-bool launch_gemv_stream(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, int n_cu,
+bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
                         hipStream_t stream, hipError_t *err) {
     *err = hipSuccess;
     switch (type) {
-#define QLIN_CASE(TT) case TT: return stream_typed<TT>(W, x, y, n_rows, n_cols, n_cu, stream, err);
+#define QLIN_CASE(TT) case TT: return stream_typed<TT>(job, x, n_cols, n_cu, stream, err);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
 #undef QLIN_CASE
     default: return false;

@@ -139,15 +139,19 @@ int weights_on_device_locked(const void *host, size_t bytes, DevBuf &buf, const 
 
 /* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the streaming kernel,
  * else (ragged or oversized shapes, unaligned pointers) the plain kernel */
+hipError_t dispatch_gemv_job(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t s) {
+    if ((job.mode == kSiluMul ? job.n_rows[0] : job.total_rows()) == 0) return hipSuccess;
+    bool w_aligned = true;
+    for (int m = 0; m < job.n_mat; m++) w_aligned = w_aligned && aligned(job.W[m], 16);
+    if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && w_aligned && aligned(x, 16))
+        return launch_gemv_q4k(job, x, n_cols, s, g.n_cu);
+    hipError_t err;
+    if (launch_gemv_stream(type, job, x, n_cols, g.n_cu, s, &err)) return err;
+    return launch_gemv_generic(type, job, x, n_cols, s);
+}
 hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y, int n_rows,
                          int n_cols, hipStream_t s) {
-    if (n_rows == 0) return hipSuccess;
-    if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && aligned(W, 16) && aligned(x, 16)) {
-        return launch_gemv_q4k(W, x, y, n_rows, n_cols, s, g.n_cu);
-    }
-    hipError_t err;
-    if (launch_gemv_stream(type, W, x, y, n_rows, n_cols, g.n_cu, s, &err)) return err;
-    return launch_gemv_generic(type, W, x, y, n_rows, n_cols, s);
+    return dispatch_gemv_job(type, single_job(W, y, n_rows), x, n_cols, s);
 }
 
 int check_linear_shape(uint32_t type, int n_rows, int n_cols) {
@@ -171,6 +175,43 @@ int matvec_host_locked(float *dst, const void *W, uint32_t type, int n_cols, con
     if (int rc = g.y[slot].ensure((size_t)n_rows * 4 + 16)) return rc;
     HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)g.y[slot].p, n_rows, n_cols, g.stream));
     HIP_TRY(hipMemcpyAsync(dst, g.y[slot].p, (size_t)n_rows * 4, hipMemcpyDeviceToHost, g.stream));
+    return QLIN_OK;
+}
+
+/* up to three matrices against one x (host pointers). Matrices of one type go out as ONE launch;
+ * otherwise one launch per matrix, with the SiLU product as a separate pass. dst[m] receives
+ * n_rows[m] floats (mode kSiluMul: dst[0] only; mode kAdd: dst[m] is read first). */
+int matvec_multi_host_locked(int n_mat, float *const dst[3], const void *const W[3], const uint32_t types[3],
+                             const int n_rows[3], int n_cols, const float *x, int mode) {
+    if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
+    HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_cols * 4, hipMemcpyHostToDevice, g.stream));
+    const void *dW[3] = {nullptr, nullptr, nullptr};
+    bool same = true;
+    for (int m = 0; m < n_mat; m++) {
+        if (n_rows[m] == 0) continue;
+        if (int rc = weights_on_device_locked(W[m], row_size(types[m], n_cols) * (size_t)n_rows[m], g.w[m], &dW[m])) return rc;
+        if (int rc = g.y[m].ensure((size_t)n_rows[m] * 4 + 16)) return rc;
+        same = same && types[m] == types[0];
+    }
+    if (mode == kAdd)
+        for (int m = 0; m < n_mat; m++)
+            if (n_rows[m]) HIP_TRY(hipMemcpyAsync(g.y[m].p, dst[m], (size_t)n_rows[m] * 4, hipMemcpyHostToDevice, g.stream));
+    const float *dx = (const float *)g.x.p;
+    if (same && n_rows[0] > 0) {
+        GemvJob job = {{dW[0], dW[1], dW[2]}, {(float *)g.y[0].p, (float *)g.y[1].p, (float *)g.y[2].p},
+                       {n_rows[0], n_rows[1], n_rows[2]}, n_mat, mode};
+        HIP_TRY(dispatch_gemv_job(types[0], job, dx, n_cols, g.stream));
+    } else {
+        for (int m = 0; m < n_mat; m++)
+            if (n_rows[m])
+                HIP_TRY(dispatch_gemv_job(types[m], single_job(dW[m], (float *)g.y[m].p, n_rows[m], mode == kAdd ? kAdd : kStore),
+                                          dx, n_cols, g.stream));
+        if (mode == kSiluMul)
+            HIP_TRY(launch_silu_mul((float *)g.y[0].p, (const float *)g.y[0].p, (const float *)g.y[1].p, n_rows[0], g.stream));
+    }
+    const int n_out = mode == kSiluMul ? 1 : n_mat;
+    for (int m = 0; m < n_out; m++)
+        if (n_rows[m]) HIP_TRY(hipMemcpyAsync(dst[m], g.y[m].p, (size_t)n_rows[m] * 4, hipMemcpyDeviceToHost, g.stream));
     return QLIN_OK;
 }
 
@@ -344,8 +385,11 @@ int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2,
     if (!dst1 || !dst2 || !W1 || !W2 || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;
-    if (int rc = matvec_host_locked(dst1, W1, type1, n_cols, x, n_rows, 0, true)) return rc;
-    if (int rc = matvec_host_locked(dst2, W2, type2, n_cols, x, n_rows, 1, false)) return rc;
+    const void *W[3] = {W1, W2, nullptr};
+    const uint32_t types[3] = {type1, type2, 0};
+    float *dst[3] = {dst1, dst2, nullptr};
+    const int rows[3] = {n_rows, n_rows, 0};
+    if (int rc = matvec_multi_host_locked(2, dst, W, types, rows, n_cols, x, kStore)) return rc;
     HIP_TRY(hipStreamSynchronize(g.stream));
     return QLIN_OK;
 }
@@ -357,15 +401,72 @@ int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k
     if (int rc = check_linear_shape(type_k, n_kv, n_cols)) return rc;
     if (int rc = check_linear_shape(type_v, n_kv, n_cols)) return rc;
     if (!x || (n_q && (!q || !Wq)) || (n_kv && (!k || !Wk || !v || !Wv))) return fail(QLIN_ERR_ARG, "null pointer");
+    if (n_q == 0 && n_kv == 0) return QLIN_OK;
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;
-    bool up = true;
-    if (n_q) { if (int rc = matvec_host_locked(q, Wq, type_q, n_cols, x, n_q, 0, up)) return rc; up = false; }
-    if (n_kv) {
-        if (int rc = matvec_host_locked(k, Wk, type_k, n_cols, x, n_kv, 1, up)) return rc;
-        if (int rc = matvec_host_locked(v, Wv, type_v, n_cols, x, n_kv, 2, false)) return rc;
-    }
+    const void *W[3] = {Wq, Wk, Wv};
+    const uint32_t types[3] = {type_q, type_k, type_v};
+    float *dst[3] = {q, k, v};
+    const int rows[3] = {n_q, n_kv, n_kv};
+    if (int rc = matvec_multi_host_locked(3, dst, W, types, rows, n_cols, x, kStore)) return rc;
     HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_matvec_silu_mul(float *dst, const void *Wgate, uint32_t type_gate, const void *Wup, uint32_t type_up,
+                         int n_cols, const float *x, int n_rows) {
+    if (int rc = check_linear_shape(type_gate, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type_up, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!dst || !Wgate || !Wup || !x) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const void *W[3] = {Wgate, Wup, nullptr};
+    const uint32_t types[3] = {type_gate, type_up, 0};
+    float *out[3] = {dst, nullptr, nullptr};
+    const int rows[3] = {n_rows, n_rows, 0};
+    if (int rc = matvec_multi_host_locked(2, out, W, types, rows, n_cols, x, kSiluMul)) return rc;
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_matvec_add(float *dst, const void *W, uint32_t type, int n_cols, const float *x, int n_rows) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!dst || !W || !x) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const void *Wm[3] = {W, nullptr, nullptr};
+    const uint32_t types[3] = {type, 0, 0};
+    float *out[3] = {dst, nullptr, nullptr};
+    const int rows[3] = {n_rows, 0, 0};
+    if (int rc = matvec_multi_host_locked(1, out, Wm, types, rows, n_cols, x, kAdd)) return rc;
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_matvec_argmax(int *index, float *value, float *logits, const void *W, uint32_t type, int n_cols,
+                       const float *x, int n_rows) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return fail(QLIN_ERR_ARG, "argmax over no rows");
+    if (!index || !W || !x) return fail(QLIN_ERR_ARG, "null pointer");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const size_t rb = row_size(type, n_cols);
+    const void *dW;
+    if (int rc = weights_on_device_locked(W, rb * (size_t)n_rows, g.w[0], &dW)) return rc;
+    if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
+    HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_cols * 4, hipMemcpyHostToDevice, g.stream));
+    if (int rc = g.y[0].ensure((size_t)n_rows * 4 + 16)) return rc;
+    if (int rc = g.tmp[0].ensure(QLIN_ARGMAX_RESULT_BYTES)) return rc;
+    HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)g.y[0].p, n_rows, n_cols, g.stream));
+    HIP_TRY(launch_argmax((const float *)g.y[0].p, n_rows, (float *)g.tmp[0].p, g.stream));
+    float res[2];
+    HIP_TRY(hipMemcpyAsync(res, g.tmp[0].p, 8, hipMemcpyDeviceToHost, g.stream));
+    if (logits) HIP_TRY(hipMemcpyAsync(logits, g.y[0].p, (size_t)n_rows * 4, hipMemcpyDeviceToHost, g.stream));
+    HIP_TRY(hipStreamSynchronize(g.stream));
+    memcpy(index, &res[0], 4);
+    if (value) *value = res[1];
     return QLIN_OK;
 }
 
@@ -515,6 +616,67 @@ int qlin_gemv_dev(uint32_t type, const void *W, const float *x, float *y, int n_
         if (int rc = ensure_init_locked(0)) return rc;
     }
     HIP_TRY(dispatch_gemv(type, W, x, y, n_rows, n_cols, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+namespace {
+int check_dev_gemv(uint32_t type, int n_rows, int n_cols, const void *W, const float *x, const float *y) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!W || !x || !y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 2) || !aligned(x, 16) || !aligned(y, 4))
+        return fail(QLIN_ERR_ARG, "W needs 2-byte, x 16-byte, y 4-byte alignment");
+    return QLIN_OK;
+}
+int init_once() {
+    std::lock_guard<std::mutex> lk(g.mu);
+    return ensure_init_locked(0);
+}
+}  // namespace
+
+int qlin_gemv_add_dev(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, void *stream) {
+    if (int rc = check_dev_gemv(type, n_rows, n_cols, W, x, y)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (int rc = init_once()) return rc;
+    HIP_TRY(dispatch_gemv_job(type, single_job(W, y, n_rows, kAdd), x, n_cols, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_gemv_silu_mul_dev(uint32_t type, const void *Wgate, const void *Wup, const float *x, float *out,
+                           int n_rows, int n_cols, void *stream) {
+    if (int rc = check_dev_gemv(type, n_rows, n_cols, Wgate, x, out)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!Wup || !aligned(Wup, 2)) return fail(QLIN_ERR_ARG, "null or misaligned up matrix");
+    if (int rc = init_once()) return rc;
+    GemvJob job = {{Wgate, Wup, nullptr}, {out, nullptr, nullptr}, {n_rows, n_rows, 0}, 2, kSiluMul};
+    HIP_TRY(dispatch_gemv_job(type, job, x, n_cols, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_gemv_multi_dev(uint32_t type, int n_mat, const void *const *W, float *const *y, const int *n_rows,
+                        const float *x, int n_cols, void *stream) {
+    if (n_mat < 1 || n_mat > 3 || !W || !y || !n_rows) return fail(QLIN_ERR_ARG, "1 to 3 matrices");
+    GemvJob job = {{nullptr, nullptr, nullptr}, {nullptr, nullptr, nullptr}, {0, 0, 0}, n_mat, kStore};
+    for (int m = 0; m < n_mat; m++) {
+        if (int rc = check_dev_gemv(type, n_rows[m], n_cols, W[m], x, y[m])) return rc;
+        job.W[m] = W[m];
+        job.y[m] = y[m];
+        job.n_rows[m] = n_rows[m];
+    }
+    if (job.total_rows() == 0) return QLIN_OK;
+    if (int rc = init_once()) return rc;
+    HIP_TRY(dispatch_gemv_job(type, job, x, n_cols, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_gemv_argmax_dev(uint32_t type, const void *W, const float *x, float *logits, void *result, int n_rows,
+                         int n_cols, void *stream) {
+    if (int rc = check_dev_gemv(type, n_rows, n_cols, W, x, logits)) return rc;
+    if (n_rows == 0) return fail(QLIN_ERR_ARG, "argmax over no rows");
+    if (!result || !aligned(result, 8)) return fail(QLIN_ERR_ARG, "result needs QLIN_ARGMAX_RESULT_BYTES bytes, 8-byte aligned");
+    if (int rc = init_once()) return rc;
+    HIP_TRY(dispatch_gemv(type, W, x, logits, n_rows, n_cols, (hipStream_t)stream));
+    HIP_TRY(launch_argmax(logits, n_rows, (float *)result, (hipStream_t)stream));
     return QLIN_OK;
 }
 

@@ -267,6 +267,23 @@ __device__ __forceinline__ void wait_vm_at_most(int n) {
     }
 }
 
+/* Kernel-side view of one fused matvec launch: up to three matrices of one block type that share
+ * x (host-side GemvJob, flattened so that nothing is indexed dynamically). mode 0: y = W.x,
+ * 1: y += W.x, 2: y0 = silu(W0.x) * (W1.x) with n0 == n1. */
+struct JobView {
+    const uint8_t *W0, *W1, *W2;
+    float *y0, *y1, *y2;
+    int n0, n1, n2;
+    int mode;
+};
+/* matrix and row of virtual row v, the rows of the matrices taken one after the other */
+__device__ __forceinline__ void job_locate(const JobView &j, int v, const uint8_t *&W, float *&y, int &r) {
+    if (v < j.n0) { W = j.W0; y = j.y0; r = v; }
+    else if (v < j.n0 + j.n1) { W = j.W1; y = j.y1; r = v - j.n0; }
+    else { W = j.W2; y = j.y2; r = v - j.n0 - j.n1; }
+}
+__device__ __forceinline__ float silu_times(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+
 /* wave64 sum: every lane ends up with the total */
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -10,6 +10,8 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include "qlin_device.h"
+
 namespace qlin {
 
 /* out[n_rows, n_cols] = decode(W); n_cols may be ragged: only n_cols / block_elems blocks per
@@ -17,16 +19,42 @@ namespace qlin {
 hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, int n_cols,
                           size_t row_bytes, hipStream_t stream);
 
-/* y[n_rows] = W . x, any supported type and any whole-block shape */
-hipError_t launch_gemv_generic(uint32_t type, const void *W, const float *x, float *y, int n_rows,
-                               int n_cols, hipStream_t stream);
+/* One matvec launch over up to three matrices of ONE block type that share x and n_cols: the
+ * fused call shapes of the reference's decode loop.
+ *   kStore    y_m[r] = W_m[r,:] . x for every matrix m (rows of the matrices are concatenated:
+ *             tf_qmatvec_fused2_pool, tf_qmatvec_fused_qkv_pool, common/transformer.h:897, :1021)
+ *   kAdd      y_m[r] += W_m[r,:] . x   (projection followed by the residual add, :4037)
+ *   kSiluMul  two matrices of equal row count: y_0[r] = silu(W_0[r,:].x) * (W_1[r,:].x)
+ *             (tf_qmatvec_fused2_silu_pool, :953; silu(g) = g / (1 + exp(-g))) */
+enum GemvMode : int { kStore = 0, kAdd = 1, kSiluMul = 2 };
+struct GemvJob {
+    const void *W[3];
+    float *y[3];
+    int n_rows[3];
+    int n_mat;   /* 1..3; kSiluMul: 2 */
+    int mode;    /* GemvMode */
+    int total_rows() const { return n_rows[0] + (n_mat > 1 ? n_rows[1] : 0) + (n_mat > 2 ? n_rows[2] : 0); }
+};
+inline GemvJob single_job(const void *W, float *y, int n_rows, int mode = kStore) {
+    GemvJob j = {{W, nullptr, nullptr}, {y, nullptr, nullptr}, {n_rows, 0, 0}, 1, mode};
+    return j;
+}
+
+inline JobView job_view(const GemvJob &job) {
+    const JobView v = {(const uint8_t *)job.W[0], (const uint8_t *)job.W[1], (const uint8_t *)job.W[2],
+                       job.y[0], job.y[1], job.y[2],
+                       job.n_rows[0], job.n_mat > 1 ? job.n_rows[1] : 0, job.n_mat > 2 ? job.n_rows[2] : 0, job.mode};
+    return v;
+}
+
+/* one job: y[n_rows] = W . x (or the fused forms above), any supported type and any whole-block shape */
+hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t stream);
 /* streaming matvec for every type; returns false if the shape rules of gemv_stream.hip do not
  * hold (nothing was launched), else true with the launch status in *err */
-bool launch_gemv_stream(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, int n_cu,
+bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
                         hipStream_t stream, hipError_t *err);
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
-hipError_t launch_gemv_q4k(const void *W, const float *x, float *y, int n_rows, int n_cols,
-                           hipStream_t stream, int n_cu);
+hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu);
 
 /* Y[t*ldy + r] = dot(W[r,:], X[t*ldx..]) in fp32 */
 hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *Y, int n_rows,
@@ -46,6 +74,10 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
 hipError_t launch_moe_route(const float *logits, int n_tok, int n_expert, int top_k, int32_t *idx,
                             float *w, hipStream_t stream);
 hipError_t launch_silu_mul(float *h, const float *gate, const float *up, int n, hipStream_t stream);
+/* result[0] = index (as int32 bits) of the first largest of v[0..n), result[1] = that value: the
+ * loop `if (v[j] > v[best]) best = j` (server/server_llm.c:224-228). result holds
+ * QLIN_ARGMAX_RESULT_BYTES bytes: the rest is scratch for the first stage. */
+hipError_t launch_argmax(const float *v, int n, float *result, hipStream_t stream);
 hipError_t launch_axpy_dev_weight(float *out, const float *q, const float *w, int widx, int n,
                                   int overwrite, hipStream_t stream);
 

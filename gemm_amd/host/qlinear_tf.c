@@ -80,6 +80,29 @@ void qtf_qmatvec_fused2_pool(const float *x, float *dst1, const qtensor *mat1, f
     }
 }
 
+void qtf_qmatvec_fused2_silu_pool(const float *x, float *dst, const qtensor *gate_mat, const qtensor *up_mat,
+                                  int n_rows) {
+    if (qlin_matvec_silu_mul(dst, gate_mat->data, gate_mat->type, up_mat->data, up_mat->type, gate_mat->n_cols, x,
+                             n_rows) != QLIN_OK) {
+        complain("qmatvec_fused2_silu");
+        zero_fill(dst, (size_t)n_rows);
+    }
+}
+
+void qtf_qmatvec_add(const float *x, float *dst, const qtensor *mat, int n_rows) {
+    /* on failure the residual stream is left as it was */
+    if (qlin_matvec_add(dst, mat->data, mat->type, mat->n_cols, x, n_rows) != QLIN_OK) complain("qmatvec_add");
+}
+
+int qtf_logits_argmax(const float *x, const qtensor *output, int n_vocab, float *logits) {
+    int index = -1;
+    if (qlin_matvec_argmax(&index, NULL, logits, output->data, output->type, output->n_cols, x, n_vocab) != QLIN_OK) {
+        complain("logits_argmax");
+        return -1;
+    }
+    return index;
+}
+
 void qtf_qmatvec_fused_qkv_pool(const float *x, float *q, const qtensor *mat_q, int n_q, float *k,
                                 const qtensor *mat_k, float *v, const qtensor *mat_v, int n_kv) {
     if (qlin_matvec_qkv(q, mat_q->data, mat_q->type, n_q, k, mat_k->data, mat_k->type, v, mat_v->data, mat_v->type,

@@ -58,6 +58,9 @@ SIGNATURES = {
     "qlin_matvec_qkv": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, _vp, C.c_uint32, _vp, _vp, C.c_uint32,
                                   C.c_int, C.c_int, _vp]),
     "qlin_matvec_expert": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, C.c_int, _vp, C.c_int]),
+    "qlin_matvec_silu_mul": (C.c_int, [_vp, _vp, C.c_uint32, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
+    "qlin_matvec_add": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
+    "qlin_matvec_argmax": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
     "qlin_gemm_tokenmajor": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "qlin_moe_ffn_token": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp]),
     "qlin_dev_alloc": (_vp, [C.c_size_t]),
@@ -67,6 +70,10 @@ SIGNATURES = {
     "qlin_dev_sync": (C.c_int, [_vp]),
     "qlin_dequant_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemv_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "qlin_gemv_add_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "qlin_gemv_silu_mul_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "qlin_gemv_multi_dev": (C.c_int, [C.c_uint32, C.c_int, _vp, _vp, _vp, _vp, C.c_int, _vp]),
+    "qlin_gemv_argmax_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemm_bf16_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp]),
     "qlin_gemm_f32_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp]),
     "qlin_moe_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
@@ -191,6 +198,60 @@ def gemm_tokenmajor(type_id, W, X, n_cols):
 
 def gemv_dev(type_id, dW, dx, dy, n_rows, n_cols, stream=None):
     check(load().qlin_gemv_dev(type_id, dW.ptr, dx.ptr, dy.ptr, n_rows, n_cols, stream))
+
+
+def gemv_add_dev(type_id, dW, dx, dy, n_rows, n_cols, stream=None):
+    check(load().qlin_gemv_add_dev(type_id, dW.ptr, dx.ptr, dy.ptr, n_rows, n_cols, stream))
+
+
+def gemv_silu_mul_dev(type_id, dWgate, dWup, dx, dout, n_rows, n_cols, stream=None):
+    check(load().qlin_gemv_silu_mul_dev(type_id, dWgate.ptr, dWup.ptr, dx.ptr, dout.ptr, n_rows, n_cols, stream))
+
+
+def gemv_multi_dev(type_id, dWs, dys, n_rows, dx, n_cols, stream=None):
+    """dWs, dys: lists of 1..3 DevBuf; n_rows: list of ints"""
+    n = len(dWs)
+    Wp = (C.c_void_p * n)(*[d.ptr for d in dWs])
+    yp = (C.c_void_p * n)(*[d.ptr for d in dys])
+    rows = (C.c_int * n)(*n_rows)
+    check(load().qlin_gemv_multi_dev(type_id, n, C.addressof(Wp), C.addressof(yp), C.addressof(rows), dx.ptr, n_cols,
+                                     stream))
+
+
+ARGMAX_RESULT_BYTES = 2056  # QLIN_ARGMAX_RESULT_BYTES of include/qlinear.h
+
+
+def gemv_argmax_dev(type_id, dW, dx, dlogits, dresult, n_rows, n_cols, stream=None):
+    check(load().qlin_gemv_argmax_dev(type_id, dW.ptr, dx.ptr, dlogits.ptr, dresult.ptr, n_rows, n_cols, stream))
+
+
+def matvec_silu_mul(type_gate, Wgate, type_up, Wup, x, n_cols):
+    Wgate, Wup = np.ascontiguousarray(Wgate, np.uint8), np.ascontiguousarray(Wup, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.zeros(Wgate.shape[0], np.float32)
+    check(load().qlin_matvec_silu_mul(_ptr(y), _ptr(Wgate), type_gate, _ptr(Wup), type_up, n_cols, _ptr(x),
+                                      Wgate.shape[0]))
+    return y
+
+
+def matvec_add(type_id, W, x, n_cols, residual):
+    W = np.ascontiguousarray(W, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.array(residual, dtype=np.float32, copy=True)
+    check(load().qlin_matvec_add(_ptr(y), _ptr(W), type_id, n_cols, _ptr(x), W.shape[0]))
+    return y
+
+
+def matvec_argmax(type_id, W, x, n_cols, want_logits=False):
+    """-> (index, value, logits or None)"""
+    W = np.ascontiguousarray(W, np.uint8)
+    x = np.ascontiguousarray(x, np.float32)
+    idx = np.zeros(1, np.int32)
+    val = np.zeros(1, np.float32)
+    logits = np.zeros(W.shape[0], np.float32) if want_logits else None
+    check(load().qlin_matvec_argmax(_ptr(idx), _ptr(val), _ptr(logits) if want_logits else None, _ptr(W), type_id,
+                                    n_cols, _ptr(x), W.shape[0]))
+    return int(idx[0]), float(val[0]), logits
 
 
 def dequant_dev(type_id, dW, dout, n_rows, n_cols, stream=None):

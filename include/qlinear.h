@@ -121,6 +121,20 @@ int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2,
 int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k, const void *Wk,
                     uint32_t type_k, float *v, const void *Wv, uint32_t type_v, int n_kv,
                     int n_cols, const float *x);
+/* dst[r] = silu(Wgate[r,:].x) * (Wup[r,:].x), silu(g) = g / (1 + exp(-g)): gate and up projection
+ * with the activation applied before anything is written
+ *                            tf_qmatvec_fused2_silu_pool, common/transformer.h:953 */
+int qlin_matvec_silu_mul(float *dst, const void *Wgate, uint32_t type_gate, const void *Wup,
+                         uint32_t type_up, int n_cols, const float *x, int n_rows);
+/* dst[r] += W[r,:].x: a projection followed by the residual add
+ *                            tf_qmatvec_pool + tf_vadd, common/transformer.h:4037, :551 */
+int qlin_matvec_add(float *dst, const void *W, uint32_t ggml_type, int n_cols, const float *x, int n_rows);
+/* output projection and greedy pick: *index = first largest of W.x (the loop of
+ * server/server_llm.c:224-228 over transformer_compute_logits, common/transformer.h:4302-4307),
+ * *value = that logit (may be NULL), logits[n_rows] = all of them (may be NULL: then only 8 bytes
+ * come back from the GPU) */
+int qlin_matvec_argmax(int *index, float *value, float *logits, const void *W, uint32_t ggml_type,
+                       int n_cols, const float *x, int n_rows);
 /* one expert of a [n_cols, rows_per_expert, n_expert] tensor: rows start at
  * W + expert * rows_per_expert * row_bytes
  *                            tf_qmatvec_expert(_pool), common/transformer.h:517, :1136 */
@@ -153,6 +167,22 @@ int qlin_dequant_dev(uint32_t ggml_type, const void *W, float *out, int n_rows, 
 /* y[n_rows] = W . x, x fp32 */
 int qlin_gemv_dev(uint32_t ggml_type, const void *W, const float *x, float *y, int n_rows,
                   int n_cols, void *stream);
+/* The fused call shapes of the decode loop, one launch each (all matrices of one ggml type):
+ *   add       y[r] += W[r,:].x                                   (projection + residual)
+ *   silu_mul  out[r] = silu(Wgate[r,:].x) * (Wup[r,:].x)         (common/transformer.h:953)
+ *   multi     y_m = W_m . x for m < n_mat <= 3 matrices sharing x (gate+up :897, Q/K/V :1021)
+ *   argmax    logits = W.x (written, n_rows floats), then result = {int32 index of the first
+ *             largest logit, float value} in the first 8 bytes of `result`, which must hold
+ *             QLIN_ARGMAX_RESULT_BYTES bytes, 8-byte aligned (the rest is scratch for the pick) */
+#define QLIN_ARGMAX_RESULT_BYTES 2056
+int qlin_gemv_add_dev(uint32_t ggml_type, const void *W, const float *x, float *y, int n_rows,
+                      int n_cols, void *stream);
+int qlin_gemv_silu_mul_dev(uint32_t ggml_type, const void *Wgate, const void *Wup, const float *x,
+                           float *out, int n_rows, int n_cols, void *stream);
+int qlin_gemv_multi_dev(uint32_t ggml_type, int n_mat, const void *const *W, float *const *y,
+                        const int *n_rows, const float *x, int n_cols, void *stream);
+int qlin_gemv_argmax_dev(uint32_t ggml_type, const void *W, const float *x, float *logits,
+                         void *result, int n_rows, int n_cols, void *stream);
 /* Y[t*ldy + r] = dot(W[r,:], X[t*ldx ...]); X bf16 (uint16 bit patterns), fp32 accumulate on
  * the matrix cores, Y fp32 token-major. Q4_K only; n_cols % 256 == 0. */
 int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,

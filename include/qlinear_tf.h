@@ -13,7 +13,11 @@
  *   qtf_qmatvec                  tf_qmatvec                    :1049-1114
  *   qtf_qmatvec_pool             tf_qmatvec_pool               :1117-1133
  *   qtf_qmatvec_fused2_pool      tf_qmatvec_fused2_pool        :897-914
+ *   qtf_qmatvec_fused2_silu_pool tf_qmatvec_fused2_silu_pool   :953-970
  *   qtf_qmatvec_fused_qkv_pool   tf_qmatvec_fused_qkv_pool     :1021-1047
+ *   qtf_qmatvec_add              tf_qmatvec_pool + tf_vadd     :4037, :551 (projection + residual)
+ *   qtf_logits_argmax            transformer_compute_logits + the greedy loop of
+ *                                server/server_llm.c:224-228   :4302-4307
  *   qtf_qmatvec_expert           tf_qmatvec_expert             :517-548
  *   qtf_qmatvec_expert_pool      tf_qmatvec_expert_pool        :1136-1158
  *   qtf_gemm_tokenmajor          tf_gemm_f16_mt_tokenmajor     :4487-4595
@@ -62,6 +66,13 @@ void qtf_qmatvec(float *dst, const qtensor *mat, const float *x, int n_rows, flo
 void qtf_qmatvec_pool(const float *x, float *dst, const qtensor *mat, int n_rows);
 void qtf_qmatvec_fused2_pool(const float *x, float *dst1, const qtensor *mat1, float *dst2,
                              const qtensor *mat2, int n_rows);
+/* dst = silu(gate_mat . x) * (up_mat . x) */
+void qtf_qmatvec_fused2_silu_pool(const float *x, float *dst, const qtensor *gate_mat, const qtensor *up_mat,
+                                  int n_rows);
+/* dst += mat . x */
+void qtf_qmatvec_add(const float *x, float *dst, const qtensor *mat, int n_rows);
+/* index of the first largest of output . x (-1 on failure); logits may be NULL */
+int  qtf_logits_argmax(const float *x, const qtensor *output, int n_vocab, float *logits);
 void qtf_qmatvec_fused_qkv_pool(const float *x, float *q, const qtensor *mat_q, int n_q, float *k,
                                 const qtensor *mat_k, float *v, const qtensor *mat_v, int n_kv);
 void qtf_qmatvec_expert(float *dst, const qtensor *mat, int expert, const float *x,
@@ -79,6 +90,7 @@ void qtf_moe_ffn(float *out, const qtensor *gate_exps, const qtensor *up_exps,
 #ifdef QLINEAR_TF_REFERENCE_NAMES
 #define tf_row_bytes                 qtf_row_bytes
 #define tf_is_supported_weight_type  qtf_is_supported_weight_type
+#define tf_qmatvec_fused2_silu_pool(m, dst, gate_mat, up_mat, x, n_rows) qtf_qmatvec_fused2_silu_pool(x, dst, gate_mat, up_mat, n_rows)
 #define tf_dequant_row               qtf_dequant_row
 #define tf_qmatvec                   qtf_qmatvec
 #define tf_qmatvec_expert            qtf_qmatvec_expert

@@ -92,6 +92,37 @@ int main(void) {
     check_rows("fused qkv k (q8_0)", &c8, 0, 96, x, y2);
     check_rows("fused qkv v (q6_K)", &c6, 0, 96, x, y3);
 
+    /* gate+up+SiLU, projection+residual, output projection + greedy pick */
+    {
+        float g[256], u[256], want[256];
+        tf_qmatvec(g, &a, x, 256, NULL);
+        tf_qmatvec(u, &b, x, 256, NULL);
+        tf_qmatvec_fused2_silu_pool(NULL, y, &a, &b, x, 256);
+        double num = 0, den = 0;
+        for (int i = 0; i < 256; i++) {
+            want[i] = (float)((double)g[i] / (1.0 + exp(-(double)g[i])) * (double)u[i]);
+            num += ((double)y[i] - want[i]) * ((double)y[i] - want[i]);
+            den += (double)want[i] * want[i];
+        }
+        printf("%-28s rel-L2 %.3e %s\n", "fused2 silu", sqrt(num / den), sqrt(num / den) <= 1e-5 ? "ok" : "FAIL");
+        if (!(sqrt(num / den) <= 1e-5)) failures++;
+        for (int i = 0; i < 256; i++) y2[i] = 0.25f * (float)i;
+        qtf_qmatvec_add(x, y2, &a, 256);
+        num = den = 0;
+        for (int i = 0; i < 256; i++) {
+            const double w = 0.25 * i + (double)g[i];
+            num += ((double)y2[i] - w) * ((double)y2[i] - w);
+            den += w * w;
+        }
+        printf("%-28s rel-L2 %.3e %s\n", "projection + residual", sqrt(num / den), sqrt(num / den) <= 1e-5 ? "ok" : "FAIL");
+        if (!(sqrt(num / den) <= 1e-5)) failures++;
+        int best = 0;
+        for (int i = 1; i < 256; i++) if (g[i] > g[best]) best = i;
+        const int got = qtf_logits_argmax(x, &a, 256, y3);
+        printf("%-28s %d vs %d %s\n", "logits argmax", got, best, got == best ? "ok" : "FAIL");
+        if (got != best) failures++;
+    }
+
     tf_qmatvec_expert(y, &a, 3, x, 64, NULL); /* 4 experts of 64 rows */
     check_rows("tf_qmatvec_expert", &a, 192, 64, x, y);
 
