@@ -66,6 +66,54 @@ def time_gemv(type_id, n_rows, n_cols, steps, warmup, min_total_bytes=320 << 20,
     return ms / steps, copies
 
 
+def time_fused(steps):
+    """Q4_K, hidden 4096, FFN 14336, 8 KV heads of 128: one launch per fused call shape against the
+    separate launches it replaces. -> {name: us}"""
+    K, FF = 4096, 14336
+    x = qlinear.DevBuf.from_numpy(synth.make_activation(K, seed=3) * np.float32(0.05))
+    h = qlinear.DevBuf.from_numpy(synth.make_activation(FF, seed=4))
+
+    def copies(rows, cols, n, seed):
+        W = synth.make_weights(Q4K, rows, cols, seed=seed)
+        return [qlinear.DevBuf.from_numpy(W) for _ in range(n)]
+
+    def run(fn, n):
+        for i in range(n):
+            fn(i)
+        qlinear.sync()
+        qlinear.timer_begin()
+        for i in range(steps):
+            fn(i % n)
+        return round(qlinear.timer_end() / steps * 1e3, 2)
+
+    out = {}
+    n = 6
+    Wg, Wu = copies(FF, K, n, 51), copies(FF, K, n, 52)
+    y1, y2 = qlinear.DevBuf(FF * 4), qlinear.DevBuf(FF * 4)
+    out["gate,up: two launches (no activation)"] = run(
+        lambda i: (qlinear.gemv_dev(Q4K, Wg[i], x, y1, FF, K), qlinear.gemv_dev(Q4K, Wu[i], x, y2, FF, K)), n)
+    out["gate+up+silu: one launch"] = run(lambda i: qlinear.gemv_silu_mul_dev(Q4K, Wg[i], Wu[i], x, y1, FF, K), n)
+    for d in Wg + Wu:
+        d.free()
+    n = 24
+    Wq, Wk, Wv = copies(4096, K, n, 53), copies(1024, K, n, 54), copies(1024, K, n, 55)
+    q, k, v = qlinear.DevBuf(4096 * 4), qlinear.DevBuf(1024 * 4), qlinear.DevBuf(1024 * 4)
+    out["q,k,v: three launches"] = run(
+        lambda i: (qlinear.gemv_dev(Q4K, Wq[i], x, q, 4096, K), qlinear.gemv_dev(Q4K, Wk[i], x, k, 1024, K),
+                   qlinear.gemv_dev(Q4K, Wv[i], x, v, 1024, K)), n)
+    out["q,k,v: one launch"] = run(
+        lambda i: qlinear.gemv_multi_dev(Q4K, [Wq[i], Wk[i], Wv[i]], [q, k, v], [4096, 1024, 1024], x, K), n)
+    for d in Wq + Wk + Wv:
+        d.free()
+    n = 12
+    Wd = copies(K, FF, n, 56)
+    out["down 4096x14336"] = run(lambda i: qlinear.gemv_dev(Q4K, Wd[i], h, q, K, FF), n)
+    out["down + residual: one launch"] = run(lambda i: qlinear.gemv_add_dev(Q4K, Wd[i], h, q, K, FF), n)
+    for d in Wd + [x, h, y1, y2, q, k, v]:
+        d.free()
+    return out
+
+
 def time_gemm(n_tok, n_rows, n_cols, steps, warmup):
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=31)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=32, tokens=n_tok))
@@ -236,6 +284,17 @@ def main():
         extra["q4k_prefill_gemm_roofline"] = {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS,
                                               "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),
                                               "traffic": None}
+
+        # every other block format at the headline shape, and the fused call shapes of the decode loop
+        other = {}
+        for tid, tname in synth.TYPE_NAMES.items():
+            if tid == Q4K:
+                continue
+            m, _ = time_gemv(tid, 14336, 4096, max(20, args.steps // 8), 4)
+            b = gemv_bytes(tid, 14336, 4096)
+            other[tname] = {"us": round(m * 1e3, 2), "GB/s": round(b / (m * 1e-3) / 1e9, 1)}
+        extra["gemv_14336x4096_all_formats"] = other
+        extra["q4k_fused_decode_shapes"] = time_fused(max(20, args.steps // 8))
 
         hb = time_host_boundary(n_rows, n_cols)
         extra["host_pointer_matvec_14336x4096"] = {"us": round(hb * 1e3, 1), "GB/s": round(nbytes / (hb * 1e-3) / 1e9, 1),

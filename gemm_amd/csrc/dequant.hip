@@ -13,8 +13,8 @@ namespace qlin {
 
 template <uint32_t T, bool VEC>
 __global__ void __launch_bounds__(256)
-dequant_kernel(const uint8_t *__restrict__ W, float *__restrict__ out, int n_rows, int n_cols,
-               size_t row_bytes, int blocks_per_row) {
+dequant_kernel(const uint8_t *__restrict__ W, const int32_t *__restrict__ row_ids, int n_src_rows,
+               float *__restrict__ out, int n_rows, int n_cols, size_t row_bytes, int blocks_per_row) {
     using C = Codec<T>;
     constexpr int GPB = C::BE / 8; /* 8-element groups per block */
     const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -24,7 +24,15 @@ dequant_kernel(const uint8_t *__restrict__ W, float *__restrict__ out, int n_row
     const int g = (int)(gid - (long long)row * groups_per_row);
     const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
     float y[8];
-    C::decode8(W + (size_t)row * row_bytes + (size_t)blk * C::BB, k0, y);
+    /* output row `row` is source row row_ids[row] when a list is given (embedding lookup); an id
+     * outside the table yields a row of zeros */
+    const int src_row = row_ids ? row_ids[row] : row;
+    if (src_row >= 0 && src_row < n_src_rows) {
+        C::decode8(W + (size_t)src_row * row_bytes + (size_t)blk * C::BB, k0, y);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) y[i] = 0.0f;
+    }
     float *o = out + (size_t)row * n_cols + (size_t)blk * C::BE + k0;
     if (VEC) {
         reinterpret_cast<float4 *>(o)[0] = make_float4(y[0], y[1], y[2], y[3]);
@@ -35,22 +43,34 @@ dequant_kernel(const uint8_t *__restrict__ W, float *__restrict__ out, int n_row
     }
 }
 
-/* F16 / BF16 / F32 rows (common/ggml_dequant.h:3251-3261) */
+/* F16 / BF16 / F32 rows (common/ggml_dequant.h:3251-3261); output row r = source row row_ids[r]
+ * when a list is given */
 __global__ void __launch_bounds__(256)
-convert_plain_kernel(uint32_t type, const uint8_t *__restrict__ src, float *__restrict__ out, long long n) {
+convert_plain_kernel(uint32_t type, const uint8_t *__restrict__ src, const int32_t *__restrict__ row_ids,
+                     int n_src_rows, float *__restrict__ out, long long n, int n_cols) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
+    long long s = i;
+    if (row_ids) {
+        const long long r = i / n_cols;
+        const int id = row_ids[r];
+        if (id < 0 || id >= n_src_rows) {
+            out[i] = 0.0f;
+            return;
+        }
+        s = (long long)id * n_cols + (i - r * n_cols);
+    }
     if (type == T_F32) {
-        reinterpret_cast<uint32_t *>(out)[i] = reinterpret_cast<const uint32_t *>(src)[i];
+        reinterpret_cast<uint32_t *>(out)[i] = reinterpret_cast<const uint32_t *>(src)[s];
     } else {
-        const uint32_t h = reinterpret_cast<const uint16_t *>(src)[i];
+        const uint32_t h = reinterpret_cast<const uint16_t *>(src)[s];
         out[i] = (type == T_F16) ? half_bits_exact(h) : __uint_as_float(h << 16);
     }
 }
 
 template <uint32_t T>
-static hipError_t launch_typed(const void *W, float *out, int n_rows, int n_cols, size_t row_bytes,
-                               hipStream_t stream) {
+static hipError_t launch_typed(const void *W, const int32_t *row_ids, int n_src_rows, float *out, int n_rows,
+                               int n_cols, size_t row_bytes, hipStream_t stream) {
     const int bpr = n_cols / Codec<T>::BE;
     const long long groups = (long long)bpr * (Codec<T>::BE / 8) * n_rows;
     if (groups == 0) return hipSuccess;
@@ -58,24 +78,25 @@ static hipError_t launch_typed(const void *W, float *out, int n_rows, int n_cols
     const bool vec = (n_cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(out) & 15u) == 0);
     if (vec)
         hipLaunchKernelGGL((dequant_kernel<T, true>), dim3(grid), dim3(256), 0, stream,
-                           (const uint8_t *)W, out, n_rows, n_cols, row_bytes, bpr);
+                           (const uint8_t *)W, row_ids, n_src_rows, out, n_rows, n_cols, row_bytes, bpr);
     else
         hipLaunchKernelGGL((dequant_kernel<T, false>), dim3(grid), dim3(256), 0, stream,
-                           (const uint8_t *)W, out, n_rows, n_cols, row_bytes, bpr);
+                           (const uint8_t *)W, row_ids, n_src_rows, out, n_rows, n_cols, row_bytes, bpr);
     return hipGetLastError();
 }
 
-hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, int n_cols,
-                          size_t row_bytes, hipStream_t stream) {
+hipError_t launch_dequant(uint32_t type, const void *W, const int32_t *row_ids, int n_src_rows, float *out,
+                          int n_rows, int n_cols, size_t row_bytes, hipStream_t stream) {
+    if (!row_ids) n_src_rows = n_rows;
     switch (type) {
-#define QLIN_CASE(TT) case TT: return launch_typed<TT>(W, out, n_rows, n_cols, row_bytes, stream);
+#define QLIN_CASE(TT) case TT: return launch_typed<TT>(W, row_ids, n_src_rows, out, n_rows, n_cols, row_bytes, stream);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
 #undef QLIN_CASE
     case T_F32: case T_F16: case T_BF16: {
         const long long n = (long long)n_rows * n_cols;
         if (n == 0) return hipSuccess;
         hipLaunchKernelGGL(convert_plain_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
-                           type, (const uint8_t *)W, out, n);
+                           type, (const uint8_t *)W, row_ids, n_src_rows, out, n, n_cols);
         return hipGetLastError();
     }
     default: return hipErrorInvalidValue;

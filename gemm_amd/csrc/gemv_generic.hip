@@ -122,6 +122,7 @@ hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x
     switch (type) {
 #define QLIN_CASE(TT) case TT: return gemv_typed<TT>(job, x, n_cols, s);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+    QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
 #undef QLIN_CASE
     default: return hipErrorInvalidValue;
     }
@@ -144,6 +145,7 @@ hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *
     switch (type) {
 #define QLIN_CASE(TT) case TT: return gemm_typed<TT>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, s);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+    QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
 #undef QLIN_CASE
     default: return hipErrorInvalidValue;
     }

@@ -602,6 +602,7 @@ bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n
     switch (type) {
 #define QLIN_CASE(TT) case TT: return stream_typed<TT>(job, x, n_cols, n_cu, stream, err);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+    QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
 #undef QLIN_CASE
     default: return false;
     }

@@ -156,8 +156,9 @@ hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y,
 
 int check_linear_shape(uint32_t type, int n_rows, int n_cols) {
     int be, bb;
-    if (!type_geometry(type, &be, &bb) || be == 1)
+    if (!type_geometry(type, &be, &bb))
         return fail(QLIN_ERR_TYPE, "unsupported weight type %u", type);
+    if (be == 1) be = 8; /* dense F16/BF16/F32 rows go through the kernels eight elements at a time */
     if (n_rows < 0 || n_cols <= 0) return fail(QLIN_ERR_ARG, "bad shape %d x %d", n_rows, n_cols);
     if (n_cols % be) return fail(QLIN_ERR_ARG, "n_cols %d is not a whole number of %d-element blocks", n_cols, be);
     return QLIN_OK;
@@ -213,6 +214,22 @@ int matvec_multi_host_locked(int n_mat, float *const dst[3], const void *const W
     for (int m = 0; m < n_out; m++)
         if (n_rows[m]) HIP_TRY(hipMemcpyAsync(dst[m], g.y[m].p, (size_t)n_rows[m] * 4, hipMemcpyDeviceToHost, g.stream));
     return QLIN_OK;
+}
+
+bool dense_type(uint32_t t) { return t == T_F16 || t == T_BF16 || t == T_F32; }
+
+/* argument checks shared by the device-resident matvec entry points */
+int check_dev_gemv(uint32_t type, int n_rows, int n_cols, const void *W, const float *x, const float *y) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!W || !x || !y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, dense_type(type) ? 16 : 2) || !aligned(x, 16) || !aligned(y, 4))
+        return fail(QLIN_ERR_ARG, "W needs 2-byte (dense types: 16-byte), x 16-byte, y 4-byte alignment");
+    return QLIN_OK;
+}
+int init_once() {
+    std::lock_guard<std::mutex> lk(g.mu);
+    return ensure_init_locked(0);
 }
 
 void void_decoder(uint32_t type, const char *name, const void *src, float *dst, int n) {
@@ -286,7 +303,7 @@ int qlin_dequant_rows(uint32_t ggml_type, const void *src, float *dst, int n_row
     if (int rc = weights_on_device_locked(src, rb * (size_t)(n_rows - 1) + (size_t)(whole / be) * bb, g.w[0], &dW)) return rc;
     const size_t out_bytes = (size_t)n_rows * n_cols * 4;
     if (int rc = g.tmp[0].ensure(out_bytes)) return rc;
-    HIP_TRY(launch_dequant(ggml_type, dW, (float *)g.tmp[0].p, n_rows, n_cols, rb, g.stream));
+    HIP_TRY(launch_dequant(ggml_type, dW, nullptr, 0, (float *)g.tmp[0].p, n_rows, n_cols, rb, g.stream));
     if (whole == n_cols) {
         HIP_TRY(hipMemcpyAsync(dst, g.tmp[0].p, out_bytes, hipMemcpyDeviceToHost, g.stream));
     } else { /* leave the undecoded tail of every row untouched in dst */
@@ -544,9 +561,8 @@ int qlin_moe_ffn_token(float *out, const void *gate_exps, const void *up_exps, c
         const uint8_t *ge = (const uint8_t *)dG + (size_t)e * n_ff * rb_in;
         const uint8_t *ue = (const uint8_t *)dU + (size_t)e * n_ff * rb_in;
         const uint8_t *de = (const uint8_t *)dD + (size_t)e * n_embd * rb_dn;
-        HIP_TRY(dispatch_gemv(type, ge, (const float *)g.x.p, (float *)g.tmp[1].p, n_ff, n_embd, g.stream));
-        HIP_TRY(dispatch_gemv(type, ue, (const float *)g.x.p, (float *)g.tmp[2].p, n_ff, n_embd, g.stream));
-        HIP_TRY(launch_silu_mul((float *)g.tmp[1].p, (const float *)g.tmp[1].p, (const float *)g.tmp[2].p, n_ff, g.stream));
+        const GemvJob gate_up = {{ge, ue, nullptr}, {(float *)g.tmp[1].p, nullptr, nullptr}, {n_ff, n_ff, 0}, 2, kSiluMul};
+        HIP_TRY(dispatch_gemv_job(type, gate_up, (const float *)g.x.p, n_embd, g.stream));
         HIP_TRY(dispatch_gemv(type, de, (const float *)g.tmp[1].p, (float *)g.tmp[3].p, n_embd, n_ff, g.stream));
         HIP_TRY(launch_axpy_dev_weight((float *)g.y[0].p, (const float *)g.tmp[3].p, d_w, k, n_embd, k == 0, g.stream));
     }
@@ -601,38 +617,33 @@ int qlin_dequant_dev(uint32_t type, const void *W, float *out, int n_rows, int n
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
-    HIP_TRY(launch_dequant(type, W, out, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));
+    HIP_TRY(launch_dequant(type, W, nullptr, 0, out, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_embed_rows_dev(uint32_t type, const void *table, int n_table_rows, const int32_t *row_ids, int n_ids,
+                        float *out, int n_cols, void *stream) {
+    if (!known_type(type)) return fail(QLIN_ERR_TYPE, "unsupported type %u", type);
+    if (n_table_rows < 0 || n_ids < 0 || n_cols < 0) return fail(QLIN_ERR_ARG, "negative size");
+    int be, bb;
+    type_geometry(type, &be, &bb);
+    if (n_cols % be) return fail(QLIN_ERR_ARG, "n_cols %d is not a whole number of %d-element blocks", n_cols, be);
+    if (n_ids == 0 || n_cols == 0) return QLIN_OK;
+    if (!table || !row_ids || !out) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(table, 2) || !aligned(row_ids, 4) || !aligned(out, 4)) return fail(QLIN_ERR_ARG, "misaligned pointer");
+    if (int rc = init_once()) return rc;
+    HIP_TRY(launch_dequant(type, table, row_ids, n_table_rows, out, n_ids, n_cols, row_size(type, n_cols),
+                           (hipStream_t)stream));
     return QLIN_OK;
 }
 
 int qlin_gemv_dev(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, void *stream) {
-    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (int rc = check_dev_gemv(type, n_rows, n_cols, W, x, y)) return rc;
     if (n_rows == 0) return QLIN_OK;
-    if (!W || !x || !y) return fail(QLIN_ERR_ARG, "null pointer");
-    if (!aligned(W, 2) || !aligned(x, 16) || !aligned(y, 4))
-        return fail(QLIN_ERR_ARG, "W needs 2-byte, x 16-byte, y 4-byte alignment");
-    {
-        std::lock_guard<std::mutex> lk(g.mu);
-        if (int rc = ensure_init_locked(0)) return rc;
-    }
+    if (int rc = init_once()) return rc;
     HIP_TRY(dispatch_gemv(type, W, x, y, n_rows, n_cols, (hipStream_t)stream));
     return QLIN_OK;
 }
-
-namespace {
-int check_dev_gemv(uint32_t type, int n_rows, int n_cols, const void *W, const float *x, const float *y) {
-    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
-    if (n_rows == 0) return QLIN_OK;
-    if (!W || !x || !y) return fail(QLIN_ERR_ARG, "null pointer");
-    if (!aligned(W, 2) || !aligned(x, 16) || !aligned(y, 4))
-        return fail(QLIN_ERR_ARG, "W needs 2-byte, x 16-byte, y 4-byte alignment");
-    return QLIN_OK;
-}
-int init_once() {
-    std::lock_guard<std::mutex> lk(g.mu);
-    return ensure_init_locked(0);
-}
-}  // namespace
 
 int qlin_gemv_add_dev(uint32_t type, const void *W, const float *x, float *y, int n_rows, int n_cols, void *stream) {
     if (int rc = check_dev_gemv(type, n_rows, n_cols, W, x, y)) return rc;

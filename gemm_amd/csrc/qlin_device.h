@@ -240,6 +240,44 @@ template <> struct Codec<T_IQ3_S> : Geom<T_IQ3_S> {
     }
 };
 
+/* Dense rows (F16, BF16, F32) seen by the matvec kernels as "blocks" of eight elements, so that
+ * they run through the same row loops: what tf_qmatvec computes for these types is the fp32 dot of
+ * the widened row with x (common/transformer.h:1051-1075, common/ggml_dequant.h:360-400, :1201-1230).
+ * type_geometry() keeps the per-element view (1 element, 2 or 4 bytes) for the codec entry points. */
+#define QLIN_FOR_EACH_DENSE_TYPE(X) X(T_F16) X(T_BF16) X(T_F32)
+template <> struct Geom<T_F16>  { static constexpr int BE = 8, BB = 16; };
+template <> struct Geom<T_BF16> { static constexpr int BE = 8, BB = 16; };
+template <> struct Geom<T_F32>  { static constexpr int BE = 8, BB = 32; };
+
+template <> struct Codec<T_F16> : Geom<T_F16> {
+    __device__ static void decode8(const uint8_t *blk, int, float (&y)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(blk);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            y[2 * i] = half_bits_exact(w[i] & 0xFFFFu);
+            y[2 * i + 1] = half_bits_exact(w[i] >> 16);
+        }
+    }
+};
+template <> struct Codec<T_BF16> : Geom<T_BF16> {
+    __device__ static void decode8(const uint8_t *blk, int, float (&y)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(blk);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            y[2 * i] = __uint_as_float(w[i] << 16);
+            y[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+        }
+    }
+};
+template <> struct Codec<T_F32> : Geom<T_F32> {
+    __device__ static void decode8(const uint8_t *blk, int, float (&y)[8]) {
+        const float4 a = reinterpret_cast<const float4 *>(blk)[0], b = reinterpret_cast<const float4 *>(blk)[1];
+        y[0] = a.x; y[1] = a.y; y[2] = a.z; y[3] = a.w; y[4] = b.x; y[5] = b.y; y[6] = b.z; y[7] = b.w;
+    }
+};
+
 }  // namespace qlin
 #include "qlin_codecs_ext.h"
 namespace qlin {

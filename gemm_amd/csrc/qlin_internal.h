@@ -15,9 +15,11 @@
 namespace qlin {
 
 /* out[n_rows, n_cols] = decode(W); n_cols may be ragged: only n_cols / block_elems blocks per
- * row are decoded, row r of W starts at r * row_bytes, row r of out at r * n_cols. */
-hipError_t launch_dequant(uint32_t type, const void *W, float *out, int n_rows, int n_cols,
-                          size_t row_bytes, hipStream_t stream);
+ * row are decoded, row r of W starts at r * row_bytes, row r of out at r * n_cols. With row_ids
+ * (device, n_rows entries) output row r is decoded from source row row_ids[r] of a table of
+ * n_src_rows rows (zeros for an id outside it); without, n_src_rows is ignored. */
+hipError_t launch_dequant(uint32_t type, const void *W, const int32_t *row_ids, int n_src_rows, float *out,
+                          int n_rows, int n_cols, size_t row_bytes, hipStream_t stream);
 
 /* One matvec launch over up to three matrices of ONE block type that share x and n_cols: the
  * fused call shapes of the reference's decode loop.

@@ -70,6 +70,7 @@ SIGNATURES = {
     "qlin_dev_sync": (C.c_int, [_vp]),
     "qlin_dequant_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemv_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
+    "qlin_embed_rows_dev": (C.c_int, [C.c_uint32, _vp, C.c_int, _vp, C.c_int, _vp, C.c_int, _vp]),
     "qlin_gemv_add_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemv_silu_mul_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemv_multi_dev": (C.c_int, [C.c_uint32, C.c_int, _vp, _vp, _vp, _vp, C.c_int, _vp]),
@@ -198,6 +199,10 @@ def gemm_tokenmajor(type_id, W, X, n_cols):
 
 def gemv_dev(type_id, dW, dx, dy, n_rows, n_cols, stream=None):
     check(load().qlin_gemv_dev(type_id, dW.ptr, dx.ptr, dy.ptr, n_rows, n_cols, stream))
+
+
+def embed_rows_dev(type_id, dtable, n_table_rows, dids, n_ids, dout, n_cols, stream=None):
+    check(load().qlin_embed_rows_dev(type_id, dtable.ptr, n_table_rows, dids.ptr, n_ids, dout.ptr, n_cols, stream))
 
 
 def gemv_add_dev(type_id, dW, dx, dy, n_rows, n_cols, stream=None):

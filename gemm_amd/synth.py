@@ -38,6 +38,9 @@ TYPE_NAMES = {GGML_Q8_0: "q8_0", GGML_Q4_K: "q4_K", GGML_Q5_K: "q5_K", GGML_Q6_K
 LINEAR_TYPES = {t: TYPE_NAMES[t] for t in (
     GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_IQ2_XXS, GGML_IQ4_NL, GGML_IQ3_S, GGML_Q4_0,
     GGML_Q2_K, GGML_Q3_K, GGML_IQ2_XS, GGML_IQ3_XXS, GGML_IQ1_S, GGML_IQ2_S, GGML_IQ4_XS, GGML_IQ1_M)}
+# dense row formats the model path also takes as weights (one element per "block")
+DENSE_TYPES = {GGML_F32: "f32", GGML_F16: "f16", GGML_BF16: "bf16"}
+BLOCK_GEOMETRY.update({GGML_F32: (1, 4), GGML_F16: (1, 2), GGML_BF16: (1, 2)})
 # offsets of the fp16 scale fields of the formats not spelled out in make_weights
 _F16_FIELDS = {
     GGML_IQ4_NL: (0,), GGML_IQ2_XXS: (0,), GGML_IQ3_S: (0,),
@@ -70,6 +73,15 @@ def make_weights(type_id, n_rows, n_cols, seed, wild=False):
     assert n_cols % be == 0, "n_cols must be a whole number of blocks"
     nb = n_cols // be
     rng = np.random.default_rng(seed)
+    if type_id in DENSE_TYPES:  # N(0, 0.02) values (wild: any bit pattern)
+        if wild:
+            return rng.integers(0, 256, size=(n_rows, nb * bb), dtype=np.uint8)
+        v = (rng.standard_normal(size=(n_rows, n_cols)) * 0.02).astype(np.float32)
+        if type_id == GGML_F16:
+            v = v.astype(np.float16)
+        elif type_id == GGML_BF16:
+            v = to_bf16_bits(v)
+        return np.ascontiguousarray(v).view(np.uint8).reshape(n_rows, nb * bb)
     blocks = rng.integers(0, 256, size=(n_rows, nb, bb), dtype=np.uint8)
     if not wild:
         if type_id == GGML_Q8_0:

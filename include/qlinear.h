@@ -164,7 +164,14 @@ int   qlin_dev_sync(void *stream);
 
 /* out[n_rows, n_cols] fp32 = decode(W); whole blocks only */
 int qlin_dequant_dev(uint32_t ggml_type, const void *W, float *out, int n_rows, int n_cols, void *stream);
-/* y[n_rows] = W . x, x fp32 */
+/* out[i, :] = decode(table row row_ids[i]) for i < n_ids: the token-embedding lookup
+ * (tf_dequant_row on token_embd, common/transformer.h:3509) for a list of device-resident ids.
+ * An id outside [0, n_table_rows) gives a row of zeros (the reference refuses such a token, :3501). */
+int qlin_embed_rows_dev(uint32_t ggml_type, const void *table, int n_table_rows, const int32_t *row_ids,
+                        int n_ids, float *out, int n_cols, void *stream);
+/* y[n_rows] = W . x, x fp32. Besides the block formats W may be dense F16, BF16 or F32 rows
+ * (n_cols a multiple of 8, W 16-byte aligned): the fp32 dot of the widened row with x, as
+ * tf_qmatvec does for these types (common/transformer.h:1051-1075). */
 int qlin_gemv_dev(uint32_t ggml_type, const void *W, const float *x, float *y, int n_rows,
                   int n_cols, void *stream);
 /* The fused call shapes of the decode loop, one launch each (all matrices of one ggml type):

@@ -92,7 +92,8 @@ def main():
     x = synth.make_activation(LIN_COLS, seed=77)
     X = synth.make_activation(LIN_COLS, seed=78, tokens=5)
     lin["x"], lin["X"] = x, X
-    for tid, name in synth.LINEAR_TYPES.items():  # the types the reference's model path accepts
+    # the types the reference's model path accepts: sixteen block formats and the dense ones
+    for tid, name in list(synth.LINEAR_TYPES.items()) + list(synth.DENSE_TYPES.items()):
         W = synth.make_weights(tid, LIN_ROWS, LIN_COLS, seed=4000 + tid)
         lin[name + "_W"] = W
         lin[name + "_y_f32"] = ref.qmatvec(tid, W, x, LIN_COLS)

@@ -120,3 +120,20 @@ def test_full_size_q4k_decode_properties(oracle):
     lo = (-dmin * 63)[..., None]
     o = out.reshape(n_rows, n_cols // 256, 256)
     assert np.all(o <= hi + 1e-6) and np.all(o >= lo - 1e-6)
+
+
+@pytest.mark.parametrize("tid,name", NAMES + list(synth.DENSE_TYPES.items()))
+def test_embedding_lookup_by_device_resident_ids(oracle, tid, name):
+    """rows picked by a list of ids, decoded bit-exactly; an id outside the table gives zeros"""
+    n_vocab, n_cols = 300, 1024
+    W = synth.make_weights(tid, n_vocab, n_cols, seed=800 + tid)
+    ids = np.array([5, 299, 0, 5, -1, 300, 123], np.int32)
+    dW, dI = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(ids)
+    dO = qlinear.DevBuf(ids.size * n_cols * 4)
+    qlinear.embed_rows_dev(tid, dW, n_vocab, dI, ids.size, dO, n_cols)
+    qlinear.sync()
+    got = dO.to_numpy(np.float32, (ids.size, n_cols))
+    dec = oracle.dequant_matrix(tid, W, n_cols)
+    for i, t in enumerate(ids):
+        want = dec[t] if 0 <= t < n_vocab else np.zeros(n_cols, np.float32)
+        assert_same_bits(got[i], want, "%s id %d" % (name, t))

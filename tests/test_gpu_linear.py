@@ -8,8 +8,10 @@ from gemm_amd import qlinear, synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu
-NAMES = list(synth.TYPE_NAMES.items())
-LINEAR = list(synth.LINEAR_TYPES.items())  # the types the reference golden outputs exist for
+# every block format, plus dense F32/F16/BF16 rows
+NAMES = list(synth.TYPE_NAMES.items()) + list(synth.DENSE_TYPES.items())
+# the types the reference golden outputs exist for: the model path's block formats and dense rows
+LINEAR = list(synth.LINEAR_TYPES.items()) + list(synth.DENSE_TYPES.items())
 TOL = 1e-5
 
 
@@ -58,7 +60,8 @@ def test_matvec_empty_and_errors():
     y = np.zeros(4, np.float32)
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_Q4_K, 512, x.ctypes.data, 0) == 0
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, 99, 512, x.ctypes.data, 4) == qlinear.ERR_TYPE
-    assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_F16, 512, x.ctypes.data, 4) == qlinear.ERR_TYPE
+    assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, 9, 512, x.ctypes.data, 4) == qlinear.ERR_TYPE  # Q8_1
+    assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_F16, 500, x.ctypes.data, 4) == qlinear.ERR_ARG
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_Q4_K, 500, x.ctypes.data, 4) == qlinear.ERR_ARG
     assert lib.qlin_matvec(None, W.ctypes.data, synth.GGML_Q4_K, 512, x.ctypes.data, 4) == qlinear.ERR_ARG
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_Q4_K, 512, x.ctypes.data, -1) == qlinear.ERR_ARG

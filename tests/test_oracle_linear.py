@@ -6,7 +6,8 @@ from gemm_amd import synth
 from tests.conftest import rel_l2
 
 NAMES = list(synth.TYPE_NAMES.items())
-LINEAR = list(synth.LINEAR_TYPES.items())  # the types the reference golden outputs exist for
+# the types the reference golden outputs exist for: the model path's block formats and dense rows
+LINEAR = list(synth.LINEAR_TYPES.items()) + list(synth.DENSE_TYPES.items())
 
 
 @pytest.mark.parametrize("tid,name", NAMES)
