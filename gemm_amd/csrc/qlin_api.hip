@@ -37,6 +37,23 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+}  // namespace
+
+namespace qlin {
+/* for the other translation units of the library: sets the text qlin_last_error() returns */
+int set_error(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    t_error = buf;
+    return code;
+}
+}  // namespace qlin
+
+namespace {
+
 #define HIP_TRY(expr)                                                                          \
     do {                                                                                       \
         hipError_t e_ = (expr);                                                                \
@@ -363,6 +380,19 @@ int qlin_weight_register(const void *host_data, size_t n_bytes) {
         return fail(QLIN_ERR_DEVICE, "upload failed: %s", hipGetErrorString(e));
     }
     g.registry[h] = Range{n_bytes, dev};
+    return QLIN_OK;
+}
+
+int qlin_weight_adopt(const void *host_data, size_t n_bytes, void *dev_copy) {
+    if (!host_data || n_bytes == 0 || !dev_copy) return fail(QLIN_ERR_ARG, "null or empty weight range");
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    const uintptr_t h = reinterpret_cast<uintptr_t>(host_data);
+    if (lookup_locked(host_data, 1) || lookup_locked((const uint8_t *)host_data + n_bytes - 1, 1))
+        return fail(QLIN_ERR_ARG, "range overlaps a registered range");
+    auto nxt = g.registry.lower_bound(h);
+    if (nxt != g.registry.end() && nxt->first < h + n_bytes) return fail(QLIN_ERR_ARG, "range overlaps a registered range");
+    g.registry[h] = Range{n_bytes, dev_copy};
     return QLIN_OK;
 }
 

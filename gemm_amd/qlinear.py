@@ -51,6 +51,7 @@ SIGNATURES = {
     "qlin_dequantize_row_bf16": (None, [_vp, _vp, C.c_int]),
     "qlin_dequant_rows": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int]),
     "qlin_weight_register": (C.c_int, [_vp, C.c_size_t]),
+    "qlin_weight_adopt": (C.c_int, [_vp, C.c_size_t, _vp]),
     "qlin_weight_unregister": (C.c_int, [_vp]),
     "qlin_weight_device_ptr": (_vp, [_vp]),
     "qlin_matvec": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
@@ -81,6 +82,26 @@ SIGNATURES = {
     "qlin_moe_route_dev": (C.c_int, [_vp, C.c_int, C.c_int, C.c_int, _vp, _vp, _vp]),
     "qlin_moe_ffn_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int,
                                    C.c_int, C.c_int, _vp, _vp]),
+    "qlin_gguf_open": (C.c_int, [C.c_char_p, _vp]),
+    "qlin_gguf_close": (None, [_vp]),
+    "qlin_gguf_version": (C.c_uint32, [_vp]),
+    "qlin_gguf_alignment": (C.c_uint32, [_vp]),
+    "qlin_gguf_data_offset": (C.c_size_t, [_vp]),
+    "qlin_gguf_data_size": (C.c_size_t, [_vp]),
+    "qlin_gguf_n_tensors": (C.c_int, [_vp]),
+    "qlin_gguf_find_tensor": (C.c_int, [_vp, C.c_char_p]),
+    "qlin_gguf_tensor_info": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "qlin_gguf_tensor_host": (_vp, [_vp, C.c_int]),
+    "qlin_gguf_tensor_dev": (_vp, [_vp, C.c_int]),
+    "qlin_gguf_upload": (C.c_int, [_vp]),
+    "qlin_gguf_n_kv": (C.c_int, [_vp]),
+    "qlin_gguf_find_key": (C.c_int, [_vp, C.c_char_p]),
+    "qlin_gguf_key": (C.c_char_p, [_vp, C.c_int]),
+    "qlin_gguf_value_type": (C.c_int, [_vp, C.c_int]),
+    "qlin_gguf_get_i64": (C.c_int, [_vp, C.c_int, _vp]),
+    "qlin_gguf_get_f64": (C.c_int, [_vp, C.c_int, _vp]),
+    "qlin_gguf_get_str": (C.c_char_p, [_vp, C.c_int]),
+    "qlin_gguf_get_array": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp]),
     "qlin_timer_begin": (C.c_int, [_vp]),
     "qlin_timer_end": (C.c_int, [_vp, _fp]),
 }

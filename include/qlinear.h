@@ -105,6 +105,9 @@ int    qlin_dequant_rows(uint32_t ggml_type, const void *src, float *dst, int n_
  * Calls with an unregistered pointer still work: the bytes are staged for that call only. */
 int  qlin_weight_register(const void *host_data, size_t n_bytes);
 int  qlin_weight_unregister(const void *host_data);
+/* Same registration for a host range whose device copy already exists (n_bytes at dev_copy, from
+ * hipMalloc): nothing is copied, the library takes ownership and frees it on unregister. */
+int  qlin_weight_adopt(const void *host_data, size_t n_bytes, void *dev_copy);
 /* Device address that mirrors host_ptr, or NULL if host_ptr is in no registered range. */
 const void *qlin_weight_device_ptr(const void *host_ptr);
 
@@ -208,6 +211,41 @@ int qlin_moe_ffn_dev(uint32_t ggml_type, const void *gate_exps, const void *up_e
                      const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
                      const float *expert_w, float *out, int n_tok, int top_k, int n_embd,
                      int n_ff, int n_expert, void *workspace, void *stream);
+
+/* ------------------------------------------------------------------ GGUF file -> HBM
+ * The tensor table and key/value pairs of a GGUF model file (versions 2 and 3, as read by
+ * gguf_open, common/gguf_loader.h:343-411) and its tensor bytes in device memory.
+ * qlin_gguf_open parses the header (no GPU needed, no tensor data read); qlin_gguf_upload streams
+ * the data section into ONE device allocation through pinned staging buffers and registers the
+ * host range of the (lazily) mapped file, so that qlin_gguf_tensor_host(i) pointers work with the
+ * host-pointer entry points above without further copies (the place of tf_load_tensor's
+ * `gguf_tensor_data` pointers, common/transformer.h:363-381) and qlin_gguf_tensor_dev(i) with the
+ * device-resident ones. Tensor sizes follow gguf_tensor_size (:520-532). */
+typedef struct qlin_gguf qlin_gguf;
+int  qlin_gguf_open(const char *path, qlin_gguf **out);
+void qlin_gguf_close(qlin_gguf *g);       /* also releases the device copy */
+uint32_t qlin_gguf_version(const qlin_gguf *g);
+uint32_t qlin_gguf_alignment(const qlin_gguf *g);
+size_t qlin_gguf_data_offset(const qlin_gguf *g);   /* file offset of the data section */
+size_t qlin_gguf_data_size(const qlin_gguf *g);     /* end of the last tensor */
+int  qlin_gguf_n_tensors(const qlin_gguf *g);
+int  qlin_gguf_find_tensor(const qlin_gguf *g, const char *name); /* index or -1 (tf_find_tensor, :355) */
+int  qlin_gguf_tensor_info(const qlin_gguf *g, int i, const char **name, uint32_t *ggml_type, int *n_dims,
+                           uint64_t dims[4], uint64_t *offset, size_t *n_bytes);
+const void *qlin_gguf_tensor_host(const qlin_gguf *g, int i);  /* address in the mapped file */
+const void *qlin_gguf_tensor_dev(const qlin_gguf *g, int i);   /* NULL before qlin_gguf_upload */
+int  qlin_gguf_upload(qlin_gguf *g);
+/* key/value pairs: index of a key or -1; value type = enum gguf_value_type (:26-41) */
+int  qlin_gguf_n_kv(const qlin_gguf *g);
+int  qlin_gguf_find_key(const qlin_gguf *g, const char *key);
+const char *qlin_gguf_key(const qlin_gguf *g, int i);
+int  qlin_gguf_value_type(const qlin_gguf *g, int i);
+int  qlin_gguf_get_i64(const qlin_gguf *g, int i, int64_t *out);   /* any integer width, bool */
+int  qlin_gguf_get_f64(const qlin_gguf *g, int i, double *out);    /* any number */
+const char *qlin_gguf_get_str(const qlin_gguf *g, int i);           /* NULL unless a string */
+/* arrays: element type, count and the address of the first element in the mapped file (strings:
+ * u64 length + bytes each, not terminated) */
+int  qlin_gguf_get_array(const qlin_gguf *g, int i, uint32_t *elem_type, uint64_t *n, const void **first);
 
 /* Elapsed milliseconds of work enqueued on `stream` between the two calls, by HIP events
  * recorded on that stream (the role of elapsed_kernel_ms in rdna4/dequant/bench_dequant.c:764-780). */

@@ -113,3 +113,38 @@ const void *ref_table(const char *name, size_t *bytes) {
     *bytes = 0;
     return NULL;
 }
+
+/* ---- GGUF loader of the reference, for the fixture of the file parser ---- */
+void *ref_gguf_open(const char *path) { return gguf_open(path, 0); }
+void ref_gguf_close(void *c) { gguf_close((gguf_context *)c); }
+uint64_t ref_gguf_n_tensors(const void *c) { return ((const gguf_context *)c)->n_tensors; }
+uint64_t ref_gguf_n_kv(const void *c) { return ((const gguf_context *)c)->n_kv; }
+uint32_t ref_gguf_version(const void *c) { return ((const gguf_context *)c)->version; }
+uint32_t ref_gguf_alignment(const void *c) { return ((const gguf_context *)c)->alignment; }
+uint64_t ref_gguf_data_offset(const void *c) { return ((const gguf_context *)c)->data_offset; }
+uint64_t ref_gguf_data_size(const void *c) { return ((const gguf_context *)c)->data_size; }
+const char *ref_gguf_tensor_name(const void *c, int i) { return gguf_tensor_name((const gguf_context *)c, i); }
+uint64_t ref_gguf_tensor_size(const void *c, int i) { return gguf_tensor_size((const gguf_context *)c, i); }
+const void *ref_gguf_tensor_data(const void *c, int i) { return gguf_tensor_data((const gguf_context *)c, i); }
+/* out: type, n_dims, dims[4], offset */
+void ref_gguf_tensor_info(const void *c, int i, uint64_t out[7]) {
+    const gguf_tensor_info *t = &((const gguf_context *)c)->tensors[i];
+    out[0] = t->type; out[1] = t->n_dims;
+    for (int d = 0; d < 4; d++) out[2 + d] = t->dims[d];
+    out[6] = t->offset;
+}
+/* the qtensor tf_load_tensor builds for a name: out = type, n_rows, n_cols, n_dims; returns the data
+ * offset from the start of the data section, or -1 if the tensor is missing */
+int64_t ref_tf_load_tensor(const void *c, const char *name, int64_t out[4]) {
+    const gguf_context *g = (const gguf_context *)c;
+    qtensor t = tf_load_tensor(g, name, 0);
+    if (!t.data) return -1;
+    out[0] = t.type; out[1] = t.n_rows; out[2] = t.n_cols; out[3] = t.n_dims;
+    return (int64_t)((const uint8_t *)t.data - g->data);
+}
+int ref_gguf_find_key(const void *c, const char *key) { return gguf_find_key((const gguf_context *)c, key); }
+uint32_t ref_gguf_kv_type(const void *c, int i) { return ((const gguf_context *)c)->kv[i].type; }
+uint64_t ref_gguf_kv_u64(const void *c, int i) { return ((const gguf_context *)c)->kv[i].value.u64; }
+const char *ref_gguf_kv_str(const void *c, int i) { return ((const gguf_context *)c)->kv[i].value.str.str; }
+uint64_t ref_gguf_kv_arr_n(const void *c, int i) { return ((const gguf_context *)c)->kv[i].value.arr.n; }
+int ref_tf_get_int(const void *c, const char *key, int dflt) { return tf_get_int((const gguf_context *)c, key, dflt); }

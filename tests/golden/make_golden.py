@@ -42,6 +42,92 @@ def canonical_nan(bits):
     return bits
 
 
+def gguf_fixture(ref):
+    """A small GGUF file (tests/golden/tiny.gguf) and what the reference's loader reads from it."""
+    import ctypes as C
+    from tests import gguf_writer as gw
+    path = os.path.join(OUT, "tiny.gguf")
+    rng = np.random.default_rng(77)
+    tensors = [
+        ("token_embd.weight", synth.GGML_Q6_K, (256, 40), synth.make_weights(synth.GGML_Q6_K, 40, 256, seed=1)),
+        ("blk.0.ffn_gate.weight", synth.GGML_Q4_K, (512, 24), synth.make_weights(synth.GGML_Q4_K, 24, 512, seed=2)),
+        ("blk.0.ffn_down_exps.weight", synth.GGML_IQ2_XS, (256, 8, 3), synth.make_weights(synth.GGML_IQ2_XS, 24, 256, seed=3)),
+        ("blk.0.attn_norm.weight", synth.GGML_F32, (256,), synth.make_activation(256, seed=4).view(np.uint8)),
+        ("output.weight", synth.GGML_Q8_0, (256, 40), synth.make_weights(synth.GGML_Q8_0, 40, 256, seed=5)),
+        ("rope_freqs", synth.GGML_F16, (31,), rng.integers(0, 256, 62, dtype=np.uint8)),  # odd size: next start is padded
+        ("blk.0.attn_q.weight", synth.GGML_BF16, (256, 16), synth.make_weights(synth.GGML_BF16, 16, 256, seed=6)),
+    ]
+    kvs = [("general.architecture", gw.STR, "qwen3"), ("qwen3.block_count", gw.U32, 1),
+           ("qwen3.embedding_length", gw.U32, 256), ("qwen3.rope.freq_base", gw.F32, 1000000.0),
+           ("qwen3.attention.layer_norm_rms_epsilon", gw.F32, 1e-6), ("general.file_type", gw.I32, -3),
+           ("some.u8", gw.U8, 200), ("some.i8", gw.I8, -100), ("some.u16", gw.U16, 60000), ("some.i16", gw.I16, -30000),
+           ("some.u64", gw.U64, 2 ** 63 + 5), ("some.i64", gw.I64, -2 ** 62), ("some.f64", gw.F64, 2.5), ("some.bool", gw.BOOL, 1),
+           ("tokenizer.ggml.tokens", gw.ARR, (gw.STR, ["<s>", "hello", "", "w\u00f6rld"])),
+           ("tokenizer.ggml.scores", gw.ARR, (gw.F32, [0.0, -1.5, 2.25])),
+           ("tokenizer.ggml.token_type", gw.ARR, (gw.I32, [1, 2, 3, 4, 5]))]
+    gw.write(path, kvs, tensors, version=3, alignment=64)
+    L = ref.lib
+    L.ref_gguf_open.restype = C.c_void_p
+    L.ref_gguf_open.argtypes = [C.c_char_p]
+    for fn, rt in (("n_tensors", C.c_uint64), ("n_kv", C.c_uint64), ("version", C.c_uint32), ("alignment", C.c_uint32),
+                   ("data_offset", C.c_uint64), ("data_size", C.c_uint64)):
+        getattr(L, "ref_gguf_" + fn).restype = rt
+        getattr(L, "ref_gguf_" + fn).argtypes = [C.c_void_p]
+    L.ref_gguf_tensor_name.restype = C.c_char_p
+    L.ref_gguf_tensor_name.argtypes = [C.c_void_p, C.c_int]
+    L.ref_gguf_tensor_size.restype = C.c_uint64
+    L.ref_gguf_tensor_size.argtypes = [C.c_void_p, C.c_int]
+    L.ref_gguf_tensor_data.restype = C.c_void_p
+    L.ref_gguf_tensor_data.argtypes = [C.c_void_p, C.c_int]
+    L.ref_gguf_tensor_info.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+    L.ref_tf_load_tensor.restype = C.c_int64
+    L.ref_tf_load_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p]
+    L.ref_gguf_find_key.argtypes = [C.c_void_p, C.c_char_p]
+    L.ref_gguf_kv_type.restype = C.c_uint32
+    L.ref_gguf_kv_type.argtypes = [C.c_void_p, C.c_int]
+    L.ref_gguf_kv_u64.restype = C.c_uint64
+    L.ref_gguf_kv_u64.argtypes = [C.c_void_p, C.c_int]
+    L.ref_gguf_kv_str.restype = C.c_char_p
+    L.ref_gguf_kv_str.argtypes = [C.c_void_p, C.c_int]
+    L.ref_gguf_kv_arr_n.restype = C.c_uint64
+    L.ref_gguf_kv_arr_n.argtypes = [C.c_void_p, C.c_int]
+    L.ref_tf_get_int.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
+    L.ref_gguf_close.argtypes = [C.c_void_p]
+    ctx = L.ref_gguf_open(path.encode())
+    assert ctx
+    out = {"file": "tiny.gguf", "file_sha256": hashlib.sha256(open(path, "rb").read()).hexdigest(),
+           "version": L.ref_gguf_version(ctx), "alignment": L.ref_gguf_alignment(ctx),
+           "data_offset": L.ref_gguf_data_offset(ctx), "data_size": L.ref_gguf_data_size(ctx),
+           "n_kv": L.ref_gguf_n_kv(ctx), "tensors": [], "kv": {}}
+    for i in range(L.ref_gguf_n_tensors(ctx)):
+        info = (C.c_uint64 * 7)()
+        L.ref_gguf_tensor_info(ctx, i, info)
+        name = L.ref_gguf_tensor_name(ctx, i)
+        size = L.ref_gguf_tensor_size(ctx, i)
+        raw = C.string_at(L.ref_gguf_tensor_data(ctx, i), size)
+        qt = (C.c_int64 * 4)()
+        qoff = L.ref_tf_load_tensor(ctx, name, qt)
+        out["tensors"].append({"name": name.decode(), "type": info[0], "n_dims": info[1], "dims": list(info[2:6]),
+                               "offset": info[6], "size": size, "data_sha256": hashlib.sha256(raw).hexdigest(),
+                               "qtensor": {"type": qt[0], "n_rows": qt[1], "n_cols": qt[2], "n_dims": qt[3],
+                                           "data_offset": qoff}})
+    for key, vtype, _ in kvs + [("general.alignment", gw.U32, 64)]:
+        i = L.ref_gguf_find_key(ctx, key.encode())
+        assert i >= 0
+        e = {"index": i, "type": L.ref_gguf_kv_type(ctx, i)}
+        if vtype == gw.STR:
+            e["str"] = L.ref_gguf_kv_str(ctx, i).decode()
+        elif vtype == gw.ARR:
+            e["n"] = L.ref_gguf_kv_arr_n(ctx, i)
+        else:
+            e["raw_u64"] = L.ref_gguf_kv_u64(ctx, i) & ((1 << (8 * {0: 1, 1: 1, 7: 1, 2: 2, 3: 2, 4: 4, 5: 4, 6: 4, 10: 8, 11: 8, 12: 8}[vtype])) - 1)
+        out["kv"][key] = e
+    out["tf_get_int"] = {k: L.ref_tf_get_int(ctx, k.encode(), -7) for k in
+                         ("qwen3.block_count", "general.file_type", "some.u16", "missing.key")}
+    L.ref_gguf_close(ctx)
+    return out
+
+
 def main():
     ref = Reference()
     manifest = {"generator": "tests/golden/make_golden.py", "source": "reference C compiled via oracle/ref_shim.c"}
@@ -102,6 +188,8 @@ def main():
         # expert slice: the 24 rows seen as 3 experts of 8 rows
         lin[name + "_y_expert1"] = ref.qmatvec_expert(tid, W, 1, x, 8, LIN_COLS)
     np.savez_compressed(os.path.join(OUT, "linear_golden.npz"), **lin)
+
+    manifest["gguf_fixture"] = gguf_fixture(ref)
 
     with open(os.path.join(OUT, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1, sort_keys=True)
