@@ -38,7 +38,7 @@ Q4K = synth.GGML_Q4_K
 # HBM bytes moved per Q4_K 14336x4096 matvec launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by what the same counters read for a device-to-device copy of known size
 # (profiles/gemv_q4k_14336x4096.md).
-MEASURED_TRAFFIC_BYTES = 33303554
+MEASURED_TRAFFIC_BYTES = 33319875
 
 
 def gemv_bytes(type_id, n_rows, n_cols):
@@ -229,6 +229,29 @@ def probe(args):
         tid, r, c = (synth.GGML_Q8_0, 4096, 4096) if args.probe == "gemv_q8_0" else (synth.GGML_Q6_K, 151936, 4096)
         ms, copies = time_gemv(tid, r, c, max(10, args.steps // 8), 3, max_copies=24 if r < 100000 else 2)
         print(json.dumps({"probe": args.probe, "ms_per_step": ms, "copies": copies}))
+    elif args.probe == "gemv_q4_0":
+        ms, copies = time_gemv(synth.GGML_Q4_0, 14336, 4096, max(10, args.steps // 4), 3)
+        print(json.dumps({"probe": args.probe, "ms_per_step": ms, "copies": copies}))
+    elif args.probe == "gemv_silu":  # only the fused gate+up+SiLU launch, 2 x (14336 x 4096) Q4_K
+        K, FF, n = 4096, 14336, 6
+        x = qlinear.DevBuf.from_numpy(synth.make_activation(K, seed=3) * np.float32(0.05))
+        Wg = [qlinear.DevBuf.from_numpy(synth.make_weights(Q4K, FF, K, seed=51)) for _ in range(n)]
+        Wu = [qlinear.DevBuf.from_numpy(synth.make_weights(Q4K, FF, K, seed=52)) for _ in range(n)]
+        y = qlinear.DevBuf(FF * 4)
+        steps = max(20, args.steps // 4)
+        for i in range(steps + 5):
+            if i == 5:
+                qlinear.sync()
+                qlinear.timer_begin()
+            qlinear.gemv_silu_mul_dev(Q4K, Wg[i % n], Wu[i % n], x, y, FF, K)
+        print(json.dumps({"probe": args.probe, "ms_per_step": qlinear.timer_end() / steps}))
+    elif args.probe == "dequant":
+        W = synth.make_weights(Q4K, 14336, 4096, seed=5)
+        dW, dO = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf(14336 * 4096 * 4)
+        for _ in range(max(5, args.steps // 20)):
+            qlinear.dequant_dev(Q4K, dW, dO, 14336, 4096)
+        qlinear.sync()
+        print(json.dumps({"probe": args.probe}))
     elif args.probe == "moe":
         m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
         print(json.dumps({"probe": "moe", "ms_per_step": m, "bytes": b, "routed": routed}))
@@ -244,7 +267,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemm", "moe"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "moe"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "

@@ -39,6 +39,46 @@ size_t qtf_row_bytes(uint32_t type, int n_cols) {
     return qtf_is_supported_weight_type(type) ? qlin_dequant_row_size(type, n_cols) : 0;
 }
 
+qtensor qtf_load_tensor(const struct qlin_gguf *gguf, const char *name, int required) {
+    qtensor t;
+    memset(&t, 0, sizeof(t));
+    const int idx = qlin_gguf_find_tensor(gguf, name);
+    if (idx < 0) {
+        if (required) fprintf(stderr, "qlinear: missing tensor '%s'\n", name);
+        return t;
+    }
+    uint32_t type = 0;
+    int n_dims = 0;
+    uint64_t dims[4] = {0, 0, 0, 0};
+    if (qlin_gguf_tensor_info(gguf, idx, NULL, &type, &n_dims, dims, NULL, NULL) != QLIN_OK) return t;
+    t.data = (void *)qlin_gguf_tensor_host(gguf, idx);
+    t.type = type;
+    t.n_dims = n_dims;
+    uint64_t n_rows = 1;
+    for (int d = 0; d < n_dims; d++) {
+        t.dims[d] = dims[d];
+        if (d > 0) n_rows *= dims[d];
+    }
+    t.n_cols = (int)dims[0];
+    t.n_rows = (int)n_rows;
+    return t;
+}
+
+int qtf_get_int(const struct qlin_gguf *gguf, const char *key, int default_val) {
+    const int i = qlin_gguf_find_key(gguf, key);
+    const int type = i < 0 ? -1 : qlin_gguf_value_type(gguf, i);
+    int64_t v;
+    if ((type != 4 && type != 5) || qlin_gguf_get_i64(gguf, i, &v) != QLIN_OK) return default_val; /* u32, i32 only */
+    return (int)v;
+}
+
+float qtf_get_float(const struct qlin_gguf *gguf, const char *key, float default_val) {
+    const int i = qlin_gguf_find_key(gguf, key);
+    double v;
+    if (i < 0 || qlin_gguf_value_type(gguf, i) != 6 || qlin_gguf_get_f64(gguf, i, &v) != QLIN_OK) return default_val;
+    return (float)v;
+}
+
 static size_t tensor_bytes(const qtensor *t) {
     return (size_t)t->n_rows * qtf_row_bytes(t->type, t->n_cols);
 }

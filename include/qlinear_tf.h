@@ -22,6 +22,8 @@
  *   qtf_qmatvec_expert_pool      tf_qmatvec_expert_pool        :1136-1158
  *   qtf_gemm_tokenmajor          tf_gemm_f16_mt_tokenmajor     :4487-4595
  *   qtf_moe_ffn                  the MoE FFN block             :4045-4131
+ *   qtf_load_tensor              tf_load_tensor                :363-381
+ *   qtf_get_int / qtf_get_float  tf_get_int / tf_get_float     :383-396
  *   qtf_register_tensor          (upload once; the reference maps the file and never copies)
  *
  * Differences, all on the caller's side of the boundary:
@@ -53,6 +55,17 @@ typedef struct {
     float    scale;      /* carried, never applied (the reference's CPU path does not read it either) */
     int      has_scale;
 } qtensor;
+
+/* an open model file (include/qlinear.h: qlin_gguf_open / qlin_gguf_upload) */
+struct qlin_gguf;
+/* the qtensor of a named tensor: data = its address in the mapped file (registered with the GPU copy
+ * once qlin_gguf_upload has run), n_cols = dims[0], n_rows = product of the other dims; data == NULL
+ * if the tensor is missing (with a message on stderr when `required`)
+ *                                tf_load_tensor, common/transformer.h:363-381 */
+qtensor qtf_load_tensor(const struct qlin_gguf *gguf, const char *name, int required);
+/* u32/i32 and f32 values with a default   tf_get_int, tf_get_float, common/transformer.h:383-396 */
+int    qtf_get_int(const struct qlin_gguf *gguf, const char *key, int default_val);
+float  qtf_get_float(const struct qlin_gguf *gguf, const char *key, float default_val);
 
 size_t qtf_row_bytes(uint32_t type, int n_cols);
 int    qtf_is_supported_weight_type(uint32_t type);

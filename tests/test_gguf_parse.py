@@ -210,3 +210,33 @@ def test_damaged_headers_are_refused(tmp_path):
         assert g.rc != 0, what
         g.close()
     assert Gguf(tmp_path / "does_not_exist.gguf").rc == qlinear.ERR_ARG
+
+
+def test_reference_shaped_loader_calls(tiny, manifest):
+    """qtf_load_tensor / qtf_get_int / qtf_get_float of the reference-named layer against what
+    tf_load_tensor / tf_get_int read from the same file"""
+    from gemm_amd import build
+
+    class QTensor(C.Structure):
+        _fields_ = [("data", C.c_void_p), ("type", C.c_uint32), ("n_rows", C.c_int), ("n_cols", C.c_int),
+                    ("n_dims", C.c_int), ("dims", C.c_uint64 * 4), ("scale", C.c_float), ("has_scale", C.c_int)]
+    if not os.path.exists(build.TF_LIB):
+        build.build_host(verbose=False)
+    tf = C.CDLL(build.TF_LIB)
+    tf.qtf_load_tensor.restype = QTensor
+    tf.qtf_load_tensor.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
+    tf.qtf_get_int.argtypes = [C.c_void_p, C.c_char_p, C.c_int]
+    tf.qtf_get_float.restype = C.c_float
+    tf.qtf_get_float.argtypes = [C.c_void_p, C.c_char_p, C.c_float]
+    ref = manifest["gguf_fixture"]
+    base = tiny.lib.qlin_gguf_tensor_host(tiny.h, 0) - ref["tensors"][0]["offset"]
+    for want in ref["tensors"]:
+        t = tf.qtf_load_tensor(tiny.h, want["name"].encode(), 1)
+        q = want["qtensor"]
+        assert (t.type, t.n_rows, t.n_cols, t.n_dims) == (q["type"], q["n_rows"], q["n_cols"], q["n_dims"])
+        assert t.data - base == q["data_offset"] and list(t.dims) == want["dims"]
+    assert tf.qtf_load_tensor(tiny.h, b"missing", 0).data is None
+    for key, want in ref["tf_get_int"].items():
+        assert tf.qtf_get_int(tiny.h, key.encode(), -7) == want, key
+    assert tf.qtf_get_float(tiny.h, b"qwen3.rope.freq_base", 0.0) == 1000000.0
+    assert tf.qtf_get_float(tiny.h, b"some.f64", 3.0) == 3.0  # f32 only, like the reference
