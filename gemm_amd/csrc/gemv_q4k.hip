@@ -54,21 +54,6 @@ constexpr int kRowImage = 2304;     /* bytes per LDS row image: 16 super-blocks 
 constexpr int kMaxDepth = Q4K_MAX_DEPTH; /* row images per wavefront */
 constexpr int kMaxRowsPerWg = 128;
 
-template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
-__device__ __forceinline__ float lane_value(float v, int lane) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
-}
-/* sum over the 64 lanes with cross-lane data-path moves (no LDS round trips); uniform result */
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-    v += dpp_mov<0xB1>(v);  /* quad_perm [1,0,3,2] */
-    v += dpp_mov<0x4E>(v);  /* quad_perm [2,3,0,1] */
-    v += dpp_mov<0x141>(v); /* row_half_mirror */
-    v += dpp_mov<0x140>(v); /* row_mirror: every lane of a 16-lane row now holds the row total */
-    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
-}
-
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 __device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_udot4(a, b, c, false); }
 

@@ -539,7 +539,7 @@ gemv_stream_kernel(const JobView job, const float *__restrict__ x, int n_cols, i
             issue(issued);
             issued++;
         }
-        const float s = wave_sum(acc);
+        const float s = wave_sum_dpp(acc);
         const uint8_t *Wm;
         float *ym;
         int r;

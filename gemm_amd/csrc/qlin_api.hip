@@ -154,8 +154,9 @@ int weights_on_device_locked(const void *host, size_t bytes, DevBuf &buf, const 
     return QLIN_OK;
 }
 
-/* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the streaming kernel,
- * else (ragged or oversized shapes, unaligned pointers) the plain kernel */
+/* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the integer-dot kernel
+ * (formats with small integer codes), else the streaming float kernel, else (ragged or oversized
+ * shapes, unaligned pointers) the plain kernel */
 hipError_t dispatch_gemv_job(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t s) {
     if ((job.mode == kSiluMul ? job.n_rows[0] : job.total_rows()) == 0) return hipSuccess;
     bool w_aligned = true;
@@ -163,6 +164,7 @@ hipError_t dispatch_gemv_job(uint32_t type, const GemvJob &job, const float *x, 
     if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && w_aligned && aligned(x, 16))
         return launch_gemv_q4k(job, x, n_cols, s, g.n_cu);
     hipError_t err;
+    if (launch_gemv_int(type, job, x, n_cols, g.n_cu, s, &err)) return err;
     if (launch_gemv_stream(type, job, x, n_cols, g.n_cu, s, &err)) return err;
     return launch_gemv_generic(type, job, x, n_cols, s);
 }

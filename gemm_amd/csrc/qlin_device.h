@@ -305,6 +305,21 @@ __device__ __forceinline__ void wait_vm_at_most(int n) {
     }
 }
 
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+/* sum over the 64 lanes with cross-lane data-path moves (no LDS round trips); uniform result */
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    v += dpp_mov<0xB1>(v);  /* quad_perm [1,0,3,2] */
+    v += dpp_mov<0x4E>(v);  /* quad_perm [2,3,0,1] */
+    v += dpp_mov<0x141>(v); /* row_half_mirror */
+    v += dpp_mov<0x140>(v); /* row_mirror: every lane of a 16-lane row now holds the row total */
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
+}
+
 /* Kernel-side view of one fused matvec launch: up to three matrices of one block type that share
  * x (host-side GemvJob, flattened so that nothing is indexed dynamically). mode 0: y = W.x,
  * 1: y += W.x, 2: y0 = silu(W0.x) * (W1.x) with n0 == n1. */

@@ -55,6 +55,9 @@ hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x
  * hold (nothing was launched), else true with the launch status in *err */
 bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
                         hipStream_t stream, hipError_t *err);
+/* integer-dot matvec (gemv_int.hip) for the formats it covers; same contract as launch_gemv_stream */
+bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
+                     hipStream_t stream, hipError_t *err);
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu);
 
