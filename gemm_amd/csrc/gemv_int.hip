@@ -426,7 +426,7 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
         for (int c0 = 0; c0 < n_chunks; c0 += 64) {
             const uint32_t m0v = __builtin_amdgcn_readfirstlane(img + 16u * (uint32_t)c0);
             if (c0 + lane < n_chunks)
-                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
                              : : "v"(gp + c0 + lane), "s"(m0v) : "memory");
         }
     };

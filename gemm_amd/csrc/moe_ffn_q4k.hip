@@ -221,7 +221,7 @@ __device__ __forceinline__ void image_from_global(uint8_t *img, const uint8_t *m
                              (size_t)sb * kQ4KBlock + 16 * c9;
         const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
         if (t < kChunks)
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0v) : "memory");
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" : : "v"(src), "s"(m0v) : "memory");
     }
 }
 
