@@ -114,6 +114,58 @@ def time_fused(steps):
     return out
 
 
+def time_decode_step_linear(n_layers=32, steps=5):
+    """The block-quantized linear operators of one decode step of a Llama-3-8B-shaped model (hidden
+    4096, FFN 14336, 32 query / 8 KV heads of 128, vocabulary 128256), all Q4_K except a Q6_K output
+    projection, each layer with its own weights (3.6 GB in all), as 4 launches per layer + 2:
+    Q/K/V in one launch, attention output + residual, gate+up+SiLU, down + residual; then the output
+    projection with the greedy pick. Attention, norms and RoPE are outside this library and not run.
+    -> dict"""
+    K, FF, KV, V = 4096, 14336, 1024, 128256
+    Q6K = synth.GGML_Q6_K
+
+    def dev(tid, rows, cols, seed):
+        return qlinear.DevBuf.from_numpy(synth.make_weights(tid, rows, cols, seed=seed))
+
+    # one set of host tensors, uploaded once per layer (the values do not matter for timing)
+    hq, hk, hv = (synth.make_weights(Q4K, r, K, seed=61 + i) for i, r in enumerate((K, KV, KV)))
+    ho, hg, hu = (synth.make_weights(Q4K, r, K, seed=64 + i) for i, r in enumerate((K, FF, FF)))
+    hd = synth.make_weights(Q4K, K, FF, seed=67)
+    layers = [[qlinear.DevBuf.from_numpy(h) for h in (hq, hk, hv, ho, hg, hu, hd)] for _ in range(n_layers)]
+    Wout = dev(Q6K, V, K, 68)
+    x = qlinear.DevBuf.from_numpy(synth.make_activation(K, seed=5) * np.float32(0.05))
+    q, k, v = qlinear.DevBuf(K * 4), qlinear.DevBuf(KV * 4), qlinear.DevBuf(KV * 4)
+    h = qlinear.DevBuf(FF * 4)
+    logits, pick = qlinear.DevBuf(V * 4), qlinear.DevBuf(qlinear.ARGMAX_RESULT_BYTES)
+
+    def step():
+        for Wq, Wk, Wv, Wo, Wg, Wu, Wd in layers:
+            qlinear.gemv_multi_dev(Q4K, [Wq, Wk, Wv], [q, k, v], [K, KV, KV], x, K)
+            qlinear.gemv_add_dev(Q4K, Wo, q, x, K, K)             # attention output (stand-in input: q) + residual
+            qlinear.gemv_silu_mul_dev(Q4K, Wg, Wu, x, h, FF, K)
+            qlinear.gemv_add_dev(Q4K, Wd, h, x, K, FF)
+        qlinear.gemv_argmax_dev(Q6K, Wout, x, logits, pick, V, K)
+
+    step()
+    qlinear.sync()
+    t_host = time.time()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        step()
+    host_ms = (time.time() - t_host) * 1e3 / steps  # time to enqueue one step from Python
+    ms = qlinear.timer_end() / steps
+    weight_bytes = n_layers * sum(a.nbytes for a in (hq, hk, hv, ho, hg, hu, hd)) + V * synth.row_bytes(Q6K, K)
+    for bufs in layers:
+        for d in bufs:
+            d.free()
+    for d in (Wout, x, q, k, v, h, logits, pick):
+        d.free()
+    return {"ms_per_token": round(ms, 4), "host_enqueue_ms": round(host_ms, 4), "launches": 4 * n_layers + 3,
+            "weight_bytes": weight_bytes,
+            "GB/s": round(weight_bytes / (ms * 1e-3) / 1e9, 1),
+            "hbm_frac": round(weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+
+
 def time_gemm(n_tok, n_rows, n_cols, steps, warmup):
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=31)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=32, tokens=n_tok))
@@ -252,6 +304,8 @@ def probe(args):
             qlinear.dequant_dev(Q4K, dW, dO, 14336, 4096)
         qlinear.sync()
         print(json.dumps({"probe": args.probe}))
+    elif args.probe == "decode_step":
+        print(json.dumps({"probe": args.probe, **time_decode_step_linear()}))
     elif args.probe == "moe":
         m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
         print(json.dumps({"probe": "moe", "ms_per_step": m, "bytes": b, "routed": routed}))
@@ -267,7 +321,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "moe"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
@@ -318,6 +372,8 @@ def main():
             other[tname] = {"us": round(m * 1e3, 2), "GB/s": round(b / (m * 1e-3) / 1e9, 1)}
         extra["gemv_14336x4096_all_formats"] = other
         extra["q4k_fused_decode_shapes"] = time_fused(max(20, args.steps // 8))
+
+        extra["q4k_llama8b_shaped_decode_step_linear_ops"] = time_decode_step_linear()
 
         hb = time_host_boundary(n_rows, n_cols)
         extra["host_pointer_matvec_14336x4096"] = {"us": round(hb * 1e3, 1), "GB/s": round(nbytes / (hb * 1e-3) / 1e9, 1),
