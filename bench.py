@@ -138,13 +138,13 @@ def time_decode_step_linear(n_layers=32, steps=5):
     h = qlinear.DevBuf(FF * 4)
     logits, pick = qlinear.DevBuf(V * 4), qlinear.DevBuf(qlinear.ARGMAX_RESULT_BYTES)
 
-    def step():
+    def step(stream=None):
         for Wq, Wk, Wv, Wo, Wg, Wu, Wd in layers:
-            qlinear.gemv_multi_dev(Q4K, [Wq, Wk, Wv], [q, k, v], [K, KV, KV], x, K)
-            qlinear.gemv_add_dev(Q4K, Wo, q, x, K, K)             # attention output (stand-in input: q) + residual
-            qlinear.gemv_silu_mul_dev(Q4K, Wg, Wu, x, h, FF, K)
-            qlinear.gemv_add_dev(Q4K, Wd, h, x, K, FF)
-        qlinear.gemv_argmax_dev(Q6K, Wout, x, logits, pick, V, K)
+            qlinear.gemv_multi_dev(Q4K, [Wq, Wk, Wv], [q, k, v], [K, KV, KV], x, K, stream)
+            qlinear.gemv_add_dev(Q4K, Wo, q, x, K, K, stream)     # attention output (stand-in input: q) + residual
+            qlinear.gemv_silu_mul_dev(Q4K, Wg, Wu, x, h, FF, K, stream)
+            qlinear.gemv_add_dev(Q4K, Wd, h, x, K, FF, stream)
+        qlinear.gemv_argmax_dev(Q6K, Wout, x, logits, pick, V, K, stream)
 
     step()
     qlinear.sync()
@@ -155,12 +155,34 @@ def time_decode_step_linear(n_layers=32, steps=5):
     host_ms = (time.time() - t_host) * 1e3 / steps  # time to enqueue one step from Python
     ms = qlinear.timer_end() / steps
     weight_bytes = n_layers * sum(a.nbytes for a in (hq, hk, hv, ho, hg, hu, hd)) + V * synth.row_bytes(Q6K, K)
+    # the same step captured once into a HIP graph and replayed (the entry points only enqueue kernels)
+    hip = ctypes.CDLL("libamdhip64.so")
+    stream, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    graph_ms = None
+    if hip.hipStreamCreate(ctypes.byref(stream)) == 0:
+        ok = hip.hipStreamBeginCapture(stream, 0) == 0
+        if ok:
+            step(stream)
+            ok = hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+        ok = ok and hip.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, ctypes.c_size_t(0)) == 0
+        if ok:
+            hip.hipGraphLaunch(gexec, stream)
+            qlinear.sync(stream)
+            qlinear.timer_begin(stream)
+            for _ in range(steps):
+                hip.hipGraphLaunch(gexec, stream)
+            graph_ms = qlinear.timer_end(stream) / steps
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        hip.hipStreamDestroy(stream)
     for bufs in layers:
         for d in bufs:
             d.free()
     for d in (Wout, x, q, k, v, h, logits, pick):
         d.free()
-    return {"ms_per_token": round(ms, 4), "host_enqueue_ms": round(host_ms, 4), "launches": 4 * n_layers + 3,
+    return {"ms_per_token": round(ms, 4), "host_enqueue_ms": round(host_ms, 4),
+            "ms_per_token_graph_replay": None if graph_ms is None else round(graph_ms, 4), "launches": 4 * n_layers + 3,
             "weight_bytes": weight_bytes,
             "GB/s": round(weight_bytes / (ms * 1e-3) / 1e9, 1),
             "hbm_frac": round(weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}

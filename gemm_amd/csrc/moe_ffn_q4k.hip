@@ -316,14 +316,17 @@ __device__ __forceinline__ TileElem tile_elem(int idx) {
 }
 
 /* ---- 2. gate and up for RT * 16 rows of one expert, all of its tokens ---- */
-#ifndef MOE_WAVES
-#define MOE_WAVES 2
+#ifndef MOE_GU_WAVES
+#define MOE_GU_WAVES 2
+#endif
+#ifndef MOE_DN_WAVES
+#define MOE_DN_WAVES 2
 #endif
 #ifndef MOE_GU_RT
 #define MOE_GU_RT 1
 #endif
 template <int RT>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_GU_WAVES)))
 moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
                    const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
                    const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
@@ -372,7 +375,7 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
 }
 
 /* ---- 3. down for 32 rows of one expert ---- */
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                 const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
                 const int32_t *__restrict__ order, const float *__restrict__ expert_w, float *__restrict__ part,
