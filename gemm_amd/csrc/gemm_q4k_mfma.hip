@@ -18,13 +18,20 @@
  * copies 4 x 16 bytes of activations into an LDS ring of three stages; the MFMA operands of a
  * tile are fetched from LDS half a tile ahead of the MFMAs that use them, the decode of tile
  * i+2 is issued in the shadow of the MFMAs of tile i, and global loads run four tiles ahead
- * (two register sets). One barrier per tile.
+ * (two register sets). One barrier per tile. When 128-row tiles would leave compute units
+ * without a workgroup (few tokens, or few rows) the same kernel runs with BN = 64: 4 x 2 waves
+ * of 64 tokens x 32 rows, eight 4-byte weight parts per row (M = 128: 66 -> 55 us).
  *
- * Measured on MI355X at M=512, N=14336, K=4096: 78 us, 0.77 PFLOP/s. Taking pieces out of the
- * loop shows what is left to win: MFMAs + barriers alone 41 us (the matrix pipe idles about
- * 500 cycles around every barrier), + operand fetches 53 us, + decode and LDS stores 78 us: the
- * three pipes (matrix, LDS, vector ALU) each need about 1000 cycles per tile and overlap only
- * partly with two waves per SIMD that are re-aligned by a barrier every tile.
+ * Measured on MI355X at M=512, N=14336, K=4096: 76-78 us, 0.78 PFLOP/s on 224 of 256 compute
+ * units. Cycle stamps (s_memtime) around the parts of one tile show a tile of about 1920 cycles
+ * at a shader clock of 1.75-1.9 GHz under this load (2.0-2.1 GHz in a light kernel), against
+ * 1024 cycles of matrix-pipe work per SIMD: the eight operand fetches that follow the barrier
+ * take 350-450 cycles to issue for the first wave of each SIMD and 650-750 for the second
+ * (about 45 cycles per ds_read_b128 and SIMD, twice what the same access pattern costs in a loop
+ * of nothing but reads), the second wave stays that far behind through the tile, and the first
+ * wave waits 600-700 cycles at the barrier. Matrix pipe, vector ALU and LDS are each busy about
+ * half of the time (SQ counters). Orders that were measured and were not faster: MFMAs ahead of
+ * the fetches, one fetch per MFMA, four MFMAs then the fetches then the rest.
  *
  * Both MFMA operands are read from LDS with the same [row][k] indexing, so the result does
  * not depend on which k a given lane/element position feeds inside the instruction.
@@ -40,7 +47,6 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef float float2v __attribute__((ext_vector_type(2)));
 
-constexpr int kBN = 128;        /* weight rows per workgroup */
 constexpr int kBK = 64;         /* k per step */
 constexpr int kRow = 136;       /* average bytes per LDS tile row: pairs of 128-byte rows + 16 bytes */
 constexpr int kStages = 3;      /* LDS ring depth */
@@ -83,18 +89,27 @@ __device__ __forceinline__ uint4 decode8(uint32_t n0, uint32_t n1, float dl, flo
     return r;
 }
 
+/* 4 nibbles of one dword -> 4 decoded weights as 2 bf16 pairs */
+__device__ __forceinline__ uint2 decode4(uint32_t n0, float dl, float ml) {
+    const float2v a = fp8_pair_lo(n0), b = fp8_pair_hi(n0);
+    return make_uint2(pack_bf16(fmaf(a.x, dl, -ml), fmaf(a.y, dl, -ml)), pack_bf16(fmaf(b.x, dl, -ml), fmaf(b.y, dl, -ml)));
+}
+
 }  // namespace
 
-template <int WM>
+/* NB = 2: 128 weight rows per workgroup (wave tile 64 tokens x 64 rows); NB = 1: 64 weight rows (wave
+ * tile 64 x 32) and twice as many workgroups, for shapes whose grid would not fill the chip */
+template <int WM, int NB>
 __global__ void __launch_bounds__(128 * WM)
 gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y,
                      int n_rows, int n_sb, int n_tok, int ldx, int ldy, int m_tiles) {
     constexpr int BM = 64 * WM, NT = 128 * WM;
     static_assert(NT == 512, "one weight-row part per thread: 512 threads");
-    constexpr int kATile = BM * kRow, kBTile = kBN * kRow;
+    constexpr int BN = 64 * NB;
+    constexpr int kATile = BM * kRow, kBTile = BN * kRow;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t *As = lds;                      /* [kStages][BM][kRow]  */
-    uint8_t *Bs = lds + kStages * kATile;   /* [kStages][kBN][kRow] */
+    uint8_t *Bs = lds + kStages * kATile;   /* [kStages][BN][kRow]  */
 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int wm = wv >> 1, wn = wv & 1;
@@ -105,12 +120,13 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int tile_m = slot % m_tiles;
     const int tile_n = (slot / m_tiles) * 8 + xcd;
-    if (tile_n * kBN >= n_rows) return;
+    if (tile_n * BN >= n_rows) return;
 
     const size_t row_bytes = (size_t)n_sb * 144;
-    /* B-tile role: weight row br, 8-byte part bp of the 32 nibble bytes of a sub-block pair */
-    const int br = tid >> 2, bp = tid & 3;
-    int w_row = tile_n * kBN + br;
+    /* B-tile role: weight row br, part bp of the 32 nibble bytes of a sub-block pair (NB = 2: four
+     * 8-byte parts per row, NB = 1: eight 4-byte parts) */
+    const int br = NB == 2 ? tid >> 2 : tid >> 3, bp = NB == 2 ? tid & 3 : tid & 7;
+    int w_row = tile_n * BN + br;
     if (w_row >= n_rows) w_row = n_rows - 1;
     const uint8_t *w_ptr = W + (size_t)w_row * row_bytes;
     /* A-tile role: chunks (token row ar + 64j, 16-byte column ac), j = 0..3 */
@@ -131,7 +147,8 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
         const int sb = step >> 2, c = step & 3;
         const uint8_t *blk = w_ptr + (size_t)sb * 144;
         r.hdr = *reinterpret_cast<const uint4 *>(blk);
-        r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * bp);
+        if (NB == 2) r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * bp);
+        else r.qs = make_uint2(*reinterpret_cast<const uint32_t *>(blk + 16 + 32 * c + 4 * bp), 0u);
         r.x0 = x_chunk(0, step); r.x1 = x_chunk(1, step); r.x2 = x_chunk(2, step); r.x3 = x_chunk(3, step);
     };
 
@@ -150,9 +167,15 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
         const float ml_a = dmin * (float)(mn2 & 0xFFu), ml_b = dmin * (float)((mn2 >> 8) & 0xFFu);
         uint8_t *bt = Bs + st * kBTile;
         /* sub-block 2c (low nibbles) -> k 0..31 = chunks 0..3, sub-block 2c+1 -> chunks 4..7 */
-        *reinterpret_cast<uint4 *>(bt + swz(br, bp)) = decode8(r.qs.x & 0x0F0F0F0Fu, r.qs.y & 0x0F0F0F0Fu, dl_a, ml_a);
-        *reinterpret_cast<uint4 *>(bt + swz(br, 4 + bp)) =
-            decode8((r.qs.x >> 4) & 0x0F0F0F0Fu, (r.qs.y >> 4) & 0x0F0F0F0Fu, dl_b, ml_b);
+        if (NB == 2) {
+            *reinterpret_cast<uint4 *>(bt + swz(br, bp)) = decode8(r.qs.x & 0x0F0F0F0Fu, r.qs.y & 0x0F0F0F0Fu, dl_a, ml_a);
+            *reinterpret_cast<uint4 *>(bt + swz(br, 4 + bp)) =
+                decode8((r.qs.x >> 4) & 0x0F0F0F0Fu, (r.qs.y >> 4) & 0x0F0F0F0Fu, dl_b, ml_b);
+        } else { /* four codes per nibble position: half a 16-byte chunk each */
+            *reinterpret_cast<uint2 *>(bt + swz(br, bp >> 1) + 8 * (bp & 1)) = decode4(r.qs.x & 0x0F0F0F0Fu, dl_a, ml_a);
+            *reinterpret_cast<uint2 *>(bt + swz(br, 4 + (bp >> 1)) + 8 * (bp & 1)) =
+                decode4((r.qs.x >> 4) & 0x0F0F0F0Fu, dl_b, ml_b);
+        }
     };
     auto stage_acts = [&](const StepRegs &r, int st) {
         uint8_t *at = As + st * kATile;
@@ -169,35 +192,35 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     /* operand fragments of two k-steps (half a tile): 2 x (2 A + 2 B) x 8 bf16 */
     struct Frags { bf16x8 a0, a1, b0, b1, c0, c1, d0, d1; };
     const int frag_row = lane & 31, kg = lane >> 5;
-    const int a_row = wm * 64 + frag_row, b_row = wn * 64 + frag_row;
+    const int a_row = wm * 64 + frag_row, b_row = wn * (32 * NB) + frag_row;
     auto load_frags = [&](Frags &f, int st, int half) {
         const uint8_t *at = As + st * kATile, *bt = Bs + st * kBTile;
         const int ch0 = 4 * half + kg, ch1 = ch0 + 2; /* logical chunks of k-steps 2*half, 2*half+1 */
         f.a0 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row, ch0));
         f.a1 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row + 32, ch0));
         f.b0 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row, ch0));
-        f.b1 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row + 32, ch0));
+        if (NB == 2) f.b1 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row + 32, ch0));
         f.c0 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row, ch1));
         f.c1 = *reinterpret_cast<const bf16x8 *>(at + swz(a_row + 32, ch1));
         f.d0 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row, ch1));
-        f.d1 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row + 32, ch1));
+        if (NB == 2) f.d1 = *reinterpret_cast<const bf16x8 *>(bt + swz(b_row + 32, ch1));
     };
     auto mma_half = [&](const Frags &f) {
         acc00 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a0, f.b0, acc00, 0, 0, 0);
-        acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a0, f.b1, acc01, 0, 0, 0);
+        if (NB == 2) acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a0, f.b1, acc01, 0, 0, 0);
         acc10 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a1, f.b0, acc10, 0, 0, 0);
-        acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a1, f.b1, acc11, 0, 0, 0);
+        if (NB == 2) acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a1, f.b1, acc11, 0, 0, 0);
         acc00 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c0, f.d0, acc00, 0, 0, 0);
-        acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c0, f.d1, acc01, 0, 0, 0);
+        if (NB == 2) acc01 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c0, f.d1, acc01, 0, 0, 0);
         acc10 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c1, f.d0, acc10, 0, 0, 0);
-        acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c1, f.d1, acc11, 0, 0, 0);
+        if (NB == 2) acc11 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c1, f.d1, acc11, 0, 0, 0);
     };
 
     /* ask the instruction scheduler for "one MFMA, then a few vector-ALU instructions" eight
      * times over, so that the decode arithmetic is issued in the shadow of the MFMAs of the same
      * wave instead of in front of them */
 #define QLIN_INTERLEAVE_8(VALU_PER_MFMA)                                  \
-    _Pragma("unroll") for (int q_ = 0; q_ < 8; q_++) {                    \
+    _Pragma("unroll") for (int q_ = 0; q_ < 4 * NB; q_++) {               \
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                \
         __builtin_amdgcn_sched_group_barrier(0x002, VALU_PER_MFMA, 0);    \
     }
@@ -266,7 +289,7 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     /* C layout of the 32x32 MFMA: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4,
      * column l%32. Columns are weight rows, contiguous in the token-major output. */
     auto store_tile = [&](const floatx16 &acc, int mi, int ni) {
-        const int n = tile_n * kBN + wn * 64 + ni * 32 + (lane & 31);
+        const int n = tile_n * BN + wn * (32 * NB) + ni * 32 + (lane & 31);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const int m = tile_m * BM + wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
@@ -274,31 +297,46 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
         }
     };
     store_tile(acc00, 0, 0);
-    store_tile(acc01, 0, 1);
     store_tile(acc10, 1, 0);
-    store_tile(acc11, 1, 1);
+    if (NB == 2) {
+        store_tile(acc01, 0, 1);
+        store_tile(acc11, 1, 1);
+    }
 }
 
-hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
-                                int n_tok, int ldx, int ldy, hipStream_t stream) {
+namespace {
+
+template <int NB>
+hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok, int ldx,
+                        int ldy, hipStream_t stream) {
     static bool lds_raised = false;
-    constexpr int WM = 4, BM = 64 * WM;
+    constexpr int WM = 4, BM = 64 * WM, BN = 64 * NB;
     const int n_sb = n_cols / 256;
     const int m_tiles = (n_tok + BM - 1) / BM;
-    const int n_tiles = (n_rows + kBN - 1) / kBN;
+    const int n_tiles = (n_rows + BN - 1) / BN;
     /* ids are dealt to 8 XCDs; pad the n-tile count to a multiple of 8 (surplus groups exit) */
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const int grid = n_tiles_pad * m_tiles;
-    const size_t lds_bytes = (size_t)kStages * (BM + kBN) * kRow;
+    const size_t lds_bytes = (size_t)kStages * (BM + BN) * kRow;
     if (!lds_raised) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemm_q4k_bf16_kernel<WM>,
+        hipError_t e = hipFuncSetAttribute((const void *)gemm_q4k_bf16_kernel<WM, NB>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         lds_raised = true;
     }
-    hipLaunchKernelGGL((gemm_q4k_bf16_kernel<WM>), dim3(grid), dim3(128 * WM), lds_bytes, stream,
+    hipLaunchKernelGGL((gemm_q4k_bf16_kernel<WM, NB>), dim3(grid), dim3(128 * WM), lds_bytes, stream,
                        (const uint8_t *)W, X, Y, n_rows, n_sb, n_tok, ldx, ldy, m_tiles);
     return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                                int n_tok, int ldx, int ldy, hipStream_t stream) {
+    /* 128-row tiles unless they would leave compute units without a workgroup */
+    const int m_tiles = (n_tok + 255) / 256, n_tiles_128 = (n_rows + 127) / 128;
+    if (m_tiles * n_tiles_128 < 200) return launch_tiled<1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    return launch_tiled<2>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
 }
 
 }  // namespace qlin

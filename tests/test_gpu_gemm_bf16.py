@@ -42,6 +42,7 @@ def references(oracle, W, Xb, n_cols):
 @pytest.mark.parametrize("n_tok,n_rows,n_cols", [
     (1, 128, 256), (7, 130, 512), (64, 256, 1024), (128, 384, 4096), (256, 128, 4096),
     (300, 257, 2048), (512, 1024, 4096), (33, 1000, 768),
+    (260, 12805, 256), (1030, 5130, 512),  # enough tiles for the 128-row variant of the kernel
 ])
 def test_gemm_bf16_shapes(oracle, n_tok, n_rows, n_cols):
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=n_rows + n_tok)
