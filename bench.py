@@ -336,6 +336,36 @@ def probe(args):
         print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
 
 
+def time_achievable():
+    """What the part sustains on the two priced resources: a register-only loop of the GEMM's matrix
+    instruction (with the shader clock it ran at) and a streaming read of 512 MiB / of the headline's
+    33 MB, both timed with the same event timer as the kernels."""
+    out = {}
+    qlinear.probe_mfma_bf16(2000); qlinear.sync()
+    best = 0.0
+    for _ in range(3):
+        qlinear.timer_begin()
+        fl = qlinear.probe_mfma_bf16(20000)
+        ms = qlinear.timer_end()
+        best = max(best, fl / (ms * 1e-3) / 1e12)
+    out["mfma_bf16_32x32x16_register_loop_TFLOP/s"] = round(best, 1)
+    out["shader_clock_MHz_in_that_loop"] = round(qlinear.probe_clocks(), 0)
+    for label, nbytes, reps in (("hbm_read_512MiB_GB/s", 512 << 20, 10), ("hbm_read_33MB_rotating_GB/s", 33030144, 40)):
+        copies = 1 if nbytes > (256 << 20) else 11
+        bufs = [qlinear.DevBuf(nbytes) for _ in range(copies)]
+        for b in bufs:
+            qlinear.probe_hbm_read(b)
+        qlinear.sync()
+        qlinear.timer_begin()
+        for i in range(reps):
+            qlinear.probe_hbm_read(bufs[i % copies])
+        ms = qlinear.timer_end() / reps
+        out[label] = round(nbytes / (ms * 1e-3) / 1e9, 1)
+        for b in bufs:
+            b.free()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -380,6 +410,7 @@ def main():
             gemm["M=%d" % M] = {"us": round(m * 1e3, 1), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}
         extra["q4k_prefill_gemm_14336x4096_bf16"] = gemm
         tf = gemm["M=512"]["TFLOP/s"]
+        extra["achievable_on_this_gpu"] = time_achievable()
         extra["q4k_prefill_gemm_roofline"] = {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS,
                                               "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),
                                               "traffic": None}

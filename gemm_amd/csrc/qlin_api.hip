@@ -798,6 +798,32 @@ int qlin_moe_ffn_dev(uint32_t type, const void *gate_exps, const void *up_exps, 
     return QLIN_OK;
 }
 
+int qlin_probe_mfma_bf16(int iters, void *stream, double *flops) {
+    if (iters <= 0 || iters > (1 << 22) || !flops) return fail(QLIN_ERR_ARG, "iters must be in 1..2^22 and flops non-null");
+    if (int rc = init_once()) return rc;
+    HIP_TRY(launch_probe_mfma(iters, g.n_cu, (hipStream_t)stream, flops));
+    return QLIN_OK;
+}
+
+int qlin_probe_clocks(void *stream, double *shader_mhz) {
+    if (!shader_mhz) return fail(QLIN_ERR_ARG, "null pointer");
+    if (int rc = init_once()) return rc;
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    uint64_t c[2] = {0, 0};
+    HIP_TRY(read_probe_clocks(c));
+    if (c[1] == 0) return fail(QLIN_ERR_ARG, "qlin_probe_mfma_bf16 has not run");
+    *shader_mhz = (double)c[0] * 100.0 / (double)c[1];
+    return QLIN_OK;
+}
+
+int qlin_probe_hbm_read(const void *buf, size_t n_bytes, void *stream) {
+    if (!buf || n_bytes < 16 || ((uintptr_t)buf & 15)) return fail(QLIN_ERR_ARG, "buffer must be 16-byte aligned and at least 16 bytes");
+    if (n_bytes / 16 / 2048 > 0x7fffffffu) return fail(QLIN_ERR_ARG, "buffer too large for one launch");
+    if (int rc = init_once()) return rc;
+    HIP_TRY(launch_probe_read(buf, n_bytes, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
 int qlin_timer_begin(void *stream) {
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;

@@ -83,6 +83,11 @@ hipError_t launch_silu_mul(float *h, const float *gate, const float *up, int n, 
  * loop `if (v[j] > v[best]) best = j` (server/server_llm.c:224-228). result holds
  * QLIN_ARGMAX_RESULT_BYTES bytes: the rest is scratch for the first stage. */
 hipError_t launch_argmax(const float *v, int n, float *result, hipStream_t stream);
+/* measurement probes (probe.hip): a register-only MFMA loop (flops issued come back in *flops) with the
+ * cycle and 100 MHz counters around it, and a streaming read of a device buffer */
+hipError_t launch_probe_mfma(int iters, int n_cu, hipStream_t stream, double *flops);
+hipError_t launch_probe_read(const void *buf, size_t n_bytes, hipStream_t stream);
+hipError_t read_probe_clocks(uint64_t out[2]);
 hipError_t launch_axpy_dev_weight(float *out, const float *q, const float *w, int widx, int n,
                                   int overwrite, hipStream_t stream);
 

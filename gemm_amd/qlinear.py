@@ -102,6 +102,9 @@ SIGNATURES = {
     "qlin_gguf_get_f64": (C.c_int, [_vp, C.c_int, _vp]),
     "qlin_gguf_get_str": (C.c_char_p, [_vp, C.c_int]),
     "qlin_gguf_get_array": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp]),
+    "qlin_probe_mfma_bf16": (C.c_int, [C.c_int, _vp, C.POINTER(C.c_double)]),
+    "qlin_probe_clocks": (C.c_int, [_vp, C.POINTER(C.c_double)]),
+    "qlin_probe_hbm_read": (C.c_int, [_vp, C.c_size_t, _vp]),
     "qlin_timer_begin": (C.c_int, [_vp]),
     "qlin_timer_end": (C.c_int, [_vp, _fp]),
 }
@@ -308,6 +311,24 @@ def moe_ffn_dev(type_id, dgate, dup, ddown, dX, didx, dw, dout, n_tok, top_k, n_
 
 def sync(stream=None):
     check(load().qlin_dev_sync(stream))
+
+
+def probe_mfma_bf16(iters, stream=None):
+    """Enqueue the register-only MFMA loop; returns the flops of the launch."""
+    flops = C.c_double(0)
+    check(load().qlin_probe_mfma_bf16(iters, stream, C.byref(flops)))
+    return flops.value
+
+
+def probe_clocks(stream=None):
+    """Shader clock (MHz) of the last probe_mfma_bf16 launch."""
+    mhz = C.c_double(0)
+    check(load().qlin_probe_clocks(stream, C.byref(mhz)))
+    return mhz.value
+
+
+def probe_hbm_read(buf, n_bytes=None, stream=None):
+    check(load().qlin_probe_hbm_read(buf.ptr, buf.nbytes if n_bytes is None else n_bytes, stream))
 
 
 def timer_begin(stream=None):
