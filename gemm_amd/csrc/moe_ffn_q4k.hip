@@ -374,38 +374,43 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
     }
 }
 
-/* ---- 3. down for 32 rows of one expert ---- */
+/* ---- 3. down for RT * 16 rows of one expert ---- */
+#ifndef MOE_DN_RT
+#define MOE_DN_RT 2
+#endif
+template <int RT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                 const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
                 const int32_t *__restrict__ order, const float *__restrict__ expert_w, float *__restrict__ part,
                 int n_embd, int n_ff) {
+    constexpr int kRows = 16 * RT;
     extern __shared__ __attribute__((aligned(16))) float red[];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
-    const int row0 = blockIdx.x * 32;
+    const int row0 = blockIdx.x * kRows;
     const int first = offsets[e], cnt = offsets[e + 1] - first;
     if (cnt == 0) return;
     const int j = lane & 15;
     const int n_sb = n_ff >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
     const uint8_t *d0 = down + ((size_t)e * n_embd + row0) * row_bytes;
-    /* LDS: red [waves][2][64][4] floats | images [waves][32 rows][144 bytes] */
-    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 512) + wv * (32 * kQ4KBlock);
+    /* LDS: red [waves][RT][64][4] floats | images [waves][RT * 16 rows][144 bytes] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * RT * 256) + wv * (kRows * kQ4KBlock);
     const bool one_sb = n_sb <= n_waves;
-    if (one_sb && wv < n_sb) image_from_global<2>(img, d0, d0, 32, row_bytes, wv, lane);
+    if (one_sb && wv < n_sb) image_from_global<RT>(img, d0, d0, kRows, row_bytes, wv, lane);
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt;
         const size_t at_a = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
         const uint16_t *const arow[2] = {h_hi + at_a, h_lo + at_a};
-        ksplit_tile<2, 2>(img, d0, d0, 32, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
+        ksplit_tile<RT, 2>(img, d0, d0, kRows, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 512; idx += blockDim.x) {
-            const TileElem t = tile_elem<2>(idx);
+        for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
+            const TileElem t = tile_elem<RT>(idx);
             float d = 0.0f;
-            for (int w = 0; w < n_waves; w++) d += red[((w * 2 + t.r) * 64 + t.lane) * 4 + t.v];
+            for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
             if (t0 + t.slot < cnt) {
                 const float w = expert_w[order[first + t0 + t.slot]];
                 part[(size_t)(first + t0 + t.slot) * n_embd + row0 + t.row] = w * d; /* w * q, as out[i] += w*q does (:4116-4127) */
@@ -452,14 +457,19 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
         if (e1 != hipSuccess) return e1;
         lds_raised = true;
     }
-    /* waves per workgroup = super-blocks of K, at most 8 */
-    const int gu_waves = n_embd / 256 < 8 ? n_embd / 256 : 8, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
+    /* waves per workgroup = super-blocks of K, at most 4 for gate/up (a wave then walks several
+     * super-blocks one after the other) and 8 for down. The gate/up kernel needs 138 registers, so a
+     * compute unit holds 12 of its waves: three 4-wave workgroups in different phases instead of one
+     * 8-wave workgroup that loads, computes and reduces with nothing beside it (75 -> 65 us). */
+    const int gu_waves = n_embd / 256 < 4 ? n_embd / 256 : 4, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
     constexpr int RT = MOE_GU_RT;
     hipLaunchKernelGGL(moe_gate_up_kernel<RT>, dim3(n_ff / (16 * RT), n_expert), dim3(64 * gu_waves),
                        (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock), stream,
                        (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
                        n_ff, top_k);
-    hipLaunchKernelGGL(moe_down_kernel, dim3(n_embd / 32, n_expert), dim3(64 * dn_waves), (size_t)dn_waves * (2 * 1024 + 32 * kQ4KBlock), stream,
+    constexpr int DRT = MOE_DN_RT;
+    hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
+                       (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
                        (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.order, w, ws.part, n_embd, n_ff);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 255) / 256), dim3(256), 0, stream, ws.part,
                        ws.slot_of, out, n_embd, top_k);
