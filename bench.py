@@ -38,7 +38,7 @@ Q4K = synth.GGML_Q4_K
 # HBM bytes moved per Q4_K 14336x4096 matvec launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # scaled by what the same counters read for a device-to-device copy of known size
 # (profiles/gemv_q4k_14336x4096.md).
-MEASURED_TRAFFIC_BYTES = 33319952
+MEASURED_TRAFFIC_BYTES = 33319932
 
 
 def gemv_bytes(type_id, n_rows, n_cols):
