@@ -75,7 +75,7 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int32_t *__restrict__ offsets,
                  int32_t *__restrict__ order, int32_t *__restrict__ slot_of) {
-    extern __shared__ int32_t lds[]; /* cnt[n_expert], cur[n_expert] */
+    extern __shared__ int32_t lds[]; /* cnt[n_expert], cur[n_expert], wave_total[16] */
     int32_t *cnt = lds, *cur = lds + n_expert;
     for (int e = threadIdx.x; e < n_expert; e += blockDim.x) cnt[e] = 0;
     __syncthreads();
@@ -84,14 +84,33 @@ moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int
         if (e >= 0 && e < n_expert) atomicAdd(&cnt[e], 1);
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        int run = 0;
-        for (int e = 0; e < n_expert; e++) {
-            offsets[e] = run;
-            cur[e] = run;
-            run += cnt[e];
+    /* exclusive prefix sum of cnt[] over the workgroup: a thread owns `per` consecutive experts, the
+     * threads' sums are scanned inside each wave by shuffles and the 16 wave totals by every thread */
+    {
+        const int per = (n_expert + (int)blockDim.x - 1) / (int)blockDim.x;
+        const int e0 = threadIdx.x * per;
+        int mine = 0;
+        for (int q = 0; q < per; q++) mine += (e0 + q < n_expert) ? cnt[e0 + q] : 0;
+        const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+        int incl = mine;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += up;
         }
-        offsets[n_expert] = run;
+        int32_t *wave_total = lds + 2 * n_expert; /* [16] */
+        if (lane == 63) wave_total[wv] = incl;
+        __syncthreads();
+        int run = incl - mine;
+        for (int w = 0; w < wv; w++) run += wave_total[w];
+        for (int q = 0; q < per; q++) {
+            if (e0 + q < n_expert) {
+                offsets[e0 + q] = run;
+                cur[e0 + q] = run;
+                run += cnt[e0 + q];
+            }
+        }
+        if (threadIdx.x == blockDim.x - 1) offsets[n_expert] = run;
     }
     __syncthreads();
     for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
@@ -425,14 +444,22 @@ __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of, float *__restrict__ out,
                    int n_embd, int top_k) {
     const int t = blockIdx.x;
-    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+    const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
     if (c >= n_embd) return;
     float4 s = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    for (int k = 0; k < top_k; k++) {
-        const int slot = slot_of[t * top_k + k];
-        if (slot < 0) continue;
-        const float4 p = *(const float4 *)(part + (size_t)slot * n_embd + c);
-        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+    /* eight experts at a time: their slots, then their rows, are requested together; the additions stay in k order */
+    for (int k0 = 0; k0 < top_k; k0 += 8) {
+        int slot[8];
+        float4 p[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) slot[q] = k0 + q < top_k ? slot_of[t * top_k + k0 + q] : -1;
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            p[q] = slot[q] >= 0 ? *(const float4 *)(part + (size_t)slot[q] * n_embd + c) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            if (slot[q] >= 0) { s.x += p[q].x; s.y += p[q].y; s.z += p[q].z; s.w += p[q].w; }
+        }
     }
     *(float4 *)(out + (size_t)t * n_embd + c) = s;
 }
@@ -448,7 +475,7 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
                               int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream) {
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)n_expert * 2 * sizeof(int32_t), stream, idx,
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), ((size_t)n_expert * 2 + 16) * sizeof(int32_t), stream, idx,
                        n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of);
     static bool lds_raised = false;
     if (!lds_raised) {
@@ -471,7 +498,7 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
     hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
                        (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
                        (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.order, w, ws.part, n_embd, n_ff);
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 255) / 256), dim3(256), 0, stream, ws.part,
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 63) / 64), dim3(64), 0, stream, ws.part,
                        ws.slot_of, out, n_embd, top_k);
     return hipGetLastError();
 }
