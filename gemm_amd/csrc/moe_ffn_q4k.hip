@@ -48,6 +48,7 @@ struct Workspace {
     int32_t *offsets;  /* [n_expert + 1] first slot of each expert */
     int32_t *order;    /* [n_pairs] slot -> pair (t*top_k + k), grouped by expert */
     int32_t *slot_of;  /* [n_pairs] pair -> slot, -1 for an expert index out of range */
+    float *w_slot;     /* [n_pairs] routing weight of the pair in each slot */
     uint16_t *h_hi;    /* [n_pairs, n_ff] bf16 head of silu(g)*u, by slot */
     uint16_t *h_lo;    /* [n_pairs, n_ff] bf16 tail */
     float *part;       /* [n_pairs, n_embd] w * down(h), by slot */
@@ -64,6 +65,7 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
     w.offsets = (int32_t *)(p + off); off += round256(((size_t)n_expert + 1) * 4);
     w.order = (int32_t *)(p + off);   off += round256(n_pairs * 4);
     w.slot_of = (int32_t *)(p + off); off += round256(n_pairs * 4);
+    w.w_slot = (float *)(p + off);    off += round256(n_pairs * 4);
     w.h_hi = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
     w.h_lo = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
     w.part = (float *)(p + off);      off += round256(n_pairs * n_embd * 4);
@@ -74,7 +76,8 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
 /* ---- 1. counting sort of pairs by expert; cnt[] and cur[] live in LDS ---- */
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int32_t *__restrict__ offsets,
-                 int32_t *__restrict__ order, int32_t *__restrict__ slot_of) {
+                 int32_t *__restrict__ order, int32_t *__restrict__ slot_of, const float *__restrict__ expert_w,
+                 float *__restrict__ w_slot) {
     extern __shared__ int32_t lds[]; /* cnt[n_expert], cur[n_expert], wave_total[16] */
     int32_t *cnt = lds, *cur = lds + n_expert;
     for (int e = threadIdx.x; e < n_expert; e += blockDim.x) cnt[e] = 0;
@@ -119,6 +122,7 @@ moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int
         if (e >= 0 && e < n_expert) {
             slot = atomicAdd(&cur[e], 1);
             order[slot] = p;
+            w_slot[slot] = expert_w[p]; /* by slot, so that the down kernel finds it with one load */
         }
         slot_of[p] = slot;
     }
@@ -401,7 +405,7 @@ template <int RT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                 const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
-                const int32_t *__restrict__ order, const float *__restrict__ expert_w, float *__restrict__ part,
+                const float *__restrict__ w_slot, float *__restrict__ part,
                 int n_embd, int n_ff) {
     constexpr int kRows = 16 * RT;
     extern __shared__ __attribute__((aligned(16))) float red[];
@@ -431,7 +435,7 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
             float d = 0.0f;
             for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
             if (t0 + t.slot < cnt) {
-                const float w = expert_w[order[first + t0 + t.slot]];
+                const float w = w_slot[first + t0 + t.slot];
                 part[(size_t)(first + t0 + t.slot) * n_embd + row0 + t.row] = w * d; /* w * q, as out[i] += w*q does (:4116-4127) */
             }
         }
@@ -476,7 +480,7 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), ((size_t)n_expert * 2 + 16) * sizeof(int32_t), stream, idx,
-                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of);
+                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, w, ws.w_slot);
     static bool lds_raised = false;
     if (!lds_raised) {
         hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<MOE_GU_RT>,
@@ -497,7 +501,7 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
     constexpr int DRT = MOE_DN_RT;
     hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
                        (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
-                       (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.order, w, ws.part, n_embd, n_ff);
+                       (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.w_slot, ws.part, n_embd, n_ff);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 63) / 64), dim3(64), 0, stream, ws.part,
                        ws.slot_of, out, n_embd, top_k);
     return hipGetLastError();
