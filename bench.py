@@ -404,7 +404,7 @@ def main():
             gemv["%s_%dx%d" % (tname, r, c)] = {"us": round(m * 1e3, 2), "GB/s": round(b / (m * 1e-3) / 1e9, 1)}
         extra["gemv_other_shapes"] = gemv
         gemm = {}
-        for M in (128, 512, 2048):
+        for M in (16, 128, 512, 2048):
             m = time_gemm(M, 14336, 4096, max(5, args.steps // 40), 2)
             fl = 2.0 * M * 14336 * 4096
             gemm["M=%d" % M] = {"us": round(m * 1e3, 1), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}

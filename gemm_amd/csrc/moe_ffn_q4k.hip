@@ -232,13 +232,16 @@ __device__ __forceinline__ void load_acts(Acts<NA> &s, const uint16_t *const (&a
  * Nothing else in these kernels uses M0. */
 template <int NW>
 __device__ __forceinline__ void image_from_global(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
-                                                  int rows_per_matrix, size_t row_bytes, int sb, int lane) {
+                                                  int rows_per_matrix, size_t row_bytes, int sb, int lane,
+                                                  int last_row = 0x7fffffff) {
     const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
     constexpr int kChunks = NW * 16 * 9;
 #pragma unroll
     for (int i = 0; i < (kChunks + 63) / 64; i++) {
         const int t = 64 * i + lane;
-        const int R = t / 9, c9 = t - 9 * R;
+        int R = t / 9;
+        const int c9 = t - 9 * R;
+        R = R < last_row ? R : last_row; /* a ragged last tile re-reads its last row; those results are not stored */
         const uint8_t *src = (R < rows_per_matrix ? m0_rows + (size_t)R * row_bytes
                                                   : m1_rows + (size_t)(R - rows_per_matrix) * row_bytes) +
                              (size_t)sb * kQ4KBlock + 16 * c9;
@@ -303,7 +306,8 @@ template <int NW, int NA>
 __device__ __forceinline__ void ksplit_tile(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
                                             int rows_per_matrix, size_t row_bytes,
                                             const uint16_t *const (&arow)[NA], int n_sb, int wv, int n_waves,
-                                            int lane, bool live, bool image_ready, float *red) {
+                                            int lane, bool live, bool image_ready, float *red,
+                                            int last_row = 0x7fffffff) {
     const int j = lane & 15, kg = lane >> 4;
     f32x4 acc[NW];
 #pragma unroll
@@ -312,7 +316,7 @@ __device__ __forceinline__ void ksplit_tile(uint8_t *img, const uint8_t *m0_rows
         Acts<NA> s;
         if (!image_ready) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous image have returned */
-            image_from_global<NW>(img, m0_rows, m1_rows, rows_per_matrix, row_bytes, sb, lane);
+            image_from_global<NW>(img, m0_rows, m1_rows, rows_per_matrix, row_bytes, sb, lane, last_row);
         }
         load_acts(s, arow, sb, kg, live);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* image (and activations) have landed */
@@ -468,7 +472,60 @@ moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ s
     *(float4 *)(out + (size_t)t * n_embd + c) = s;
 }
 
+/* ---- 5. dense GEMM for a handful of tokens on the same machinery ----
+ * Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k] for RT * 16 rows per workgroup and 16 tokens at a
+ * time: one "expert" with every token routed to it. The weights stay exact (4-bit codes through the
+ * matrix instruction, block scales applied in fp32), so this path is closer to the oracle than the
+ * bf16-weights tile kernel; it streams the weights once per 16 tokens, which is what a few tokens need
+ * (common/transformer.h:4535-4572 decodes a row and dots it with every token). */
+template <int RT>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
+gemm_q4k_fewtok_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y,
+                       int n_rows, int n_sb, int n_tok, int ldx, int ldy) {
+    constexpr int kRows = 16 * RT;
+    extern __shared__ __attribute__((aligned(16))) float red[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * kRows;
+    const int j = lane & 15;
+    const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
+    const uint8_t *w0 = W + (size_t)row0 * row_bytes;
+    const int last_row = n_rows - 1 - row0; /* >= 0: the grid covers n_rows */
+    /* LDS: red [waves][RT][64][4] floats | images [waves][RT * 16 rows][144 bytes] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * RT * 256) + wv * (kRows * kQ4KBlock);
+    const bool one_sb = n_sb <= n_waves;
+    if (one_sb && wv < n_sb) image_from_global<RT>(img, w0, w0, kRows, row_bytes, wv, lane, last_row);
+
+    for (int t0 = 0; t0 < n_tok; t0 += 16) {
+        const bool live = t0 + j < n_tok;
+        const uint16_t *const arow[1] = {X + (size_t)(live ? t0 + j : 0) * ldx};
+        ksplit_tile<RT, 1>(img, w0, w0, kRows, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red, last_row);
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
+            const TileElem t = tile_elem<RT>(idx);
+            float d = 0.0f;
+            for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
+            if (t0 + t.slot < n_tok && row0 + t.row < n_rows) Y[(size_t)(t0 + t.slot) * ldy + row0 + t.row] = d;
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace
+
+hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
+                                  int ldx, int ldy, hipStream_t stream) {
+    /* 32 rows and 4 waves per workgroup measured best at 14336 x 4096 (12.8 us for one token, 14.8 for
+     * 16, 27 for 32); 16 rows: 21 us at 16 tokens, 64 rows: 15.5 us at one, 8 waves: +1 us from 16 tokens on */
+    constexpr int RT = 2;
+    const int n_sb = n_cols / 256;
+    const int waves = n_sb < 4 ? n_sb : 4;
+    const int grid = (n_rows + 16 * RT - 1) / (16 * RT);
+    hipLaunchKernelGGL(gemm_q4k_fewtok_kernel<RT>, dim3(grid), dim3(64 * waves),
+                       (size_t)waves * RT * (1024 + 16 * kQ4KBlock), stream, (const uint8_t *)W, X, Y, n_rows, n_sb,
+                       n_tok, ldx, ldy);
+    return hipGetLastError();
+}
 
 size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
     return carve(nullptr, n_tok, top_k, n_embd, n_ff, n_expert).bytes;

@@ -66,6 +66,11 @@ hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *
                            int n_cols, int n_tok, int ldx, int ldy, hipStream_t stream);
 
 /* Q4_K x bf16 on the matrix cores */
+/* the same contraction for a handful of tokens: exact 4-bit codes through the matrix instruction, block
+ * scales in fp32, weights streamed once per 16 tokens (moe_ffn_q4k.hip) */
+constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
+hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
+                                  int ldx, int ldy, hipStream_t stream);
 hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
                                 int n_tok, int ldx, int ldy, hipStream_t stream);
 

@@ -3,9 +3,10 @@
 Two bars per case:
   * the contract: relative L2 <= 2e-3 against a double-precision-accumulated reference that
     uses the EXACT fp32 decoded weights (the CPU oracle) and the same bf16-rounded activations;
-  * the arithmetic: relative L2 <= 2e-5 against a double-precision reference that uses the
-    decoded weights rounded to bf16 (nearest even): what the kernel is designed to compute,
-    so that only fp32 accumulation order is left.
+  * the arithmetic: relative L2 <= 2e-5 against a double-precision reference of what the kernel
+    is designed to compute, so that only fp32 accumulation order is left: from 49 tokens on
+    the decoded weights rounded to bf16 (nearest even), up to FEW_TOKENS = 48 tokens the exact
+    weights (the few-token kernel does not round them).
 """
 import numpy as np
 import pytest
@@ -15,6 +16,7 @@ from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu
 Q4K = synth.GGML_Q4_K
+FEW_TOKENS = 48  # kFewTokens of the library: up to here the weights stay exact
 
 
 def run_gemm(W, Xb, n_rows, n_cols, n_tok, ldx=None, ldy=None):
@@ -36,12 +38,13 @@ def references(oracle, W, Xb, n_cols):
     exact = Xf @ dec.astype(np.float64).T
     dec_bf16 = synth.bf16_bits_to_f32(synth.to_bf16_bits(dec)).astype(np.float64)
     designed = Xf @ dec_bf16.T
-    return exact, designed
+    return exact, (exact if Xb.shape[0] <= FEW_TOKENS else designed)
 
 
 @pytest.mark.parametrize("n_tok,n_rows,n_cols", [
     (1, 128, 256), (7, 130, 512), (64, 256, 1024), (128, 384, 4096), (256, 128, 4096),
-    (300, 257, 2048), (512, 1024, 4096), (33, 1000, 768),
+    (300, 257, 2048), (512, 1024, 4096), (33, 1000, 768), (16, 14336, 256), (17, 48, 512), (48, 100, 256),
+    (49, 100, 256), (3, 16, 2560),
     (260, 12805, 256), (1030, 5130, 512),  # enough tiles for the 128-row variant of the kernel
 ])
 def test_gemm_bf16_shapes(oracle, n_tok, n_rows, n_cols):
@@ -53,8 +56,9 @@ def test_gemm_bf16_shapes(oracle, n_tok, n_rows, n_cols):
     assert rel_l2(Y, exact) <= 2e-3, (n_tok, n_rows, n_cols)
 
 
-def test_gemm_bf16_strides_and_untouched_padding(oracle):
-    n_tok, n_rows, n_cols = 40, 200, 1024
+@pytest.mark.parametrize("n_tok", [40, 72])  # few-token kernel, tile kernel
+def test_gemm_bf16_strides_and_untouched_padding(oracle, n_tok):
+    n_rows, n_cols = 200, 1024
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=3)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=4, tokens=n_tok))
     Y = run_gemm(W, Xb, n_rows, n_cols, n_tok, ldx=n_cols + 64, ldy=n_rows + 12)
@@ -74,8 +78,14 @@ def test_gemm_bf16_equals_per_token_matvec(oracle):
         X[i, k] = 1.0
     Y = run_gemm(W, synth.to_bf16_bits(X), n_rows, n_cols, len(ks))
     dec = oracle.dequant_matrix(Q4K, W, n_cols)
+    assert np.array_equal(Y, dec[:, ks].T)  # ten tokens: exact weights, bit for bit the codec's values
+    # the same probes inside a batch that takes the tile kernel: the bf16 rounding of those values
+    Xbig = np.zeros((FEW_TOKENS + 16, n_cols), np.float32)
+    Xbig[:len(ks)] = X
+    Ybig = run_gemm(W, synth.to_bf16_bits(Xbig), n_rows, n_cols, Xbig.shape[0])
     want = synth.bf16_bits_to_f32(synth.to_bf16_bits(dec[:, ks].T.copy()))
-    assert np.array_equal(Y, want)
+    assert np.array_equal(Ybig[:len(ks)], want)
+    assert not Ybig[len(ks):].any()
 
 
 def test_gemm_bf16_argument_checks():
