@@ -336,6 +336,25 @@ def probe(args):
         print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
 
 
+def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
+    """Prefill GEMM for any format: decode to bf16 in a workspace + dense library GEMM. -> ms per step"""
+    W = synth.make_weights(type_id, n_rows, n_cols, seed=70 + type_id)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=71, tokens=n_tok))
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xb)
+    dY = qlinear.DevBuf(n_tok * n_rows * 4)
+    ws = qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+    for _ in range(warmup):
+        qlinear.gemm_bf16_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        qlinear.gemm_bf16_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
+    ms = qlinear.timer_end() / steps
+    for b in (dW, dX, dY, ws):
+        b.free()
+    return ms
+
+
 def time_achievable():
     """What the part sustains on the two priced resources: a register-only loop of the GEMM's matrix
     instruction (with the shader clock it ran at) and a streaming read of 512 MiB / of the headline's
@@ -410,6 +429,13 @@ def main():
             gemm["M=%d" % M] = {"us": round(m * 1e3, 1), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}
         extra["q4k_prefill_gemm_14336x4096_bf16"] = gemm
         tf = gemm["M=512"]["TFLOP/s"]
+        anyfmt = {}
+        for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("q8_0", synth.GGML_Q8_0, 512), ("q5_K", synth.GGML_Q5_K, 512),
+                              ("iq4_nl", synth.GGML_IQ4_NL, 512), ("bf16", synth.GGML_BF16, 512), ("q4_K", Q4K, 2048),
+                              ("q6_K", synth.GGML_Q6_K, 2048)):
+            m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
+            anyfmt["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
+        extra["prefill_gemm_any_format_14336x4096_decode_to_bf16_plus_library_gemm"] = anyfmt
         extra["achievable_on_this_gpu"] = time_achievable()
         extra["q4k_prefill_gemm_roofline"] = {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS,
                                               "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libqlinear.so")
 TF_LIB = os.path.join(HERE, "libqlinear_tf.so")
-SOURCES = ["qlin_api.hip", "dequant.hip", "gemv_generic.hip", "gemv_q4k.hip", "gemv_stream.hip", "gemv_int.hip", "gemm_q4k_mfma.hip", "moe.hip", "moe_ffn_q4k.hip", "argmax.hip", "gguf_upload.hip", "probe.hip"]
+SOURCES = ["qlin_api.hip", "dequant.hip", "gemv_generic.hip", "gemv_q4k.hip", "gemv_stream.hip", "gemv_int.hip", "gemm_q4k_mfma.hip", "moe.hip", "moe_ffn_q4k.hip", "argmax.hip", "gguf_upload.hip", "probe.hip", "gemm_dense_lt.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -37,7 +37,7 @@ def build(verbose=True):
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(_compile, SOURCES))
-    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs + ["-lhipblaslt"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)

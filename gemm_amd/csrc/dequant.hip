@@ -68,6 +68,46 @@ convert_plain_kernel(uint32_t type, const uint8_t *__restrict__ src, const int32
     }
 }
 
+/* the same decode with the result rounded once to bf16 (nearest even) and stored 8 values = 16 bytes per
+ * thread: the weight operand of the dense matrix-core GEMM */
+template <uint32_t T>
+__global__ void __launch_bounds__(256)
+dequant_bf16_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, int n_rows, int n_cols,
+                    size_t row_bytes, int blocks_per_row) {
+    using C = Codec<T>;
+    constexpr int GPB = C::BE / 8;
+    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long groups_per_row = (long long)blocks_per_row * GPB;
+    if (gid >= groups_per_row * n_rows) return;
+    const int row = (int)(gid / groups_per_row);
+    const int g = (int)(gid - (long long)row * groups_per_row);
+    const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+    float y[8];
+    C::decode8(W + (size_t)row * row_bytes + (size_t)blk * C::BB, k0, y);
+    typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+    uint4 v;
+    uint32_t *vp = &v.x;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        bf16x2 r;
+        r[0] = (__bf16)y[2 * i];
+        r[1] = (__bf16)y[2 * i + 1];
+        vp[i] = __builtin_bit_cast(uint32_t, r);
+    }
+    *reinterpret_cast<uint4 *>(out + (size_t)row * n_cols + (size_t)blk * C::BE + k0) = v;
+}
+
+template <uint32_t T>
+static hipError_t launch_bf16_typed(const void *W, uint16_t *out, int n_rows, int n_cols, size_t row_bytes,
+                                    hipStream_t stream) {
+    const int bpr = n_cols / Codec<T>::BE;
+    const long long groups = (long long)bpr * (Codec<T>::BE / 8) * n_rows;
+    if (groups == 0) return hipSuccess;
+    hipLaunchKernelGGL((dequant_bf16_kernel<T>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream,
+                       (const uint8_t *)W, out, n_rows, n_cols, row_bytes, bpr);
+    return hipGetLastError();
+}
+
 template <uint32_t T>
 static hipError_t launch_typed(const void *W, const int32_t *row_ids, int n_src_rows, float *out, int n_rows,
                                int n_cols, size_t row_bytes, hipStream_t stream) {
@@ -99,6 +139,18 @@ hipError_t launch_dequant(uint32_t type, const void *W, const int32_t *row_ids, 
                            type, (const uint8_t *)W, row_ids, n_src_rows, out, n, n_cols);
         return hipGetLastError();
     }
+    default: return hipErrorInvalidValue;
+    }
+}
+
+/* out[r * n_cols + k] = bf16(decode(W)[r][k]); out 16-byte aligned, n_cols a multiple of the block size */
+hipError_t launch_dequant_bf16(uint32_t type, const void *W, uint16_t *out, int n_rows, int n_cols, size_t row_bytes,
+                               hipStream_t stream) {
+    switch (type) {
+#define QLIN_CASE(TT) case TT: return launch_bf16_typed<TT>(W, out, n_rows, n_cols, row_bytes, stream);
+    QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+    QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
+#undef QLIN_CASE
     default: return hipErrorInvalidValue;
     }
 }

@@ -755,6 +755,42 @@ int qlin_gemm_bf16_dev(uint32_t type, const void *W, const uint16_t *X, float *Y
     return QLIN_OK;
 }
 
+static constexpr size_t kDenseLibWorkspace = (size_t)32 << 20;
+
+size_t qlin_gemm_bf16_any_workspace_bytes(int n_rows, int n_cols) {
+    if (n_rows <= 0 || n_cols <= 0) return 0;
+    return dense_gemm_weight_bytes(n_rows, n_cols) + kDenseLibWorkspace;
+}
+
+int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                           int n_tok, int ldx, int ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_tok < 0 || ldx < n_cols || ldy < n_rows) return fail(QLIN_ERR_ARG, "bad token count or leading dimension");
+    if (n_rows == 0 || n_tok == 0) return QLIN_OK;
+    if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
+        return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
+    /* Q4_K up to 512 tokens: the fused kernels, which need no workspace */
+    if (type == T_Q4_K && n_tok <= 512 && n_cols % 256 == 0)
+        return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+        return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    const uint16_t *Wd = (const uint16_t *)W; /* bf16 weights are used where they are */
+    if (type != T_BF16) {
+        HIP_TRY(launch_dequant_bf16(type, W, (uint16_t *)workspace, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));
+        Wd = (const uint16_t *)workspace;
+    }
+    void *lib_ws = (char *)workspace + dense_gemm_weight_bytes(n_rows, n_cols);
+    if (const char *err = launch_gemm_dense_bf16(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, lib_ws, kDenseLibWorkspace,
+                                                 (hipStream_t)stream))
+        return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+    return QLIN_OK;
+}
+
 int qlin_moe_route_dev(const float *router_logits, int n_tok, int n_expert, int top_k, int32_t *expert_idx,
                        float *expert_w, void *stream) {
     if (n_tok < 0 || n_expert <= 0 || top_k <= 0 || top_k > n_expert || n_expert > 8192)

@@ -68,6 +68,12 @@ hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *
 /* Q4_K x bf16 on the matrix cores */
 /* the same contraction for a handful of tokens: exact 4-bit codes through the matrix instruction, block
  * scales in fp32, weights streamed once per 16 tokens (moe_ffn_q4k.hip) */
+/* any format: decode to bf16 (dequant.hip), then the dense library GEMM (gemm_dense_lt.hip) */
+hipError_t launch_dequant_bf16(uint32_t type, const void *W, uint16_t *out, int n_rows, int n_cols, size_t row_bytes,
+                               hipStream_t stream);
+size_t dense_gemm_weight_bytes(int n_rows, int n_cols);
+const char *launch_gemm_dense_bf16(const uint16_t *Wd, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
+                                   int ldx, int ldy, void *lib_ws, size_t lib_ws_bytes, hipStream_t stream);
 constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
 hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                   int ldx, int ldy, hipStream_t stream);

@@ -200,6 +200,18 @@ int qlin_gemv_argmax_dev(uint32_t ggml_type, const void *W, const float *x, floa
  * applied in fp32 (~1e-6). */
 int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,
                        int n_cols, int n_tok, int ldx, int ldy, void *stream);
+/* The same contraction for EVERY weight format (block-quantized and dense F16/BF16/F32), the role of
+ * tf_gemm_f16_mt_tokenmajor for the formats it re-decodes once per token (common/transformer.h:4535-4572):
+ * W is decoded once to bf16 (nearest even) into `workspace` and multiplied by the dense matrix-core GEMM of
+ * the vendor library. Q4_K with at most 512 tokens takes the fused kernels of qlin_gemm_bf16_dev instead
+ * and leaves the workspace alone. workspace: device memory, 256-byte aligned, at least
+ * qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes (2 bytes per weight + 32 MiB for the library);
+ * calls that share a workspace must be ordered on one stream. Relative L2 of Y against exact weights
+ * <= 2e-3. */
+size_t qlin_gemm_bf16_any_workspace_bytes(int n_rows, int n_cols);
+int qlin_gemm_bf16_any_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,
+                           int n_cols, int n_tok, int ldx, int ldy, void *workspace, size_t workspace_bytes,
+                           void *stream);
 /* Same contraction in fp32 (X fp32, no rounding of weights or activations); any supported type. */
 int qlin_gemm_f32_dev(uint32_t ggml_type, const void *W, const float *X, float *Y, int n_rows,
                       int n_cols, int n_tok, int ldx, int ldy, void *stream);

@@ -1,0 +1,109 @@
+"""GPU parity of the prefill GEMM for every weight format (decode once to bf16, then the dense
+matrix-core GEMM), through the C ABI. Two bars, as for the fused Q4_K kernel: relative L2 <= 2e-3 against
+the oracle's exact decoded weights, and <= 2e-5 against the same weights rounded to bf16 (nearest even),
+which is what the path is designed to compute."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gemm_amd import qlinear, synth
+from tests.conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+Q4K = synth.GGML_Q4_K
+ALL = dict(synth.TYPE_NAMES)
+ALL.update(synth.DENSE_TYPES)
+
+
+def run(tid, W, Xb, n_rows, n_cols, n_tok, ldx=None, ldy=None, ws=None):
+    ldx, ldy = ldx or n_cols, ldy or n_rows
+    Xpad = np.zeros((n_tok, ldx), np.uint16)
+    Xpad[:, :n_cols] = Xb
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xpad)
+    dY = qlinear.DevBuf.from_numpy(np.full((n_tok, ldy), -3.0, np.float32))
+    dws = ws or qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+    qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, dws)
+    qlinear.sync()
+    Y = dY.to_numpy(np.float32, (n_tok, ldy))
+    for b in (dW, dX, dY) + (() if ws else (dws,)):
+        b.free()
+    return Y
+
+
+def references(oracle, tid, W, Xb, n_cols):
+    dec = oracle.dequant_matrix(tid, W, n_cols)
+    Xf = synth.bf16_bits_to_f32(Xb).astype(np.float64)
+    exact = Xf @ dec.astype(np.float64).T
+    designed = Xf @ synth.bf16_bits_to_f32(synth.to_bf16_bits(dec)).astype(np.float64).T
+    return exact, designed
+
+
+@pytest.mark.parametrize("tid", sorted(ALL), ids=lambda t: ALL[t])
+def test_every_format(oracle, tid):
+    n_tok, n_rows, n_cols = 72, 160, 512
+    W = synth.make_weights(tid, n_rows, n_cols, seed=500 + tid)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=600 + tid, tokens=n_tok))
+    Y = run(tid, W, Xb, n_rows, n_cols, n_tok)
+    exact, designed = references(oracle, tid, W, Xb, n_cols)
+    assert rel_l2(Y, designed) <= 2e-5, ALL[tid]
+    # F32 weights carry 24 significant bits, everything else at most 11 + a few: rounding to bf16 is 2^-9 each
+    assert rel_l2(Y, exact) <= 3e-3, ALL[tid]
+
+
+@pytest.mark.parametrize("tid,n_tok,n_rows,n_cols", [
+    (synth.GGML_Q6_K, 1, 16, 256), (synth.GGML_Q6_K, 515, 1000, 1024), (synth.GGML_Q8_0, 130, 257, 96),
+    (synth.GGML_Q5_K, 64, 2048, 768), (synth.GGML_IQ4_NL, 200, 130, 4096), (Q4K, 513, 384, 512),
+    (Q4K, 1100, 300, 256), (synth.GGML_BF16, 33, 100, 264), (synth.GGML_F16, 300, 64, 1000),
+])
+def test_shapes(oracle, tid, n_tok, n_rows, n_cols):
+    W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + n_tok)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=n_cols + n_tok, tokens=n_tok))
+    Y = run(tid, W, Xb, n_rows, n_cols, n_tok)
+    exact, designed = references(oracle, tid, W, Xb, n_cols)
+    assert rel_l2(Y, designed) <= 2e-5, (ALL[tid], n_tok, n_rows, n_cols)
+    assert rel_l2(Y, exact) <= 3e-3
+
+
+def test_q4k_up_to_512_tokens_is_the_fused_path_and_needs_no_workspace(oracle):
+    n_tok, n_rows, n_cols = 40, 96, 512
+    W = synth.make_weights(Q4K, n_rows, n_cols, seed=1)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=2, tokens=n_tok))
+    dW, dX, dY = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xb), qlinear.DevBuf(n_tok * n_rows * 4)
+    qlinear.gemm_bf16_any_dev(Q4K, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, None)
+    qlinear.sync()
+    exact, _ = references(oracle, Q4K, W, Xb, n_cols)
+    assert rel_l2(dY.to_numpy(np.float32, (n_tok, n_rows)), exact) <= 2e-5  # few-token kernel: exact weights
+
+
+def test_strides_padding_and_workspace_reuse(oracle):
+    tid, n_tok, n_rows, n_cols = synth.GGML_Q6_K, 90, 200, 1024
+    ws = qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+    for seed in (3, 4):  # two different tensors through one workspace, back to back
+        W = synth.make_weights(tid, n_rows, n_cols, seed=seed)
+        Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=seed + 10, tokens=n_tok))
+        Y = run(tid, W, Xb, n_rows, n_cols, n_tok, ldx=n_cols + 64, ldy=n_rows + 12, ws=ws)
+        _, designed = references(oracle, tid, W, Xb, n_cols)
+        assert rel_l2(Y[:, :n_rows], designed) <= 2e-5
+        assert np.all(Y[:, n_rows:] == -3.0)
+    ws.free()
+
+
+def test_argument_checks():
+    lib = qlinear.load()
+    d = qlinear.DevBuf(1 << 20)
+    need = qlinear.gemm_bf16_any_workspace_bytes(128, 256)
+    assert need == 128 * 256 * 2 + (32 << 20)
+    ws = qlinear.DevBuf(need)
+    f = lib.qlin_gemm_bf16_any_dev
+    Q6K = synth.GGML_Q6_K
+    assert f(9, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, ws.ptr, need, None) == qlinear.ERR_TYPE
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 300, 4, 304, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ragged K
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 260, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ldx % 8
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 100, ws.ptr, need, None) == qlinear.ERR_ARG      # ldy < rows
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 0, 256, 4, 256, 128, None, 0, None) == 0
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 0, 256, 128, None, 0, None) == 0
+    assert lib.qlin_gemm_bf16_any_workspace_bytes(0, 256) == 0
