@@ -334,6 +334,12 @@ def probe(args):
     elif args.probe == "gemm":
         ms = time_gemm(512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
+    elif args.probe == "gemm_any_q6_K":  # decode to bf16 + dense library GEMM, Q6_K, 512 tokens
+        ms = time_gemm_any(synth.GGML_Q6_K, 512, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_any_q6_K", "ms_per_step": ms}))
+    elif args.probe == "gemm_fewtok":  # the few-token kernel at 16 tokens
+        ms = time_gemm(16, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_fewtok", "ms_per_step": ms}))
 
 
 def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
@@ -392,7 +398,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
