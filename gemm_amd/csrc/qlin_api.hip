@@ -653,6 +653,19 @@ int qlin_dequant_dev(uint32_t type, const void *W, float *out, int n_rows, int n
     return QLIN_OK;
 }
 
+int qlin_dequant_bf16_dev(uint32_t type, const void *W, uint16_t *out, int n_rows, int n_cols, void *stream) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_rows == 0) return QLIN_OK;
+    if (!W || !out) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 16) || !aligned(out, 16)) return fail(QLIN_ERR_ARG, "W and out need 16-byte alignment");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    HIP_TRY(launch_dequant_bf16(type, W, out, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));
+    return QLIN_OK;
+}
+
 int qlin_embed_rows_dev(uint32_t type, const void *table, int n_table_rows, const int32_t *row_ids, int n_ids,
                         float *out, int n_cols, void *stream) {
     if (!known_type(type)) return fail(QLIN_ERR_TYPE, "unsupported type %u", type);

@@ -102,6 +102,7 @@ SIGNATURES = {
     "qlin_gguf_get_f64": (C.c_int, [_vp, C.c_int, _vp]),
     "qlin_gguf_get_str": (C.c_char_p, [_vp, C.c_int]),
     "qlin_gguf_get_array": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp]),
+    "qlin_dequant_bf16_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemm_bf16_any_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "qlin_gemm_bf16_any_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, C.c_size_t, _vp]),
     "qlin_probe_mfma_bf16": (C.c_int, [C.c_int, _vp, C.POINTER(C.c_double)]),
@@ -295,6 +296,10 @@ def gemm_bf16_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, stream=N
 
 def gemm_f32_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, stream=None):
     check(load().qlin_gemm_f32_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy, stream))
+
+
+def dequant_bf16_dev(type_id, dW, dout, n_rows, n_cols, stream=None):
+    check(load().qlin_dequant_bf16_dev(type_id, dW.ptr, dout.ptr, n_rows, n_cols, stream))
 
 
 def gemm_bf16_any_workspace_bytes(n_rows, n_cols):

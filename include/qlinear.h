@@ -167,6 +167,11 @@ int   qlin_dev_sync(void *stream);
 
 /* out[n_rows, n_cols] fp32 = decode(W); whole blocks only */
 int qlin_dequant_dev(uint32_t ggml_type, const void *W, float *out, int n_rows, int n_cols, void *stream);
+/* out[n_rows, n_cols] bf16 (bit patterns) = decode(W) rounded to nearest even: the weight operand of
+ * qlin_gemm_bf16_any_dev. An engine with HBM to spare decodes the tensors its prefill uses most once and
+ * passes the copy as GGML_TYPE_BF16 (the decode is 35-45 us of a 90 us call at 14336 x 4096 x 512 tokens).
+ * W and out 16-byte aligned, n_cols a whole number of blocks (dense types: a multiple of 8). */
+int qlin_dequant_bf16_dev(uint32_t ggml_type, const void *W, uint16_t *out, int n_rows, int n_cols, void *stream);
 /* out[i, :] = decode(table row row_ids[i]) for i < n_ids: the token-embedding lookup
  * (tf_dequant_row on token_embd, common/transformer.h:3509) for a list of device-resident ids.
  * An id outside [0, n_table_rows) gives a row of zeros (the reference refuses such a token, :3501). */

@@ -107,3 +107,24 @@ def test_argument_checks():
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 0, 256, 4, 256, 128, None, 0, None) == 0
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 0, 256, 128, None, 0, None) == 0
     assert lib.qlin_gemm_bf16_any_workspace_bytes(0, 256) == 0
+
+
+@pytest.mark.parametrize("tid", sorted(ALL), ids=lambda t: ALL[t])
+def test_decode_to_bf16_is_the_codec_rounded_once(oracle, tid):
+    n_rows, n_cols = 37, 1024
+    W = synth.make_weights(tid, n_rows, n_cols, seed=40 + tid)
+    dW, dout = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf(n_rows * n_cols * 2)
+    qlinear.dequant_bf16_dev(tid, dW, dout, n_rows, n_cols)
+    qlinear.sync()
+    got = dout.to_numpy(np.uint16, (n_rows, n_cols))
+    want = synth.to_bf16_bits(oracle.dequant_matrix(tid, W, n_cols))
+    assert np.array_equal(got, want), ALL[tid]
+    # a cached bf16 copy is a weight tensor of its own
+    n_tok = 70
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=7, tokens=n_tok))
+    Y_cached = run(synth.GGML_BF16, got.view(np.uint8).reshape(n_rows, -1), Xb, n_rows, n_cols, n_tok)
+    Y_direct = run(tid, W, Xb, n_rows, n_cols, n_tok) if not (tid == Q4K) else None
+    if Y_direct is not None:
+        assert np.array_equal(Y_cached, Y_direct)
+    dW.free()
+    dout.free()
