@@ -402,7 +402,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
-              "weight rows with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "weight rows with no exchange)" % args.gpus, file=sys.stderr)
         return 2
     if args.probe:
         probe(args)
@@ -473,7 +473,7 @@ def main():
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "Q4_K GEMV 14336x4096, batch 1, x fp32 (BASELINE configs[1])",
+        "config": {"workload": "Q4_K GEMV 14336x4096, batch 1, x fp32 (the configuration the headline metric is quoted on)",
                    "bytes_per_step": nbytes, "weight_copies_rotated": copies, "device": name.strip(),
                    "compute_units": n_cu},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
