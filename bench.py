@@ -188,6 +188,43 @@ def time_decode_step_linear(n_layers=32, steps=5):
             "hbm_frac": round(weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
 
 
+def time_prefill_chunk_linear(n_tok=512, n_layers=32, steps=3):
+    """The block-quantized linear operators of one 512-token prefill chunk of the same Llama-3-8B-shaped
+    model: seven Q4_K x bf16 GEMMs per layer (Q, K, V, attention output, gate, up, down) through
+    qlin_gemm_bf16_any_dev (fused tile kernel for gate and up, decode + library GEMM for the 4096- and
+    1024-row tensors), each layer with its own weights; inputs are bf16 buffers of the right shapes (attention, norms, the SiLU product and
+    the fp32 -> bf16 conversions between the operators are not run). -> dict"""
+    K, FF, KV = 4096, 14336, 1024
+    shapes = ((K, K), (KV, K), (KV, K), (K, K), (FF, K), (FF, K), (K, FF))
+    host = [synth.make_weights(Q4K, r, c, seed=81 + i) for i, (r, c) in enumerate(shapes)]
+    layers = [[qlinear.DevBuf.from_numpy(h) for h in host] for _ in range(n_layers)]
+    xk = qlinear.DevBuf.from_numpy(synth.to_bf16_bits(synth.make_activation(K, seed=6, tokens=n_tok)))
+    xff = qlinear.DevBuf.from_numpy(synth.to_bf16_bits(synth.make_activation(FF, seed=7, tokens=n_tok)))
+    out = qlinear.DevBuf(n_tok * FF * 4)
+    ws = qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(FF, K))
+
+    def step():
+        for W in layers:
+            for i, (r, c) in enumerate(shapes):
+                qlinear.gemm_bf16_any_dev(Q4K, W[i], xff if c == FF else xk, out, r, c, n_tok, c, r, ws)
+
+    step()
+    qlinear.sync()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        step()
+    ms = qlinear.timer_end() / steps
+    flops = 2.0 * n_tok * n_layers * sum(r * c for r, c in shapes)
+    for bufs in layers:
+        for d in bufs:
+            d.free()
+    for d in (xk, xff, out, ws):
+        d.free()
+    return {"ms_per_chunk": round(ms, 3), "tokens": n_tok, "tokens_per_s": round(n_tok / (ms * 1e-3)),
+            "launches": 7 * n_layers, "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
+            "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4)}
+
+
 def time_gemm(n_tok, n_rows, n_cols, steps, warmup):
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=31)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=32, tokens=n_tok))
@@ -459,6 +496,7 @@ def main():
         extra["q4k_fused_decode_shapes"] = time_fused(max(20, args.steps // 8))
 
         extra["q4k_llama8b_shaped_decode_step_linear_ops"] = time_decode_step_linear()
+        extra["q4k_llama8b_shaped_prefill_512tok_linear_ops"] = time_prefill_chunk_linear()
 
         hb = time_host_boundary(n_rows, n_cols)
         extra["host_pointer_matvec_14336x4096"] = {"us": round(hb * 1e3, 1), "GB/s": round(nbytes / (hb * 1e-3) / 1e9, 1),

@@ -20,7 +20,10 @@
  * i+2 is issued in the shadow of the MFMAs of tile i, and global loads run four tiles ahead
  * (two register sets). One barrier per tile. When 128-row tiles would leave compute units
  * without a workgroup (few tokens, or few rows) the same kernel runs with BN = 64: 4 x 2 waves
- * of 64 tokens x 32 rows, eight 4-byte weight parts per row (M = 128: 66 -> 55 us).
+ * of 64 tokens x 32 rows, eight 4-byte weight parts per row (M = 128: 66 -> 55 us). When even those
+ * tiles number 128 or fewer (4096 rows at 512 tokens), K is cut in two halves that add their results to
+ * a zeroed Y (4096 x 14336 at 512 tokens: 166 -> 108 us; two addends onto zero commute, so the result
+ * does not depend on which half arrives first).
  *
  * Measured on MI355X at M=512, N=14336, K=4096: 76-78 us, 0.78 PFLOP/s on 224 of 256 compute
  * units. Cycle stamps (s_memtime) around the parts of one tile show a tile of about 1920 cycles
@@ -102,7 +105,7 @@ __device__ __forceinline__ uint2 decode4(uint32_t n0, float dl, float ml) {
 template <int WM, int NB>
 __global__ void __launch_bounds__(128 * WM)
 gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y,
-                     int n_rows, int n_sb, int n_tok, int ldx, int ldy, int m_tiles) {
+                     int n_rows, int n_sb, int n_tok, int ldx, int ldy, int m_tiles, int k_split) {
     constexpr int BM = 64 * WM, NT = 128 * WM;
     static_assert(NT == 512, "one weight-row part per thread: 512 threads");
     constexpr int BN = 64 * NB;
@@ -131,7 +134,10 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     const uint8_t *w_ptr = W + (size_t)w_row * row_bytes;
     /* A-tile role: chunks (token row ar + 64j, 16-byte column ac), j = 0..3 */
     const int ar = tid >> 3, ac = tid & 7;
-    const int n_steps = n_sb * 4;
+    /* blockIdx.y = which part of K (k_split parts of equal, even length); with more than one part the
+     * results are added to a zeroed Y */
+    const int n_steps = (int)(blockIdx.y + 1) * (n_sb * 4 / k_split);
+    const int step0 = (int)blockIdx.y * (n_sb * 4 / k_split);
 
     /* register set of one tile in flight from global memory; named members only (a set that
      * lives across the tile loop stays in registers only when nothing indexes it) */
@@ -233,19 +239,19 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
      * Stage (i+2) % 3 held tile i-1, whose last fragments were read before the barrier that
      * opens tile i; tile i+1 was completed before that same barrier. */
     StepRegs r0, r1;
-    fetch(r0, 0);
-    fetch(r1, 1);
-    stage_weights(r0, 0, 0);
+    fetch(r0, step0);
+    fetch(r1, step0 + 1);
+    stage_weights(r0, step0, 0);
     stage_acts(r0, 0);
-    fetch(r0, 2);
-    stage_weights(r1, 1, 1);
+    fetch(r0, step0 + 2);
+    stage_weights(r1, step0 + 1, 1);
     stage_acts(r1, 1);
-    fetch(r1, 3);
+    fetch(r1, step0 + 3);
     __syncthreads();
     Frags f0, f1;
     load_frags(f0, 0, 0);
     int st = 0; /* stage of the current tile */
-    for (int step = 0; step < n_steps; step += 2) {
+    for (int step = step0; step < n_steps; step += 2) {
         /* even tile: registers r0 hold tile step+2 */
         {
             const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
@@ -293,7 +299,10 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const int m = tile_m * BM + wm * 64 + mi * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-            if (m < n_tok && n < n_rows) Y[(size_t)m * ldy + n] = acc[v];
+            if (m < n_tok && n < n_rows) {
+                if (k_split == 1) Y[(size_t)m * ldy + n] = acc[v];
+                else unsafeAtomicAdd(&Y[(size_t)m * ldy + n], acc[v]); /* two addends onto zero: the order cannot matter */
+            }
         }
     };
     store_tile(acc00, 0, 0);
@@ -305,6 +314,11 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
 }
 
 namespace {
+
+__global__ void __launch_bounds__(256) zero_rows_kernel(float *__restrict__ Y, int n_rows, int ldy) {
+    const int n = blockIdx.x * 256 + threadIdx.x;
+    if (n < n_rows) Y[(size_t)blockIdx.y * ldy + n] = 0.0f;
+}
 
 template <int NB>
 hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok, int ldx,
@@ -318,14 +332,21 @@ hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, 
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
     const int grid = n_tiles_pad * m_tiles;
     const size_t lds_bytes = (size_t)kStages * (BM + BN) * kRow;
+    /* half a chip's worth of tiles or less (4096 rows at 512 tokens: 128): each tile's K range is cut in
+     * two halves that add their results to a zeroed Y; a + b onto zero is the same in either order, so
+     * the result stays deterministic (three or more parts would not) */
+    const int k_split = (NB == 1 && n_tiles * m_tiles <= 128 && n_sb >= 4) ? 2 : 1;
+    if (k_split > 1) {
+        hipLaunchKernelGGL(zero_rows_kernel, dim3((n_rows + 255) / 256, n_tok), dim3(256), 0, stream, Y, n_rows, ldy);
+    }
     if (!lds_raised) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_q4k_bf16_kernel<WM, NB>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         lds_raised = true;
     }
-    hipLaunchKernelGGL((gemm_q4k_bf16_kernel<WM, NB>), dim3(grid), dim3(128 * WM), lds_bytes, stream,
-                       (const uint8_t *)W, X, Y, n_rows, n_sb, n_tok, ldx, ldy, m_tiles);
+    hipLaunchKernelGGL((gemm_q4k_bf16_kernel<WM, NB>), dim3(grid, k_split), dim3(128 * WM), lds_bytes, stream,
+                       (const uint8_t *)W, X, Y, n_rows, n_sb, n_tok, ldx, ldy, m_tiles, k_split);
     return hipGetLastError();
 }
 

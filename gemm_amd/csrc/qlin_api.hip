@@ -783,9 +783,14 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
     if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
         return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
-    /* Q4_K up to 512 tokens: the fused kernels, which need no workspace */
-    if (type == T_Q4_K && n_tok <= 512 && n_cols % 256 == 0)
-        return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    /* Q4_K: the fused kernels (no workspace) for a few tokens, and up to 512 tokens where their 256-token x
+     * 128-row tiles fill the chip; with fewer than 200 tiles (4096 rows: 64) the decode + library route is
+     * faster (4096 x 14336 at 512 tokens: 105 vs 162 us; 14336 x 4096: 96 vs 77 us) */
+    if (type == T_Q4_K) {
+        const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
+        if (n_tok <= kFewTokens || (n_tok <= 512 && tiles >= 200))
+            return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    }
     if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols))
         return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes");
     {

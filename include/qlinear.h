@@ -208,8 +208,9 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
 /* The same contraction for EVERY weight format (block-quantized and dense F16/BF16/F32), the role of
  * tf_gemm_f16_mt_tokenmajor for the formats it re-decodes once per token (common/transformer.h:4535-4572):
  * W is decoded once to bf16 (nearest even) into `workspace` and multiplied by the dense matrix-core GEMM of
- * the vendor library. Q4_K with at most 512 tokens takes the fused kernels of qlin_gemm_bf16_dev instead
- * and leaves the workspace alone. workspace: device memory, 256-byte aligned, at least
+ * the vendor library. Q4_K takes the fused kernels of qlin_gemm_bf16_dev instead, and leaves the
+ * workspace alone, for up to 48 tokens and for up to 512 tokens when the tensor has enough rows to fill
+ * the chip with their tiles (about 12800 rows at 512 tokens). workspace: device memory, 256-byte aligned, at least
  * qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes (2 bytes per weight + 32 MiB for the library);
  * calls that share a workspace must be ordered on one stream. Relative L2 of Y against exact weights
  * <= 2e-3. */

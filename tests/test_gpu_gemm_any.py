@@ -54,7 +54,7 @@ def test_every_format(oracle, tid):
 @pytest.mark.parametrize("tid,n_tok,n_rows,n_cols", [
     (synth.GGML_Q6_K, 1, 16, 256), (synth.GGML_Q6_K, 515, 1000, 1024), (synth.GGML_Q8_0, 130, 257, 96),
     (synth.GGML_Q5_K, 64, 2048, 768), (synth.GGML_IQ4_NL, 200, 130, 4096), (Q4K, 513, 384, 512),
-    (Q4K, 1100, 300, 256), (synth.GGML_BF16, 33, 100, 264), (synth.GGML_F16, 300, 64, 1000),
+    (Q4K, 1100, 300, 256), (Q4K, 300, 25700, 256), (synth.GGML_BF16, 33, 100, 264), (synth.GGML_F16, 300, 64, 1000),
 ])
 def test_shapes(oracle, tid, n_tok, n_rows, n_cols):
     W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + n_tok)
@@ -65,7 +65,7 @@ def test_shapes(oracle, tid, n_tok, n_rows, n_cols):
     assert rel_l2(Y, exact) <= 3e-3
 
 
-def test_q4k_up_to_512_tokens_is_the_fused_path_and_needs_no_workspace(oracle):
+def test_q4k_few_tokens_is_the_fused_path_and_needs_no_workspace(oracle):
     n_tok, n_rows, n_cols = 40, 96, 512
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=1)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=2, tokens=n_tok))
