@@ -96,6 +96,7 @@ struct State {
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::map<uintptr_t, Range> registry; /* host begin -> range */
     DevBuf w[3], x, y[3], tmp[4];
+    bool prefill_bf16 = false; /* qlin_gemm_tokenmajor on the matrix cores (opt-in: costs accuracy) */
 } g;
 
 int ensure_init_locked(int device) {
@@ -112,6 +113,7 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipEventCreate(&g.ev0));
     HIP_TRY(hipEventCreate(&g.ev1));
     g.device = device;
+    if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
     g.ready = true;
     return QLIN_OK;
 }
@@ -545,11 +547,43 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
     if (int rc = g.tmp[1].ensure((size_t)n_tok * n_rows * 4)) return rc;
     HIP_TRY(hipMemcpy2DAsync(g.tmp[0].p, (size_t)n_cols * 4, X, (size_t)x_stride * 4, (size_t)n_cols * 4,
                              (size_t)n_tok, hipMemcpyHostToDevice, g.stream));
-    HIP_TRY(launch_gemm_f32(type, dW, (const float *)g.tmp[0].p, (float *)g.tmp[1].p, n_rows, n_cols, n_tok,
-                            n_cols, n_rows, g.stream));
+    if (g.prefill_bf16 && n_tok >= 8 && n_cols % 8 == 0) {
+        /* opted in: activations rounded to bf16 on the device, then the matrix-core route of
+         * qlin_gemm_bf16_any_dev with internal scratch */
+        const size_t ws_bytes = dense_gemm_weight_bytes(n_rows, n_cols) + ((size_t)32 << 20);
+        if (int rc = g.tmp[2].ensure((size_t)n_tok * n_cols * 2)) return rc;
+        if (int rc = g.tmp[3].ensure(ws_bytes)) return rc;
+        HIP_TRY(launch_dequant_bf16(T_F32, g.tmp[0].p, (uint16_t *)g.tmp[2].p, n_tok, n_cols, (size_t)n_cols * 4, g.stream));
+        const uint16_t *Xb = (const uint16_t *)g.tmp[2].p;
+        float *Yd = (float *)g.tmp[1].p;
+        const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
+        if (type == T_Q4_K && (n_tok <= kFewTokens || (n_tok <= 512 && tiles >= 200))) {
+            HIP_TRY(launch_gemm_q4k_bf16(dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
+        } else {
+            const uint16_t *Wd = (const uint16_t *)dW;
+            if (type != T_BF16) {
+                HIP_TRY(launch_dequant_bf16(type, dW, (uint16_t *)g.tmp[3].p, n_rows, n_cols, rb, g.stream));
+                Wd = (const uint16_t *)g.tmp[3].p;
+            }
+            void *lib_ws = (char *)g.tmp[3].p + dense_gemm_weight_bytes(n_rows, n_cols);
+            if (const char *err = launch_gemm_dense_bf16(Wd, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, lib_ws,
+                                                         (size_t)32 << 20, g.stream))
+                return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+        }
+    } else {
+        HIP_TRY(launch_gemm_f32(type, dW, (const float *)g.tmp[0].p, (float *)g.tmp[1].p, n_rows, n_cols, n_tok,
+                                n_cols, n_rows, g.stream));
+    }
     HIP_TRY(hipMemcpy2DAsync(Y, (size_t)out_stride * 4, g.tmp[1].p, (size_t)n_rows * 4, (size_t)n_rows * 4,
                              (size_t)n_tok, hipMemcpyDeviceToHost, g.stream));
     HIP_TRY(hipStreamSynchronize(g.stream));
+    return QLIN_OK;
+}
+
+int qlin_set_prefill_matrix_cores(int enable) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    g.prefill_bf16 = enable != 0;
     return QLIN_OK;
 }
 

@@ -128,3 +128,25 @@ def test_decode_to_bf16_is_the_codec_rounded_once(oracle, tid):
         assert np.array_equal(Y_cached, Y_direct)
     dW.free()
     dout.free()
+
+
+@pytest.mark.parametrize("tid", [Q4K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ3_S, synth.GGML_F16],
+                         ids=lambda t: ALL[t])
+def test_host_pointer_prefill_on_the_matrix_cores_when_opted_in(oracle, tid):
+    lib = qlinear.load()
+    n_tok, n_rows, n_cols = 60, 300, 1024
+    W = synth.make_weights(tid, n_rows, n_cols, seed=77 + tid)
+    X = synth.make_activation(n_cols, seed=78, tokens=n_tok)
+    want = X.astype(np.float64) @ oracle.dequant_matrix(tid, W, n_cols).astype(np.float64).T
+    exact = qlinear.gemm_tokenmajor(tid, W, X, n_cols)
+    assert rel_l2(exact, want) <= 1e-5
+    assert lib.qlin_set_prefill_matrix_cores(1) == 0
+    try:
+        fast = qlinear.gemm_tokenmajor(tid, W, X, n_cols)
+        few = qlinear.gemm_tokenmajor(tid, W, X[:5], n_cols)  # fewer than 8 tokens stay on the fp32 path
+    finally:
+        assert lib.qlin_set_prefill_matrix_cores(0) == 0
+    err = rel_l2(fast, want)
+    assert 1e-5 < err <= 3e-3, err  # the bf16 route really ran, and inside its contract
+    assert rel_l2(few, want[:5]) <= 1e-5
+    assert rel_l2(qlinear.gemm_tokenmajor(tid, W, X, n_cols), want) <= 1e-5  # and the switch is off again
