@@ -260,11 +260,13 @@ def time_host_boundary(n_rows, n_cols, calls=200):
     return dt * 1e3
 
 
-def time_moe(steps, warmup, n_expert=128, n_embd=2048, n_ff=768, top_k=8, n_tok=64, copies=2):
-    """Grouped MoE expert FFN: -> (ms per step, algorithmic bytes per step, flops per step)"""
+def time_moe(steps, warmup, n_expert=128, n_embd=2048, n_ff=768, top_k=8, n_tok=64, copies=2, types=None):
+    """Grouped MoE expert FFN: -> (ms per step, algorithmic bytes per step, flops per step).
+    types = formats of (gate, up, down); default all Q4_K"""
+    types = types or (Q4K, Q4K, Q4K)
     sets = []
     for c in range(copies):
-        sets.append([qlinear.DevBuf.from_numpy(synth.make_weights(Q4K, n_expert * r, k, seed=900 + 3 * c + i))
+        sets.append([qlinear.DevBuf.from_numpy(synth.make_weights(types[i], n_expert * r, k, seed=900 + 3 * c + i))
                      for i, (r, k) in enumerate(((n_ff, n_embd), (n_ff, n_embd), (n_embd, n_ff)))])
     Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=41, tokens=n_tok))
     dX = qlinear.DevBuf.from_numpy(Xb)
@@ -278,7 +280,7 @@ def time_moe(steps, warmup, n_expert=128, n_embd=2048, n_ff=768, top_k=8, n_tok=
 
     def step(i):
         g, u, d = sets[i % copies]
-        qlinear.moe_ffn_dev(Q4K, g, u, d, dX, di, dw, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
+        qlinear.moe_ffn_types_dev(types, g, u, d, dX, di, dw, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
 
     for i in range(warmup):
         step(i)
@@ -287,7 +289,8 @@ def time_moe(steps, warmup, n_expert=128, n_embd=2048, n_ff=768, top_k=8, n_tok=
     for i in range(steps):
         step(i)
     ms = qlinear.timer_end()
-    expert_bytes = 2 * n_ff * synth.row_bytes(Q4K, n_embd) + n_embd * synth.row_bytes(Q4K, n_ff)
+    expert_bytes = (n_ff * (synth.row_bytes(types[0], n_embd) + synth.row_bytes(types[1], n_embd)) +
+                    n_embd * synth.row_bytes(types[2], n_ff))
     nbytes = routed * expert_bytes + n_tok * n_embd * 2 + n_tok * n_embd * 4 + n_tok * top_k * 8
     flops = 2.0 * n_tok * top_k * 3 * n_ff * n_embd
     for b in [x for st in sets for x in st] + [dX, dl, di, dw, dout, dws]:
@@ -502,6 +505,12 @@ def main():
         extra["host_pointer_matvec_14336x4096"] = {"us": round(hb * 1e3, 1), "GB/s": round(nbytes / (hb * 1e-3) / 1e9, 1),
                                                   "note": "W registered; x H2D and y D2H every call"}
         m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
+        Q6K = synth.GGML_Q6_K
+        for label, tys in (("q4k_q4k_q6k", (Q4K, Q4K, Q6K)), ("q6k", (Q6K, Q6K, Q6K))):
+            mm, bb, _, _ = time_moe(max(5, args.steps // 40), 2, types=tys)
+            extra["moe_ffn_128x(768x2048)_64tok_top8_%s" % label] = {
+                "us": round(mm * 1e3, 1), "bytes": bb, "GB/s": round(bb / (mm * 1e-3) / 1e9, 1),
+                "hbm_frac": round(bb / (mm * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
         extra["q4k_moe_ffn_128x(768x2048)_64tok_top8"] = {
             "us": round(m * 1e3, 1), "routed_experts": routed, "bytes": b, "GB/s": round(b / (m * 1e-3) / 1e9, 1),
             "hbm_frac": round(b / (m * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}

@@ -52,6 +52,7 @@ struct Workspace {
     uint16_t *h_hi;    /* [n_pairs, n_ff] bf16 head of silu(g)*u, by slot */
     uint16_t *h_lo;    /* [n_pairs, n_ff] bf16 tail */
     float *part;       /* [n_pairs, n_embd] w * down(h), by slot */
+    float *g32, *u32;  /* [n_pairs, n_ff] each: gate and up results of the any-format kernels, by slot */
     size_t bytes;
 };
 
@@ -69,6 +70,8 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
     w.h_hi = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
     w.h_lo = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
     w.part = (float *)(p + off);      off += round256(n_pairs * n_embd * 4);
+    w.g32 = (float *)(p + off);       off += round256(n_pairs * n_ff * 4);
+    w.u32 = (float *)(p + off);       off += round256(n_pairs * n_ff * 4);
     w.bytes = off;
     return w;
 }
@@ -472,6 +475,118 @@ moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ s
     *(float4 *)(out + (size_t)t * n_embd + c) = s;
 }
 
+/* ---- 6. the expert matrices of any format: rows of one matrix for all tokens of an expert ----
+ * A wavefront owns one row of one expert, decodes it (the bit-exact codec, 8 elements per lane and
+ * step) once per 8 of the expert's tokens and dots it with their activation rows in fp32:
+ * what tf_qmatvec_expert computes per token (common/transformer.h:517-548), grouped by expert.
+ * NX = 1: activations are the tokens' bf16 rows X[token] (gate, up); NX = 2: the bf16 head and tail
+ * of the intermediate, by slot (down), and the result is scaled by the pair's routing weight. */
+template <uint32_t T, int NX>
+__global__ void __launch_bounds__(256)
+moe_rows_any_kernel(const uint8_t *__restrict__ W, int rows_per_expert, int n_cols, size_t row_bytes,
+                    const int32_t *__restrict__ offsets, const int32_t *__restrict__ order, int top_k,
+                    const uint16_t *__restrict__ X0, const uint16_t *__restrict__ X1,
+                    const float *__restrict__ w_slot, float *__restrict__ out) {
+    using C = Codec<T>;
+    constexpr int GPB = C::BE / 8, TT = 8;
+    const int e = blockIdx.y;
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= rows_per_expert) return; /* whole waves leave; there is no barrier below */
+    const uint8_t *Wr = W + ((size_t)e * rows_per_expert + row) * row_bytes;
+    const int groups = (n_cols / C::BE) * GPB;
+    for (int t0 = 0; t0 < cnt; t0 += TT) {
+        const uint16_t *xa[TT], *xb[TT];
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const int slot = first + (t0 + t < cnt ? t0 + t : t0); /* past the end: a valid row, result unused */
+            if (NX == 1) {
+                xa[t] = X0 + (size_t)(order[slot] / top_k) * n_cols;
+                xb[t] = nullptr;
+            } else {
+                xa[t] = X0 + (size_t)slot * n_cols;
+                xb[t] = X1 + (size_t)slot * n_cols;
+            }
+        }
+        float acc[TT];
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[t] = 0.0f;
+        for (int g = lane; g < groups; g += 64) {
+            const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+            float w[8];
+            C::decode8(Wr + (size_t)blk * C::BB, k0, w);
+            const size_t at = (size_t)blk * C::BE + k0;
+#pragma unroll
+            for (int t = 0; t < TT; t++) {
+                if (t0 + t < cnt) {
+                    const uint4 a = *reinterpret_cast<const uint4 *>(xa[t] + at);
+                    const uint32_t av[4] = {a.x, a.y, a.z, a.w};
+                    float x[8];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        x[2 * i] = __uint_as_float(av[i] << 16);
+                        x[2 * i + 1] = __uint_as_float(av[i] & 0xFFFF0000u);
+                    }
+                    if (NX == 2) {
+                        const uint4 b = *reinterpret_cast<const uint4 *>(xb[t] + at);
+                        const uint32_t bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            x[2 * i] += __uint_as_float(bv[i] << 16);
+                            x[2 * i + 1] += __uint_as_float(bv[i] & 0xFFFF0000u);
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[t] = fmaf(w[i], x[i], acc[t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const float sum = wave_sum_dpp(acc[t]);
+            if (lane == 0 && t0 + t < cnt) {
+                const int slot = first + t0 + t;
+                out[(size_t)slot * rows_per_expert + row] = w_slot ? w_slot[slot] * sum : sum;
+            }
+        }
+    }
+}
+
+/* h = silu(g) * u (tf_silu_mul, common/transformer.h:4679-4694) as a bf16 head and tail, by slot */
+__global__ void __launch_bounds__(256)
+moe_silu_split_kernel(const float *__restrict__ g32, const float *__restrict__ u32, uint16_t *__restrict__ h_hi,
+                      uint16_t *__restrict__ h_lo, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    const float g = g32[i];
+    const float h = g / (1.0f + expf(-g)) * u32[i];
+    const __bf16 hi = (__bf16)h;
+    const __bf16 lo = (__bf16)(h - (float)hi);
+    h_hi[i] = __builtin_bit_cast(uint16_t, hi);
+    h_lo[i] = __builtin_bit_cast(uint16_t, lo);
+}
+
+template <int NX>
+hipError_t launch_rows_any(uint32_t type, const void *W, int rows_per_expert, int n_cols, int n_expert,
+                           const Workspace &ws, int top_k, const uint16_t *X0, const uint16_t *X1,
+                           const float *w_slot, float *out, hipStream_t stream) {
+    const dim3 grid((rows_per_expert + 3) / 4, n_expert);
+    switch (type) {
+#define QLIN_CASE(TT)                                                                                              \
+    case TT:                                                                                                       \
+        hipLaunchKernelGGL((moe_rows_any_kernel<TT, NX>), grid, dim3(256), 0, stream, (const uint8_t *)W,          \
+                           rows_per_expert, n_cols, (size_t)(n_cols / Codec<TT>::BE) * Codec<TT>::BB, ws.offsets,  \
+                           ws.order, top_k, X0, X1, w_slot, out);                                                  \
+        return hipGetLastError();
+    QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
+    QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
+#undef QLIN_CASE
+    default: return hipErrorInvalidValue;
+    }
+}
+
 /* ---- 5. dense GEMM for a handful of tokens on the same machinery ----
  * Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k] for RT * 16 rows per workgroup and 16 tokens at a
  * time: one "expert" with every token routed to it. The weights stay exact (4-bit codes through the
@@ -531,9 +646,9 @@ size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_exp
     return carve(nullptr, n_tok, top_k, n_embd, n_ff, n_expert).bytes;
 }
 
-hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down, const uint16_t *X,
-                              const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
-                              int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream) {
+hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
+                          const void *down, const uint16_t *X, const int32_t *idx, const float *w, float *out, int n_tok,
+                          int top_k, int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream) {
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), ((size_t)n_expert * 2 + 16) * sizeof(int32_t), stream, idx,
@@ -545,20 +660,40 @@ hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down
         if (e1 != hipSuccess) return e1;
         lds_raised = true;
     }
+    /* Q4_K matrices take the matrix-core kernels; any other format (or a shape their tiles do not divide)
+     * the any-format kernel, matrix by matrix: gate and up -> fp32 by slot -> silu(g)*u as head + tail */
+    const bool fast_gu = type_gate == T_Q4_K && type_up == T_Q4_K && n_embd % 256 == 0 && n_ff % (16 * MOE_GU_RT) == 0;
+    const bool fast_dn = type_down == T_Q4_K && n_ff % 256 == 0 && n_embd % (16 * MOE_DN_RT) == 0;
     /* waves per workgroup = super-blocks of K, at most 4 for gate/up (a wave then walks several
      * super-blocks one after the other) and 8 for down. The gate/up kernel needs 138 registers, so a
      * compute unit holds 12 of its waves: three 4-wave workgroups in different phases instead of one
      * 8-wave workgroup that loads, computes and reduces with nothing beside it (75 -> 65 us). */
     const int gu_waves = n_embd / 256 < 4 ? n_embd / 256 : 4, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
-    constexpr int RT = MOE_GU_RT;
-    hipLaunchKernelGGL(moe_gate_up_kernel<RT>, dim3(n_ff / (16 * RT), n_expert), dim3(64 * gu_waves),
-                       (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock), stream,
-                       (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
-                       n_ff, top_k);
-    constexpr int DRT = MOE_DN_RT;
-    hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
-                       (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
-                       (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.w_slot, ws.part, n_embd, n_ff);
+    if (fast_gu) {
+        constexpr int RT = MOE_GU_RT;
+        hipLaunchKernelGGL(moe_gate_up_kernel<RT>, dim3(n_ff / (16 * RT), n_expert), dim3(64 * gu_waves),
+                           (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock), stream,
+                           (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
+                           n_ff, top_k);
+    } else {
+        hipError_t e1 = launch_rows_any<1>(type_gate, gate, n_ff, n_embd, n_expert, ws, top_k, X, nullptr, nullptr, ws.g32, stream);
+        if (e1 != hipSuccess) return e1;
+        e1 = launch_rows_any<1>(type_up, up, n_ff, n_embd, n_expert, ws, top_k, X, nullptr, nullptr, ws.u32, stream);
+        if (e1 != hipSuccess) return e1;
+        const size_t n = (size_t)n_pairs * n_ff;
+        hipLaunchKernelGGL(moe_silu_split_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, ws.g32, ws.u32,
+                           ws.h_hi, ws.h_lo, n);
+    }
+    if (fast_dn) {
+        constexpr int DRT = MOE_DN_RT;
+        hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
+                           (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
+                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.w_slot, ws.part, n_embd, n_ff);
+    } else {
+        hipError_t e1 = launch_rows_any<2>(type_down, down, n_embd, n_ff, n_expert, ws, top_k, ws.h_hi, ws.h_lo, ws.w_slot,
+                                           ws.part, stream);
+        if (e1 != hipSuccess) return e1;
+    }
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 63) / 64), dim3(64), 0, stream, ws.part,
                        ws.slot_of, out, n_embd, top_k);
     return hipGetLastError();

@@ -861,12 +861,14 @@ size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int 
     return moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert);
 }
 
-int qlin_moe_ffn_dev(uint32_t type, const void *gate_exps, const void *up_exps, const void *down_exps,
-                     const uint16_t *X, const int32_t *expert_idx, const float *expert_w, float *out,
-                     int n_tok, int top_k, int n_embd, int n_ff, int n_expert, void *workspace, void *stream) {
-    if (type != T_Q4_K) return fail(QLIN_ERR_TYPE, "grouped MoE FFN takes Q4_K experts only (got %u)", type);
-    if (int rc = check_linear_shape(type, n_ff, n_embd)) return rc;
-    if (int rc = check_linear_shape(type, n_embd, n_ff)) return rc;
+int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
+                           const void *up_exps, const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
+                           const float *expert_w, float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert,
+                           void *workspace, void *stream) {
+    if (int rc = check_linear_shape(type_gate, n_ff, n_embd)) return rc;
+    if (int rc = check_linear_shape(type_up, n_ff, n_embd)) return rc;
+    if (int rc = check_linear_shape(type_down, n_embd, n_ff)) return rc;
+    if (n_embd % 8 || n_ff % 8) return fail(QLIN_ERR_ARG, "n_embd and n_ff must be multiples of 8");
     if (n_tok < 0 || n_expert <= 0 || top_k <= 0 || top_k > n_expert) return fail(QLIN_ERR_ARG, "bad MoE shape");
     if (n_expert > 4096) return fail(QLIN_ERR_ARG, "grouped MoE FFN handles at most 4096 experts (got %d)", n_expert);
     if ((long long)n_tok * top_k > (1 << 24))
@@ -881,9 +883,16 @@ int qlin_moe_ffn_dev(uint32_t type, const void *gate_exps, const void *up_exps, 
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
-    HIP_TRY(launch_moe_ffn_q4k(gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out, n_tok, top_k,
-                               n_embd, n_ff, n_expert, workspace, (hipStream_t)stream));
+    HIP_TRY(launch_moe_ffn(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
+                           n_tok, top_k, n_embd, n_ff, n_expert, workspace, (hipStream_t)stream));
     return QLIN_OK;
+}
+
+int qlin_moe_ffn_dev(uint32_t type, const void *gate_exps, const void *up_exps, const void *down_exps,
+                     const uint16_t *X, const int32_t *expert_idx, const float *expert_w, float *out,
+                     int n_tok, int top_k, int n_embd, int n_ff, int n_expert, void *workspace, void *stream) {
+    return qlin_moe_ffn_types_dev(type, type, type, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out, n_tok,
+                                  top_k, n_embd, n_ff, n_expert, workspace, stream);
 }
 
 int qlin_probe_mfma_bf16(int iters, void *stream, double *flops) {

@@ -80,11 +80,12 @@ hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, in
 hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
                                 int n_tok, int ldx, int ldy, hipStream_t stream);
 
-/* grouped MoE expert FFN on the matrix cores (Q4_K experts, bf16 activations) */
+/* grouped MoE expert FFN (bf16 activations): Q4_K matrices on the matrix cores, any other format through
+ * the bit-exact codec in fp32; the three matrices may have different formats */
 size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
-hipError_t launch_moe_ffn_q4k(const void *gate, const void *up, const void *down, const uint16_t *X,
-                              const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
-                              int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream);
+hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
+                          const void *down, const uint16_t *X, const int32_t *idx, const float *w, float *out, int n_tok,
+                          int top_k, int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream);
 
 /* MoE pieces */
 hipError_t launch_moe_route(const float *logits, int n_tok, int n_expert, int top_k, int32_t *idx,

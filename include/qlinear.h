@@ -225,10 +225,13 @@ int qlin_gemm_bf16_any_dev(uint32_t ggml_type, const void *W, const uint16_t *X,
 /* Same contraction in fp32 (X fp32, no rounding of weights or activations); any supported type. */
 int qlin_gemm_f32_dev(uint32_t ggml_type, const void *W, const float *X, float *Y, int n_rows,
                       int n_cols, int n_tok, int ldx, int ldy, void *stream);
-/* Grouped MoE expert FFN over n_tok tokens:
+/* Grouped MoE expert FFN over n_tok tokens (the block of common/transformer.h:4045-4131 after the router):
  *   X bf16 [n_tok, n_embd]; expert_idx int32 [n_tok, top_k]; expert_w fp32 [n_tok, top_k];
  *   gate/up: [n_expert][n_ff][n_embd] blocks, down: [n_expert][n_embd][n_ff] blocks;
- *   out fp32 [n_tok, n_embd] (overwritten). workspace: qlin_moe_workspace_bytes() bytes. */
+ *   out fp32 [n_tok, n_embd] (overwritten). workspace: qlin_moe_workspace_bytes() bytes.
+ * Q4_K matrices run on the matrix cores with unrounded codes; every other format (block-quantized or dense)
+ * runs through the bit-exact decoder in fp32, several times slower. qlin_moe_ffn_types_dev takes one format
+ * per tensor: K-quant mixes store part of the down projections as Q6_K beside Q4_K gate and up. */
 size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
 int qlin_moe_route_dev(const float *router_logits, int n_tok, int n_expert, int top_k,
                        int32_t *expert_idx, float *expert_w, void *stream);
@@ -236,6 +239,10 @@ int qlin_moe_ffn_dev(uint32_t ggml_type, const void *gate_exps, const void *up_e
                      const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
                      const float *expert_w, float *out, int n_tok, int top_k, int n_embd,
                      int n_ff, int n_expert, void *workspace, void *stream);
+int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
+                           const void *up_exps, const void *down_exps, const uint16_t *X,
+                           const int32_t *expert_idx, const float *expert_w, float *out, int n_tok, int top_k,
+                           int n_embd, int n_ff, int n_expert, void *workspace, void *stream);
 
 /* ------------------------------------------------------------------ GGUF file -> HBM
  * The tensor table and key/value pairs of a GGUF model file (versions 2 and 3, as read by

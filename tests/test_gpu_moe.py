@@ -17,23 +17,28 @@ from tests.conftest import rel_l2
 pytestmark = pytest.mark.gpu
 Q4K = synth.GGML_Q4_K
 CONTRACT, DESIGNED = 2e-3, 2e-5
+ALL_NAMES = dict(synth.TYPE_NAMES)
+ALL_NAMES.update(synth.DENSE_TYPES)
 
 
-def make_experts(n_expert, n_embd, n_ff, seed):
-    gate = synth.make_weights(Q4K, n_expert * n_ff, n_embd, seed=seed)
-    up = synth.make_weights(Q4K, n_expert * n_ff, n_embd, seed=seed + 1)
-    down = synth.make_weights(Q4K, n_expert * n_embd, n_ff, seed=seed + 2)
+def make_experts(n_expert, n_embd, n_ff, seed, types=(Q4K, Q4K, Q4K)):
+    gate = synth.make_weights(types[0], n_expert * n_ff, n_embd, seed=seed)
+    up = synth.make_weights(types[1], n_expert * n_ff, n_embd, seed=seed + 1)
+    down = synth.make_weights(types[2], n_expert * n_embd, n_ff, seed=seed + 2)
     return gate, up, down
 
 
-def run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, fill=-7.0):
+def run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, fill=-7.0, types=None):
     n_tok, top_k = idx.shape
     bufs = [qlinear.DevBuf.from_numpy(a) for a in (gate, up, down, Xb, idx.astype(np.int32), w.astype(np.float32))]
     out0 = np.full((max(n_tok, 1), n_embd), fill, np.float32)
     dout = qlinear.DevBuf.from_numpy(out0)
     nws = qlinear.moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert)
     dws = qlinear.DevBuf(max(nws, 256))
-    qlinear.moe_ffn_dev(Q4K, *bufs, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
+    if types is None:
+        qlinear.moe_ffn_dev(Q4K, *bufs, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
+    else:
+        qlinear.moe_ffn_types_dev(types, *bufs, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws)
     qlinear.sync()
     out = dout.to_numpy(np.float32, out0.shape)[:n_tok]
     for b in bufs + [dout, dws]:
@@ -55,17 +60,17 @@ def oracle_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff):
                      for t in range(X.shape[0])])
 
 
-def numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff):
+def numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=(Q4K, Q4K, Q4K)):
     """float64 restatement grouped by expert: decode each routed expert once."""
     X = synth.bf16_bits_to_f32(Xb).astype(np.float64)
     out = np.zeros((X.shape[0], n_embd), np.float64)
-    gb, db = synth.row_bytes(Q4K, n_embd), synth.row_bytes(Q4K, n_ff)
+    gb, ub, db = synth.row_bytes(types[0], n_embd), synth.row_bytes(types[1], n_embd), synth.row_bytes(types[2], n_ff)
     for e in np.unique(idx):
         if e < 0:
             continue
-        G = oracle.dequant_matrix(Q4K, gate[e * n_ff:(e + 1) * n_ff].reshape(n_ff, gb), n_embd).astype(np.float64)
-        U = oracle.dequant_matrix(Q4K, up[e * n_ff:(e + 1) * n_ff].reshape(n_ff, gb), n_embd).astype(np.float64)
-        D = oracle.dequant_matrix(Q4K, down[e * n_embd:(e + 1) * n_embd].reshape(n_embd, db), n_ff).astype(np.float64)
+        G = oracle.dequant_matrix(types[0], gate[e * n_ff:(e + 1) * n_ff].reshape(n_ff, gb), n_embd).astype(np.float64)
+        U = oracle.dequant_matrix(types[1], up[e * n_ff:(e + 1) * n_ff].reshape(n_ff, ub), n_embd).astype(np.float64)
+        D = oracle.dequant_matrix(types[2], down[e * n_embd:(e + 1) * n_embd].reshape(n_embd, db), n_ff).astype(np.float64)
         toks, ks = np.nonzero(idx == e)
         g, u = X[toks] @ G.T, X[toks] @ U.T
         with np.errstate(over="ignore"):  # exp(-g) -> inf gives h -> 0, as in fp32
@@ -133,7 +138,9 @@ def test_grouped_ffn_rejects_other_types_and_shapes():
     lib = qlinear.load()
     d = qlinear.DevBuf(4096)
     p = d.ptr
-    assert lib.qlin_moe_ffn_dev(synth.GGML_Q8_0, p, p, p, p, p, p, p, 1, 1, 256, 256, 2, p, None) == qlinear.ERR_TYPE
+    assert lib.qlin_moe_ffn_dev(9, p, p, p, p, p, p, p, 1, 1, 256, 256, 2, p, None) == qlinear.ERR_TYPE
+    assert lib.qlin_moe_ffn_types_dev(Q4K, Q4K, 9, p, p, p, p, p, p, p, 1, 1, 256, 256, 2, p, None) == qlinear.ERR_TYPE
+    assert lib.qlin_moe_ffn_types_dev(Q4K, Q4K, synth.GGML_Q8_0, p, p, p, p, p, p, p, 1, 1, 256, 250, 2, p, None) == qlinear.ERR_ARG
     assert lib.qlin_moe_ffn_dev(Q4K, p, p, p, p, p, p, p, 1, 1, 250, 256, 2, p, None) == qlinear.ERR_ARG
     assert lib.qlin_moe_ffn_dev(Q4K, p, p, p, p, p, p, p, 1, 3, 256, 256, 2, p, None) == qlinear.ERR_ARG
     assert lib.qlin_moe_ffn_dev(Q4K, p, p, p, p, p, p, p, 1, 1, 256, 256, 2, None, None) == qlinear.ERR_ARG
@@ -163,3 +170,40 @@ def test_grouped_ffn_full_size(oracle):
         one = oracle.moe_ffn_token(Q4K, gate, up, down, n_embd, n_ff, synth.bf16_bits_to_f32(Xb[t]), idx[t], w[t], f64=True)
         assert rel_l2(want[t], one) <= 1e-6
         assert rel_l2(got[t], one) <= 10 * DESIGNED
+
+
+Q6K, Q8_0 = synth.GGML_Q6_K, synth.GGML_Q8_0
+
+
+@pytest.mark.parametrize("types", [
+    (Q4K, Q4K, Q6K),                                    # what K-quant mixes store for part of the layers
+    (Q6K, Q6K, Q6K), (Q8_0, Q8_0, Q8_0), (Q4K, Q6K, Q4K),
+    (synth.GGML_IQ4_NL, synth.GGML_IQ4_NL, synth.GGML_Q5_K), (synth.GGML_BF16, synth.GGML_F16, synth.GGML_F32),
+    (synth.GGML_IQ2_XXS, synth.GGML_IQ3_S, synth.GGML_Q4_0),
+], ids=lambda t: "-".join(ALL_NAMES[x] for x in t))
+@pytest.mark.parametrize("n_tok", [3, 40])
+def test_grouped_ffn_other_and_mixed_formats(oracle, types, n_tok):
+    n_expert, n_embd, n_ff, k = 8, 512, 256, 3
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=700, types=types)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=710 + n_tok, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=720 + n_tok), k)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
+    err = rel_l2(got, want)
+    assert err <= DESIGNED, (err, types)
+    for t in range(n_tok):
+        assert rel_l2(got[t], want[t]) <= 10 * DESIGNED, t
+
+
+def test_grouped_ffn_mixed_formats_many_tokens_per_expert_and_ragged_shapes(oracle):
+    """two experts, 50 tokens: 8-token passes of the any-format kernel with a ragged tail; n_ff = 96 is not a
+    multiple of the matrix-core tiles, so Q4_K gate/up cannot be used and Q8_0 (32-element blocks) is"""
+    types = (Q8_0, Q8_0, Q8_0)
+    n_expert, n_embd, n_ff, k, n_tok = 2, 160, 96, 2, 50
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=800, types=types)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=801, tokens=n_tok))
+    idx = np.tile(np.array([[1, 0]], np.int32), (n_tok, 1))
+    w = np.tile(np.array([[0.6, 0.4]], np.float32), (n_tok, 1))
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
+    assert rel_l2(got, want) <= DESIGNED
