@@ -590,19 +590,26 @@ int qlin_set_prefill_matrix_cores(int enable) {
 int qlin_moe_ffn_token(float *out, const void *gate_exps, const void *up_exps, const void *down_exps,
                        uint32_t type, int n_embd, int n_ff, int n_expert, int top_k,
                        const float *router_logits, const float *x) {
-    if (int rc = check_linear_shape(type, n_ff, n_embd)) return rc;
-    if (int rc = check_linear_shape(type, n_embd, n_ff)) return rc;
+    return qlin_moe_ffn_token_types(out, gate_exps, up_exps, down_exps, type, type, type, n_embd, n_ff, n_expert, top_k,
+                                    router_logits, x);
+}
+
+int qlin_moe_ffn_token_types(float *out, const void *gate_exps, const void *up_exps, const void *down_exps,
+                             uint32_t type_gate, uint32_t type_up, uint32_t type_down, int n_embd, int n_ff,
+                             int n_expert, int top_k, const float *router_logits, const float *x) {
+    if (int rc = check_linear_shape(type_gate, n_ff, n_embd)) return rc;
+    if (int rc = check_linear_shape(type_up, n_ff, n_embd)) return rc;
+    if (int rc = check_linear_shape(type_down, n_embd, n_ff)) return rc;
     if (n_expert <= 0 || top_k <= 0 || top_k > n_expert || top_k > 64 || n_expert > 8192)
         return fail(QLIN_ERR_ARG, "bad expert counts (n_expert %d, top_k %d)", n_expert, top_k);
     if (!out || !gate_exps || !up_exps || !down_exps || !router_logits || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;
-    const size_t rb_in = row_size(type, n_embd), rb_dn = row_size(type, n_ff);
-    const size_t bytes_in = rb_in * (size_t)n_ff * n_expert, bytes_dn = rb_dn * (size_t)n_embd * n_expert;
+    const size_t rb_g = row_size(type_gate, n_embd), rb_u = row_size(type_up, n_embd), rb_dn = row_size(type_down, n_ff);
     const void *dG, *dU, *dD;
-    if (int rc = weights_on_device_locked(gate_exps, bytes_in, g.w[0], &dG)) return rc;
-    if (int rc = weights_on_device_locked(up_exps, bytes_in, g.w[1], &dU)) return rc;
-    if (int rc = weights_on_device_locked(down_exps, bytes_dn, g.w[2], &dD)) return rc;
+    if (int rc = weights_on_device_locked(gate_exps, rb_g * (size_t)n_ff * n_expert, g.w[0], &dG)) return rc;
+    if (int rc = weights_on_device_locked(up_exps, rb_u * (size_t)n_ff * n_expert, g.w[1], &dU)) return rc;
+    if (int rc = weights_on_device_locked(down_exps, rb_dn * (size_t)n_embd * n_expert, g.w[2], &dD)) return rc;
     /* tmp[0]: logits | idx | w ; tmp[1]: gate ; tmp[2]: up ; tmp[3]: down out ; y[0]: accumulated out */
     const size_t off_idx = ((size_t)n_expert * 4 + 255) & ~(size_t)255;
     const size_t off_w = off_idx + 256;
@@ -624,12 +631,18 @@ int qlin_moe_ffn_token(float *out, const void *gate_exps, const void *up_exps, c
     for (int k = 0; k < top_k; k++) {
         const int e = h_idx[k];
         if (e < 0 || e >= n_expert) return fail(QLIN_ERR_DEVICE, "router produced expert %d", e);
-        const uint8_t *ge = (const uint8_t *)dG + (size_t)e * n_ff * rb_in;
-        const uint8_t *ue = (const uint8_t *)dU + (size_t)e * n_ff * rb_in;
+        const uint8_t *ge = (const uint8_t *)dG + (size_t)e * n_ff * rb_g;
+        const uint8_t *ue = (const uint8_t *)dU + (size_t)e * n_ff * rb_u;
         const uint8_t *de = (const uint8_t *)dD + (size_t)e * n_embd * rb_dn;
-        const GemvJob gate_up = {{ge, ue, nullptr}, {(float *)g.tmp[1].p, nullptr, nullptr}, {n_ff, n_ff, 0}, 2, kSiluMul};
-        HIP_TRY(dispatch_gemv_job(type, gate_up, (const float *)g.x.p, n_embd, g.stream));
-        HIP_TRY(dispatch_gemv(type, de, (const float *)g.tmp[1].p, (float *)g.tmp[3].p, n_embd, n_ff, g.stream));
+        if (type_gate == type_up) { /* one launch: silu(gate x) * (up x) */
+            const GemvJob gate_up = {{ge, ue, nullptr}, {(float *)g.tmp[1].p, nullptr, nullptr}, {n_ff, n_ff, 0}, 2, kSiluMul};
+            HIP_TRY(dispatch_gemv_job(type_gate, gate_up, (const float *)g.x.p, n_embd, g.stream));
+        } else {
+            HIP_TRY(dispatch_gemv(type_gate, ge, (const float *)g.x.p, (float *)g.tmp[1].p, n_ff, n_embd, g.stream));
+            HIP_TRY(dispatch_gemv(type_up, ue, (const float *)g.x.p, (float *)g.tmp[2].p, n_ff, n_embd, g.stream));
+            HIP_TRY(launch_silu_mul((float *)g.tmp[1].p, (const float *)g.tmp[1].p, (const float *)g.tmp[2].p, n_ff, g.stream));
+        }
+        HIP_TRY(dispatch_gemv(type_down, de, (const float *)g.tmp[1].p, (float *)g.tmp[3].p, n_embd, n_ff, g.stream));
         HIP_TRY(launch_axpy_dev_weight((float *)g.y[0].p, (const float *)g.tmp[3].p, d_w, k, n_embd, k == 0, g.stream));
     }
     HIP_TRY(hipMemcpyAsync(out, g.y[0].p, (size_t)n_embd * 4, hipMemcpyDeviceToHost, g.stream));

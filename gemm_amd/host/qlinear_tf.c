@@ -180,9 +180,8 @@ void qtf_gemm_tokenmajor(float *Y_out, const qtensor *mat, const float *X, int n
 void qtf_moe_ffn(float *out, const qtensor *gate_exps, const qtensor *up_exps, const qtensor *down_exps,
                  int n_expert, int top_k, int n_ff_expert, const float *router_logits, const float *x) {
     const int n_embd = gate_exps->n_cols;
-    if (up_exps->type != gate_exps->type || down_exps->type != gate_exps->type ||
-        qlin_moe_ffn_token(out, gate_exps->data, up_exps->data, down_exps->data, gate_exps->type, n_embd,
-                           n_ff_expert, n_expert, top_k, router_logits, x) != QLIN_OK) {
+    if (qlin_moe_ffn_token_types(out, gate_exps->data, up_exps->data, down_exps->data, gate_exps->type, up_exps->type,
+                                 down_exps->type, n_embd, n_ff_expert, n_expert, top_k, router_logits, x) != QLIN_OK) {
         complain("moe_ffn");
         zero_fill(out, (size_t)n_embd);
     }

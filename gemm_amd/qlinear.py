@@ -64,6 +64,8 @@ SIGNATURES = {
     "qlin_matvec_argmax": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int]),
     "qlin_gemm_tokenmajor": (C.c_int, [_vp, _vp, C.c_uint32, C.c_int, _vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "qlin_moe_ffn_token": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp]),
+    "qlin_moe_ffn_token_types": (C.c_int, [_vp, _vp, _vp, _vp, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_int, C.c_int,
+                                           C.c_int, _vp, _vp]),
     "qlin_dev_alloc": (_vp, [C.c_size_t]),
     "qlin_dev_free": (None, [_vp]),
     "qlin_dev_upload": (C.c_int, [_vp, _vp, C.c_size_t]),

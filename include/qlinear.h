@@ -158,6 +158,10 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t ggml_type, int n_cols
 int qlin_moe_ffn_token(float *out, const void *gate_exps, const void *up_exps, const void *down_exps,
                        uint32_t ggml_type, int n_embd, int n_ff_expert, int n_expert, int top_k,
                        const float *router_logits, const float *x);
+/* the same with one format per tensor (the down projections of K-quant mixes are partly Q6_K) */
+int qlin_moe_ffn_token_types(float *out, const void *gate_exps, const void *up_exps, const void *down_exps,
+                             uint32_t type_gate, uint32_t type_up, uint32_t type_down, int n_embd, int n_ff,
+                             int n_expert, int top_k, const float *router_logits, const float *x);
 
 /* ------------------------------------------------------------------ device-resident
  * All pointers are device addresses; `stream` is a hipStream_t passed as void* (NULL = the

@@ -188,3 +188,30 @@ def test_moe_route_and_token_ffn(oracle):
         assert np.array_equal(oi[order_o], gi[t][order_g])
         assert np.allclose(ow[order_o], gw[t][order_g], rtol=1e-5, atol=1e-8)
         assert np.all(np.diff(gw[t]) <= 0)  # descending weight order
+
+
+@pytest.mark.parametrize("types", [(synth.GGML_Q4_K, synth.GGML_Q4_K, synth.GGML_Q6_K),
+                                   (synth.GGML_Q4_K, synth.GGML_Q6_K, synth.GGML_Q8_0),
+                                   (synth.GGML_IQ4_NL, synth.GGML_IQ4_NL, synth.GGML_F16)])
+def test_token_ffn_with_one_format_per_tensor(oracle, types):
+    """the down projections of K-quant mixes are partly Q6_K beside Q4_K gate and up"""
+    lib = qlinear.load()
+    n_expert, n_embd, n_ff, k = 8, 512, 256, 3
+    gate = synth.make_weights(types[0], n_expert * n_ff, n_embd, seed=41)
+    up = synth.make_weights(types[1], n_expert * n_ff, n_embd, seed=42)
+    down = synth.make_weights(types[2], n_expert * n_embd, n_ff, seed=43)
+    x = synth.make_activation(n_embd, seed=44)
+    logits = synth.make_router_logits(1, n_expert, seed=45)[0]
+    idx, w = oracle.moe_route(logits, k)
+    want = np.zeros(n_embd, np.float64)
+    for e, we in zip(idx, w):
+        G = oracle.dequant_matrix(types[0], gate[e * n_ff:(e + 1) * n_ff], n_embd).astype(np.float64)
+        U = oracle.dequant_matrix(types[1], up[e * n_ff:(e + 1) * n_ff], n_embd).astype(np.float64)
+        D = oracle.dequant_matrix(types[2], down[e * n_embd:(e + 1) * n_embd], n_ff).astype(np.float64)
+        g, u = G @ x.astype(np.float64), U @ x.astype(np.float64)
+        want += float(we) * (D @ (g / (1.0 + np.exp(-g)) * u))
+    out = np.zeros(n_embd, np.float32)
+    assert lib.qlin_moe_ffn_token_types(out.ctypes.data, gate.ctypes.data, up.ctypes.data, down.ctypes.data, types[0],
+                                        types[1], types[2], n_embd, n_ff, n_expert, k, logits.ctypes.data,
+                                        x.ctypes.data) == 0
+    assert rel_l2(out, want) <= TOL
