@@ -476,11 +476,15 @@ moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ s
 }
 
 /* ---- 6. the expert matrices of any format: rows of one matrix for all tokens of an expert ----
- * A wavefront owns one row of one expert, decodes it (the bit-exact codec, 8 elements per lane and
- * step) once per 8 of the expert's tokens and dots it with their activation rows in fp32:
- * what tf_qmatvec_expert computes per token (common/transformer.h:517-548), grouped by expert.
+ * A workgroup of four waves owns 16 rows of one expert. The activations of 8 of the expert's tokens
+ * are staged in LDS as fp32, 1024 elements of K at a time; a wave then walks its 4 rows, decodes each
+ * with the bit-exact codec (8 elements per lane and step) and dots it with the staged rows: what
+ * tf_qmatvec_expert computes per token (common/transformer.h:517-548), grouped by expert so that a
+ * row is decoded once per 8 tokens.
  * NX = 1: activations are the tokens' bf16 rows X[token] (gate, up); NX = 2: the bf16 head and tail
  * of the intermediate, by slot (down), and the result is scaled by the pair's routing weight. */
+constexpr int kAnyRows = 16, kAnyTok = 8, kAnyChunk = 1024;
+
 template <uint32_t T, int NX>
 __global__ void __launch_bounds__(256)
 moe_rows_any_kernel(const uint8_t *__restrict__ W, int rows_per_expert, int n_cols, size_t row_bytes,
@@ -488,67 +492,85 @@ moe_rows_any_kernel(const uint8_t *__restrict__ W, int rows_per_expert, int n_co
                     const uint16_t *__restrict__ X0, const uint16_t *__restrict__ X1,
                     const float *__restrict__ w_slot, float *__restrict__ out) {
     using C = Codec<T>;
-    constexpr int GPB = C::BE / 8, TT = 8;
+    constexpr int GPB = C::BE / 8, RW = kAnyRows / 4; /* rows per wave */
+    static_assert(kAnyChunk % 256 == 0, "a chunk is a whole number of blocks of every format");
+    extern __shared__ __attribute__((aligned(16))) float xs[]; /* [kAnyTok][chunk] */
     const int e = blockIdx.y;
     const int first = offsets[e], cnt = offsets[e + 1] - first;
     if (cnt == 0) return;
-    const int lane = threadIdx.x & 63;
-    const int row = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    if (row >= rows_per_expert) return; /* whole waves leave; there is no barrier below */
-    const uint8_t *Wr = W + ((size_t)e * rows_per_expert + row) * row_bytes;
-    const int groups = (n_cols / C::BE) * GPB;
-    for (int t0 = 0; t0 < cnt; t0 += TT) {
-        const uint16_t *xa[TT], *xb[TT];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int row0 = blockIdx.x * kAnyRows + wv * RW;
+    const int chunk = n_cols < kAnyChunk ? n_cols : kAnyChunk;
+    for (int t0 = 0; t0 < cnt; t0 += kAnyTok) {
+        const int n_live = cnt - t0 < kAnyTok ? cnt - t0 : kAnyTok;
+        float acc[RW][kAnyTok];
 #pragma unroll
-        for (int t = 0; t < TT; t++) {
-            const int slot = first + (t0 + t < cnt ? t0 + t : t0); /* past the end: a valid row, result unused */
-            if (NX == 1) {
-                xa[t] = X0 + (size_t)(order[slot] / top_k) * n_cols;
-                xb[t] = nullptr;
-            } else {
-                xa[t] = X0 + (size_t)slot * n_cols;
-                xb[t] = X1 + (size_t)slot * n_cols;
-            }
-        }
-        float acc[TT];
+        for (int r = 0; r < RW; r++)
 #pragma unroll
-        for (int t = 0; t < TT; t++) acc[t] = 0.0f;
-        for (int g = lane; g < groups; g += 64) {
-            const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
-            float w[8];
-            C::decode8(Wr + (size_t)blk * C::BB, k0, w);
-            const size_t at = (size_t)blk * C::BE + k0;
+            for (int t = 0; t < kAnyTok; t++) acc[r][t] = 0.0f;
+        for (int c0 = 0; c0 < n_cols; c0 += chunk) {
+            const int c_len = n_cols - c0 < chunk ? n_cols - c0 : chunk;
+            __syncthreads(); /* the previous chunk has been consumed */
+            /* stage: 8 elements per thread and step */
+            for (int i = threadIdx.x; i < n_live * (c_len / 8); i += 256) {
+                const int t = i / (c_len / 8), k8 = i - t * (c_len / 8);
+                const int slot = first + t0 + t;
+                const size_t src = (NX == 1 ? (size_t)(order[slot] / top_k) : (size_t)slot) * n_cols + c0 + 8 * k8;
+                const uint4 a = *reinterpret_cast<const uint4 *>(X0 + src);
+                const uint32_t av[4] = {a.x, a.y, a.z, a.w};
+                float x[8];
 #pragma unroll
-            for (int t = 0; t < TT; t++) {
-                if (t0 + t < cnt) {
-                    const uint4 a = *reinterpret_cast<const uint4 *>(xa[t] + at);
-                    const uint32_t av[4] = {a.x, a.y, a.z, a.w};
-                    float x[8];
+                for (int q = 0; q < 4; q++) {
+                    x[2 * q] = __uint_as_float(av[q] << 16);
+                    x[2 * q + 1] = __uint_as_float(av[q] & 0xFFFF0000u);
+                }
+                if (NX == 2) {
+                    const uint4 b = *reinterpret_cast<const uint4 *>(X1 + src);
+                    const uint32_t bv[4] = {b.x, b.y, b.z, b.w};
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        x[2 * i] = __uint_as_float(av[i] << 16);
-                        x[2 * i + 1] = __uint_as_float(av[i] & 0xFFFF0000u);
+                    for (int q = 0; q < 4; q++) {
+                        x[2 * q] += __uint_as_float(bv[q] << 16);
+                        x[2 * q + 1] += __uint_as_float(bv[q] & 0xFFFF0000u);
                     }
-                    if (NX == 2) {
-                        const uint4 b = *reinterpret_cast<const uint4 *>(xb[t] + at);
-                        const uint32_t bv[4] = {b.x, b.y, b.z, b.w};
+                }
+                float4 *dst = reinterpret_cast<float4 *>(xs + (size_t)t * chunk + 8 * k8);
+                dst[0] = make_float4(x[0], x[1], x[2], x[3]);
+                dst[1] = make_float4(x[4], x[5], x[6], x[7]);
+            }
+            __syncthreads();
+            const int groups = c_len / 8, g0 = c0 / 8;
+            for (int g = lane; g < groups; g += 64) {
+                const int gg = g0 + g, blk = gg / GPB, k0 = (gg - blk * GPB) * 8;
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            x[2 * i] += __uint_as_float(bv[i] << 16);
-                            x[2 * i + 1] += __uint_as_float(bv[i] & 0xFFFF0000u);
+                for (int r = 0; r < RW; r++) {
+                    const int row = row0 + r < rows_per_expert ? row0 + r : rows_per_expert - 1;
+                    float w[8];
+                    C::decode8(W + ((size_t)e * rows_per_expert + row) * row_bytes + (size_t)blk * C::BB, k0, w);
+#pragma unroll
+                    for (int t = 0; t < kAnyTok; t++) {
+                        if (t < n_live) {
+                            const float4 xa = *reinterpret_cast<const float4 *>(xs + (size_t)t * chunk + 8 * g);
+                            const float4 xb = *reinterpret_cast<const float4 *>(xs + (size_t)t * chunk + 8 * g + 4);
+                            float a = acc[r][t];
+                            a = fmaf(w[0], xa.x, a); a = fmaf(w[1], xa.y, a); a = fmaf(w[2], xa.z, a); a = fmaf(w[3], xa.w, a);
+                            a = fmaf(w[4], xb.x, a); a = fmaf(w[5], xb.y, a); a = fmaf(w[6], xb.z, a); a = fmaf(w[7], xb.w, a);
+                            acc[r][t] = a;
                         }
                     }
-#pragma unroll
-                    for (int i = 0; i < 8; i++) acc[t] = fmaf(w[i], x[i], acc[t]);
                 }
             }
         }
 #pragma unroll
-        for (int t = 0; t < TT; t++) {
-            const float sum = wave_sum_dpp(acc[t]);
-            if (lane == 0 && t0 + t < cnt) {
-                const int slot = first + t0 + t;
-                out[(size_t)slot * rows_per_expert + row] = w_slot ? w_slot[slot] * sum : sum;
+        for (int r = 0; r < RW; r++) {
+#pragma unroll
+            for (int t = 0; t < kAnyTok; t++) {
+                if (t < n_live) { /* uniform over the wave: the reduction runs with all lanes */
+                    const float sum = wave_sum_dpp(acc[r][t]);
+                    if (lane == 0 && row0 + r < rows_per_expert) {
+                        const int slot = first + t0 + t;
+                        out[(size_t)slot * rows_per_expert + row0 + r] = w_slot ? w_slot[slot] * sum : sum;
+                    }
+                }
             }
         }
     }
@@ -568,18 +590,31 @@ moe_silu_split_kernel(const float *__restrict__ g32, const float *__restrict__ u
     h_lo[i] = __builtin_bit_cast(uint16_t, lo);
 }
 
+template <uint32_t T, int NX>
+hipError_t launch_rows_any_typed(const void *W, int rows_per_expert, int n_cols, int n_expert, const Workspace &ws,
+                                 int top_k, const uint16_t *X0, const uint16_t *X1, const float *w_slot, float *out,
+                                 hipStream_t stream) {
+    static bool lds_raised = false;
+    const size_t lds = (size_t)kAnyTok * (n_cols < kAnyChunk ? n_cols : kAnyChunk) * sizeof(float);
+    if (!lds_raised) { /* 8 x 1024 floats = 32 KB: several workgroups per compute unit */
+        hipError_t e = hipFuncSetAttribute((const void *)moe_rows_any_kernel<T, NX>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)((size_t)kAnyTok * kAnyChunk * sizeof(float)));
+        if (e != hipSuccess) return e;
+        lds_raised = true;
+    }
+    hipLaunchKernelGGL((moe_rows_any_kernel<T, NX>), dim3((rows_per_expert + kAnyRows - 1) / kAnyRows, n_expert), dim3(256),
+                       lds, stream, (const uint8_t *)W, rows_per_expert, n_cols,
+                       (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB, ws.offsets, ws.order, top_k, X0, X1, w_slot, out);
+    return hipGetLastError();
+}
+
 template <int NX>
 hipError_t launch_rows_any(uint32_t type, const void *W, int rows_per_expert, int n_cols, int n_expert,
                            const Workspace &ws, int top_k, const uint16_t *X0, const uint16_t *X1,
                            const float *w_slot, float *out, hipStream_t stream) {
-    const dim3 grid((rows_per_expert + 3) / 4, n_expert);
     switch (type) {
-#define QLIN_CASE(TT)                                                                                              \
-    case TT:                                                                                                       \
-        hipLaunchKernelGGL((moe_rows_any_kernel<TT, NX>), grid, dim3(256), 0, stream, (const uint8_t *)W,          \
-                           rows_per_expert, n_cols, (size_t)(n_cols / Codec<TT>::BE) * Codec<TT>::BB, ws.offsets,  \
-                           ws.order, top_k, X0, X1, w_slot, out);                                                  \
-        return hipGetLastError();
+#define QLIN_CASE(TT) \
+    case TT: return launch_rows_any_typed<TT, NX>(W, rows_per_expert, n_cols, n_expert, ws, top_k, X0, X1, w_slot, out, stream);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
     QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
 #undef QLIN_CASE
