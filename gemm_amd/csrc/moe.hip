@@ -13,23 +13,77 @@
 
 namespace qlin {
 
+/* Probabilities live in registers, PL per lane (expert e = lane + 64 j); every selection step is one
+ * wave maximum on the cross-lane data path plus a ballot for the lowest expert index holding it. The
+ * general form (more than 64 * 8 experts) keeps them in LDS and reads them back per step. */
+template <int PL>
 __global__ void __launch_bounds__(64)
 moe_route_kernel(const float *__restrict__ logits, int n_expert, int top_k, int32_t *__restrict__ idx,
                  float *__restrict__ wgt) {
+    const int tok = blockIdx.x, lane = threadIdx.x;
+    const float *lg = logits + (size_t)tok * n_expert;
+    float p[PL];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PL; j++) {
+        const int e = lane + 64 * j;
+        p[j] = e < n_expert ? lg[e] : -INFINITY;
+        mx = fmaxf(mx, p[j]);
+    }
+    mx = wave_max_dpp(mx);
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < PL; j++) {
+        const int e = lane + 64 * j;
+        p[j] = e < n_expert ? expf(p[j] - mx) : -1.0f; /* empty slots never win */
+        sum += e < n_expert ? p[j] : 0.0f;
+    }
+    sum = wave_sum_dpp(sum);
+#pragma unroll
+    for (int j = 0; j < PL; j++)
+        if (lane + 64 * j < n_expert) p[j] /= sum;
+    float wsum = 0.0f, mine = 0.0f; /* lane k keeps the k-th weight (top_k <= 64) */
+    int mine_idx = 0;
+    for (int k = 0; k < top_k; k++) {
+        float best = -1.0f;
+#pragma unroll
+        for (int j = 0; j < PL; j++) best = fmaxf(best, p[j]);
+        best = wave_max_dpp(best);
+        /* the lowest expert index among those that hold the maximum: slots j in order, lowest lane first */
+        int bi = 0x7FFFFFFF;
+#pragma unroll
+        for (int j = 0; j < PL; j++) {
+            const unsigned long long m = __ballot(p[j] == best);
+            if (bi == 0x7FFFFFFF && m != 0ull) bi = __builtin_ctzll(m) + 64 * j;
+        }
+#pragma unroll
+        for (int j = 0; j < PL; j++)
+            if (lane + 64 * j == bi) p[j] = -2.0f;
+        if (lane == k) { mine = best; mine_idx = bi; }
+        wsum += best;
+    }
+    if (lane < top_k) {
+        idx[(size_t)tok * top_k + lane] = mine_idx;
+        wgt[(size_t)tok * top_k + lane] = wsum > 0.0f ? mine / wsum : mine;
+    }
+}
+
+__global__ void __launch_bounds__(64)
+moe_route_lds_kernel(const float *__restrict__ logits, int n_expert, int top_k, int32_t *__restrict__ idx,
+                     float *__restrict__ wgt) {
     extern __shared__ float prob[]; /* n_expert floats */
     const int tok = blockIdx.x, lane = threadIdx.x;
     const float *lg = logits + (size_t)tok * n_expert;
     float mx = -INFINITY;
     for (int e = lane; e < n_expert; e += 64) mx = fmaxf(mx, lg[e]);
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    mx = wave_max_dpp(mx);
     float sum = 0.0f;
     for (int e = lane; e < n_expert; e += 64) {
         const float p = expf(lg[e] - mx);
         prob[e] = p;
         sum += p;
     }
-    sum = wave_sum(sum);
+    sum = wave_sum_dpp(sum);
     __syncthreads();
     for (int e = lane; e < n_expert; e += 64) prob[e] /= sum;
     __syncthreads();
@@ -80,8 +134,19 @@ axpy_dev_weight_kernel(float *__restrict__ out, const float *__restrict__ q, con
 hipError_t launch_moe_route(const float *logits, int n_tok, int n_expert, int top_k, int32_t *idx,
                             float *w, hipStream_t s) {
     if (n_tok == 0) return hipSuccess;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(n_tok), dim3(64), (size_t)n_expert * sizeof(float), s,
-                       logits, n_expert, top_k, idx, w);
+    if (top_k <= 64 && n_expert <= 64 * 8) {
+        if (n_expert <= 64)
+            hipLaunchKernelGGL(moe_route_kernel<1>, dim3(n_tok), dim3(64), 0, s, logits, n_expert, top_k, idx, w);
+        else if (n_expert <= 128)
+            hipLaunchKernelGGL(moe_route_kernel<2>, dim3(n_tok), dim3(64), 0, s, logits, n_expert, top_k, idx, w);
+        else if (n_expert <= 256)
+            hipLaunchKernelGGL(moe_route_kernel<4>, dim3(n_tok), dim3(64), 0, s, logits, n_expert, top_k, idx, w);
+        else
+            hipLaunchKernelGGL(moe_route_kernel<8>, dim3(n_tok), dim3(64), 0, s, logits, n_expert, top_k, idx, w);
+    } else {
+        hipLaunchKernelGGL(moe_route_lds_kernel, dim3(n_tok), dim3(64), (size_t)n_expert * sizeof(float), s,
+                           logits, n_expert, top_k, idx, w);
+    }
     return hipGetLastError();
 }
 

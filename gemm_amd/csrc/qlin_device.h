@@ -320,6 +320,15 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
     return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 
+/* maximum over the 64 lanes, same moves; uniform result. NaN inputs are ignored (fmaxf). */
+__device__ __forceinline__ float wave_max_dpp(float v) {
+    v = fmaxf(v, dpp_mov<0xB1>(v));
+    v = fmaxf(v, dpp_mov<0x4E>(v));
+    v = fmaxf(v, dpp_mov<0x141>(v));
+    v = fmaxf(v, dpp_mov<0x140>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
+}
+
 /* Kernel-side view of one fused matvec launch: up to three matrices of one block type that share
  * x (host-side GemvJob, flattened so that nothing is indexed dynamically). mode 0: y = W.x,
  * 1: y += W.x, 2: y0 = silu(W0.x) * (W1.x) with n0 == n1. */

@@ -215,3 +215,43 @@ def test_token_ffn_with_one_format_per_tensor(oracle, types):
                                         types[1], types[2], n_embd, n_ff, n_expert, k, logits.ctypes.data,
                                         x.ctypes.data) == 0
     assert rel_l2(out, want) <= TOL
+
+
+@pytest.mark.parametrize("n_expert,k", [(5, 1), (5, 5), (64, 8), (65, 8), (128, 8), (200, 64), (300, 4), (512, 8),
+                                        (513, 8), (1000, 2), (128, 100)])
+def test_routing_over_expert_counts(oracle, n_expert, k):
+    """register-resident form up to 512 experts and 64 picks, LDS form beyond; same experts and weights as
+    the oracle, in descending weight order"""
+    lib = qlinear.load()
+    n_tok = 9
+    lg = synth.make_router_logits(n_tok, n_expert, seed=n_expert + k)
+    dl = qlinear.DevBuf.from_numpy(lg)
+    di, dw = qlinear.DevBuf(n_tok * k * 4), qlinear.DevBuf(n_tok * k * 4)
+    assert lib.qlin_moe_route_dev(dl.ptr, n_tok, n_expert, k, di.ptr, dw.ptr, None) == 0
+    qlinear.sync()
+    gi, gw = di.to_numpy(np.int32, (n_tok, k)), dw.to_numpy(np.float32, (n_tok, k))
+    for t in range(n_tok):
+        oi, ow = oracle.moe_route(lg[t], k)
+        order_o, order_g = np.argsort(oi), np.argsort(gi[t])
+        assert np.array_equal(oi[order_o], gi[t][order_g]), (t, n_expert, k)
+        assert np.allclose(ow[order_o], gw[t][order_g], rtol=1e-5, atol=1e-8)
+        assert np.all(np.diff(gw[t]) <= 0)
+    for b in (dl, di, dw):
+        b.free()
+
+
+@pytest.mark.parametrize("n_expert", [100, 600])
+def test_routing_ties_take_the_lower_expert_index(n_expert):
+    lib = qlinear.load()
+    lg = np.zeros((1, n_expert), np.float32)          # all equal: the first k experts, in index order
+    lg[0, 70] = 1.0                                   # one clear winner first
+    k = 6
+    dl = qlinear.DevBuf.from_numpy(lg)
+    di, dw = qlinear.DevBuf(k * 4), qlinear.DevBuf(k * 4)
+    assert lib.qlin_moe_route_dev(dl.ptr, 1, n_expert, k, di.ptr, dw.ptr, None) == 0
+    qlinear.sync()
+    assert list(di.to_numpy(np.int32, (k,))) == [70, 0, 1, 2, 3, 4]
+    w = dw.to_numpy(np.float32, (k,))
+    assert abs(float(w.sum()) - 1.0) < 1e-6 and w[0] > w[1] and np.all(w[1:] == w[1])
+    for b in (dl, di, dw):
+        b.free()
