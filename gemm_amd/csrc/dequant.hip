@@ -76,25 +76,32 @@ dequant_bf16_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, i
                     size_t row_bytes, int blocks_per_row) {
     using C = Codec<T>;
     constexpr int GPB = C::BE / 8;
-    const long long gid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    /* a thread decodes two 8-element groups half a workgroup's span apart, so that each of its two
+     * 16-byte stores is part of a contiguous 4 KB of the workgroup */
     const long long groups_per_row = (long long)blocks_per_row * GPB;
-    if (gid >= groups_per_row * n_rows) return;
-    const int row = (int)(gid / groups_per_row);
-    const int g = (int)(gid - (long long)row * groups_per_row);
-    const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
-    float y[8];
-    C::decode8(W + (size_t)row * row_bytes + (size_t)blk * C::BB, k0, y);
+    const long long n_groups = groups_per_row * n_rows;
+    const long long base = (long long)blockIdx.x * 512 + threadIdx.x;
     typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
-    uint4 v;
-    uint32_t *vp = &v.x;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        bf16x2 r;
-        r[0] = (__bf16)y[2 * i];
-        r[1] = (__bf16)y[2 * i + 1];
-        vp[i] = __builtin_bit_cast(uint32_t, r);
+    for (int h = 0; h < 2; h++) {
+        const long long gid = base + 256 * h;
+        if (gid >= n_groups) return;
+        const int row = (int)(gid / groups_per_row);
+        const int g = (int)(gid - (long long)row * groups_per_row);
+        const int blk = g / GPB, k0 = (g - blk * GPB) * 8;
+        float y[8];
+        C::decode8(W + (size_t)row * row_bytes + (size_t)blk * C::BB, k0, y);
+        uint4 v;
+        uint32_t *vp = &v.x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            bf16x2 r;
+            r[0] = (__bf16)y[2 * i];
+            r[1] = (__bf16)y[2 * i + 1];
+            vp[i] = __builtin_bit_cast(uint32_t, r);
+        }
+        *reinterpret_cast<uint4 *>(out + (size_t)row * n_cols + (size_t)blk * C::BE + k0) = v;
     }
-    *reinterpret_cast<uint4 *>(out + (size_t)row * n_cols + (size_t)blk * C::BE + k0) = v;
 }
 
 template <uint32_t T>
@@ -103,7 +110,7 @@ static hipError_t launch_bf16_typed(const void *W, uint16_t *out, int n_rows, in
     const int bpr = n_cols / Codec<T>::BE;
     const long long groups = (long long)bpr * (Codec<T>::BE / 8) * n_rows;
     if (groups == 0) return hipSuccess;
-    hipLaunchKernelGGL((dequant_bf16_kernel<T>), dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, stream,
+    hipLaunchKernelGGL((dequant_bf16_kernel<T>), dim3((unsigned)((groups + 511) / 512)), dim3(256), 0, stream,
                        (const uint8_t *)W, out, n_rows, n_cols, row_bytes, bpr);
     return hipGetLastError();
 }
