@@ -35,7 +35,17 @@ struct Plan {
 
 std::mutex g_mu;
 hipblasLtHandle_t g_handle = nullptr;
-std::map<std::array<long long, 5>, Plan> g_plans; /* (n_rows, n_cols, n_tok, ldx, ldy) -> plan; lives for the process */
+std::map<std::array<long long, 5>, Plan> g_plans; /* (n_rows, n_cols, n_tok, ldx, ldy) -> plan; at most kMaxPlans */
+
+constexpr size_t kMaxPlans = 512;
+
+void destroy_plan(Plan &p) {
+    if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+    if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+    if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    p = Plan();
+}
 
 const char *make_plan(Plan &p, long long n_rows, long long n_cols, long long n_tok, long long ldx, long long ldy,
                       size_t lib_ws_bytes) {
@@ -78,8 +88,15 @@ const char *launch_gemm_dense_bf16(const uint16_t *Wd, const uint16_t *X, float 
     const std::array<long long, 5> key = {n_rows, n_cols, n_tok, ldx, ldy};
     auto it = g_plans.find(key);
     if (it == g_plans.end()) {
+        if (g_plans.size() >= kMaxPlans) { /* a caller with ever-changing token counts: start over */
+            for (auto &kv : g_plans) destroy_plan(kv.second);
+            g_plans.clear();
+        }
         Plan p;
-        if (const char *err = make_plan(p, n_rows, n_cols, n_tok, ldx, ldy, lib_ws_bytes)) return err;
+        if (const char *err = make_plan(p, n_rows, n_cols, n_tok, ldx, ldy, lib_ws_bytes)) {
+            destroy_plan(p);
+            return err;
+        }
         it = g_plans.emplace(key, p).first;
     }
     const Plan &p = it->second;

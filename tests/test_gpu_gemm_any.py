@@ -150,3 +150,28 @@ def test_host_pointer_prefill_on_the_matrix_cores_when_opted_in(oracle, tid):
     assert 1e-5 < err <= 3e-3, err  # the bf16 route really ran, and inside its contract
     assert rel_l2(few, want[:5]) <= 1e-5
     assert rel_l2(qlinear.gemm_tokenmajor(tid, W, X, n_cols), want) <= 1e-5  # and the switch is off again
+
+
+def test_more_shapes_than_the_plan_cache_holds():
+    """the dense GEMM keeps one library plan per shape, at most 512: a caller with ever-changing token counts
+    makes it start over, and results stay right on both sides of that"""
+    n_rows, n_cols = 64, 64
+    rng = np.random.default_rng(5)
+    Wf = rng.standard_normal((n_rows, n_cols)).astype(np.float32)
+    Wb = synth.to_bf16_bits(Wf)
+    Wd = synth.bf16_bits_to_f32(Wb).astype(np.float64)
+    dW = qlinear.DevBuf.from_numpy(Wb.view(np.uint8))
+    ws = qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+    n_max = 530
+    Xb = synth.to_bf16_bits(rng.standard_normal((n_max, n_cols)).astype(np.float32))
+    dX, dY = qlinear.DevBuf.from_numpy(Xb), qlinear.DevBuf(n_max * n_rows * 4)
+    want = synth.bf16_bits_to_f32(Xb).astype(np.float64) @ Wd.T
+    for n_tok in range(1, n_max + 1):
+        qlinear.gemm_bf16_any_dev(synth.GGML_BF16, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
+        if n_tok in (1, 2, 511, 512, 513, 514, n_max):
+            qlinear.sync()
+            got = dY.to_numpy(np.float32, (n_max, n_rows))[:n_tok]
+            assert rel_l2(got, want[:n_tok]) <= 2e-5, n_tok
+    qlinear.sync()
+    for b in (dW, ws, dX, dY):
+        b.free()
