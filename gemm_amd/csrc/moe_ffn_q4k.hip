@@ -501,6 +501,12 @@ moe_rows_any_kernel(const uint8_t *__restrict__ W, int rows_per_expert, int n_co
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int row0 = blockIdx.x * kAnyRows + wv * RW;
     const int chunk = n_cols < kAnyChunk ? n_cols : kAnyChunk;
+    const uint8_t *wrow[RW];
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+        const int row = row0 + r < rows_per_expert ? row0 + r : rows_per_expert - 1;
+        wrow[r] = W + ((size_t)e * rows_per_expert + row) * row_bytes;
+    }
     for (int t0 = 0; t0 < cnt; t0 += kAnyTok) {
         const int n_live = cnt - t0 < kAnyTok ? cnt - t0 : kAnyTok;
         float acc[RW][kAnyTok];
@@ -541,19 +547,22 @@ moe_rows_any_kernel(const uint8_t *__restrict__ W, int rows_per_expert, int n_co
             const int groups = c_len / 8, g0 = c0 / 8;
             for (int g = lane; g < groups; g += 64) {
                 const int gg = g0 + g, blk = gg / GPB, k0 = (gg - blk * GPB) * 8;
+                float w[RW][8];
 #pragma unroll
                 for (int r = 0; r < RW; r++) {
-                    const int row = row0 + r < rows_per_expert ? row0 + r : rows_per_expert - 1;
-                    float w[8];
-                    C::decode8(W + ((size_t)e * rows_per_expert + row) * row_bytes + (size_t)blk * C::BB, k0, w);
+                    C::decode8(wrow[r] + (size_t)blk * C::BB, k0, w[r]);
+                }
 #pragma unroll
-                    for (int t = 0; t < kAnyTok; t++) {
-                        if (t < n_live) {
-                            const float4 xa = *reinterpret_cast<const float4 *>(xs + (size_t)t * chunk + 8 * g);
-                            const float4 xb = *reinterpret_cast<const float4 *>(xs + (size_t)t * chunk + 8 * g + 4);
+                for (int t = 0; t < kAnyTok; t++) {
+                    if (t < n_live) { /* one read of the token's 8 activations serves the 4 rows */
+                        const float4 xa = *reinterpret_cast<const float4 *>(xs + (size_t)t * chunk + 8 * g);
+                        const float4 xb = *reinterpret_cast<const float4 *>(xs + (size_t)t * chunk + 8 * g + 4);
+#pragma unroll
+                        for (int r = 0; r < RW; r++) {
                             float a = acc[r][t];
-                            a = fmaf(w[0], xa.x, a); a = fmaf(w[1], xa.y, a); a = fmaf(w[2], xa.z, a); a = fmaf(w[3], xa.w, a);
-                            a = fmaf(w[4], xb.x, a); a = fmaf(w[5], xb.y, a); a = fmaf(w[6], xb.z, a); a = fmaf(w[7], xb.w, a);
+                            a = fmaf(w[r][0], xa.x, a); a = fmaf(w[r][1], xa.y, a); a = fmaf(w[r][2], xa.z, a);
+                            a = fmaf(w[r][3], xa.w, a); a = fmaf(w[r][4], xb.x, a); a = fmaf(w[r][5], xb.y, a);
+                            a = fmaf(w[r][6], xb.z, a); a = fmaf(w[r][7], xb.w, a);
                             acc[r][t] = a;
                         }
                     }

@@ -80,25 +80,22 @@ __device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) { /* 2-byte alig
     return ld_u16(p) | (ld_u16(p + 2) << 16);
 }
 
-/* IEEE half -> float, bit-exact for every input like common/ggml_dequant.h:206-229: NaN
- * payloads pass through unquieted, subnormals become m * 2^-24 (exact, and a normal float,
- * so the result does not depend on the denormal mode). */
-__device__ __forceinline__ float half_bits_exact(uint32_t h) {
-    const uint32_t sign = (h & 0x8000u) << 16;
-    const uint32_t e = (h >> 10) & 31u;
-    const uint32_t m = h & 1023u;
-    uint32_t bits;
-    if (e == 31u) bits = sign | 0x7F800000u | (m << 13);
-    else if (e != 0u) bits = sign | ((e + 112u) << 23) | (m << 13);
-    else bits = sign | __float_as_uint((float)m * 0x1p-24f);
-    return __uint_as_float(bits);
-}
-
-/* hardware conversion: exact for finite inputs, may quiet a signalling NaN */
+/* hardware conversion: exact for every finite input (subnormals included) and for infinities;
+ * quiets a signalling NaN */
 __device__ __forceinline__ float half_bits_fast(uint32_t h) {
     union { unsigned short u; _Float16 f; } v;
     v.u = (unsigned short)h;
     return (float)v.f;
+}
+
+/* IEEE half -> float, bit-exact for every input like common/ggml_dequant.h:206-229, whose NaN
+ * payloads pass through unquieted: the hardware conversion, with the bits of a NaN rebuilt by
+ * hand. Written without a branch on the loaded value, so that the loads of several blocks can be
+ * in flight before the first conversion. */
+__device__ __forceinline__ float half_bits_exact(uint32_t h) {
+    const float f = half_bits_fast(h);
+    const uint32_t nan_bits = ((h & 0x8000u) << 16) | 0x7F800000u | ((h & 1023u) << 13);
+    return (h & 0x7FFFu) > 0x7C00u ? __uint_as_float(nan_bits) : f;
 }
 
 /* sign byte of the 2/3-bit i-quants: 7 stored bits + their parity in bit 7
@@ -177,6 +174,9 @@ template <> struct Codec<T_Q5_K> : Geom<T_Q5_K> {
 };
 
 template <> struct Codec<T_Q6_K> : Geom<T_Q6_K> {
+    /* four codes at a time: the low nibbles and the two high bits are combined bytewise into q + 32
+     * (0..63); (float)byte - 32.0f is exact and equals (float)(q), so dl * that rounds like the
+     * reference's d * sc * q. */
     __device__ static void decode8(const uint8_t *blk, int k0, float (&y)[8]) {
         const float d = half_bits_exact(ld_u16(blk + 208));
         const int half = k0 >> 7, r = k0 & 127, seg = r >> 5, l0 = r & 31;
@@ -186,9 +186,11 @@ template <> struct Codec<T_Q6_K> : Geom<T_Q6_K> {
         const float dl = d * (float)sc;
         const int nsh = (seg >> 1) * 4, hsh = 2 * seg;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int q = (((ql[i] >> nsh) & 15) | (((qh[i] >> hsh) & 3) << 4)) - 32;
-            y[i] = dl * (float)q;
+        for (int j = 0; j < 2; j++) {
+            const uint32_t lo = ld_u32_a2(ql + 4 * j), hi = ld_u32_a2(qh + 4 * j);
+            const uint32_t q4 = ((lo >> nsh) & 0x0F0F0F0Fu) | (((hi >> hsh) & 0x03030303u) << 4);
+#pragma unroll
+            for (int i = 0; i < 4; i++) y[4 * j + i] = dl * ((float)((q4 >> (8 * i)) & 255u) - 32.0f);
         }
     }
 };
