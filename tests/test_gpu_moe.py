@@ -195,6 +195,20 @@ def test_grouped_ffn_other_and_mixed_formats(oracle, types, n_tok):
         assert rel_l2(got[t], want[t]) <= 10 * DESIGNED, t
 
 
+@pytest.mark.parametrize("type_id", sorted(synth.TYPE_NAMES), ids=lambda t: ALL_NAMES[t])
+def test_grouped_ffn_every_block_format(oracle, type_id):
+    """all three expert tensors in each of the 24 block formats (Q4_K: the matrix-core kernels; every other
+    format: the any-format kernel with that format's codec)"""
+    types = (type_id, type_id, type_id)
+    n_expert, n_embd, n_ff, k, n_tok = 4, 512, 256, 2, 11
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=900 + type_id, types=types)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=901, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=902), k)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
+    assert rel_l2(got, want) <= DESIGNED, ALL_NAMES[type_id]
+
+
 def test_grouped_ffn_mixed_formats_many_tokens_per_expert_and_ragged_shapes(oracle):
     """two experts, 50 tokens: 8-token passes of the any-format kernel with a ragged tail; n_ff = 96 is not a
     multiple of the matrix-core tiles, so Q4_K gate/up cannot be used and Q8_0 (32-element blocks) is"""
