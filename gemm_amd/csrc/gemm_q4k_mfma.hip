@@ -141,7 +141,11 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
 
     /* register set of one tile in flight from global memory; named members only (a set that
      * lives across the tile loop stays in registers only when nothing indexes it) */
-    struct StepRegs { uint4 x0, x1, x2, x3, hdr; uint2 qs; };
+    struct StepRegs { uint4 x0, x1, x2, x3; uint2 qs; };
+    /* d, dmin and the 6-bit scales and mins of one super-block of this thread's weight row, unpacked once
+     * per super-block (four tiles): bytes 0..3 of sc_lo / mn_lo belong to sub-blocks 0..3, of sc_hi / mn_hi
+     * to sub-blocks 4..7 */
+    struct SbScales { float d, dmin; uint32_t sc_lo, sc_hi, mn_lo, mn_hi; };
     auto x_chunk = [&](int j, int step) {
         /* token rows past the end re-read row 0: their products land in accumulator rows that
          * are never stored */
@@ -152,25 +156,31 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
         if (step >= n_steps) step = n_steps - 1; /* harmless re-read past the end */
         const int sb = step >> 2, c = step & 3;
         const uint8_t *blk = w_ptr + (size_t)sb * 144;
-        r.hdr = *reinterpret_cast<const uint4 *>(blk);
         if (NB == 2) r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * bp);
         else r.qs = make_uint2(*reinterpret_cast<const uint32_t *>(blk + 16 + 32 * c + 4 * bp), 0u);
         r.x0 = x_chunk(0, step); r.x1 = x_chunk(1, step); r.x2 = x_chunk(2, step); r.x3 = x_chunk(3, step);
     };
 
     const float unit = 1.0f / fp8_pair_lo(1u).x;
-    /* the two halves of the work that puts one tile into LDS stage `st` */
-    auto stage_weights = [&](const StepRegs &r, int step, int st) {
-        const int c = step & 3;
-        const uint4 h = r.hdr;
-        const float d = half_bits_fast(h.x & 0xFFFFu) * unit, dmin = half_bits_fast(h.x >> 16);
-        const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
-        const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
-        const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-        const uint32_t sc2 = ((c & 2) ? sc_hi : sc_lo) >> ((c & 1) * 16);
-        const uint32_t mn2 = ((c & 2) ? mn_hi : mn_lo) >> ((c & 1) * 16);
-        const float dl_a = d * (float)(sc2 & 0xFFu), dl_b = d * (float)((sc2 >> 8) & 0xFFu);
-        const float ml_a = dmin * (float)(mn2 & 0xFFu), ml_b = dmin * (float)((mn2 >> 8) & 0xFFu);
+    auto load_hdr = [&](int sb) {
+        if (sb * 4 >= n_steps) sb = n_steps / 4 - 1; /* harmless re-read past the end */
+        return *reinterpret_cast<const uint4 *>(w_ptr + (size_t)sb * 144);
+    };
+    auto unpack_hdr = [&](const uint4 &h, SbScales &sc) {
+        sc.d = half_bits_fast(h.x & 0xFFFFu) * unit;
+        sc.dmin = half_bits_fast(h.x >> 16);
+        sc.sc_lo = h.y & 0x3F3F3F3Fu;
+        sc.mn_lo = h.z & 0x3F3F3F3Fu;
+        sc.sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+        sc.mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+    };
+    /* the two halves of the work that puts one tile into LDS stage `st`; c = which quarter of the
+     * super-block, a constant at every call site */
+    auto stage_weights = [&](const StepRegs &r, const SbScales &sc, int c, int st) {
+        const uint32_t sc2 = ((c & 2) ? sc.sc_hi : sc.sc_lo) >> ((c & 1) * 16);
+        const uint32_t mn2 = ((c & 2) ? sc.mn_hi : sc.mn_lo) >> ((c & 1) * 16);
+        const float dl_a = sc.d * (float)(sc2 & 0xFFu), dl_b = sc.d * (float)((sc2 >> 8) & 0xFFu);
+        const float ml_a = sc.dmin * (float)(mn2 & 0xFFu), ml_b = sc.dmin * (float)((mn2 >> 8) & 0xFFu);
         uint8_t *bt = Bs + st * kBTile;
         /* sub-block 2c (low nibbles) -> k 0..31 = chunks 0..3, sub-block 2c+1 -> chunks 4..7 */
         if (NB == 2) {
@@ -239,58 +249,56 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
      * Stage (i+2) % 3 held tile i-1, whose last fragments were read before the barrier that
      * opens tile i; tile i+1 was completed before that same barrier. */
     StepRegs r0, r1;
+    SbScales sbs;
+    uint4 hdr_next;
     fetch(r0, step0);
     fetch(r1, step0 + 1);
-    stage_weights(r0, step0, 0);
+    unpack_hdr(load_hdr(step0 >> 2), sbs);
+    hdr_next = load_hdr((step0 >> 2) + 1);
+    stage_weights(r0, sbs, 0, 0);
     stage_acts(r0, 0);
     fetch(r0, step0 + 2);
-    stage_weights(r1, step0 + 1, 1);
+    stage_weights(r1, sbs, 1, 1);
     stage_acts(r1, 1);
     fetch(r1, step0 + 3);
     __syncthreads();
     Frags f0, f1;
     load_frags(f0, 0, 0);
     int st = 0; /* stage of the current tile */
-    for (int step = step0; step < n_steps; step += 2) {
-        /* even tile: registers r0 hold tile step+2 */
-        {
-            const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
-            load_frags(f1, st, 1);
-            __builtin_amdgcn_sched_barrier(0); /* keep the operand fetch ahead of the MFMAs it hides behind */
-            stage_weights(r0, step + 2, st2);
-            mma_half(f0);
-            QLIN_INTERLEAVE_8(8)
-            __builtin_amdgcn_sched_barrier(0);
-            load_frags(f0, st1, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            stage_acts(r0, st2);
-            fetch(r0, step + 4);
-            mma_half(f1);
-            QLIN_INTERLEAVE_8(5)
-            __builtin_amdgcn_sched_barrier(0);
-            st = st1;
-        }
-        __syncthreads();
-        /* odd tile: registers r1 hold tile step+3 */
-        {
-            const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
-            load_frags(f1, st, 1);
-            __builtin_amdgcn_sched_barrier(0); /* keep the operand fetch ahead of the MFMAs it hides behind */
-            stage_weights(r1, step + 3, st2);
-            mma_half(f0);
-            QLIN_INTERLEAVE_8(8)
-            __builtin_amdgcn_sched_barrier(0);
-            load_frags(f0, st1, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            stage_acts(r1, st2);
-            fetch(r1, step + 5);
-            mma_half(f1);
-            QLIN_INTERLEAVE_8(5)
-            __builtin_amdgcn_sched_barrier(0);
-            st = st1;
-        }
-        __syncthreads();
+    /* tile STEP + U of a super-block (U = 0..3, a constant); registers R hold tile STEP + U + 2, quarter
+     * (U + 2) % 4 of its super-block, which for U >= 2 is the next one: its header was requested four
+     * tiles ago and is unpacked here, and the one after it is requested */
+#define QLIN_GEMM_TILE(R, STEP, U)                                                                     \
+    {                                                                                                  \
+        const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;                            \
+        load_frags(f1, st, 1);                                                                         \
+        __builtin_amdgcn_sched_barrier(0); /* keep the operand fetch ahead of the MFMAs it hides behind */ \
+        if ((U) == 2) {                                                                                \
+            unpack_hdr(hdr_next, sbs);                                                                 \
+            hdr_next = load_hdr(((STEP) >> 2) + 2);                                                    \
+        }                                                                                              \
+        stage_weights(R, sbs, ((U) + 2) & 3, st2);                                                     \
+        mma_half(f0);                                                                                  \
+        QLIN_INTERLEAVE_8(8)                                                                           \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        load_frags(f0, st1, 0);                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        stage_acts(R, st2);                                                                            \
+        fetch(R, (STEP) + (U) + 4);                                                                    \
+        mma_half(f1);                                                                                  \
+        QLIN_INTERLEAVE_8(5)                                                                           \
+        __builtin_amdgcn_sched_barrier(0);                                                             \
+        st = st1;                                                                                      \
+    }                                                                                                  \
+    __syncthreads();
+
+    for (int step = step0; step < n_steps; step += 4) { /* one super-block of K per pass */
+        QLIN_GEMM_TILE(r0, step, 0)
+        QLIN_GEMM_TILE(r1, step, 1)
+        QLIN_GEMM_TILE(r0, step, 2)
+        QLIN_GEMM_TILE(r1, step, 3)
     }
+#undef QLIN_GEMM_TILE
 
     /* C layout of the 32x32 MFMA: register v of lane l holds row 8*(v/4) + 4*(l/32) + v%4,
      * column l%32. Columns are weight rows, contiguous in the token-major output. */
@@ -335,7 +343,7 @@ hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, 
     /* half a chip's worth of tiles or less (4096 rows at 512 tokens: 128): each tile's K range is cut in
      * two halves that add their results to a zeroed Y; a + b onto zero is the same in either order, so
      * the result stays deterministic (three or more parts would not) */
-    const int k_split = (NB == 1 && n_tiles * m_tiles <= 128 && n_sb >= 4) ? 2 : 1;
+    const int k_split = (NB == 1 && n_tiles * m_tiles <= 128 && n_sb >= 4 && n_sb % 2 == 0) ? 2 : 1;
     if (k_split > 1) {
         hipLaunchKernelGGL(zero_rows_kernel, dim3((n_rows + 255) / 256, n_tok), dim3(256), 0, stream, Y, n_rows, ldy);
     }
