@@ -18,14 +18,16 @@
  * copies 4 x 16 bytes of activations into an LDS ring of three stages; the MFMA operands of a
  * tile are fetched from LDS half a tile ahead of the MFMAs that use them, the decode of tile
  * i+2 is issued in the shadow of the MFMAs of tile i, and global loads run four tiles ahead
- * (two register sets). One barrier per tile. When 128-row tiles would leave compute units
+ * (two register sets). One barrier per tile. The loop is unrolled by the four tiles of a
+ * super-block: d, dmin and the packed scales of the thread's row are unpacked once per super-block.
+ * When 128-row tiles would leave compute units
  * without a workgroup (few tokens, or few rows) the same kernel runs with BN = 64: 4 x 2 waves
  * of 64 tokens x 32 rows, eight 4-byte weight parts per row (M = 128: 66 -> 55 us). When even those
  * tiles number 128 or fewer (4096 rows at 512 tokens), K is cut in two halves that add their results to
  * a zeroed Y (4096 x 14336 at 512 tokens: 166 -> 108 us; two addends onto zero commute, so the result
  * does not depend on which half arrives first).
  *
- * Measured on MI355X at M=512, N=14336, K=4096: 76-78 us, 0.78 PFLOP/s on 224 of 256 compute
+ * Measured on MI355X at M=512, N=14336, K=4096: 76-77 us, 0.79 PFLOP/s on 224 of 256 compute
  * units. Cycle stamps (s_memtime) around the parts of one tile show a tile of about 1920 cycles
  * at a shader clock of 1.75-1.9 GHz under this load (2.0-2.1 GHz in a light kernel), against
  * 1024 cycles of matrix-pipe work per SIMD: the eight operand fetches that follow the barrier
