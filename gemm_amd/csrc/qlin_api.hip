@@ -10,6 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -531,6 +532,9 @@ int qlin_matvec_expert(float *dst, const void *W, uint32_t type, int n_cols, int
     return qlin_matvec(dst, slice, type, n_cols, x, rows_per_expert);
 }
 
+static constexpr size_t kDenseLibWorkspace = (size_t)32 << 20; /* handed to the library GEMM */
+static constexpr int kDenseMinTokens = 8;                     /* below this the vector-ALU kernel is faster than decode + GEMM */
+
 int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, const float *X, int n_rows,
                          int n_tok, int out_stride, int x_stride) {
     if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
@@ -569,6 +573,27 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
             if (const char *err = launch_gemm_dense_bf16(Wd, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, lib_ws,
                                                          (size_t)32 << 20, g.stream))
                 return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+        }
+    } else if (n_tok >= kDenseMinTokens) {
+        /* exact weights, fp32 activations, fp32 accumulation on the matrix cores: bands of rows are decoded
+         * to fp32 scratch (at most 512 MiB at a time) and multiplied by the library's dense fp32 GEMM */
+        int band = (int)std::min<size_t>((size_t)n_rows, std::max<size_t>(256, (((size_t)512 << 20) / ((size_t)n_cols * 4)) & ~(size_t)255));
+        const size_t w_bytes = dense_gemm_weight_bytes_f32(band, n_cols);
+        if (int rc = g.tmp[3].ensure(w_bytes + kDenseLibWorkspace)) return rc;
+        float *Wf = (float *)g.tmp[3].p;
+        void *lib_ws = (char *)g.tmp[3].p + w_bytes;
+        for (int r0 = 0; r0 < n_rows; r0 += band) {
+            const int nr = std::min(band, n_rows - r0);
+            const uint8_t *Wb = (const uint8_t *)dW + (size_t)r0 * rb;
+            const float *Wd = (const float *)Wb; /* fp32 weights are used where they are */
+            if (type != T_F32) {
+                HIP_TRY(launch_dequant(type, Wb, nullptr, nr, Wf, nr, n_cols, rb, g.stream));
+                Wd = Wf;
+            }
+            float *Yd = (float *)g.tmp[1].p + r0;
+            if (launch_gemm_dense(true, Wd, g.tmp[0].p, Yd, nr, n_cols, n_tok, n_cols, n_rows, lib_ws, kDenseLibWorkspace,
+                                  g.stream) != nullptr) /* a shape the library has no kernel for */
+                HIP_TRY(launch_gemm_f32(type, Wb, (const float *)g.tmp[0].p, Yd, nr, n_cols, n_tok, n_cols, n_rows, g.stream));
         }
     } else {
         HIP_TRY(launch_gemm_f32(type, dW, (const float *)g.tmp[0].p, (float *)g.tmp[1].p, n_rows, n_cols, n_tok,
@@ -815,8 +840,6 @@ int qlin_gemm_bf16_dev(uint32_t type, const void *W, const uint16_t *X, float *Y
     return QLIN_OK;
 }
 
-static constexpr size_t kDenseLibWorkspace = (size_t)32 << 20;
-
 size_t qlin_gemm_bf16_any_workspace_bytes(int n_rows, int n_cols) {
     if (n_rows <= 0 || n_cols <= 0) return 0;
     return dense_gemm_weight_bytes(n_rows, n_cols) + kDenseLibWorkspace;
@@ -853,6 +876,40 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     if (const char *err = launch_gemm_dense_bf16(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, lib_ws, kDenseLibWorkspace,
                                                  (hipStream_t)stream))
         return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+    return QLIN_OK;
+}
+
+size_t qlin_gemm_f32_any_workspace_bytes(int n_rows, int n_cols) {
+    if (n_rows <= 0 || n_cols <= 0) return 0;
+    return dense_gemm_weight_bytes_f32(n_rows, n_cols) + kDenseLibWorkspace;
+}
+
+int qlin_gemm_f32_any_dev(uint32_t type, const void *W, const float *X, float *Y, int n_rows, int n_cols,
+                          int n_tok, int ldx, int ldy, void *workspace, size_t workspace_bytes, void *stream) {
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_tok < 0 || ldx < n_cols || ldy < n_rows) return fail(QLIN_ERR_ARG, "bad token count or leading dimension");
+    if (n_rows == 0 || n_tok == 0) return QLIN_OK;
+    if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, type == T_F32 ? 4 : 2) || !aligned(X, 4) || !aligned(Y, 4)) return fail(QLIN_ERR_ARG, "misaligned pointer");
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    if (n_tok < kDenseMinTokens) { /* a few tokens: the vector-ALU kernel, no workspace */
+        HIP_TRY(launch_gemm_f32(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        return QLIN_OK;
+    }
+    if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_f32_any_workspace_bytes(n_rows, n_cols))
+        return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_f32_any_workspace_bytes(n_rows, n_cols) bytes");
+    const float *Wd = (const float *)W; /* fp32 weights are used where they are */
+    if (type != T_F32) {
+        HIP_TRY(launch_dequant(type, W, nullptr, n_rows, (float *)workspace, n_rows, n_cols, row_size(type, n_cols),
+                               (hipStream_t)stream));
+        Wd = (const float *)workspace;
+    }
+    void *lib_ws = (char *)workspace + dense_gemm_weight_bytes_f32(n_rows, n_cols);
+    if (launch_gemm_dense(true, Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, lib_ws, kDenseLibWorkspace, (hipStream_t)stream) != nullptr)
+        HIP_TRY(launch_gemm_f32(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream)); /* no library kernel for this shape */
     return QLIN_OK;
 }
 

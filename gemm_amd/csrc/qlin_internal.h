@@ -72,6 +72,9 @@ hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *
 hipError_t launch_dequant_bf16(uint32_t type, const void *W, uint16_t *out, int n_rows, int n_cols, size_t row_bytes,
                                hipStream_t stream);
 size_t dense_gemm_weight_bytes(int n_rows, int n_cols);
+size_t dense_gemm_weight_bytes_f32(int n_rows, int n_cols);
+const char *launch_gemm_dense(bool fp32_operands, const void *Wd, const void *X, float *Y, int n_rows, int n_cols,
+                              int n_tok, int ldx, int ldy, void *lib_ws, size_t lib_ws_bytes, hipStream_t stream);
 const char *launch_gemm_dense_bf16(const uint16_t *Wd, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                    int ldx, int ldy, void *lib_ws, size_t lib_ws_bytes, hipStream_t stream);
 constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */

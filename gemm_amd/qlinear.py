@@ -110,6 +110,8 @@ SIGNATURES = {
     "qlin_dequant_bf16_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemm_bf16_any_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "qlin_gemm_bf16_any_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, C.c_size_t, _vp]),
+    "qlin_gemm_f32_any_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
+    "qlin_gemm_f32_any_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, C.c_size_t, _vp]),
     "qlin_probe_mfma_bf16": (C.c_int, [C.c_int, _vp, C.POINTER(C.c_double)]),
     "qlin_probe_clocks": (C.c_int, [_vp, C.POINTER(C.c_double)]),
     "qlin_probe_hbm_read": (C.c_int, [_vp, C.c_size_t, _vp]),
@@ -314,6 +316,15 @@ def gemm_bf16_any_workspace_bytes(n_rows, n_cols):
 def gemm_bf16_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, dws, stream=None):
     check(load().qlin_gemm_bf16_any_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy,
                                         dws.ptr if dws is not None else None, dws.nbytes if dws is not None else 0, stream))
+
+
+def gemm_f32_any_workspace_bytes(n_rows, n_cols):
+    return load().qlin_gemm_f32_any_workspace_bytes(n_rows, n_cols)
+
+
+def gemm_f32_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, dws, stream=None):
+    check(load().qlin_gemm_f32_any_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy,
+                                       dws.ptr if dws is not None else None, dws.nbytes if dws is not None else 0, stream))
 
 
 def moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert):

@@ -144,11 +144,13 @@ int qlin_matvec_argmax(int *index, float *value, float *logits, const void *W, u
 int qlin_matvec_expert(float *dst, const void *W, uint32_t ggml_type, int n_cols, int expert,
                        const float *x, int rows_per_expert);
 /* prefill: Y[t*out_stride + r] = dot(W[r,:], X[t*x_stride ...]), r < n_rows, t < n_tok; X fp32.
- * Computed in fp32 (no bf16 rounding) so that it can stand in for the CPU path exactly.
+ * Computed in fp32 (no bf16 rounding) so that it can stand in for the CPU path exactly: with 8 tokens or
+ * more the weights are decoded to fp32 device scratch (bands of at most 512 MiB) and multiplied by the
+ * vendor library's dense fp32 GEMM on the matrix cores; fewer tokens run a vector-ALU kernel.
  *                            tf_gemm_f16_mt_tokenmajor, common/transformer.h:4487
  * qlin_set_prefill_matrix_cores(1), or QLIN_PREFILL_MATRIX_CORES=1 in the environment when the library
- * initialises, sends calls with 8 tokens or more through the matrix cores instead (activations and decoded
- * weights rounded to bf16: relative L2 <= 3e-3 instead of 1e-6; 40x less kernel time at 512 tokens). */
+ * initialises, sends calls with 8 tokens or more through the bf16 matrix-core route instead (activations
+ * and decoded weights rounded to bf16: relative L2 <= 3e-3 instead of 1e-6; 5x less kernel time again). */
 int qlin_set_prefill_matrix_cores(int enable);
 int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t ggml_type, int n_cols, const float *X,
                          int n_rows, int n_tok, int out_stride, int x_stride);
@@ -226,9 +228,22 @@ size_t qlin_gemm_bf16_any_workspace_bytes(int n_rows, int n_cols);
 int qlin_gemm_bf16_any_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,
                            int n_cols, int n_tok, int ldx, int ldy, void *workspace, size_t workspace_bytes,
                            void *stream);
-/* Same contraction in fp32 (X fp32, no rounding of weights or activations); any supported type. */
+/* Same contraction in fp32 (X fp32, no rounding of weights or activations); any supported type.
+ * Vector-ALU kernel, no workspace: the choice for a few tokens. */
 int qlin_gemm_f32_dev(uint32_t ggml_type, const void *W, const float *X, float *Y, int n_rows,
                       int n_cols, int n_tok, int ldx, int ldy, void *stream);
+/* The fp32 contraction for many tokens, any supported type: W is decoded once to fp32 (bit-exact, as
+ * qlin_dequant_dev) into `workspace` and multiplied by the vendor library's dense fp32 GEMM (fp32 operands,
+ * fp32 accumulation on the matrix cores) -- what tf_gemm_f16_mt_tokenmajor (common/transformer.h:4487)
+ * computes for fp32 activations, without the 16-bit rounding of its fast paths. Relative L2 against a
+ * double-precision reference <= 1e-5. Fewer than 8 tokens run the kernel of qlin_gemm_f32_dev and leave the
+ * workspace alone (it may then be NULL). workspace: device memory, 256-byte aligned, at least
+ * qlin_gemm_f32_any_workspace_bytes(n_rows, n_cols) bytes (4 bytes per weight + 32 MiB for the library);
+ * calls that share a workspace must be ordered on one stream. */
+size_t qlin_gemm_f32_any_workspace_bytes(int n_rows, int n_cols);
+int qlin_gemm_f32_any_dev(uint32_t ggml_type, const void *W, const float *X, float *Y, int n_rows,
+                          int n_cols, int n_tok, int ldx, int ldy, void *workspace, size_t workspace_bytes,
+                          void *stream);
 /* Grouped MoE expert FFN over n_tok tokens (the block of common/transformer.h:4045-4131 after the router):
  *   X bf16 [n_tok, n_embd]; expert_idx int32 [n_tok, top_k]; expert_w fp32 [n_tok, top_k];
  *   gate/up: [n_expert][n_ff][n_embd] blocks, down: [n_expert][n_embd][n_ff] blocks;
