@@ -33,6 +33,7 @@ from gemm_amd import qlinear, synth  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
+FP32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 MFMA, published
 Q4K = synth.GGML_Q4_K
 
 # HBM bytes moved per Q4_K 14336x4096 matvec launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
@@ -404,6 +405,9 @@ def probe(args):
     elif args.probe == "gemm_any_q6_K":  # decode to bf16 + dense library GEMM, Q6_K, 512 tokens
         ms = time_gemm_any(synth.GGML_Q6_K, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_any_q6_K", "ms_per_step": ms}))
+    elif args.probe == "gemm_f32_any_q4_K":  # decode to fp32 + dense fp32 library GEMM, Q4_K, 512 tokens
+        ms = time_gemm_f32_any(Q4K, 512, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_f32_any_q4_K", "ms_per_step": ms}))
     elif args.probe == "gemm_fewtok":  # the few-token kernel at 16 tokens
         ms = time_gemm(16, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_fewtok", "ms_per_step": ms}))
@@ -422,6 +426,26 @@ def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
     qlinear.timer_begin()
     for _ in range(steps):
         qlinear.gemm_bf16_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
+    ms = qlinear.timer_end() / steps
+    for b in (dW, dX, dY, ws):
+        b.free()
+    return ms
+
+
+def time_gemm_f32_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
+    """Exact prefill GEMM for any format: decode to fp32 in a workspace + the library's dense fp32 GEMM
+    (fp32 operands and accumulation). -> ms per step"""
+    W = synth.make_weights(type_id, n_rows, n_cols, seed=70 + type_id)
+    X = synth.make_activation(n_cols, seed=71, tokens=n_tok)
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(X)
+    dY = qlinear.DevBuf(n_tok * n_rows * 4)
+    ws = qlinear.DevBuf(qlinear.gemm_f32_any_workspace_bytes(n_rows, n_cols))
+    for _ in range(warmup):
+        qlinear.gemm_f32_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        qlinear.gemm_f32_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
     ms = qlinear.timer_end() / steps
     for b in (dW, dX, dY, ws):
         b.free()
@@ -465,7 +489,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
@@ -509,6 +533,13 @@ def main():
             m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
             anyfmt["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
         extra["prefill_gemm_any_format_14336x4096_decode_to_bf16_plus_library_gemm"] = anyfmt
+        exact = {}
+        for tname, tid, M in (("q4_K", Q4K, 512), ("q6_K", synth.GGML_Q6_K, 512), ("q4_K", Q4K, 64)):
+            m = time_gemm_f32_any(tid, M, 14336, 4096, max(3, args.steps // 60), 1)
+            tfl = 2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12
+            exact["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(tfl, 1),
+                                             "fp32_mfma_frac": round(tfl / FP32_PEAK_TFLOPS, 4)}
+        extra["prefill_gemm_exact_fp32_14336x4096_decode_to_fp32_plus_library_gemm"] = exact
         extra["achievable_on_this_gpu"] = time_achievable()
         extra["q4k_prefill_gemm_roofline"] = {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS,
                                               "unit": "TFLOP/s", "frac": round(tf / BF16_PEAK_TFLOPS, 4),
