@@ -577,7 +577,8 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
     } else if (n_tok >= kDenseMinTokens) {
         /* exact weights, fp32 activations, fp32 accumulation on the matrix cores: bands of rows are decoded
          * to fp32 scratch (at most 512 MiB at a time) and multiplied by the library's dense fp32 GEMM */
-        int band = (int)std::min<size_t>((size_t)n_rows, std::max<size_t>(256, (((size_t)512 << 20) / ((size_t)n_cols * 4)) & ~(size_t)255));
+        const size_t rows_in_512mib = (((size_t)512 << 20) / ((size_t)n_cols * 4)) & ~(size_t)255;
+        const int band = (int)std::min<size_t>((size_t)n_rows, std::max<size_t>(256, rows_in_512mib));
         const size_t w_bytes = dense_gemm_weight_bytes_f32(band, n_cols);
         if (int rc = g.tmp[3].ensure(w_bytes + kDenseLibWorkspace)) return rc;
         float *Wf = (float *)g.tmp[3].p;
