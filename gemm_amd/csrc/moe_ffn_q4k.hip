@@ -450,6 +450,83 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
     }
 }
 
+/* ---- 3b. down for NT consecutive groups of RT * 16 rows of one expert, K <= 256 * waves ----
+ * The same arithmetic as moe_down_kernel, with the workgroup walking NT row groups: the weight image of
+ * group r + 1 is in flight while group r is multiplied, reduced over the waves and stored, and the
+ * expert's activations and routing weights are fetched once for all NT groups. A (expert, 32 rows)
+ * workgroup lives for four or five memory round trips and moves 14 KB of weights; with a handful of them
+ * on a compute unit that bounded the kernel at a quarter of HBM speed. */
+#ifndef MOE_DN_NT
+#define MOE_DN_NT 4
+#endif
+template <int RT, int NT>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
+moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
+                     const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
+                     const float *__restrict__ w_slot, float *__restrict__ part, int n_embd, int n_ff) {
+    constexpr int kRows = 16 * RT, kImage = kRows * kQ4KBlock;
+    constexpr int kImageLoads = (kRows * 9 + 63) / 64; /* direct-to-LDS instructions per image and wave */
+    constexpr int kElems = 256 * RT;                   /* results of one row group and token tile */
+    static_assert(kImageLoads <= 15, "the wait below counts outstanding loads up to 15");
+    extern __shared__ __attribute__((aligned(16))) float red[];
+    const int e = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * (kRows * NT);
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int j = lane & 15, kg = lane >> 4;
+    const int n_sb = n_ff >> 8; /* <= n_waves: wave wv owns super-block wv */
+    const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
+    const uint8_t *d0 = down + ((size_t)e * n_embd + row0) * row_bytes;
+    /* LDS: red [waves][RT][64][4] floats | images [waves][2][RT * 16 rows][144 bytes] | routing weights [16] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * kElems) + wv * (2 * kImage);
+    float *wl = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(red + n_waves * kElems) + n_waves * (2 * kImage));
+    const bool has_k = wv < n_sb;
+
+    for (int t0 = 0; t0 < cnt; t0 += 16) {
+        const bool live = t0 + j < cnt;
+        const size_t at_a = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
+        const uint16_t *const arow[2] = {h_hi + at_a, h_lo + at_a};
+        Acts<2> s;
+        if (has_k) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous token tile's images have returned */
+            image_from_global<RT>(img, d0, d0, kRows, row_bytes, wv, lane);
+            load_acts(s, arow, wv, kg, live);
+        }
+        /* the tile's routing weights go to LDS once: a global load inside the walk would make the compiler
+         * wait for the image in flight as well (the first barrier of the walk publishes them) */
+        if (threadIdx.x < 16) wl[threadIdx.x] = t0 + (int)threadIdx.x < cnt ? w_slot[first + t0 + threadIdx.x] : 0.0f;
+        for (int rt = 0; rt < NT; rt++) {
+            f32x4 acc[RT];
+#pragma unroll
+            for (int w = 0; w < RT; w++) acc[w] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (has_k) {
+                if (rt + 1 < NT) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the other image has been read */
+                    const uint8_t *dn = d0 + (size_t)(rt + 1) * kRows * row_bytes;
+                    image_from_global<RT>(img + ((rt + 1) & 1) * kImage, dn, dn, kRows, row_bytes, wv, lane);
+                    wait_vm_at_most(kImageLoads); /* everything older than those: this group's image, the activations */
+                } else {
+                    wait_vm_at_most(0);
+                }
+                step_math<RT, 2>(img + (rt & 1) * kImage, j, kg, s, acc);
+            }
+#pragma unroll
+            for (int w = 0; w < RT; w++) *reinterpret_cast<f32x4 *>(red + ((wv * RT + w) * 64 + lane) * 4) = acc[w];
+            __syncthreads();
+            for (int idx = threadIdx.x; idx < kElems; idx += blockDim.x) {
+                const TileElem t = tile_elem<RT>(idx);
+                float d = 0.0f;
+                for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
+                if (t0 + t.slot < cnt)
+                    part[(size_t)(first + t0 + t.slot) * n_embd + row0 + rt * kRows + t.row] = wl[t.slot] * d;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 /* ---- 4. out[t] = sum over k, in k order ---- */
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of, float *__restrict__ out,
@@ -728,7 +805,19 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         hipLaunchKernelGGL(moe_silu_split_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, ws.g32, ws.u32,
                            ws.h_hi, ws.h_lo, n);
     }
-    if (fast_dn) {
+    if (fast_dn && n_ff / 256 <= dn_waves && n_embd % (16 * MOE_DN_RT * MOE_DN_NT) == 0) {
+        constexpr int DRT = MOE_DN_RT, DNT = MOE_DN_NT;
+        static bool walk_lds_raised = false;
+        if (!walk_lds_raised) { /* 8 waves: 90 KB */
+            hipError_t e1 = hipFuncSetAttribute((const void *)moe_down_walk_kernel<DRT, DNT>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e1 != hipSuccess) return e1;
+            walk_lds_raised = true;
+        }
+        hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
+                           (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock) + 64, stream,
+                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.w_slot, ws.part, n_embd, n_ff);
+    } else if (fast_dn) {
         constexpr int DRT = MOE_DN_RT;
         hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,

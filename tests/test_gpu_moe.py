@@ -209,6 +209,25 @@ def test_grouped_ffn_every_block_format(oracle, type_id):
     assert rel_l2(got, want) <= DESIGNED, ALL_NAMES[type_id]
 
 
+@pytest.mark.parametrize("types,n_embd,n_ff", [
+    ((Q4K, Q4K, Q4K), 256, 2304),      # 9 super-blocks of K for down: more than its 8 waves, one row group per workgroup
+    ((Q8_0, Q8_0, Q4K), 160, 256),     # 160 rows of down: not a whole number of the four-group walks
+    ((Q4K, Q4K, Q4K), 1024, 512),      # the walk: 8 groups of 4 x 32 rows, two super-blocks of K
+], ids=["long_k", "rows_not_multiple_of_128", "walk"])
+def test_grouped_ffn_down_kernel_variants(oracle, types, n_embd, n_ff):
+    """the Q4_K down projection has two kernels: one row group of 32 per workgroup, and a walk over four
+    groups with the next weight image in flight (K up to 2048, rows a multiple of 128)"""
+    n_expert, k, n_tok = 3, 2, 21
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=950, types=types)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=951, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=952), k)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
+    assert rel_l2(got, want) <= DESIGNED
+    for t in range(n_tok):
+        assert rel_l2(got[t], want[t]) <= 10 * DESIGNED, t
+
+
 def test_grouped_ffn_mixed_formats_many_tokens_per_expert_and_ragged_shapes(oracle):
     """two experts, 50 tokens: 8-token passes of the any-format kernel with a ragged tail; n_ff = 96 is not a
     multiple of the matrix-core tiles, so Q4_K gate/up cannot be used and Q8_0 (32-element blocks) is"""
