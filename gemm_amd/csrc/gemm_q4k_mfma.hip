@@ -333,7 +333,7 @@ __global__ void __launch_bounds__(256) zero_rows_kernel(float *__restrict__ Y, i
 template <int NB>
 hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok, int ldx,
                         int ldy, hipStream_t stream) {
-    static bool lds_raised = false;
+    static OnceFlag lds_raised;
     constexpr int WM = 4, BM = 64 * WM, BN = 64 * NB;
     const int n_sb = n_cols / 256;
     const int m_tiles = (n_tok + BM - 1) / BM;
@@ -349,11 +349,11 @@ hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, 
     if (k_split > 1) {
         hipLaunchKernelGGL(zero_rows_kernel, dim3((n_rows + 255) / 256, n_tok), dim3(256), 0, stream, Y, n_rows, ldy);
     }
-    if (!lds_raised) {
+    if (!lds_raised.is_set()) {
         hipError_t e = hipFuncSetAttribute((const void *)gemm_q4k_bf16_kernel<WM, NB>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
-        lds_raised = true;
+        lds_raised.set();
     }
     hipLaunchKernelGGL((gemm_q4k_bf16_kernel<WM, NB>), dim3(grid, k_split), dim3(128 * WM), lds_bytes, stream,
                        (const uint8_t *)W, X, Y, n_rows, n_sb, n_tok, ldx, ldy, m_tiles, k_split);

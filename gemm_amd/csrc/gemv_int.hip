@@ -571,17 +571,17 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = x_bytes + (size_t)waves * depth * row_bytes + 16; /* + slack for the funnel-shift reads */
     const int n_groups = n_cols >> 5;
-    auto launch = [&](auto kernel, bool &raised) {
-        if (!raised) {
+    auto launch = [&](auto kernel, OnceFlag &raised) {
+        if (!raised.is_set()) {
             *err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (*err != hipSuccess) return;
-            raised = true;
+            raised.set();
         }
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds_bytes, stream, job_view(job), x, n_cols,
                            (int)row_bytes, depth, rows_per_wg);
         *err = hipGetLastError();
     };
-    static bool raised[3] = {false, false, false};
+    static OnceFlag raised[3];
     if (n_groups <= 64) launch(gemv_int_kernel<T, 1>, raised[1]);
     else if (n_groups <= 128) launch(gemv_int_kernel<T, 2>, raised[2]);
     else launch(gemv_int_kernel<T, 0>, raised[0]);

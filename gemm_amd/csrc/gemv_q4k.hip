@@ -286,7 +286,7 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int n_
 /* Launch geometry: one 16-wave workgroup per block of rows, sized so that the grid covers the
  * compute units once (more workgroups only when a block would exceed kMaxRowsPerWg rows). */
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu) {
-    static bool lds_raised = false;
+    static OnceFlag lds_raised;
     const int n_sb = n_cols / 256;
     if (n_sb > 64 || n_sb < 1) return hipErrorInvalidValue;
     const int n_slices = n_sb <= 16 ? 1 : n_sb <= 32 ? 2 : 4;
@@ -304,11 +304,11 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
     int depth = (int)((160 * 1024 - fixed_bytes) / ((size_t)kWaves * kRowImage));
     if (depth > kMaxDepth) depth = kMaxDepth;
     const size_t lds_bytes = fixed_bytes + (size_t)kWaves * depth * kRowImage;
-    if (!lds_raised) {
+    if (!lds_raised.is_set()) {
         hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_kernel,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
-        lds_raised = true;
+        lds_raised.set();
     }
     const JobView view = job_view(job);
     hipLaunchKernelGGL(gemv_q4k_kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, view, x, n_sb, n_slices,

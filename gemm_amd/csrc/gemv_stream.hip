@@ -580,12 +580,12 @@ bool stream_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipS
     if (rows_per_wg < 1) rows_per_wg = 1;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = x_bytes + (size_t)waves * depth * row_bytes + 16; /* + slack for ld8_at */
-    static bool raised = false;
-    if (!raised) {
+    static OnceFlag raised;
+    if (!raised.is_set()) {
         *err = hipFuncSetAttribute((const void *)gemv_stream_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    160 * 1024);
         if (*err != hipSuccess) return true;
-        raised = true;
+        raised.set();
     }
     const JobView view = job_view(job);
     hipLaunchKernelGGL((gemv_stream_kernel<T>), dim3(grid), dim3(waves * 64), lds_bytes, stream, view, x, n_cols,

@@ -680,13 +680,13 @@ template <uint32_t T, int NX>
 hipError_t launch_rows_any_typed(const void *W, int rows_per_expert, int n_cols, int n_expert, const Workspace &ws,
                                  int top_k, const uint16_t *X0, const uint16_t *X1, const float *w_slot, float *out,
                                  hipStream_t stream) {
-    static bool lds_raised = false;
+    static OnceFlag lds_raised;
     const size_t lds = (size_t)kAnyTok * (n_cols < kAnyChunk ? n_cols : kAnyChunk) * sizeof(float);
-    if (!lds_raised) { /* 8 x 1024 floats = 32 KB: several workgroups per compute unit */
+    if (!lds_raised.is_set()) { /* 8 x 1024 floats = 32 KB: several workgroups per compute unit */
         hipError_t e = hipFuncSetAttribute((const void *)moe_rows_any_kernel<T, NX>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)((size_t)kAnyTok * kAnyChunk * sizeof(float)));
         if (e != hipSuccess) return e;
-        lds_raised = true;
+        lds_raised.set();
     }
     hipLaunchKernelGGL((moe_rows_any_kernel<T, NX>), dim3((rows_per_expert + kAnyRows - 1) / kAnyRows, n_expert), dim3(256),
                        lds, stream, (const uint8_t *)W, rows_per_expert, n_cols,
@@ -774,12 +774,12 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
     const int n_pairs = n_tok * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), ((size_t)n_expert * 2 + 16) * sizeof(int32_t), stream, idx,
                        n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, w, ws.w_slot);
-    static bool lds_raised = false;
-    if (!lds_raised) {
+    static OnceFlag lds_raised;
+    if (!lds_raised.is_set()) {
         hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<MOE_GU_RT>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e1 != hipSuccess) return e1;
-        lds_raised = true;
+        lds_raised.set();
     }
     /* Q4_K matrices take the matrix-core kernels; any other format (or a shape their tiles do not divide)
      * the any-format kernel, matrix by matrix: gate and up -> fp32 by slot -> silu(g)*u as head + tail */
@@ -807,12 +807,12 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
     }
     if (fast_dn && n_ff / 256 <= dn_waves && n_embd % (16 * MOE_DN_RT * MOE_DN_NT) == 0) {
         constexpr int DRT = MOE_DN_RT, DNT = MOE_DN_NT;
-        static bool walk_lds_raised = false;
-        if (!walk_lds_raised) { /* 8 waves: 90 KB */
+        static OnceFlag walk_lds_raised;
+        if (!walk_lds_raised.is_set()) { /* 8 waves: 90 KB */
             hipError_t e1 = hipFuncSetAttribute((const void *)moe_down_walk_kernel<DRT, DNT>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e1 != hipSuccess) return e1;
-            walk_lds_raised = true;
+            walk_lds_raised.set();
         }
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock) + 64, stream,

@@ -7,12 +7,22 @@
 #define QLIN_INTERNAL_H
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
 #include "qlin_device.h"
 
 namespace qlin {
+
+/* "this kernel's dynamic LDS limit has been raised": set after hipFuncSetAttribute succeeded. Device entry
+ * points may be called from several threads; raising the limit twice is harmless, a torn flag is not. */
+struct OnceFlag {
+    std::atomic<bool> done{false};
+    bool is_set() const { return done.load(std::memory_order_acquire); }
+    void set() { done.store(true, std::memory_order_release); }
+};
 
 /* out[n_rows, n_cols] = decode(W); n_cols may be ragged: only n_cols / block_elems blocks per
  * row are decoded, row r of W starts at r * row_bytes, row r of out at r * n_cols. With row_ids
