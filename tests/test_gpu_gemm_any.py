@@ -89,14 +89,16 @@ def test_strides_padding_and_workspace_reuse(oracle):
     ws.free()
 
 
+@pytest.mark.parametrize("pad", [0, 12])
 @pytest.mark.parametrize("n_tok,n_rows,n_cols", [(9, 300, 8192), (512, 300, 8192), (64, 4096, 16384)])
-def test_padded_output_with_long_rows(n_tok, n_rows, n_cols):
+def test_padded_output_with_long_rows(n_tok, n_rows, n_cols, pad):
     """few output tiles and a long K: the library's kernels that split K and reduce through a workspace wrote
-    a padded Y (ldy > n_rows) as if it were dense; the plan for such a call offers them no workspace"""
+    a padded Y (ldy > n_rows) as if it were dense; the plan for such a call offers them no workspace
+    (pad = 0: the same shapes with a dense Y, where those kernels are used)"""
     rng = np.random.default_rng(n_tok + n_cols)
     Wb = synth.to_bf16_bits(rng.standard_normal((n_rows, n_cols)).astype(np.float32))
     Xb = synth.to_bf16_bits(rng.standard_normal((n_tok, n_cols)).astype(np.float32))
-    Y = run(synth.GGML_BF16, Wb.view(np.uint8), Xb, n_rows, n_cols, n_tok, ldx=n_cols + 64, ldy=n_rows + 12)
+    Y = run(synth.GGML_BF16, Wb.view(np.uint8), Xb, n_rows, n_cols, n_tok, ldx=n_cols + 64, ldy=n_rows + pad)
     want = synth.bf16_bits_to_f32(Xb).astype(np.float64) @ synth.bf16_bits_to_f32(Wb).astype(np.float64).T
     assert rel_l2(Y[:, :n_rows], want) <= 2e-5
     assert np.all(Y[:, n_rows:] == -3.0)

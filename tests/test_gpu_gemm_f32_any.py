@@ -90,14 +90,16 @@ def test_strides_padding_and_workspace_reuse(oracle):
     ws.free()
 
 
+@pytest.mark.parametrize("pad", [0, 12])
 @pytest.mark.parametrize("n_tok,n_rows,n_cols", [(9, 300, 8192), (512, 300, 8192), (64, 4096, 16384)])
-def test_padded_output_with_long_rows(oracle, n_tok, n_rows, n_cols):
+def test_padded_output_with_long_rows(oracle, n_tok, n_rows, n_cols, pad):
     """few output tiles and a long K: the library's kernels that split K and reduce through a workspace wrote
-    a padded Y (ldy > n_rows) as if it were dense; the plan for such a call offers them no workspace"""
+    a padded Y (ldy > n_rows) as if it were dense; the plan for such a call offers them no workspace
+    (pad = 0: the same shapes with a dense Y, where those kernels are used)"""
     rng = np.random.default_rng(n_tok + n_cols)
     W = rng.standard_normal((n_rows, n_cols)).astype(np.float32)
     X = rng.standard_normal((n_tok, n_cols)).astype(np.float32)
-    Y = run(synth.GGML_F32, W.view(np.uint8), X, n_rows, n_cols, ldx=n_cols + 64, ldy=n_rows + 12)
+    Y = run(synth.GGML_F32, W.view(np.uint8), X, n_rows, n_cols, ldx=n_cols + 64, ldy=n_rows + pad)
     assert rel_l2(Y[:, :n_rows], X.astype(np.float64) @ W.astype(np.float64).T) <= TOL
     assert np.all(Y[:, n_rows:] == -3.0)
 
