@@ -153,6 +153,30 @@ def test_greedy_pick_skips_nan_and_keeps_first():
     assert lib.qlin_matvec_argmax(None, None, None, W.ctypes.data, Q80, 32, x.ctypes.data, n) == qlinear.ERR_ARG
 
 
+@pytest.mark.parametrize("offset_floats", [0, 1])
+@pytest.mark.parametrize("n", [1, 5, 1023, 1024, 1025, 151936])
+def test_greedy_pick_sizes_and_logit_alignment(n, offset_floats):
+    """the pick reads the logits four at a time when their address allows it and one at a time otherwise;
+    slices of the vector end inside a group of four for most n"""
+    lib = qlinear.load()
+    rng = np.random.default_rng(n)
+    q = rng.integers(-127, 120, n).astype(np.int8)
+    hot = sorted({n - 1, n // 2, (n * 3) // 4})
+    q[hot] = 127  # ties: the first of them wins
+    W = np.zeros((n, 34), np.uint8)
+    W[:, 0:2] = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    W[:, 2] = q.view(np.uint8)
+    x = np.zeros(32, np.float32)
+    x[0] = 1.0
+    dW, dx = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(x)
+    dl, dr = qlinear.DevBuf((n + 4) * 4), qlinear.DevBuf(qlinear.ARGMAX_RESULT_BYTES)
+    assert lib.qlin_gemv_argmax_dev(Q80, dW.ptr, dx.ptr, dl.ptr + 4 * offset_floats, dr.ptr, n, 32, None) == 0
+    qlinear.sync()
+    assert dr.to_numpy(np.int32, (2,))[0] == hot[0] and dr.to_numpy(np.float32, (2,))[1] == 127.0
+    for b in (dW, dx, dl, dr):
+        b.free()
+
+
 def test_fused_errors():
     lib = qlinear.load()
     W = synth.make_weights(Q4K, 4, 512, seed=1)
