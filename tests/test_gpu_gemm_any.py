@@ -145,8 +145,8 @@ def test_decode_to_bf16_is_the_codec_rounded_once(oracle, tid):
     dout.free()
 
 
-@pytest.mark.parametrize("tid", [Q4K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ3_S, synth.GGML_F16],
-                         ids=lambda t: ALL[t])
+@pytest.mark.parametrize("tid", [Q4K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ3_S, synth.GGML_F16, synth.GGML_F32,
+                                 synth.GGML_BF16], ids=lambda t: ALL[t])
 def test_host_pointer_prefill_on_the_matrix_cores_when_opted_in(oracle, tid):
     lib = qlinear.load()
     n_tok, n_rows, n_cols = 60, 300, 1024
