@@ -9,8 +9,8 @@
  *
  * Four launches:
  *   1. group:   counting sort of the (token, k) pairs by expert (one workgroup).
- *   2. gate_up: one wavefront per (expert, 32 rows of gate and of up). For every 32-element
- *               sub-block it issues v_mfma_f32_16x16x32_bf16 with
+ *   2. gate_up: one workgroup per (expert, 16 rows of gate and of up), its waves splitting K. For
+ *               every 32-element sub-block a wave issues v_mfma_f32_16x16x32_bf16 with
  *                   A = 16 of the expert's tokens x 32 activations (bf16, as given),
  *                   B = 32 raw 4-bit codes x 16 rows, the codes 0..15 converted to bf16
  *                       (exact), two per instruction, by the scaled fp8 conversion,
@@ -20,7 +20,9 @@
  *               same lanes as S. silu(g)*u is then split into a bf16 head and a bf16 tail
  *               (h = hi + lo up to 2^-17 relative), so the second GEMM sees h to ~fp32.
  *   3. down:    same scheme over K = n_ff with A = hi and A = lo accumulated in one
- *               accumulator; writes w[t,k] * result per pair.
+ *               accumulator; writes w[t,k] * result per pair. A workgroup walks four groups of 32
+ *               rows with the next group's weights in flight (one group per workgroup when K
+ *               exceeds 2048 or the rows are not a multiple of 128).
  *   4. combine: out[t] = the token's top_k partial rows added in k order (deterministic).
  *
  * Lane layout of the 16x16x32 MFMA (A: tokens i, B: rows j): lane l feeds A[i = l%16]
