@@ -1,104 +1,95 @@
 /*
- * gemv_q4k.hip - batch-1 Q4_K matvec tuned for HBM streaming on gfx950.
+ * gemv_q4k.hip - batch-1 Q4_K matvec for gfx950: inner products on the 8-bit integer matrix
+ * instruction, weights read straight from HBM in the operand layout (no LDS staging).
  *
- * Structure (one workgroup of 16 wavefronts per block of rows, about one per compute unit):
+ * y[r] = sum over super-blocks of d*sum_s sc_s*(q_s . x_s) - dmin*sum_s m_s*sum(x_s)
+ * (the factored form of common/ggml_dequant.h:1592-1618 dotted with x; sub-block s = 32 elements,
+ * 6-bit sc/m from get_scale_min_k4, :1582-1590).
  *
- *  1. x -> fixed point, once per workgroup. Each 32-element sub-block of x (the Q4_K scale
- *     granularity, common/ggml_dequant.h:71-76) is scaled by a power of two so that
- *     X = rint(x * 2^(22-e)) fits 23 bits, and the three bytes of X are stored as three
- *     "digit planes" in LDS (top byte signed, lower two unsigned) together with 2^(e-22) and
- *     the fp32 sum of the sub-block. Quantisation error is 2^-23 of the sub-block's largest
- *     |x|; measured end-to-end error is ~7e-7 relative L2 against the double-precision oracle.
- *  2. Weights are streamed as a FLAT byte stream: a wavefront moves a row (or a slice of at
- *     most 16 super-blocks = 2304 bytes of it) with up to three fully contiguous
- *     16-byte-per-lane loads that write straight into a private LDS row image
- *     (global_load_lds_dwordx4: no registers are held while the data is in flight). Only the
- *     flat pattern reaches the streaming rate of a plain copy kernel; lane-owned strided
- *     16-byte loads cost 40 % more time on this part. One row per wavefront in flight (16
- *     per compute unit, 9.4 MB over the chip) already runs HBM at the rate it gives a burst of
- *     this size; deeper rings (the code takes up to four images) measured slower, because
- *     they only lengthen the queue in front of the x loads and of each wave's last row.
- *     The x loads of all 16 waves are issued before any row load (a barrier separates them),
- *     so the x preparation overlaps the first rows instead of waiting behind them.
- *  3. Arithmetic re-reads the row image in the layout it wants: four lanes per super-block,
- *     lane c takes nibble bytes qs[32c..32c+31] = sub-blocks 2c (low nibbles) and 2c+1 (high
- *     nibbles). The nibbles are masked into bytes and multiplied with the digit planes by
- *     4-way integer dot instructions: 48 per row and lane instead of 128 converts and FMAs.
- *     Per sub-block: S = top*65536 + mid*256 + low, y += d*sc*2^(e-22)*S - dmin*m*sum(x)
- *     (the factored form of common/ggml_dequant.h:1592-1618 dotted with x; scales unpacked
- *     four at a time from the 12 packed bytes, get_scale_min_k4, :1582-1590).
- *  4. Rows longer than 16 super-blocks are cut into S = 2 or 4 slices; slice s of a row is
- *     handled by a wave with (wave % S) == s, so every wave keeps ONE slice of the digit
- *     planes in registers for all its rows. Partial sums meet in LDS at the end.
+ *  1. x -> fixed point per 32-element sub-block: X = rint(x * 2^(30-e)), e the exponent of the
+ *     sub-block's largest |x|, written as four SIGNED base-256 digits (top in [-64,64], the others in
+ *     [-128,127]). q_s . x_s = 2^(e-30) * sum_k 256^k * D_k with D_k the exact integer inner products of
+ *     the 4-bit codes with the digit planes. An element keeps all 24 bits of its significand unless it
+ *     is more than 2^7 times smaller than the largest of its sub-block; the error is at most 2^-31 of
+ *     that largest |x| per element, so an outlier 10^5 times the bulk still leaves its 31 neighbours
+ *     14 bits.
+ *  2. The inner products run on v_mfma_i32_16x16x64_i8: 16 weight rows (B operand: the codes, one
+ *     byte each) against 16 "x rows" (A operand). Wave w of a 16-wave workgroup owns super-block w
+ *     (w+16, w+32, w+48 for longer rows) of every row, so it prepares only ITS 256 elements of x - one
+ *     16-byte load per lane, no workgroup-wide x pass, no barrier before the weights are requested.
+ *     Per super-block two chains of two instructions: chain p covers the 64 code bytes [64p, 64p+64)
+ *     = sub-blocks 4p..4p+3; lane group g = lane/16 supplies 16 of those bytes, low nibbles in operand
+ *     registers 0-1, high nibbles in 2-3. The A operand is block-diagonal to match: x-row 4*s'+digit
+ *     (s' = 0..3, digit 3..0) holds the digits of sub-block 4p+s' at exactly the k positions
+ *     that carry that sub-block's codes and zeros elsewhere, so result register r of lane group s' is
+ *     digit plane r of sub-block 4p+s' for weight row lane%16: all 16 x-rows and all 64 lanes are used
+ *     (2 shift-adds, 2 converts, 4 multiply-adds per sub-block and row). About 60 vector instructions per
+ *     (16 rows x super-block) instead of the ~150 per row of a v_dot4 formulation.
+ *  3. Lane (n, g) loads the header and its two 16-byte code chunks of row 16*rg + n directly from HBM:
+ *     per instruction 16 rows x 64 contiguous bytes. Four row groups (12 loads) are in flight per
+ *     wave before the first is used; waves never wait for each other until the final sum over the 16
+ *     super-block shares of a row, which meets in LDS.
+ *
+ * Measured alternatives on this part (14336x4096, period per launch; a bare read of the same bytes with
+ * contiguous 1 KB-per-instruction loads is 6.2 us, with this kernel's access pattern 7.3 us): rows copied
+ * to LDS by global_load_lds as contiguous streams with 16-row tiles handed over by workgroup barriers
+ * 10.3-11.2 us (waves stuck in issue reach the barrier late, and LDS instructions of other waves slow
+ * the incoming copy stream); dedicated copying waves that publish their progress in LDS 10.4 us; each
+ * wave gathering its own 144-byte blocks into LDS 16 us (a gather of short runs costs one access per
+ * lane); a v_dot4 kernel with one row per wave in LDS 8.3-8.6 us, the same as this one, which needs a
+ * third of the vector instructions and no LDS for the weights.
  *
  * A non-finite x makes every output NaN (the fixed-point form cannot carry Inf).
  */
 #include "qlin_device.h"
 #include "qlin_internal.h"
+#include <type_traits>
 
 namespace qlin {
 
 namespace {
 
-#ifndef Q4K_WAVES
-#define Q4K_WAVES 16
-#endif
-constexpr int kWaves = Q4K_WAVES;   /* wavefronts per workgroup: 16 or 8 (a multiple of 4, the most slices) */
-constexpr int kThreads = kWaves * 64;
-constexpr int kChunk = 52;          /* dwords per 64-element x chunk: 3 planes x 16, padded so that
-                                       consecutive lanes' 16-byte reads fall on distinct banks */
-constexpr int kRowImage = 2304;     /* bytes per LDS row image: 16 super-blocks */
-#ifndef Q4K_MAX_DEPTH
-#define Q4K_MAX_DEPTH 1
-#endif
-constexpr int kMaxDepth = Q4K_MAX_DEPTH; /* row images per wavefront */
-constexpr int kMaxRowsPerWg = 128;
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
-__device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_udot4(a, b, c, false); }
+constexpr int kWaves = 16;             /* wavefronts per workgroup */
+constexpr int kMaxKc = 4;               /* 16-super-block column chunks: K <= 16384 */
+constexpr int kMaxRowsPerWg = 128;
+constexpr int kXScratch = 1088;         /* per wave: 4 digit planes x 256 B + 8 x (2^(e-30), sum) */
+/* x operand of one super-block: A[2p+h] for chain p, instruction h; scale[p] = 2^(e-30) and
+ * sum[p] = sum of x for sub-block 4p + lane/16 */
+struct XOperand {
+    v4i A[4];
+    float scale[2], sum[2];
+};
 
 }  // namespace
 
-__global__ void __launch_bounds__(kThreads)
-gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int n_slices, int slice_sb,
-                int rows_per_wg, int depth) {
+template <int NKC>
+__global__ void __launch_bounds__(kWaves * 64)
+gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    /* LDS map: planes [n_sb*4][kChunk] dwords | meta [n_sb*4] float4 | row images [16][depth][kRowImage] |
-     * partial sums [rows_per_wg * n_slices] floats (padded to 16 bytes) | raw x [n_sb*256] floats */
-    uint32_t *planes = reinterpret_cast<uint32_t *>(lds);
-    float4 *meta = reinterpret_cast<float4 *>(planes + n_sb * 4 * kChunk);
-    uint8_t *images = reinterpret_cast<uint8_t *>(meta + n_sb * 4);
-    float *partial = reinterpret_cast<float *>(images + kWaves * depth * kRowImage);
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15, g = lane >> 4;
+
     /* a workgroup owns rows_per_wg rows: of the concatenated matrices, or, where two results are
      * combined (mode 2), the same rows of both matrices (local rows: first matrix, then second) */
     const bool paired = job.mode == 2;
     const int n_mats_here = paired ? 2 : 1;
-    const float4 *xraw = reinterpret_cast<const float4 *>(partial + ((rows_per_wg * n_mats_here * n_slices + 3) & ~3));
-
-    const int lane = threadIdx.x & 63;
-    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); /* wave-uniform, and the compiler is told so */
-    const int c = lane & 3;
-    const int slice = wv % n_slices;
-    const int sb0 = slice * slice_sb;
-    int sb_cnt = n_sb - sb0;
-    if (sb_cnt > slice_sb) sb_cnt = slice_sb;
-    const bool active = (lane >> 2) < sb_cnt;
-    const int sb_local = active ? (lane >> 2) : 0;
-    const size_t row_bytes = (size_t)n_sb * 144;
-    const int n_chunks = sb_cnt * 9;                  /* 16-byte chunks in this wave's slice of a row */
-    const int loads_per_row = (n_chunks + 63) >> 6;   /* wave-uniform: 1, 2 or 3 */
-
     const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
-    const int row0 = blockIdx.x * rows_per_wg; /* first row of this workgroup */
+    const int row0 = blockIdx.x * rows_per_wg;
     int rows_here = n_rows - row0;
     if (rows_here > rows_per_wg) rows_here = rows_per_wg;
-    const int n_lrows = rows_here * n_mats_here;  /* local rows */
-    const int n_vrows = n_lrows * n_slices;       /* (local row, slice) pairs of this workgroup */
+    const int n_lrows = rows_here * n_mats_here;
+    const int n_rg = (n_lrows + 15) >> 4;
+    const size_t row_bytes = (size_t)n_sb * 144;
+    const int n_kc = wv < n_sb ? ((n_sb - wv + 15) >> 4) : 0; /* this wave's super-blocks: wv, wv+16, ... */
 
-    /* this wave's virtual rows: wv, wv + 16, ... ; virtual row j = (row j / S, slice j % S), and
-     * 16 % S == 0 keeps the slice of a wave fixed. my_rows of them, numbered i = 0.. */
-    const int my_rows = wv < n_vrows ? (n_vrows - wv + kWaves - 1) / kWaves : 0;
-    /* where local row lr lives: matrix and row */
+    /* LDS map: x scratch [kWaves][kXScratch] | partial sums [rows][kWaves] */
+    uint8_t *xs = lds + wv * kXScratch;
+    float *partial = reinterpret_cast<float *>(lds + kWaves * kXScratch);
+
     auto locate = [&](int lr, const uint8_t *&Wm, float *&ym, int &r) {
         if (paired) {
             const bool second = lr >= rows_here;
@@ -109,169 +100,201 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int n_
             job_locate(job, row0 + lr, Wm, ym, r);
         }
     };
-    uint8_t *my_images = images + wv * (depth * kRowImage);
-    const uint32_t my_images_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)my_images;
-    /* Row i of this wave -> image slot i % depth; exactly loads_per_row instructions are issued.
-     * Each is a 16-byte-per-lane load whose data goes to LDS at M0 + 16*lane instead of to
-     * registers. They are written as instructions: for the builtin form the compiler, which
-     * cannot tell the images apart, waits for every outstanding one before any LDS access, and
-     * that would serialise the ring. The waits this kernel needs are placed by hand
-     * (wait_vm_at_most before an image is read, lgkmcnt(0) before its slot is refilled).
-     * Nothing else in this kernel uses M0. The rows are marked non-temporal: every weight byte is
-     * read once, and without the mark a launch pushes x, the kernel arguments and its own code out
-     * of the L2 for the next launch (measured: 0.6 us per launch). */
-    auto issue = [&](int i) {
-        const int j = wv + i * kWaves;
+
+    v4f xr[NKC];
+#pragma unroll
+    for (int kc = 0; kc < NKC; kc++) {
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (kc < n_kc) v = *reinterpret_cast<const v4f *>(x + (16 * kc + wv) * 256 + 4 * lane);
+        xr[kc] = v;
+    }
+        /* x -> signed digit planes -> A operands, wave-private */
+    auto prepare = [&](v4f v, XOperand &xo) {
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        float sum = (v.x + v.y) + (v.z + v.w);
+        /* 8 consecutive lanes share one 32-element sub-block */
+        amax = fmaxf(amax, dpp_mov<0xB1>(amax));
+        amax = fmaxf(amax, dpp_mov<0x4E>(amax));
+        amax = fmaxf(amax, dpp_mov<0x141>(amax));
+        sum += dpp_mov<0xB1>(sum);
+        sum += dpp_mov<0x4E>(sum);
+        sum += dpp_mov<0x141>(sum);
+        int e = (int)(__float_as_uint(amax) >> 23) - 126; /* amax in [2^(e-1), 2^e) */
+        if (e < -96) e = -96;                              /* zero and tiny sub-blocks */
+        const float up = __uint_as_float((uint32_t)(127 + 30 - e) << 23);
+        float down = __uint_as_float((uint32_t)(127 - 30 + e) << 23);
+        if (!(amax <= 3.0e38f)) down = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
+        const int X[4] = {__float2int_rn(v.x * up), __float2int_rn(v.y * up), __float2int_rn(v.z * up),
+                          __float2int_rn(v.w * up)};
+        int X1[4], X2[4], X3[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            X1[k] = (X[k] + 128) >> 8;  /* X = 256*X1 + d0, d0 = (int8)X */
+            X2[k] = (X1[k] + 128) >> 8; /* X1 = 256*X2 + d1 */
+            X3[k] = (X2[k] + 128) >> 8; /* X2 = 256*X3 + d2; d3 = X3 in [-64, 64] */
+        }
+        /* byte 0 of four values -> one dword (selector 0-3: second operand, 4-7: first, 0x0c: zero) */
+        auto pack = [](const int (&a)[4]) {
+            const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)a[1], (uint32_t)a[0], 0x0c0c0400u);
+            const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)a[3], (uint32_t)a[2], 0x0c0c0400u);
+            return __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+        };
+        uint32_t *pl = reinterpret_cast<uint32_t *>(xs);
+        pl[lane] = pack(X3);       /* digit 3 (top) */
+        pl[64 + lane] = pack(X2);  /* digit 2 */
+        pl[128 + lane] = pack(X1); /* digit 1 */
+        pl[192 + lane] = pack(X);  /* digit 0 */
+        if ((lane & 7) == 0) reinterpret_cast<float2 *>(xs + 1024)[lane >> 3] = make_float2(down, sum);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        /* A operand: x-row i = lane%16 = 4*s' + plane; k group lane/16 carries sub-blocks 2*(g>>1)
+         * (registers 0-1) and 2*(g>>1)+1 (registers 2-3) of the chain, elements 16*(g&1) + 8h .. +7 */
+        const int sq = n >> 2, plane = n & 3;
+        const bool live = (g >> 1) == (sq >> 1);
+        const uint8_t *src = xs + plane * 256 + 32 * sq + 16 * (g & 1);
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint2 d = *reinterpret_cast<const uint2 *>(src + 128 * p + 8 * h);
+                const bool lo = live && !(sq & 1), hi = live && (sq & 1);
+                v4i a;
+                a.x = lo ? (int)d.x : 0;
+                a.y = lo ? (int)d.y : 0;
+                a.z = hi ? (int)d.x : 0;
+                a.w = hi ? (int)d.y : 0;
+                xo.A[2 * p + h] = a;
+            }
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            const float2 m = reinterpret_cast<const float2 *>(xs + 1024)[4 * p + g];
+            xo.scale[p] = m.x;
+            xo.sum[p] = m.y;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+
+    /* one super-block of 16 rows: header h, code bytes q0 (chain 0) and q1 (chain 1) of this lane */
+    auto item = [&](const XOperand &xo, const uint4 hh, const uint4 qa, const uint4 qb) {
+        constexpr uint32_t M = 0x0F0F0F0Fu;
+        v4i c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
+        v4i b;
+        b.x = (int)(qa.x & M); b.y = (int)(qa.y & M); b.z = (int)((qa.x >> 4) & M); b.w = (int)((qa.y >> 4) & M);
+        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[0], b, c0, 0, 0, 0);
+        b.x = (int)(qb.x & M); b.y = (int)(qb.y & M); b.z = (int)((qb.x >> 4) & M); b.w = (int)((qb.y >> 4) & M);
+        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2], b, c1, 0, 0, 0);
+        b.x = (int)(qa.z & M); b.y = (int)(qa.w & M); b.z = (int)((qa.z >> 4) & M); b.w = (int)((qa.w >> 4) & M);
+        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[1], b, c0, 0, 0, 0);
+        b.x = (int)(qb.z & M); b.y = (int)(qb.w & M); b.z = (int)((qb.z >> 4) & M); b.w = (int)((qb.w >> 4) & M);
+        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[3], b, c1, 0, 0, 0);
+        /* 6-bit scale and min of sub-blocks g (chain 0) and 4+g (chain 1) */
+        const uint32_t sh = 8u * (uint32_t)g;
+        const uint32_t sc0 = __builtin_amdgcn_ubfe(hh.y, sh, 6), mn0 = __builtin_amdgcn_ubfe(hh.z, sh, 6);
+        const uint32_t sc1 = __builtin_amdgcn_ubfe(hh.w, sh, 4) | (__builtin_amdgcn_ubfe(hh.y, sh + 6, 2) << 4);
+        const uint32_t mn1 = __builtin_amdgcn_ubfe(hh.w, sh + 4, 4) | (__builtin_amdgcn_ubfe(hh.z, sh + 6, 2) << 4);
+        const float d = half_bits_fast(hh.x & 0xFFFFu), dmin = half_bits_fast(hh.x >> 16);
+        /* digit sums: |top| <= 32*15*64, the others <= 32*15*128, so each pair below is an integer of less
+         * than 24 bits and its conversion is exact; one rounding in the multiply-add that joins them */
+        const float s0 = fmaf((float)((c0.x << 8) + c0.y), 65536.0f, (float)((c0.z << 8) + c0.w));
+        const float s1 = fmaf((float)((c1.x << 8) + c1.y), 65536.0f, (float)((c1.z << 8) + c1.w));
+        const float z0 = s0 * xo.scale[0], z1 = s1 * xo.scale[1];
+        const float dots = (float)sc0 * z0 + (float)sc1 * z1;
+        const float mins = (float)mn0 * xo.sum[0] + (float)mn1 * xo.sum[1];
+        return d * dots - dmin * mins;
+    };
+    auto row_pointer = [&](int rg) { /* this lane's row of row group rg (rows past the end: the last one, never stored) */
+        int lr = 16 * rg + n;
+        if (lr >= n_lrows) lr = n_lrows - 1;
         const uint8_t *Wm;
         float *ym;
         int r;
-        locate(j / n_slices, Wm, ym, r);
-        const uint4 *g = reinterpret_cast<const uint4 *>(Wm + (size_t)r * row_bytes + (size_t)sb0 * 144);
-        const uint32_t img = __builtin_amdgcn_readfirstlane(my_images_lds + (uint32_t)((i % depth) * kRowImage));
-#define QLIN_LOAD_TO_LDS(chunk0)                                                                          \
-        if ((chunk0) + lane < n_chunks)                                                                   \
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"                 \
-                         : : "v"(g + (chunk0) + lane), "s"(img + 16u * (chunk0)) : "memory")
-        QLIN_LOAD_TO_LDS(0);
-        QLIN_LOAD_TO_LDS(64);
-        QLIN_LOAD_TO_LDS(128);
-#undef QLIN_LOAD_TO_LDS
+        locate(lr, Wm, ym, r);
+        return Wm + (size_t)r * row_bytes + (size_t)wv * 144;
     };
-
-    /* x is requested first, so that it does not queue behind the weight stream: like the rows it
-     * goes straight to LDS (a raw fp32 copy, 1 KB per instruction and wave), so no register holds
-     * data that is still in flight. A barrier makes every wave's x request precede every row
-     * request; then up to `depth` rows per wave are put in flight while x is being prepared.
-     * Loads retire in order, so "at most the row loads outstanding" means that this wave's part
-     * of x has landed; each thread then prepares exactly the elements its own wave fetched. */
-    const int n4 = n_sb * 64;
-    const float4 *xg = reinterpret_cast<const float4 *>(x);
-    const uint32_t xraw_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)xraw;
-    for (int base = wv * 64; base < n4; base += kThreads) { /* uniform per wave */
-        const uint32_t m0v = __builtin_amdgcn_readfirstlane(xraw_lds + 16u * (uint32_t)base);
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     : : "v"(xg + base + lane), "s"(m0v) : "memory");
-    }
-    asm volatile("s_barrier" ::: "memory");
-    int issued = 0;
-    for (; issued < depth && issued < my_rows; issued++) issue(issued);
-    wait_vm_at_most(issued * loads_per_row);
-
-    /* ---- x -> digit planes (whole workgroup, 4 elements per thread and step); no loads in here,
-     * so nothing in it waits for the weights */
-    auto quantize = [&](int idx, const float4 v) {
-            const bool mine = idx < n4;
-            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-            float sum = (v.x + v.y) + (v.z + v.w);
-            /* 8 consecutive threads share one 32-element sub-block */
-            amax = fmaxf(amax, dpp_mov<0xB1>(amax));
-            amax = fmaxf(amax, dpp_mov<0x4E>(amax));
-            amax = fmaxf(amax, dpp_mov<0x141>(amax));
-            sum += dpp_mov<0xB1>(sum);
-            sum += dpp_mov<0x4E>(sum);
-            sum += dpp_mov<0x141>(sum);
-            int e = (int)(__float_as_uint(amax) >> 23) - 126; /* amax in [2^(e-1), 2^e) */
-            if (e < -100) e = -100;                            /* zero and tiny blocks */
-            const float scale = __uint_as_float((uint32_t)(127 + 22 - e) << 23);
-            float inv = __uint_as_float((uint32_t)(127 - 22 + e) << 23);
-            if (!(amax <= 3.0e38f)) inv = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
-            const uint32_t X0 = (uint32_t)__float2int_rn(v.x * scale), X1 = (uint32_t)__float2int_rn(v.y * scale);
-            const uint32_t X2 = (uint32_t)__float2int_rn(v.z * scale), X3 = (uint32_t)__float2int_rn(v.w * scale);
-            /* byte transpose: plane k = byte k of X0..X3 (selector 0-3: second operand, 4-7: first) */
-            const uint32_t lo01 = __builtin_amdgcn_perm(X1, X0, 0x05010400u); /* X0.b0 X1.b0 X0.b1 X1.b1 */
-            const uint32_t lo23 = __builtin_amdgcn_perm(X3, X2, 0x05010400u);
-            const uint32_t hi01 = __builtin_amdgcn_perm(X1, X0, 0x07030602u); /* X0.b2 X1.b2 X0.b3 X1.b3 */
-            const uint32_t hi23 = __builtin_amdgcn_perm(X3, X2, 0x07030602u);
-            const uint32_t pl_low = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); /* bytes 0 of X0..X3 */
-            const uint32_t pl_mid = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u); /* bytes 1 */
-            const uint32_t pl_top = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u); /* bytes 2 */
-            const int sub = idx >> 3, j = idx & 7;
-            const int chunk = sub >> 1, is_b = sub & 1;
-            uint32_t *dst = planes + chunk * kChunk + is_b * 8 + j;
-            if (mine) {
-                dst[0] = pl_top;
-                dst[16] = pl_mid;
-                dst[32] = pl_low;
-            }
-            if (mine && j == 0) {
-                float *m = reinterpret_cast<float *>(meta + chunk);
-                m[is_b] = inv;
-                m[2 + is_b] = sum;
-            }
+    auto store_partial = [&](int rg, float v, bool add) { /* the four lane groups hold four sub-blocks' shares of the same row */
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        const int lr = 16 * rg + n;
+        if (lane < 16 && lr < n_lrows) {
+            float *p = partial + lr * kWaves + wv;
+            *p = add ? *p + v : v;
+        }
     };
-    for (int idx = threadIdx.x; idx < n4; idx += kThreads) quantize(idx, xraw[idx]);
-    __syncthreads();
-
-    /* this lane's x: 16 dwords per plane (8 for sub-block 2c, 8 for 2c+1) */
-    uint32_t xt[16], xm[16], xl[16];
-    {
-        const uint4 *pp = reinterpret_cast<const uint4 *>(planes + ((sb0 + sb_local) * 4 + c) * kChunk);
+    XOperand xo;
+    /* NG row groups of column chunk kc: every block is requested before the first is used */
+    auto run_group = [&](int rg0, int kc, auto ng_tag) {
+        constexpr int NG = decltype(ng_tag)::value;
+        uint4 h[NG], q0[NG], q1[NG];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint4 t = pp[i], m = pp[4 + i], l = pp[8 + i];
-            xt[4 * i] = t.x; xt[4 * i + 1] = t.y; xt[4 * i + 2] = t.z; xt[4 * i + 3] = t.w;
-            xm[4 * i] = m.x; xm[4 * i + 1] = m.y; xm[4 * i + 2] = m.z; xm[4 * i + 3] = m.w;
-            xl[4 * i] = l.x; xl[4 * i + 1] = l.y; xl[4 * i + 2] = l.z; xl[4 * i + 3] = l.w;
+        for (int q = 0; q < NG; q++) {
+            const uint8_t *blk = row_pointer(rg0 + q) + (size_t)kc * (16 * 144);
+            h[q] = *reinterpret_cast<const uint4 *>(blk);
+            q0[q] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+            q1[q] = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
         }
-    }
-    const float4 mt = meta[(sb0 + sb_local) * 4 + c];
-    const float inv_a = mt.x, inv_b = mt.y, sum_a = mt.z, sum_b = mt.w;
-
-    for (int i = 0; i < my_rows; i++) {
-        /* rows i .. issued-1 are in flight; row i is the oldest */
-        wait_vm_at_most((issued - i - 1) * loads_per_row);
-        const uint8_t *blk = my_images + (i % depth) * kRowImage + sb_local * 144;
-        const uint4 h = *reinterpret_cast<const uint4 *>(blk);
-        const uint4 qa = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c);
-        const uint4 qb = *reinterpret_cast<const uint4 *>(blk + 32 + 32 * c);
-        /* the image may be overwritten once these reads have returned */
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (issued < my_rows) {
-            issue(issued);
-            issued++;
-        }
-        const float d = half_bits_fast(h.x & 0xFFFFu), dmin = half_bits_fast(h.x >> 16);
-        /* bytes of sc_lo: scales 0..3, mn_lo: mins 0..3, sc_hi: scales 4..7, mn_hi: mins 4..7 */
-        const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
-        const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
-        const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
-        const uint32_t sc2 = ((c & 2) ? sc_hi : sc_lo) >> ((c & 1) * 16);
-        const uint32_t mn2 = ((c & 2) ? mn_hi : mn_lo) >> ((c & 1) * 16);
-        const uint32_t w[8] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
-        int at = 0, bt = 0;
-        uint32_t am = 0, al = 0, bm = 0, bl = 0;
+        if (rg0 == 0) { /* x is prepared while the first blocks are on their way */
+            v4f v = xr[0];
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const uint32_t lo = w[k] & 0x0F0F0F0Fu, hi = (w[k] >> 4) & 0x0F0F0F0Fu;
-            at = sdot4(lo, xt[k], at);
-            am = udot4(lo, xm[k], am);
-            al = udot4(lo, xl[k], al);
-            bt = sdot4(hi, xt[8 + k], bt);
-            bm = udot4(hi, xm[8 + k], bm);
-            bl = udot4(hi, xl[8 + k], bl);
+            for (int kk = 1; kk < NKC; kk++) v = kc == kk ? xr[kk] : v;
+            prepare(v, xo);
         }
-        /* |top| <= 32*15*64, mid/low <= 32*15*255: the low part fits an int exactly */
-        const float fa = fmaf((float)at, 65536.0f, (float)((am << 8) + al)) * inv_a;
-        const float fb = fmaf((float)bt, 65536.0f, (float)((bm << 8) + bl)) * inv_b;
-        const float da = d * (float)(sc2 & 0xFFu), db = d * (float)((sc2 >> 8) & 0xFFu);
-        const float ma = dmin * (float)(mn2 & 0xFFu), mb = dmin * (float)((mn2 >> 8) & 0xFFu);
-        float v = active ? (da * fa + db * fb - (ma * sum_a + mb * sum_b)) : 0.0f;
-        v = wave_sum_dpp(v);
-        if (lane == 0) partial[wv + i * kWaves] = v;
+#pragma unroll
+        for (int q = 0; q < NG; q++) store_partial(rg0 + q, item(xo, h[q], q0[q], q1[q]), kc > 0);
+    };
+    if (n_kc == 0) { /* a wave without a super-block (K < 4096) contributes zeros */
+        for (int rg = 0; rg < n_rg; rg++) store_partial(rg, 0.0f, false);
+    } else if (NKC == 1 || n_rg >= 2) {
+        for (int kc = 0; kc < n_kc; kc++) {
+            int rg0 = 0;
+            for (; rg0 + 4 <= n_rg; rg0 += 4) run_group(rg0, kc, std::integral_constant<int, 4>());
+            if (rg0 + 2 <= n_rg) {
+                run_group(rg0, kc, std::integral_constant<int, 2>());
+                rg0 += 2;
+            }
+            if (rg0 < n_rg) run_group(rg0, kc, std::integral_constant<int, 1>());
+        }
+    } else {
+        /* long rows, one row group: the wave's up to NKC super-blocks of the row are requested together */
+        const uint8_t *blk0 = row_pointer(0);
+        uint4 h[NKC], q0[NKC], q1[NKC];
+#pragma unroll
+        for (int kc = 0; kc < NKC; kc++)
+            if (kc < n_kc) {
+                const uint8_t *blk = blk0 + (size_t)kc * (16 * 144);
+                h[kc] = *reinterpret_cast<const uint4 *>(blk);
+                q0[kc] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+                q1[kc] = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
+            }
+        float acc = 0.0f;
+#pragma unroll
+        for (int kc = 0; kc < NKC; kc++)
+            if (kc < n_kc) {
+                prepare(xr[kc], xo);
+                acc += item(xo, h[kc], q0[kc], q1[kc]);
+            }
+        store_partial(0, acc, false);
     }
     __syncthreads();
 
-    /* combine the slices of each row and store */
+    /* sum the waves' shares of each row and store */
     auto row_total = [&](int lr) {
+        const float4 *p = reinterpret_cast<const float4 *>(partial + lr * kWaves);
         float s = 0.0f;
-        for (int k = 0; k < n_slices; k++) s += partial[lr * n_slices + k];
+#pragma unroll
+        for (int k = 0; k < kWaves / 4; k++) {
+            const float4 v = p[k];
+            s += (v.x + v.y) + (v.z + v.w);
+        }
         return s;
     };
     if (paired) {
-        for (int lr = threadIdx.x; lr < rows_here; lr += kThreads)
+        for (int lr = threadIdx.x; lr < rows_here; lr += kWaves * 64)
             job.y0[row0 + lr] = silu_times(row_total(lr), row_total(rows_here + lr));
     } else {
-        for (int lr = threadIdx.x; lr < n_lrows; lr += kThreads) {
+        for (int lr = threadIdx.x; lr < n_lrows; lr += kWaves * 64) {
             const uint8_t *Wm;
             float *ym;
             int r;
@@ -280,17 +303,11 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int n_
             ym[r] = job.mode == 1 ? ym[r] + s : s;
         }
     }
-
 }
 
-/* Launch geometry: one 16-wave workgroup per block of rows, sized so that the grid covers the
- * compute units once (more workgroups only when a block would exceed kMaxRowsPerWg rows). */
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu) {
-    static OnceFlag lds_raised;
     const int n_sb = n_cols / 256;
-    if (n_sb > 64 || n_sb < 1) return hipErrorInvalidValue;
-    const int n_slices = n_sb <= 16 ? 1 : n_sb <= 32 ? 2 : 4;
-    const int slice_sb = (n_sb + n_slices - 1) / n_slices;
+    if (n_sb > 16 * kMaxKc || n_sb < 1) return hipErrorInvalidValue;
     const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     if (n_rows == 0) return hipSuccess;
@@ -298,21 +315,14 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
     if (rows_per_wg < 1) rows_per_wg = 1;
     if (rows_per_wg * n_mats_here > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / n_mats_here;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
-    const size_t fixed_bytes = (size_t)n_sb * 4 * kChunk * 4 + (size_t)n_sb * 4 * 16 +
-                               (size_t)((rows_per_wg * n_mats_here * n_slices + 3) & ~3) * 4 + (size_t)n_sb * 256 * 4;
-    if (fixed_bytes + (size_t)kWaves * kRowImage > 160 * 1024) return hipErrorInvalidValue;
-    int depth = (int)((160 * 1024 - fixed_bytes) / ((size_t)kWaves * kRowImage));
-    if (depth > kMaxDepth) depth = kMaxDepth;
-    const size_t lds_bytes = fixed_bytes + (size_t)kWaves * depth * kRowImage;
-    if (!lds_raised.is_set()) {
-        hipError_t e = hipFuncSetAttribute((const void *)gemv_q4k_kernel,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return e;
-        lds_raised.set();
-    }
+    const size_t lds_bytes = (size_t)kWaves * kXScratch + (size_t)rows_per_wg * n_mats_here * kWaves * 4;
     const JobView view = job_view(job);
-    hipLaunchKernelGGL(gemv_q4k_kernel, dim3(grid), dim3(kThreads), lds_bytes, stream, view, x, n_sb, n_slices,
-                       slice_sb, rows_per_wg, depth);
+    if (n_sb <= 16)
+        hipLaunchKernelGGL(gemv_q4k_kernel<1>, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb,
+                           rows_per_wg);
+    else
+        hipLaunchKernelGGL(gemv_q4k_kernel<kMaxKc>, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb,
+                           rows_per_wg);
     return hipGetLastError();
 }
 
