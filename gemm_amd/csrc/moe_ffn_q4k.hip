@@ -837,4 +837,34 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
     return hipGetLastError();
 }
 
+/* ---- scratch of the entry point that allocates nothing (qlin_moe_ffn_static_dev): the workspace of
+ * launch_moe_ffn as a file-scope device array. Every GPU the library's code object is loaded on holds its
+ * own copy at its own address until the process ends; host code never uses the array's name as an address,
+ * only what hipGetSymbolAddress returned for the device that was current. */
+static __device__ __align__(256) unsigned char scratch[kMoeStaticScratchBytes];
+static void *g_scratch_ptr[kMaxScratchDevices]; /* written under the caller's lock, once per device */
+
+hipError_t moe_static_scratch_setup(int device) {
+    if (device < 0 || device >= kMaxScratchDevices) return hipErrorInvalidDevice;
+    if (g_scratch_ptr[device]) return hipSuccess;
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = p;
+    return hipSuccess;
+}
+
+hipError_t launch_moe_ffn_static(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate,
+                                 const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
+                                 float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int device,
+                                 hipStream_t stream) {
+    if (device < 0 || device >= kMaxScratchDevices || !g_scratch_ptr[device]) return hipErrorNotInitialized;
+    if (moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert) > kMoeStaticScratchBytes) return hipErrorInvalidValue;
+    /* nothing in the workspace has to start at zero: the grouping kernel writes every offset, slot and weight
+     * it later reads, and the expert kernels write every slot row the combine step reads */
+    return launch_moe_ffn(type_gate, type_up, type_down, gate, up, down, X, idx, w, out, n_tok, top_k, n_embd, n_ff,
+                          n_expert, g_scratch_ptr[device], stream);
+}
+
 }  // namespace qlin

@@ -115,6 +115,7 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipEventCreate(&g.ev1));
     g.device = device;
     if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
+    HIP_TRY(moe_static_scratch_setup(device)); /* address of the no-allocation entry point's scratch on this device */
     g.ready = true;
     return QLIN_OK;
 }
@@ -932,10 +933,11 @@ size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int 
     return moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert);
 }
 
-int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
-                           const void *up_exps, const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
-                           const float *expert_w, float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert,
-                           void *workspace, void *stream) {
+static_assert(kMoeStaticScratchBytes == QLIN_MOE_STATIC_SCRATCH_BYTES, "the header states the size of the scratch");
+
+static int check_moe_args(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
+                          const void *up_exps, const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
+                          const float *expert_w, float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
     if (int rc = check_linear_shape(type_gate, n_ff, n_embd)) return rc;
     if (int rc = check_linear_shape(type_up, n_ff, n_embd)) return rc;
     if (int rc = check_linear_shape(type_down, n_embd, n_ff)) return rc;
@@ -945,17 +947,53 @@ int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_d
     if ((long long)n_tok * top_k > (1 << 24))
         return fail(QLIN_ERR_ARG, "grouped MoE FFN handles at most 2^24 (token, expert) pairs per call");
     if (n_tok == 0) return QLIN_OK;
-    if (!gate_exps || !up_exps || !down_exps || !X || !expert_idx || !expert_w || !out || !workspace)
+    if (!gate_exps || !up_exps || !down_exps || !X || !expert_idx || !expert_w || !out)
         return fail(QLIN_ERR_ARG, "null pointer");
-    if (!aligned(gate_exps, 16) || !aligned(up_exps, 16) || !aligned(down_exps, 16) || !aligned(X, 16) ||
-        !aligned(out, 16) || !aligned(workspace, 256))
-        return fail(QLIN_ERR_ARG, "misaligned pointer (16 bytes; workspace 256)");
+    if (!aligned(gate_exps, 16) || !aligned(up_exps, 16) || !aligned(down_exps, 16) || !aligned(X, 16) || !aligned(out, 16))
+        return fail(QLIN_ERR_ARG, "misaligned pointer (16 bytes)");
+    return QLIN_OK;
+}
+
+int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
+                           const void *up_exps, const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
+                           const float *expert_w, float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert,
+                           void *workspace, void *stream) {
+    if (int rc = check_moe_args(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
+                                n_tok, top_k, n_embd, n_ff, n_expert))
+        return rc;
+    if (n_tok == 0) return QLIN_OK;
+    if (!workspace) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(workspace, 256)) return fail(QLIN_ERR_ARG, "misaligned pointer (workspace: 256 bytes)");
     {
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
     HIP_TRY(launch_moe_ffn(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
                            n_tok, top_k, n_embd, n_ff, n_expert, workspace, (hipStream_t)stream));
+    return QLIN_OK;
+}
+
+int qlin_moe_ffn_static_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
+                            const void *up_exps, const void *down_exps, const uint16_t *X, const int32_t *expert_idx,
+                            const float *expert_w, float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert,
+                            void *stream) {
+    if (int rc = check_moe_args(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
+                                n_tok, top_k, n_embd, n_ff, n_expert))
+        return rc;
+    if (n_tok == 0) return QLIN_OK;
+    const size_t need = moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert);
+    if (need > (size_t)QLIN_MOE_STATIC_SCRATCH_BYTES)
+        return fail(QLIN_ERR_ARG, "this shape needs %zu bytes of scratch, the built-in scratch holds %zu: use qlin_moe_ffn_types_dev "
+                                  "with a workspace", need, (size_t)QLIN_MOE_STATIC_SCRATCH_BYTES);
+    int device;
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (!g.ready) /* initialising would allocate (stream, events): that is qlin_init's job, not this call's */
+            return fail(QLIN_ERR_DEVICE, "qlin_init() must have run before qlin_moe_ffn_static_dev");
+        device = g.device;
+    }
+    HIP_TRY(launch_moe_ffn_static(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
+                                  n_tok, top_k, n_embd, n_ff, n_expert, device, (hipStream_t)stream));
     return QLIN_OK;
 }
 

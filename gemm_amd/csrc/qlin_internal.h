@@ -100,6 +100,16 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                           const void *down, const uint16_t *X, const int32_t *idx, const float *w, float *out, int n_tok,
                           int top_k, int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream);
 
+/* the same with the workspace in a device array of the library (at most kMoeStaticScratchBytes); setup once per
+ * device with that device current, before the first launch there */
+constexpr size_t kMoeStaticScratchBytes = (size_t)16 << 20; /* = QLIN_MOE_STATIC_SCRATCH_BYTES of the public header */
+constexpr int kMaxScratchDevices = 64;
+hipError_t moe_static_scratch_setup(int device);
+hipError_t launch_moe_ffn_static(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate,
+                                 const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
+                                 float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int device,
+                                 hipStream_t stream);
+
 /* MoE pieces */
 hipError_t launch_moe_route(const float *logits, int n_tok, int n_expert, int top_k, int32_t *idx,
                             float *w, hipStream_t stream);

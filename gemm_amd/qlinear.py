@@ -86,6 +86,8 @@ SIGNATURES = {
                                    C.c_int, C.c_int, _vp, _vp]),
     "qlin_moe_ffn_types_dev": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                          C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, _vp]),
+    "qlin_moe_ffn_static_dev": (C.c_int, [C.c_uint32, C.c_uint32, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                          C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp]),
     "qlin_gguf_open": (C.c_int, [C.c_char_p, _vp]),
     "qlin_gguf_close": (None, [_vp]),
     "qlin_gguf_version": (C.c_uint32, [_vp]),
@@ -344,6 +346,11 @@ def moe_ffn_dev(type_id, dgate, dup, ddown, dX, didx, dw, dout, n_tok, top_k, n_
 def moe_ffn_types_dev(types, dgate, dup, ddown, dX, didx, dw, dout, n_tok, top_k, n_embd, n_ff, n_expert, dws, stream=None):
     check(load().qlin_moe_ffn_types_dev(types[0], types[1], types[2], dgate.ptr, dup.ptr, ddown.ptr, dX.ptr, didx.ptr,
                                         dw.ptr, dout.ptr, n_tok, top_k, n_embd, n_ff, n_expert, dws.ptr, stream))
+
+
+def moe_ffn_static_dev(types, dgate, dup, ddown, dX, didx, dw, dout, n_tok, top_k, n_embd, n_ff, n_expert, stream=None):
+    check(load().qlin_moe_ffn_static_dev(types[0], types[1], types[2], dgate.ptr, dup.ptr, ddown.ptr, dX.ptr, didx.ptr,
+                                         dw.ptr, dout.ptr, n_tok, top_k, n_embd, n_ff, n_expert, stream))
 
 
 def sync(stream=None):

@@ -262,6 +262,23 @@ int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_d
                            const void *up_exps, const void *down_exps, const uint16_t *X,
                            const int32_t *expert_idx, const float *expert_w, float *out, int n_tok, int top_k,
                            int n_embd, int n_ff, int n_expert, void *workspace, void *stream);
+/* qlin_moe_ffn_types_dev without the workspace argument and without any allocation: the scratch its kernels
+ * need (slot tables, the intermediate activations by slot, the per-slot down projections) lives in a device
+ * array inside the library, QLIN_MOE_STATIC_SCRATCH_BYTES per GPU, held until the process ends. No counterpart
+ * in the reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc. Same arguments, results and error codes as qlin_moe_ffn_types_dev, plus:
+ *   - QLIN_ERR_ARG if qlin_moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert) exceeds
+ *     QLIN_MOE_STATIC_SCRATCH_BYTES (64 tokens x top-8 x 2048/768 x 128 experts needs 8.7 MB);
+ *   - QLIN_ERR_DEVICE if qlin_init() has not run (initialising creates a stream and events, which this call
+ *     must not do); the scratch address of the device is looked up there, once.
+ * The call enqueues kernels on `stream` and returns. Every call on a GPU shares that GPU's scratch and leaves
+ * its contents behind: calls whose kernels could overlap (different streams, different host threads) race -
+ * order them on one stream. */
+#define QLIN_MOE_STATIC_SCRATCH_BYTES (16u << 20)
+int qlin_moe_ffn_static_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate_exps,
+                            const void *up_exps, const void *down_exps, const uint16_t *X,
+                            const int32_t *expert_idx, const float *expert_w, float *out, int n_tok, int top_k,
+                            int n_embd, int n_ff, int n_expert, void *stream);
 
 /* ------------------------------------------------------------------ GGUF file -> HBM
  * The tensor table and key/value pairs of a GGUF model file (versions 2 and 3, as read by
