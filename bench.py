@@ -29,7 +29,8 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-from gemm_amd import qlinear, synth  # noqa: E402
+from gemm_amd import qlinear
+import synth  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
@@ -353,6 +354,64 @@ def cpu_baseline(n_rows, n_cols, budget_s=12.0):
     }
 
 
+def cpu_baselines_other(budget_s=14.0):
+    """The reference's CPU path (compiled from its sources) on the other benchmark shapes, bounded
+    samples: matvecs on one thread and on all cores, the prefill GEMM entry point on a 128-token
+    sample, the MoE block as per-token expert-slice matvecs on a 4-token sample. Empty where the
+    compiled reference is absent."""
+    from oracle import pyoracle  # reported baseline only
+    if not pyoracle.Reference.available():
+        return {}
+    ref = pyoracle.Reference()
+    cores = max(1, min(len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1), 64))
+    out = {"cores": cores, "kind": "reference"}
+    shapes = [("q8_0", synth.GGML_Q8_0, 4096, 4096), ("q4_K", Q4K, 4096, 4096), ("q4_K", Q4K, 4096, 14336),
+              ("q5_K", synth.GGML_Q5_K, 4096, 4096), ("iq4_nl", synth.GGML_IQ4_NL, 14336, 4096),
+              ("iq2_xxs", synth.GGML_IQ2_XXS, 4096, 14336), ("iq3_s", synth.GGML_IQ3_S, 4096, 14336),
+              ("q6_K", synth.GGML_Q6_K, 151936, 4096)]
+    per_shape = budget_s * 0.5 / len(shapes)
+    mv = {}
+    for tname, tid, r, c in shapes:
+        W = synth.make_weights(tid, r, c, seed=20260 + tid)
+        x = synth.make_activation(c, seed=7)
+        b = gemv_bytes(tid, r, c)
+        tn = ref.qmatvec_pool_time(tid, W, x, c, cores, 1)
+        tn = ref.qmatvec_pool_time(tid, W, x, c, cores, max(1, int(per_shape * 0.6 / max(tn, 1e-6))))
+        rows1 = min(r, 4096)  # one thread: a slice of the rows is enough
+        t1 = ref.qmatvec_pool_time(tid, W[:rows1], x, c, 1, 1)
+        t1 = ref.qmatvec_pool_time(tid, W[:rows1], x, c, 1, max(1, int(per_shape * 0.4 / max(t1, 1e-6))))
+        mv["%s_%dx%d" % (tname, r, c)] = {"ms_all_cores": round(tn * 1e3, 3), "GB/s_all_cores": round(b / tn / 1e9, 2),
+                                          "GB/s_1_thread": round(gemv_bytes(tid, rows1, c) / t1 / 1e9, 3)}
+    out["matvec"] = mv
+    # prefill: tf_gemm_f16_mt_tokenmajor on Q4_K 14336x4096 (per-token fallback for this type), 128 tokens
+    n_tok, r, c = 128, 14336, 4096
+    W = synth.make_weights(Q4K, r, c, seed=60)
+    X = synth.make_activation(c, seed=61, tokens=n_tok)
+    t0 = time.time()
+    ref.gemm_tokenmajor(Q4K, W, X, c, n_threads=cores)
+    dt = time.time() - t0
+    out["prefill_q4_K_14336x4096"] = {"sample": "%d tokens through tf_gemm_f16_mt_tokenmajor on %d threads" % (n_tok, cores),
+                                      "ms_per_token": round(dt / n_tok * 1e3, 3),
+                                      "TFLOP/s": round(2.0 * n_tok * r * c / dt / 1e12, 4)}
+    # MoE: per token top-8 experts x (gate, up, down) expert-slice matvecs, one thread (tf_qmatvec_expert)
+    n_expert, n_embd, n_ff, top_k, sample_tok = 128, 2048, 768, 8, 4
+    g = synth.make_weights(Q4K, n_expert * n_ff, n_embd, seed=31)
+    d = synth.make_weights(Q4K, n_expert * n_embd, n_ff, seed=33)
+    xt = synth.make_activation(n_embd, seed=41)
+    ht = synth.make_activation(n_ff, seed=43)
+    t0 = time.time()
+    for t in range(sample_tok):
+        for k in range(top_k):
+            e = (17 * t + 5 * k) % n_expert
+            ref.qmatvec_expert(Q4K, g, e, xt, n_ff, n_embd)
+            ref.qmatvec_expert(Q4K, g, e, xt, n_ff, n_embd)  # up: same shape and type as gate
+            ref.qmatvec_expert(Q4K, d, e, ht, n_embd, n_ff)
+    dt = (time.time() - t0) / sample_tok
+    out["moe_ffn_128x(768x2048)_top8"] = {"sample": "%d tokens x 8 experts x 3 expert-slice matvecs (tf_qmatvec_expert), 1 thread" % sample_tok,
+                                         "ms_per_token": round(dt * 1e3, 3), "ms_for_64_tokens": round(dt * 64 * 1e3, 1)}
+    return out
+
+
 def probe(args):
     """Helper for counter collection (see profiles/): run only the named device work."""
     if args.probe == "copy":
@@ -586,6 +645,8 @@ def main():
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n_rows, n_cols)
+        if extra:
+            extra["cpu_reference_other_shapes"] = cpu_baselines_other()
     if extra:
         out["extra"] = extra
     out["wall_s"] = round(time.time() - t0, 1)

@@ -71,6 +71,58 @@ gemv_generic_kernel(const JobView job, const float *__restrict__ x, int n_cols, 
     }
 }
 
+/* dense rows whose length is not a multiple of eight elements, or that start off a 16-byte boundary: one
+ * wave per row (mode 2: per row pair), one element per lane and step, scalar loads. tf_qmatvec takes such
+ * rows (common/transformer.h:1049-1114: F32/F16/BF16 rows are dotted element by element). */
+template <uint32_t T>
+__global__ void __launch_bounds__(256)
+gemv_dense_ragged_kernel(const JobView job, const float *__restrict__ x, int n_cols) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const bool paired = job.mode == 2;
+    const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
+    if (wave >= n_rows) return;
+    auto dot = [&](const uint8_t *W, int r) {
+        float acc = 0.0f;
+        if (T == T_F32) {
+            const float *row = reinterpret_cast<const float *>(W) + (size_t)r * n_cols;
+            for (int k = lane; k < n_cols; k += 64) acc += row[k] * x[k];
+        } else {
+            const uint16_t *row = reinterpret_cast<const uint16_t *>(W) + (size_t)r * n_cols;
+            for (int k = lane; k < n_cols; k += 64) {
+                const uint32_t h = row[k];
+                acc += (T == T_F16 ? half_bits_exact(h) : __uint_as_float(h << 16)) * x[k];
+            }
+        }
+        return wave_sum(acc);
+    };
+    if (paired) {
+        const float g = dot(job.W0, wave), u = dot(job.W1, wave);
+        if (lane == 0) job.y0[wave] = silu_times(g, u);
+    } else {
+        const uint8_t *Wm;
+        float *ym;
+        int r;
+        job_locate(job, wave, Wm, ym, r);
+        const float s = dot(Wm, r);
+        if (lane == 0) ym[r] = job.mode == 1 ? ym[r] + s : s;
+    }
+}
+
+hipError_t launch_gemv_dense_ragged(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t s) {
+    const int waves = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
+    if (waves == 0) return hipSuccess;
+    const JobView view = job_view(job);
+    const dim3 grid((waves + 3) / 4), block(256);
+    switch (type) {
+    case T_F32: hipLaunchKernelGGL((gemv_dense_ragged_kernel<T_F32>), grid, block, 0, s, view, x, n_cols); break;
+    case T_F16: hipLaunchKernelGGL((gemv_dense_ragged_kernel<T_F16>), grid, block, 0, s, view, x, n_cols); break;
+    case T_BF16: hipLaunchKernelGGL((gemv_dense_ragged_kernel<T_BF16>), grid, block, 0, s, view, x, n_cols); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 /* prefill in fp32: a wavefront owns one weight row and TT tokens at a time; the row is
  * decoded once per token tile. Y is token-major. (Semantics of the reference's generic
  * prefill path, common/transformer.h:4535-4572.) */

@@ -3,8 +3,11 @@
  *
  *   route:    softmax over all experts, keep the top_k largest, renormalise by their sum
  *             (:4054-4091). One wavefront per token. The k survivors are written in
- *             descending weight order (ties: lower expert index first); the reference's heap
- *             leaves them in heap order, which only changes the order of the final fp32 sum.
+ *             descending weight order; the reference's heap leaves them in heap order, which only
+ *             changes the order of the final fp32 sum. Where the choice itself depends on the heap -
+ *             the k-th and (k+1)-th largest probabilities are equal, or probabilities are NaN - one
+ *             lane replays the reference's min-heap literally (:4057-4091), so the SET of experts
+ *             and their weights are the reference's in every case.
  *   silu_mul: h = gate/(1+exp(-gate)) * up (:4108, scalar form :4690)
  *   axpy:     out += w * q (:4116-4127)
  */
@@ -12,6 +15,45 @@
 #include "qlin_internal.h"
 
 namespace qlin {
+
+/* the reference's selection, statement for statement (common/transformer.h:4057-4091): a min-heap of the
+ * top_k largest so far over one pass, then the weights divided by their sum. One lane; heap in idx/w. */
+__device__ void route_heap(const float *prob, int n_expert, int top_k, int32_t *idx, float *w) {
+    int k = 0;
+    for (int e = 0; e < n_expert; e++) {
+        const float pe = prob[e];
+        if (k < top_k) {
+            idx[k] = e;
+            w[k] = pe;
+            k++;
+            for (int j = k - 1; j > 0;) {
+                const int parent = (j - 1) / 2;
+                if (w[j] < w[parent]) {
+                    const float tv = w[j]; w[j] = w[parent]; w[parent] = tv;
+                    const int ti = idx[j]; idx[j] = idx[parent]; idx[parent] = ti;
+                    j = parent;
+                } else break;
+            }
+        } else if (pe > w[0]) {
+            w[0] = pe;
+            idx[0] = e;
+            for (int j = 0;;) {
+                int s = j;
+                const int l = 2 * j + 1, r = 2 * j + 2;
+                if (l < top_k && w[l] < w[s]) s = l;
+                if (r < top_k && w[r] < w[s]) s = r;
+                if (s == j) break;
+                const float tv = w[j]; w[j] = w[s]; w[s] = tv;
+                const int ti = idx[j]; idx[j] = idx[s]; idx[s] = ti;
+                j = s;
+            }
+        }
+    }
+    float wsum = 0.0f;
+    for (int i = 0; i < top_k; i++) wsum += w[i];
+    if (wsum > 0.0f)
+        for (int i = 0; i < top_k; i++) w[i] /= wsum;
+}
 
 /* Probabilities live in registers, PL per lane (expert e = lane + 64 j); every selection step is one
  * wave maximum on the cross-lane data path plus a ballot for the lowest expert index holding it. The
@@ -39,11 +81,16 @@ moe_route_kernel(const float *__restrict__ logits, int n_expert, int top_k, int3
         sum += e < n_expert ? p[j] : 0.0f;
     }
     sum = wave_sum_dpp(sum);
+    __shared__ float prob_copy[64 * PL];
 #pragma unroll
-    for (int j = 0; j < PL; j++)
+    for (int j = 0; j < PL; j++) {
         if (lane + 64 * j < n_expert) p[j] /= sum;
+        prob_copy[lane + 64 * j] = p[j];
+    }
     float wsum = 0.0f, mine = 0.0f; /* lane k keeps the k-th weight (top_k <= 64) */
     int mine_idx = 0;
+    bool replay = false; /* the heap decides: a pick found nothing (NaN), or the last pick ties with what is left */
+    float last = 0.0f;
     for (int k = 0; k < top_k; k++) {
         float best = -1.0f;
 #pragma unroll
@@ -56,11 +103,25 @@ moe_route_kernel(const float *__restrict__ logits, int n_expert, int top_k, int3
             const unsigned long long m = __ballot(p[j] == best);
             if (bi == 0x7FFFFFFF && m != 0ull) bi = __builtin_ctzll(m) + 64 * j;
         }
+        if (bi >= n_expert) { bi = 0; best = 0.0f; replay = true; } /* NaN probabilities compare false everywhere */
 #pragma unroll
         for (int j = 0; j < PL; j++)
             if (lane + 64 * j == bi) p[j] = -2.0f;
         if (lane == k) { mine = best; mine_idx = bi; }
         wsum += best;
+        last = best;
+    }
+    {
+        float rest = -1.0f;
+#pragma unroll
+        for (int j = 0; j < PL; j++) rest = fmaxf(rest, p[j]);
+        rest = wave_max_dpp(rest);
+        if (top_k < n_expert && rest == last) replay = true;
+    }
+    if (replay) { /* uniform: every lane holds the same flags */
+        __syncthreads();
+        if (lane == 0) route_heap(prob_copy, n_expert, top_k, idx + (size_t)tok * top_k, wgt + (size_t)tok * top_k);
+        return;
     }
     if (lane < top_k) {
         idx[(size_t)tok * top_k + lane] = mine_idx;
@@ -87,7 +148,8 @@ moe_route_lds_kernel(const float *__restrict__ logits, int n_expert, int top_k, 
     __syncthreads();
     for (int e = lane; e < n_expert; e += 64) prob[e] /= sum;
     __syncthreads();
-    float wsum = 0.0f;
+    float wsum = 0.0f, last = 0.0f;
+    bool replay = false;
     for (int k = 0; k < top_k; k++) {
         /* arg-max over what is left: larger weight wins, then the lower index */
         float best = -1.0f;
@@ -102,13 +164,30 @@ moe_route_lds_kernel(const float *__restrict__ logits, int n_expert, int top_k, 
             const int oi = __shfl_xor(bi, off, 64);
             if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
         }
+        if (bi >= n_expert) { replay = true; break; } /* NaN probabilities compare false everywhere */
         if (lane == 0) {
             idx[(size_t)tok * top_k + k] = bi;
             wgt[(size_t)tok * top_k + k] = best;
-            prob[bi] = -2.0f;
+            prob[bi] = -2.0f - (float)k; /* marks pick k; undone below if the heap has to decide */
         }
         wsum += best;
+        last = best;
         __syncthreads();
+    }
+    if (!replay && top_k < n_expert) { /* does the last pick tie with what is left? */
+        float rest = -1.0f;
+        for (int e = lane; e < n_expert; e += 64) rest = fmaxf(rest, prob[e]);
+        rest = wave_max_dpp(rest);
+        replay = rest == last;
+    }
+    if (replay) { /* uniform; put the picked probabilities back and replay the reference's heap */
+        __syncthreads();
+        if (lane == 0) {
+            for (int e = 0; e < n_expert; e++)
+                if (prob[e] <= -2.0f) prob[e] = wgt[(size_t)tok * top_k + (int)(-2.0f - prob[e])];
+            route_heap(prob, n_expert, top_k, idx + (size_t)tok * top_k, wgt + (size_t)tok * top_k);
+        }
+        return;
     }
     if (wsum > 0.0f)
         for (int k = lane; k < top_k; k += 64) wgt[(size_t)tok * top_k + k] /= wsum;

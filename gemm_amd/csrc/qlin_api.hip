@@ -7,6 +7,7 @@
  * no CPU fallback: if the GPU cannot be used every call fails.
  */
 #include "../../include/qlinear.h"
+#include "../../include/qlinear_bench.h"
 
 #include <hip/hip_runtime.h>
 
@@ -94,7 +95,6 @@ struct State {
     int device = 0;
     int n_cu = 256;
     hipStream_t stream = nullptr;
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
     std::map<uintptr_t, Range> registry; /* host begin -> range */
     DevBuf w[3], x, y[3], tmp[4];
     bool prefill_bf16 = false; /* qlin_gemm_tokenmajor on the matrix cores (opt-in: costs accuracy) */
@@ -111,8 +111,6 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipGetDeviceProperties(&prop, device));
     g.n_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     HIP_TRY(hipStreamCreate(&g.stream));
-    HIP_TRY(hipEventCreate(&g.ev0));
-    HIP_TRY(hipEventCreate(&g.ev1));
     g.device = device;
     if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
     HIP_TRY(moe_static_scratch_setup(device)); /* address of the no-allocation entry point's scratch on this device */
@@ -165,6 +163,8 @@ hipError_t dispatch_gemv_job(uint32_t type, const GemvJob &job, const float *x, 
     if ((job.mode == kSiluMul ? job.n_rows[0] : job.total_rows()) == 0) return hipSuccess;
     bool w_aligned = true;
     for (int m = 0; m < job.n_mat; m++) w_aligned = w_aligned && aligned(job.W[m], 16);
+    if ((type == T_F16 || type == T_BF16 || type == T_F32) && (n_cols % 8 != 0 || !w_aligned))
+        return launch_gemv_dense_ragged(type, job, x, n_cols, s); /* rows that are not whole 16-byte groups */
     if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && w_aligned && aligned(x, 16))
         return launch_gemv_q4k(job, x, n_cols, s, g.n_cu);
     hipError_t err;
@@ -177,11 +177,13 @@ hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y,
     return dispatch_gemv_job(type, single_job(W, y, n_rows), x, n_cols, s);
 }
 
-int check_linear_shape(uint32_t type, int n_rows, int n_cols) {
+/* any_dense_length: the matvec paths take dense F32/F16/BF16 rows of any length, as tf_qmatvec does
+ * (common/transformer.h:1049-1114); the GEMM and MoE paths want whole groups of eight elements */
+int check_linear_shape(uint32_t type, int n_rows, int n_cols, bool any_dense_length = false) {
     int be, bb;
     if (!type_geometry(type, &be, &bb))
         return fail(QLIN_ERR_TYPE, "unsupported weight type %u", type);
-    if (be == 1) be = 8; /* dense F16/BF16/F32 rows go through the kernels eight elements at a time */
+    if (be == 1 && !any_dense_length) be = 8; /* dense rows go through those kernels eight elements at a time */
     if (n_rows < 0 || n_cols <= 0) return fail(QLIN_ERR_ARG, "bad shape %d x %d", n_rows, n_cols);
     if (n_cols % be) return fail(QLIN_ERR_ARG, "n_cols %d is not a whole number of %d-element blocks", n_cols, be);
     return QLIN_OK;
@@ -243,11 +245,11 @@ bool dense_type(uint32_t t) { return t == T_F16 || t == T_BF16 || t == T_F32; }
 
 /* argument checks shared by the device-resident matvec entry points */
 int check_dev_gemv(uint32_t type, int n_rows, int n_cols, const void *W, const float *x, const float *y) {
-    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type, n_rows, n_cols, true)) return rc;
     if (n_rows == 0) return QLIN_OK;
     if (!W || !x || !y) return fail(QLIN_ERR_ARG, "null pointer");
-    if (!aligned(W, dense_type(type) ? 16 : 2) || !aligned(x, 16) || !aligned(y, 4))
-        return fail(QLIN_ERR_ARG, "W needs 2-byte (dense types: 16-byte), x 16-byte, y 4-byte alignment");
+    if (!aligned(W, type == T_F32 ? 4 : 2) || !aligned(x, 16) || !aligned(y, 4))
+        return fail(QLIN_ERR_ARG, "W needs 2-byte (F32: 4-byte), x 16-byte, y 4-byte alignment");
     return QLIN_OK;
 }
 int init_once() {
@@ -285,8 +287,6 @@ void qlin_shutdown(void) {
     for (auto &b : g.y) b.release();
     for (auto &b : g.tmp) b.release();
     g.x.release();
-    (void)hipEventDestroy(g.ev0);
-    (void)hipEventDestroy(g.ev1);
     (void)hipStreamDestroy(g.stream);
     g.stream = nullptr;
     g.ready = false;
@@ -420,7 +420,7 @@ const void *qlin_weight_device_ptr(const void *host_ptr) {
 /* ------------------------------------------------------------------ linear, host pointers */
 
 int qlin_matvec(float *dst, const void *W, uint32_t type, int n_cols, const float *x, int n_rows) {
-    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type, n_rows, n_cols, true)) return rc;
     if (n_rows == 0) return QLIN_OK;
     if (!dst || !W || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
@@ -432,8 +432,8 @@ int qlin_matvec(float *dst, const void *W, uint32_t type, int n_cols, const floa
 
 int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2, const void *W2,
                        uint32_t type2, int n_cols, const float *x, int n_rows) {
-    if (int rc = check_linear_shape(type1, n_rows, n_cols)) return rc;
-    if (int rc = check_linear_shape(type2, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type1, n_rows, n_cols, true)) return rc;
+    if (int rc = check_linear_shape(type2, n_rows, n_cols, true)) return rc;
     if (n_rows == 0) return QLIN_OK;
     if (!dst1 || !dst2 || !W1 || !W2 || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
@@ -450,9 +450,9 @@ int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2,
 int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k, const void *Wk,
                     uint32_t type_k, float *v, const void *Wv, uint32_t type_v, int n_kv,
                     int n_cols, const float *x) {
-    if (int rc = check_linear_shape(type_q, n_q, n_cols)) return rc;
-    if (int rc = check_linear_shape(type_k, n_kv, n_cols)) return rc;
-    if (int rc = check_linear_shape(type_v, n_kv, n_cols)) return rc;
+    if (int rc = check_linear_shape(type_q, n_q, n_cols, true)) return rc;
+    if (int rc = check_linear_shape(type_k, n_kv, n_cols, true)) return rc;
+    if (int rc = check_linear_shape(type_v, n_kv, n_cols, true)) return rc;
     if (!x || (n_q && (!q || !Wq)) || (n_kv && (!k || !Wk || !v || !Wv))) return fail(QLIN_ERR_ARG, "null pointer");
     if (n_q == 0 && n_kv == 0) return QLIN_OK;
     std::lock_guard<std::mutex> lk(g.mu);
@@ -468,8 +468,8 @@ int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k
 
 int qlin_matvec_silu_mul(float *dst, const void *Wgate, uint32_t type_gate, const void *Wup, uint32_t type_up,
                          int n_cols, const float *x, int n_rows) {
-    if (int rc = check_linear_shape(type_gate, n_rows, n_cols)) return rc;
-    if (int rc = check_linear_shape(type_up, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type_gate, n_rows, n_cols, true)) return rc;
+    if (int rc = check_linear_shape(type_up, n_rows, n_cols, true)) return rc;
     if (n_rows == 0) return QLIN_OK;
     if (!dst || !Wgate || !Wup || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
@@ -484,7 +484,7 @@ int qlin_matvec_silu_mul(float *dst, const void *Wgate, uint32_t type_gate, cons
 }
 
 int qlin_matvec_add(float *dst, const void *W, uint32_t type, int n_cols, const float *x, int n_rows) {
-    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type, n_rows, n_cols, true)) return rc;
     if (n_rows == 0) return QLIN_OK;
     if (!dst || !W || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
@@ -500,7 +500,7 @@ int qlin_matvec_add(float *dst, const void *W, uint32_t type, int n_cols, const 
 
 int qlin_matvec_argmax(int *index, float *value, float *logits, const void *W, uint32_t type, int n_cols,
                        const float *x, int n_rows) {
-    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (int rc = check_linear_shape(type, n_rows, n_cols, true)) return rc;
     if (n_rows == 0) return fail(QLIN_ERR_ARG, "argmax over no rows");
     if (!index || !W || !x) return fail(QLIN_ERR_ARG, "null pointer");
     std::lock_guard<std::mutex> lk(g.mu);
@@ -525,7 +525,7 @@ int qlin_matvec_argmax(int *index, float *value, float *logits, const void *W, u
 
 int qlin_matvec_expert(float *dst, const void *W, uint32_t type, int n_cols, int expert, const float *x,
                        int rows_per_expert) {
-    if (int rc = check_linear_shape(type, rows_per_expert, n_cols)) return rc;
+    if (int rc = check_linear_shape(type, rows_per_expert, n_cols, true)) return rc;
     if (expert < 0) return fail(QLIN_ERR_ARG, "negative expert index");
     if (!W) return fail(QLIN_ERR_ARG, "null pointer");
     const size_t rb = row_size(type, n_cols);
@@ -1030,20 +1030,36 @@ int qlin_probe_hbm_read(const void *buf, size_t n_bytes, void *stream) {
     return QLIN_OK;
 }
 
+/* the event pair belongs to the calling thread, so that threads timing their own streams do not overwrite
+ * each other's start event */
+namespace {
+struct ThreadTimer {
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool begun = false;
+};
+thread_local ThreadTimer t_timer;
+}  // namespace
+
 int qlin_timer_begin(void *stream) {
-    std::lock_guard<std::mutex> lk(g.mu);
-    if (int rc = ensure_init_locked(0)) return rc;
-    HIP_TRY(hipEventRecord(g.ev0, (hipStream_t)stream));
+    {
+        std::lock_guard<std::mutex> lk(g.mu);
+        if (int rc = ensure_init_locked(0)) return rc;
+    }
+    if (!t_timer.ev0) {
+        HIP_TRY(hipEventCreate(&t_timer.ev0));
+        HIP_TRY(hipEventCreate(&t_timer.ev1));
+    }
+    HIP_TRY(hipEventRecord(t_timer.ev0, (hipStream_t)stream));
+    t_timer.begun = true;
     return QLIN_OK;
 }
 
 int qlin_timer_end(void *stream, float *ms) {
-    std::lock_guard<std::mutex> lk(g.mu);
-    if (!g.ready) return fail(QLIN_ERR_ARG, "qlin_timer_begin was not called");
+    if (!t_timer.begun) return fail(QLIN_ERR_ARG, "qlin_timer_begin was not called on this thread");
     if (!ms) return fail(QLIN_ERR_ARG, "null pointer");
-    HIP_TRY(hipEventRecord(g.ev1, (hipStream_t)stream));
-    HIP_TRY(hipEventSynchronize(g.ev1));
-    HIP_TRY(hipEventElapsedTime(ms, g.ev0, g.ev1));
+    HIP_TRY(hipEventRecord(t_timer.ev1, (hipStream_t)stream));
+    HIP_TRY(hipEventSynchronize(t_timer.ev1));
+    HIP_TRY(hipEventElapsedTime(ms, t_timer.ev0, t_timer.ev1));
     return QLIN_OK;
 }
 

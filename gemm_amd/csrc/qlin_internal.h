@@ -61,6 +61,8 @@ inline JobView job_view(const GemvJob &job) {
 
 /* one job: y[n_rows] = W . x (or the fused forms above), any supported type and any whole-block shape */
 hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t stream);
+/* dense F32/F16/BF16 rows of any length and element alignment, one element per lane and step */
+hipError_t launch_gemv_dense_ragged(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t stream);
 /* streaming matvec for every type; returns false if the shape rules of gemv_stream.hip do not
  * hold (nothing was launched), else true with the launch status in *err */
 bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,

@@ -7,9 +7,11 @@
  * call them where it calls its CPU path today; the third group works on device-resident
  * buffers (no copies per call) for engines that keep activations on the GPU.
  *
- * Supported ggml types (ids are enum ggml_dtype, common/gguf_loader.h:45-85):
- *   Q8_0 = 8, Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16, IQ4_NL = 20, IQ3_S = 21,
- *   and F32 = 0 / F16 = 1 / BF16 = 30 in the codec group only.
+ * Supported ggml types (ids are enum ggml_dtype, common/gguf_loader.h:45-85): all 24 block formats with
+ * a decoder in common/ggml_dequant.h - Q4_0 = 2, Q4_1 = 3, Q5_0 = 6, Q5_1 = 7, Q8_0 = 8, Q2_K = 10,
+ * Q3_K = 11, Q4_K = 12, Q5_K = 13, Q6_K = 14, IQ2_XXS = 16, IQ2_XS = 17, IQ3_XXS = 18, IQ1_S = 19,
+ * IQ4_NL = 20, IQ3_S = 21, IQ2_S = 22, IQ4_XS = 23, IQ1_M = 29, TQ1_0 = 34, TQ2_0 = 35, MXFP4 = 39,
+ * NVFP4 = 40, Q1_0 = 41 - and the dense F32 = 0 / F16 = 1 / BF16 = 30 rows.
  *
  * Every function returns a status (0 = ok, negative = error) unless it mirrors a `void`
  * reference function, in which case it reports on stderr and zero-fills its output the way
@@ -17,9 +19,15 @@
  * There is no CPU fallback anywhere: without a usable GPU every call fails with
  * QLIN_ERR_DEVICE.
  *
- * Threading: all entry points are serialised on one internal mutex; host-pointer calls run on
- * the library's own stream and return after the result is in host memory. Device-resident
- * calls are asynchronous on the stream they are given.
+ * Threading: host-pointer entry points are serialised on one internal mutex, run on the library's
+ * own stream and return after the result is in host memory. Device-resident calls may be made from
+ * several threads at once; they are asynchronous on the stream they are given. qlin_timer_begin/end
+ * keep their events per calling thread.
+ *
+ * First call and stream capture: the first call of a device-resident entry point for a given kernel
+ * variant raises that kernel's LDS limit (hipFuncSetAttribute), and the routes through the vendor's
+ * dense GEMM create its handle and a plan per shape. Neither may happen while a stream is being
+ * captured into a graph: run every call shape once before hipStreamBeginCapture.
  */
 #ifndef QLINEAR_H
 #define QLINEAR_H
@@ -314,18 +322,6 @@ const char *qlin_gguf_get_str(const qlin_gguf *g, int i);           /* NULL unle
 /* arrays: element type, count and the address of the first element in the mapped file (strings:
  * u64 length + bytes each, not terminated) */
 int  qlin_gguf_get_array(const qlin_gguf *g, int i, uint32_t *elem_type, uint64_t *n, const void **first);
-
-/* Measurement probes: what this GPU sustains on the two resources the kernels are priced against (the
- * reference prints a peak beside every measured rate, rdna4/dequant/bench_dequant.c:1043-1110). All three
- * only enqueue; time them with qlin_timer_begin/end.
- *   qlin_probe_mfma_bf16: register-only loop of the prefill GEMM's matrix instruction on every compute
- *     unit, `iters` x 4 instructions per wave; *flops receives the flops of the launch.
- *   qlin_probe_clocks: waits for the stream, then returns the shader clock (MHz) that the last
- *     qlin_probe_mfma_bf16 launch ran at (cycle counter against the 100 MHz counter).
- *   qlin_probe_hbm_read: streaming read of n_bytes (16-byte aligned) of device memory. */
-int qlin_probe_mfma_bf16(int iters, void *stream, double *flops);
-int qlin_probe_clocks(void *stream, double *shader_mhz);
-int qlin_probe_hbm_read(const void *buf, size_t n_bytes, void *stream);
 
 /* Elapsed milliseconds of work enqueued on `stream` between the two calls, by HIP events
  * recorded on that stream (the role of elapsed_kernel_ms in rdna4/dequant/bench_dequant.c:764-780). */

@@ -2,9 +2,12 @@
  * qlinear_tf.h - the reference's quantized-linear call shapes on top of the C ABI of qlinear.h.
  *
  * The reference keeps this path as `static` functions of a header-only library
- * (common/transformer.h). The functions below take the same arguments in the same order and
- * behave the same on failure (a message on stderr and a zero-filled output; they return void),
- * so a C engine written against transformer.h can call them in place of its own:
+ * (common/transformer.h). The functions below take the same arguments and behave the same on
+ * failure (a message on stderr and a zero-filled output; they return void). The single-thread
+ * forms keep the reference's argument order; the `_pool` forms take the activation first instead of
+ * the model pointer, and the QLINEAR_TF_REFERENCE_NAMES macros at the end of this header restore
+ * the reference's names AND argument order for all of them, so a C engine written against
+ * transformer.h compiles against this header unchanged:
  *
  *   qtensor                      common/transformer.h:34-43 (same fields, same order)
  *   qtf_row_bytes                tf_row_bytes                  :489-514
@@ -30,8 +33,9 @@
  *   - the `transformer_model *m` of the pool variants is replaced by the activation pointer the
  *     reference reads from it (m->xb); thread counts and scratch rows (`tmp`) are accepted and
  *     ignored: the GPU needs neither.
- *   - supported weight types are the seven block formats of qlinear.h; F32/F16/BF16 and the other
- *     block formats report "unsupported" exactly as an unknown type does in the reference.
+ *   - supported weight types are the sixteen block formats plus F32/F16/BF16 that the reference's model
+ *     path accepts (tf_is_supported_weight_type, :462-487); any other type reports "unsupported"
+ *     exactly as an unknown type does in the reference.
  * Define QLINEAR_TF_REFERENCE_NAMES before including this header to also get the reference's own
  * names (tf_qmatvec, ...) as macros.
  */
@@ -108,6 +112,14 @@ void qtf_moe_ffn(float *out, const qtensor *gate_exps, const qtensor *up_exps,
 #define tf_qmatvec                   qtf_qmatvec
 #define tf_qmatvec_expert            qtf_qmatvec_expert
 #define tf_gemm_f16_mt_tokenmajor    qtf_gemm_tokenmajor
+/* the pool variants, in the reference's argument order (common/transformer.h:1117, :897, :1021, :1136): the
+ * model pointer is dropped, except that the fused Q/K/V call reads its activation from it (m->xb, as the
+ * reference does, :1027-1029), so `m` must point to a struct with a `const float *xb` member there */
+#define tf_qmatvec_pool(m, dst, mat, x, n_rows) qtf_qmatvec_pool(x, dst, mat, n_rows)
+#define tf_qmatvec_fused2_pool(m, dst1, mat1, dst2, mat2, x, n_rows) qtf_qmatvec_fused2_pool(x, dst1, mat1, dst2, mat2, n_rows)
+#define tf_qmatvec_fused_qkv_pool(m, q, mat_q, n_q, k, mat_k, v, mat_v, n_kv) \
+    qtf_qmatvec_fused_qkv_pool((m)->xb, q, mat_q, n_q, k, mat_k, v, mat_v, n_kv)
+#define tf_qmatvec_expert_pool(m, dst, mat, expert, x, rows_per_expert) qtf_qmatvec_expert_pool(x, dst, mat, expert, rows_per_expert)
 #endif
 
 #ifdef __cplusplus

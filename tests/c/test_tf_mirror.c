@@ -80,14 +80,15 @@ int main(void) {
     tf_qmatvec(y, &a, x, 256, NULL);
     check_rows("tf_qmatvec q4_K", &a, 0, 256, x, y);
     if (qtf_register_tensor(&a) != 0) { printf("register FAIL\n"); failures++; }
-    qtf_qmatvec_pool(x, y, &a, 200); /* fewer rows than the tensor holds */
+    struct { const float *xb; } model = {x}, *m = &model; /* what the reference's pool calls read from the model */
+    tf_qmatvec_pool(m, y, &a, x, 200); /* fewer rows than the tensor holds */
     check_rows("qmatvec_pool registered", &a, 0, 200, x, y);
 
-    qtf_qmatvec_fused2_pool(x, y, &a, y2, &b, 256);
+    tf_qmatvec_fused2_pool(m, y, &a, y2, &b, x, 256);
     check_rows("fused2 first", &a, 0, 256, x, y);
     check_rows("fused2 second", &b, 0, 256, x, y2);
 
-    qtf_qmatvec_fused_qkv_pool(x, y, &a, 256, y2, &c8, y3, &c6, 96);
+    tf_qmatvec_fused_qkv_pool(m, y, &a, 256, y2, &c8, y3, &c6, 96);
     check_rows("fused qkv q (q4_K)", &a, 0, 256, x, y);
     check_rows("fused qkv k (q8_0)", &c8, 0, 96, x, y2);
     check_rows("fused qkv v (q6_K)", &c6, 0, 96, x, y3);
@@ -125,6 +126,8 @@ int main(void) {
 
     tf_qmatvec_expert(y, &a, 3, x, 64, NULL); /* 4 experts of 64 rows */
     check_rows("tf_qmatvec_expert", &a, 192, 64, x, y);
+    tf_qmatvec_expert_pool(m, y, &a, 2, x, 64);
+    check_rows("tf_qmatvec_expert_pool", &a, 128, 64, x, y);
 
     /* prefill, token-major with strides wider than the data */
     float *Y = (float *)malloc(sizeof(float) * 3 * 300);

@@ -19,7 +19,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 sys.path.insert(0, ROOT)
-from gemm_amd import synth  # noqa: E402
+import synth  # noqa: E402
 from oracle.pyoracle import Reference  # noqa: E402
 
 OUT = os.path.dirname(os.path.abspath(__file__))

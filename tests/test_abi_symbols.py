@@ -11,9 +11,13 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "qlinear.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(qlin_[a-z0-9_A-Z]+)\s*\(", text)))
+    """every function of the engine's header and of the bench-only probe header"""
+    names = set()
+    for header in ("qlinear.h", "qlinear_bench.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(qlin_[a-z0-9_A-Z]+)\s*\(", text))
+    return sorted(names)
 
 
 @pytest.fixture(scope="module")

@@ -8,7 +8,8 @@ import struct
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests import gguf_writer as gw
 from tests.conftest import GOLDEN
 

@@ -4,7 +4,8 @@ Tolerance: relative L2 <= 1e-5 like every fp32 matvec path."""
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu

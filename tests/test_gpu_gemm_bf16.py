@@ -11,7 +11,8 @@ Two bars per case:
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu

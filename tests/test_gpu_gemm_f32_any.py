@@ -6,7 +6,8 @@ oracle's decoded weights with the same activations."""
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu

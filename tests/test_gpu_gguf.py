@@ -6,7 +6,8 @@ import os
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests import gguf_writer as gw
 from tests.conftest import GOLDEN, rel_l2
 from tests.test_gguf_parse import Gguf

@@ -4,7 +4,8 @@ Tolerance: relative L2 <= 1e-5 for every fp32 path."""
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu
@@ -61,7 +62,7 @@ def test_matvec_empty_and_errors():
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_Q4_K, 512, x.ctypes.data, 0) == 0
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, 99, 512, x.ctypes.data, 4) == qlinear.ERR_TYPE
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, 9, 512, x.ctypes.data, 4) == qlinear.ERR_TYPE  # Q8_1
-    assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_F16, 500, x.ctypes.data, 4) == qlinear.ERR_ARG
+    assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_F16, 500, x.ctypes.data, 4) == 0  # dense rows: any length
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_Q4_K, 500, x.ctypes.data, 4) == qlinear.ERR_ARG
     assert lib.qlin_matvec(None, W.ctypes.data, synth.GGML_Q4_K, 512, x.ctypes.data, 4) == qlinear.ERR_ARG
     assert lib.qlin_matvec(y.ctypes.data, W.ctypes.data, synth.GGML_Q4_K, 512, x.ctypes.data, -1) == qlinear.ERR_ARG
@@ -240,18 +241,53 @@ def test_routing_over_expert_counts(oracle, n_expert, k):
         b.free()
 
 
-@pytest.mark.parametrize("n_expert", [100, 600])
-def test_routing_ties_take_the_lower_expert_index(n_expert):
-    lib = qlinear.load()
-    lg = np.zeros((1, n_expert), np.float32)          # all equal: the first k experts, in index order
-    lg[0, 70] = 1.0                                   # one clear winner first
-    k = 6
+def _route_on_device(lg, k):
+    n_tok, n_expert = lg.shape
     dl = qlinear.DevBuf.from_numpy(lg)
-    di, dw = qlinear.DevBuf(k * 4), qlinear.DevBuf(k * 4)
-    assert lib.qlin_moe_route_dev(dl.ptr, 1, n_expert, k, di.ptr, dw.ptr, None) == 0
+    di, dw = qlinear.DevBuf(n_tok * k * 4), qlinear.DevBuf(n_tok * k * 4)
+    assert qlinear.load().qlin_moe_route_dev(dl.ptr, n_tok, n_expert, k, di.ptr, dw.ptr, None) == 0
     qlinear.sync()
-    assert list(di.to_numpy(np.int32, (k,))) == [70, 0, 1, 2, 3, 4]
-    w = dw.to_numpy(np.float32, (k,))
-    assert abs(float(w.sum()) - 1.0) < 1e-6 and w[0] > w[1] and np.all(w[1:] == w[1])
+    idx, w = di.to_numpy(np.int32, (n_tok, k)), dw.to_numpy(np.float32, (n_tok, k))
     for b in (dl, di, dw):
         b.free()
+    return idx, w
+
+
+@pytest.mark.parametrize("n_expert", [100, 600])  # probabilities in registers / in LDS
+def test_routing_ties_choose_the_experts_the_reference_heap_keeps(oracle, n_expert):
+    """Equal probabilities around the k-th place: which of them survive is decided by the reference's
+    min-heap (common/transformer.h:4057-4086), not by the index. The device must keep the same experts
+    with the same weights; where the heap decides it also emits them in heap order."""
+    rng = np.random.default_rng(77 + n_expert)
+    k = 6
+    lg = rng.integers(0, 3, size=(40, n_expert)).astype(np.float32) * np.float32(0.5)  # three levels: ties everywhere
+    lg[0] = 0.0
+    lg[0, 70] = 1.0                       # one winner, everything else equal
+    lg[1] = 0.25                          # all equal
+    idx, w = _route_on_device(lg, k)
+    for t in range(lg.shape[0]):
+        oi, ow = oracle.moe_route(lg[t], k)
+        got = dict(zip(idx[t].tolist(), w[t].tolist()))
+        want = dict(zip(oi.tolist(), ow.tolist()))
+        assert set(got) == set(want), (t, sorted(got), sorted(want))
+        for e in want:
+            assert abs(got[e] - want[e]) <= 1e-6 * want[e], (t, e)
+    # all equal: the heap keeps the first k experts it saw, root first
+    assert idx[1].tolist() == oracle.moe_route(lg[1], k)[0].tolist()
+
+
+@pytest.mark.parametrize("n_expert", [100, 600])
+def test_routing_with_non_finite_logits_follows_the_reference(oracle, n_expert):
+    """A NaN or +Inf logit makes every probability NaN (softmax divides by a NaN sum); the reference's heap
+    then keeps the first k experts with NaN weights (every comparison is false). Same here."""
+    k = 4
+    lg = np.random.default_rng(5).standard_normal((3, n_expert)).astype(np.float32)
+    lg[0, 17] = np.nan
+    lg[1, 3] = np.inf
+    idx, w = _route_on_device(lg, k)
+    for t in (0, 1):
+        oi, ow = oracle.moe_route(lg[t], k)
+        assert idx[t].tolist() == oi.tolist() == list(range(k))
+        assert np.all(np.isnan(w[t])) and np.all(np.isnan(ow))
+    oi, ow = oracle.moe_route(lg[2], k)  # the finite token beside them is untouched
+    assert set(idx[2].tolist()) == set(oi.tolist()) and abs(float(w[2].sum()) - 1.0) < 1e-6

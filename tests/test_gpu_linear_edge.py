@@ -6,7 +6,8 @@ import threading
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu
@@ -155,3 +156,34 @@ def test_concurrent_host_threads(oracle):
     assert not errors, errors
     for tid, n_rows, n_cols, W, x, serial in jobs:
         assert rel_l2(serial, oracle.gemv_f64(tid, W, x, n_cols)) <= TOL
+
+
+@pytest.mark.parametrize("tid,name", list(synth.DENSE_TYPES.items()))
+@pytest.mark.parametrize("n_cols", [1, 7, 1001, 4100])
+def test_dense_rows_of_any_length(tid, name, n_cols):
+    """tf_qmatvec dots F32/F16/BF16 rows element by element, whatever their length
+    (common/transformer.h:1049-1114); so does the matvec here, on host and on device pointers, also when a
+    matrix starts off a 16-byte boundary."""
+    n_rows = 37
+    W = synth.make_weights(tid, n_rows, n_cols, seed=900 + tid)
+    x = synth.make_activation(n_cols, seed=901)
+    if tid == synth.GGML_F32:
+        dec = W.view(np.float32).reshape(n_rows, n_cols)
+    elif tid == synth.GGML_F16:
+        dec = W.view(np.float16).reshape(n_rows, n_cols).astype(np.float32)
+    else:
+        dec = synth.bf16_bits_to_f32(W.view(np.uint16).reshape(n_rows, n_cols))
+    want = dec.astype(np.float64) @ x.astype(np.float64)
+    got = qlinear.matvec(tid, W, x, n_cols)
+    assert rel_l2(got, want) <= TOL, (name, n_cols, rel_l2(got, want))
+    # device pointers, the matrix one element past a 16-byte boundary
+    elem = 4 if tid == synth.GGML_F32 else 2
+    raw = np.concatenate([np.zeros(elem, np.uint8), W.reshape(-1)])
+    dW, dx, dy = qlinear.DevBuf.from_numpy(raw), qlinear.DevBuf.from_numpy(x), qlinear.DevBuf(n_rows * 4)
+    lib = qlinear.load()
+    assert lib.qlin_gemv_dev(tid, dW.ptr + elem, dx.ptr, dy.ptr, n_rows, n_cols, None) == 0
+    qlinear.sync()
+    got = dy.to_numpy(np.float32, (n_rows,))
+    assert rel_l2(got, want) <= TOL, (name, n_cols, "offset", rel_l2(got, want))
+    for b in (dW, dx, dy):
+        b.free()

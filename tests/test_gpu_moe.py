@@ -11,7 +11,8 @@ activation as a bf16 head + tail, so it is held to 2e-5 here.
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu

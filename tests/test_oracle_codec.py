@@ -5,7 +5,7 @@ import hashlib
 import numpy as np
 import pytest
 
-from gemm_amd import synth
+import synth
 from tests import formulas
 
 NAMES = list(synth.TYPE_NAMES.items())

@@ -2,7 +2,7 @@
 import numpy as np
 import pytest
 
-from gemm_amd import synth
+import synth
 from tests.conftest import rel_l2
 
 NAMES = list(synth.TYPE_NAMES.items())
@@ -76,6 +76,22 @@ def test_moe_route_invariants(oracle):
         sm /= sm.sum()
         assert np.allclose(w, sm, rtol=2e-6, atol=1e-8)
         assert w[0] == w.min()  # heap order: the root is the smallest survivor
+
+
+def test_moe_route_ties_follow_the_heap(oracle):
+    """Worked by hand from common/transformer.h:4057-4086 with probabilities (0.2, 0.2, 0.6), k = 2: experts 0
+    and 1 fill the heap (root 0), expert 2 replaces the root and sinks below expert 1 -> heap (1, 2). A
+    selection by index order would keep expert 0."""
+    idx, w = oracle.moe_route(np.log(np.array([0.2, 0.2, 0.6], np.float32)), 2)
+    assert idx.tolist() == [1, 2]
+    assert np.allclose(w, [0.25, 0.75], rtol=1e-6)
+    # all equal: nothing ever beats the root, the first k stay, in fill order
+    idx, w = oracle.moe_route(np.zeros(10, np.float32), 4)
+    assert idx.tolist() == [0, 1, 2, 3] and np.allclose(w, 0.25)
+    # four experts (0.1, 0.4, 0.1, 0.4), k = 2: fill (0, 1); expert 2 ties with the root and stays out;
+    # expert 3 replaces the root (0.1) and stays on top of the equal 0.4 -> heap (3, 1)
+    idx, w = oracle.moe_route(np.log(np.array([0.1, 0.4, 0.1, 0.4], np.float32)), 2)
+    assert idx.tolist() == [3, 1] and np.allclose(w, [0.5, 0.5], rtol=1e-6)
 
 
 def test_moe_ffn_token_against_numpy(oracle):

@@ -5,7 +5,8 @@ Collected last: it must pass alone in a fresh process and after every other test
 import numpy as np
 import pytest
 
-from gemm_amd import qlinear, synth
+from gemm_amd import qlinear
+import synth
 from tests.conftest import rel_l2
 
 pytestmark = pytest.mark.gpu
