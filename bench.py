@@ -430,6 +430,11 @@ def probe(args):
         tid, r, c = (synth.GGML_Q8_0, 4096, 4096) if args.probe == "gemv_q8_0" else (synth.GGML_Q6_K, 151936, 4096)
         ms, copies = time_gemv(tid, r, c, max(10, args.steps // 8), 3, max_copies=24 if r < 100000 else 2)
         print(json.dumps({"probe": args.probe, "ms_per_step": ms, "copies": copies}))
+    elif args.probe == "gemv_any":  # --ptype NAME --prows R --pcols C: that matvec only
+        tid = {v: k for k, v in list(synth.TYPE_NAMES.items()) + list(synth.DENSE_TYPES.items())}[args.ptype]
+        ms, copies = time_gemv(tid, args.prows, args.pcols, max(10, args.steps // 4), 3)
+        print(json.dumps({"probe": "gemv_any %s %dx%d" % (args.ptype, args.prows, args.pcols), "ms_per_step": ms,
+                          "copies": copies, "bytes": gemv_bytes(tid, args.prows, args.pcols)}))
     elif args.probe == "gemv_q4_0":
         ms, copies = time_gemv(synth.GGML_Q4_0, 14336, 4096, max(10, args.steps // 4), 3)
         print(json.dumps({"probe": args.probe, "ms_per_step": ms, "copies": copies}))
@@ -548,7 +553,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the GEMM and the other shapes")
-    ap.add_argument("--probe", choices=["copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--ptype", default="iq2_xxs", help="--probe gemv_any: format name")
+    ap.add_argument("--prows", type=int, default=4096)
+    ap.add_argument("--pcols", type=int, default=14336)
+    ap.add_argument("--probe", choices=["gemv_any", "copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "

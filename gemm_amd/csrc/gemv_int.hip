@@ -59,7 +59,14 @@ template <int N> __device__ __forceinline__ void ld_dwords_at(const uint8_t *img
 __device__ __forceinline__ uint32_t spread4(uint32_t v) { return ((v & 15u) * 0x00204081u) & 0x01010101u; }
 
 /* 16-entry byte table lookup of four nibbles (bytes 0..15 in t0..t3): two byte permutes + select */
-struct Table16 { uint32_t t0, t1, t2, t3; };
+struct Table16 {
+    uint32_t t0, t1, t2, t3;
+    /* the grid formats: their codebook in LDS, and byte masks of the eight signs of a group of eight
+     * elements (0xFF where the element is negative), by sign byte and by the 7-bit index of the 2/3-bit
+     * i-quants (eighth sign = parity) */
+    const uint32_t *grid;
+    const uint2 *sign256, *sign128;
+};
 __device__ __forceinline__ uint32_t look4(uint32_t n, const Table16 &t) {
     const uint32_t sel = n & 0x07070707u;
     const uint32_t lo = __builtin_amdgcn_perm(t.t1, t.t0, sel), hi = __builtin_amdgcn_perm(t.t3, t.t2, sel);
@@ -317,7 +324,91 @@ template <> struct IntFmt<T_MXFP4> {
     }
 };
 
+/* magnitudes m (four bytes, each 1..127: no grid of these formats holds a zero) with the signs of mask s
+ * (0xFF = negative) -> signed bytes: (m ^ s) + (s & 1) per byte; a nonzero m keeps the +1 inside its byte */
+__device__ __forceinline__ uint32_t apply_signs(uint32_t m, uint32_t s) { return (m ^ s) + (s & 0x01010101u); }
+
+/* IQ2_XXS [d][8 x (4 grid indices, 4 x 7 sign bits + 4-bit scale)]: d*(0.5+s)*0.25 * grid byte * sign
+ * (common/ggml_dequant.h:2793-2816); 66-byte blocks */
+template <> struct IntFmt<T_IQ2_XXS> {
+    static constexpr bool kSigned = true, kPer16 = false;
+    __device__ static Codes get(const uint8_t *img, int g, const Table16 &t) {
+        Codes r;
+        const int off = (g >> 3) * 66;
+        uint32_t a[2];
+        ld_dwords_at<2>(img, off + 2 + 8 * (g & 7), a);
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint2 m = grid[(a[0] >> (8 * l)) & 255u];
+            const uint2 sg = t.sign128[(a[1] >> (7 * l)) & 127u];
+            r.c[2 * l] = apply_signs(m.x, sg.x);
+            r.c[2 * l + 1] = apply_signs(m.y, sg.y);
+        }
+        r.s_lo = half_bits_fast(ld_u16(img + off)) * (0.5f + (float)(a[1] >> 28)) * 0.25f;
+        r.o_lo = 0.0f;
+        return r;
+    }
+};
+
+/* IQ3_XXS [d][qs 64][8 x (4 x 7 sign bits + 4-bit scale)]: d*(0.5+s)*0.5 * grid byte * sign, a four-byte
+ * grid entry per index byte (:2916-2940); 98-byte blocks */
+template <> struct IntFmt<T_IQ3_XXS> {
+    static constexpr bool kSigned = true, kPer16 = false;
+    __device__ static Codes get(const uint8_t *img, int g, const Table16 &t) {
+        Codes r;
+        const int off = (g >> 3) * 98, gi = g & 7;
+        uint32_t q[2], w[1];
+        ld_dwords_at<2>(img, off + 2 + 8 * gi, q);
+        ld_dwords_at<1>(img, off + 66 + 4 * gi, w);
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint32_t pair = (l < 2 ? q[0] : q[1]) >> (16 * (l & 1));
+            const uint2 sg = t.sign128[(w[0] >> (7 * l)) & 127u];
+            r.c[2 * l] = apply_signs(t.grid[pair & 255u], sg.x);
+            r.c[2 * l + 1] = apply_signs(t.grid[(pair >> 8) & 255u], sg.y);
+        }
+        r.s_lo = half_bits_fast(ld_u16(img + off)) * (0.5f + (float)(w[0] >> 28)) * 0.5f;
+        r.o_lo = 0.0f;
+        return r;
+    }
+};
+
+/* IQ3_S [d][qs 64][qh 8][signs 32][scales 4]: d*(1+2s) * grid byte * sign, 9-bit grid indices (:3022-3058);
+ * 110-byte blocks */
+template <> struct IntFmt<T_IQ3_S> {
+    static constexpr bool kSigned = true, kPer16 = false;
+    __device__ static Codes get(const uint8_t *img, int g, const Table16 &t) {
+        Codes r;
+        const int off = (g >> 3) * 110, gi = g & 7;
+        uint32_t q[2], sb[1];
+        ld_dwords_at<2>(img, off + 2 + 8 * gi, q);
+        ld_dwords_at<1>(img, off + 74 + 4 * gi, sb);
+        const uint32_t qh = img[off + 66 + gi];
+        const uint32_t nib = (img[off + 106 + (gi >> 1)] >> (4 * (gi & 1))) & 15u;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint32_t pair = (l < 2 ? q[0] : q[1]) >> (16 * (l & 1));
+            const uint32_t i0 = (pair & 255u) | (((qh >> (2 * l)) & 1u) << 8);
+            const uint32_t i1 = ((pair >> 8) & 255u) | (((qh >> (2 * l + 1)) & 1u) << 8);
+            const uint2 sg = t.sign256[(sb[0] >> (8 * l)) & 255u];
+            r.c[2 * l] = apply_signs(t.grid[i0], sg.x);
+            r.c[2 * l + 1] = apply_signs(t.grid[i1], sg.y);
+        }
+        r.s_lo = half_bits_fast(ld_u16(img + off)) * (float)(1u + 2u * nib);
+        r.o_lo = 0.0f;
+        return r;
+    }
+};
+
 template <uint32_t T> constexpr bool kUsesTable = (T == T_IQ4_NL || T == T_IQ4_XS || T == T_MXFP4);
+/* codebook of the grid formats: bytes staged in LDS and their source */
+template <uint32_t T> struct IntGrid { static constexpr int kBytes = 0; __device__ static const uint32_t *src() { return nullptr; } };
+template <> struct IntGrid<T_IQ2_XXS> { static constexpr int kBytes = 2048; __device__ static const uint32_t *src() { return reinterpret_cast<const uint32_t *>(qlin_iq2xxs_grid); } };
+template <> struct IntGrid<T_IQ3_XXS> { static constexpr int kBytes = 1024; __device__ static const uint32_t *src() { return qlin_iq3xxs_grid; } };
+template <> struct IntGrid<T_IQ3_S> { static constexpr int kBytes = 2048; __device__ static const uint32_t *src() { return qlin_iq3s_grid; } };
+constexpr int kSignTableBytes = (256 + 128) * 8;
+template <uint32_t T> constexpr int kAuxBytes = IntGrid<T>::kBytes > 0 ? IntGrid<T>::kBytes + kSignTableBytes : 0;
 
 /* planes and constants of one x group, as read from LDS */
 struct XGroup {
@@ -381,15 +472,17 @@ template <typename F> __device__ __forceinline__ float group_dot(const Codes &cd
 /* NG > 0: a lane's groups (lane, lane + 64, ... : at most NG of them) keep their x planes in registers
  * for all rows; NG == 0: any row length, the planes are read from LDS for every row */
 template <uint32_t T, int NG>
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(NG > 2 ? 512 : 1024)
 gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int row_bytes, int depth, int rows_per_wg) {
     using F = IntFmt<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    /* LDS map: x groups [n_cols/32][28 dwords] | raw x [n_cols] floats | row images [waves][depth][row_bytes] */
+    /* LDS map: x groups [n_cols/32][28 dwords] | raw x [n_cols] floats | codebook and sign masks of the grid
+     * formats | row images [waves][depth][row_bytes] */
     const int n_groups = n_cols >> 5;
     uint32_t *planes = reinterpret_cast<uint32_t *>(lds);
     const float4 *xraw = reinterpret_cast<const float4 *>(planes + n_groups * kGroupDw);
-    uint8_t *images = lds + (size_t)n_groups * kGroupDw * 4 + (size_t)n_cols * 4;
+    uint8_t *aux = lds + (size_t)n_groups * kGroupDw * 4 + (size_t)n_cols * 4;
+    uint8_t *images = aux + kAuxBytes<T>;
 
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -495,7 +588,19 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
             if (j == 4) dst[27] = __float_as_uint(sum);
         }
     }
-    Table16 tab = {0, 0, 0, 0};
+    Table16 tab = {0, 0, 0, 0, nullptr, nullptr, nullptr};
+    if (IntGrid<T>::kBytes > 0) {
+        uint32_t *grid = reinterpret_cast<uint32_t *>(aux);
+        uint2 *sign256 = reinterpret_cast<uint2 *>(aux + IntGrid<T>::kBytes), *sign128 = sign256 + 256;
+        for (int t = threadIdx.x; t < IntGrid<T>::kBytes / 4; t += n_threads) grid[t] = IntGrid<T>::src()[t];
+        if (threadIdx.x < 384) {
+            const uint32_t i = threadIdx.x, sb = i < 256 ? i : iq_sign_byte(i - 256);
+            sign256[i] = make_uint2(spread4(sb) * 0xFFu, spread4(sb >> 4) * 0xFFu);
+        }
+        tab.grid = grid;
+        tab.sign256 = sign256;
+        tab.sign128 = sign128;
+    }
     if (kUsesTable<T>) {
         const uint4 v = *reinterpret_cast<const uint4 *>(T == T_MXFP4 ? qlin_mxfp4_values : qlin_iq4nl_values);
         tab.t0 = v.x; tab.t1 = v.y; tab.t2 = v.z; tab.t3 = v.w;
@@ -558,9 +663,13 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
         if ((uintptr_t)job.W[m] & 15) return false;
     if ((uintptr_t)x & 15) return false;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
-    const size_t x_bytes = (size_t)(n_cols >> 5) * kGroupDw * 4 + (size_t)n_cols * 4;
+    const size_t x_bytes = (size_t)(n_cols >> 5) * kGroupDw * 4 + (size_t)n_cols * 4 + (size_t)kAuxBytes<T>;
     const size_t lds_cap = 160 * 1024 - 16;
-    int waves = 16, depth = 2;
+    const int n_groups = n_cols >> 5;
+    /* long rows of the grid formats: eight waves of 256 registers, so that a lane keeps the x planes of its
+     * seven groups for all its rows (read from LDS for every row they are what the kernel waits for) */
+    const bool wide = IntGrid<T>::kBytes > 0 && n_groups > 128 && n_groups <= 448;
+    int waves = wide ? 8 : 16, depth = 2;
     if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) depth = 1;
     if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) { waves = 8; depth = 2; }
     if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) depth = 1;
@@ -570,7 +679,6 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
     if (rows_per_wg < 1) rows_per_wg = 1;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = x_bytes + (size_t)waves * depth * row_bytes + 16; /* + slack for the funnel-shift reads */
-    const int n_groups = n_cols >> 5;
     auto launch = [&](auto kernel, OnceFlag &raised) {
         if (!raised.is_set()) {
             *err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -581,9 +689,10 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
                            (int)row_bytes, depth, rows_per_wg);
         *err = hipGetLastError();
     };
-    static OnceFlag raised[3];
+    static OnceFlag raised[4];
     if (n_groups <= 64) launch(gemv_int_kernel<T, 1>, raised[1]);
     else if (n_groups <= 128) launch(gemv_int_kernel<T, 2>, raised[2]);
+    else if (wide && waves == 8) launch(gemv_int_kernel<T, (IntGrid<T>::kBytes > 0) ? 7 : 0>, raised[3]);
     else launch(gemv_int_kernel<T, 0>, raised[0]);
     return true;
 }
@@ -606,6 +715,9 @@ bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_co
     case T_IQ4_NL: return int_typed<T_IQ4_NL>(job, x, n_cols, n_cu, stream, err);
     case T_IQ4_XS: return int_typed<T_IQ4_XS>(job, x, n_cols, n_cu, stream, err);
     case T_MXFP4: return int_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ2_XXS: return int_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ3_XXS: return int_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ3_S: return int_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err);
     default: return false;
     }
 }
