@@ -17,6 +17,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <vector>
 #include <mutex>
 #include <string>
 
@@ -88,6 +89,7 @@ struct DevBuf {
 };
 
 struct Range { size_t bytes; void *dev; };
+constexpr size_t kPinnedHalf = (size_t)2 << 20; /* bytes of pinned staging per direction */
 
 struct State {
     std::mutex mu;
@@ -97,10 +99,20 @@ struct State {
     hipStream_t stream = nullptr;
     std::map<uintptr_t, Range> registry; /* host begin -> range */
     DevBuf w[3], x, y[3], tmp[4];
+    /* pinned host staging for the small per-call transfers of the host-pointer entry points (x up, y down):
+     * a copy between pageable memory and the GPU is staged and waited for by the runtime one at a time */
+    uint8_t *pinned = nullptr;
+    size_t up_used = 0, down_used = 0;
+    struct Pending { void *host; const void *staged; size_t bytes; };
+    std::vector<Pending> pending;
     bool prefill_bf16 = false; /* qlin_gemm_tokenmajor on the matrix cores (opt-in: costs accuracy) */
 } g;
 
 int ensure_init_locked(int device) {
+    if (!g.pending.empty() || g.up_used || g.down_used) { /* left by a call that failed before it finished */
+        g.pending.clear();
+        g.up_used = g.down_used = 0;
+    }
     if (g.ready) return QLIN_OK;
     int count = 0;
     if (hipGetDeviceCount(&count) != hipSuccess || count <= 0)
@@ -113,6 +125,10 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipStreamCreate(&g.stream));
     g.device = device;
     if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
+    if (hipHostMalloc((void **)&g.pinned, 2 * kPinnedHalf, hipHostMallocDefault) != hipSuccess) {
+        g.pinned = nullptr; /* transfers then go straight from and to the caller's memory */
+        (void)hipGetLastError();
+    }
     HIP_TRY(moe_static_scratch_setup(device)); /* address of the no-allocation entry point's scratch on this device */
     g.ready = true;
     return QLIN_OK;
@@ -142,6 +158,43 @@ const void *lookup_locked(const void *host, size_t need) {
     --it;
     if (h < it->first || h + need > it->first + it->second.bytes) return nullptr;
     return static_cast<const uint8_t *>(it->second.dev) + (h - it->first);
+}
+
+/* host -> device on the library's stream; small transfers go through the pinned buffer */
+int upload_locked(void *dev, const void *host, size_t bytes) {
+    const size_t need = (bytes + 255) & ~(size_t)255;
+    if (g.pinned && g.up_used + need <= kPinnedHalf) {
+        uint8_t *st = g.pinned + g.up_used;
+        g.up_used += need;
+        memcpy(st, host, bytes);
+        HIP_TRY(hipMemcpyAsync(dev, st, bytes, hipMemcpyHostToDevice, g.stream));
+    } else {
+        HIP_TRY(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, g.stream));
+    }
+    return QLIN_OK;
+}
+/* device -> host on the library's stream; the bytes are in `host` after finish_locked() */
+int download_locked(void *host, const void *dev, size_t bytes) {
+    const size_t need = (bytes + 255) & ~(size_t)255;
+    if (g.pinned && g.down_used + need <= kPinnedHalf) {
+        uint8_t *st = g.pinned + kPinnedHalf + g.down_used;
+        g.down_used += need;
+        HIP_TRY(hipMemcpyAsync(st, dev, bytes, hipMemcpyDeviceToHost, g.stream));
+        g.pending.push_back({host, st, bytes});
+    } else {
+        HIP_TRY(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, g.stream));
+    }
+    return QLIN_OK;
+}
+/* waits for the library's stream and hands the staged results over */
+int finish_locked() {
+    const hipError_t e = hipStreamSynchronize(g.stream);
+    if (e == hipSuccess)
+        for (const State::Pending &pd : g.pending) memcpy(pd.host, pd.staged, pd.bytes);
+    g.pending.clear();
+    g.up_used = g.down_used = 0;
+    if (e != hipSuccess) return fail(QLIN_ERR_DEVICE, "hipStreamSynchronize failed: %s", hipGetErrorString(e));
+    return QLIN_OK;
 }
 
 /* device view of host weights: the registered copy, or a staged copy in `buf` */
@@ -196,11 +249,11 @@ int matvec_host_locked(float *dst, const void *W, uint32_t type, int n_cols, con
     if (int rc = weights_on_device_locked(W, rb * (size_t)n_rows, g.w[slot], &dW)) return rc;
     if (upload_x) {
         if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
-        HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_cols * 4, hipMemcpyHostToDevice, g.stream));
+        if (int rc = upload_locked(g.x.p, x, (size_t)n_cols * 4)) return rc;
     }
     if (int rc = g.y[slot].ensure((size_t)n_rows * 4 + 16)) return rc;
     HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)g.y[slot].p, n_rows, n_cols, g.stream));
-    HIP_TRY(hipMemcpyAsync(dst, g.y[slot].p, (size_t)n_rows * 4, hipMemcpyDeviceToHost, g.stream));
+    if (int rc = download_locked(dst, g.y[slot].p, (size_t)n_rows * 4)) return rc;
     return QLIN_OK;
 }
 
@@ -210,7 +263,7 @@ int matvec_host_locked(float *dst, const void *W, uint32_t type, int n_cols, con
 int matvec_multi_host_locked(int n_mat, float *const dst[3], const void *const W[3], const uint32_t types[3],
                              const int n_rows[3], int n_cols, const float *x, int mode) {
     if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
-    HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_cols * 4, hipMemcpyHostToDevice, g.stream));
+    if (int rc = upload_locked(g.x.p, x, (size_t)n_cols * 4)) return rc;
     const void *dW[3] = {nullptr, nullptr, nullptr};
     bool same = true;
     for (int m = 0; m < n_mat; m++) {
@@ -221,7 +274,7 @@ int matvec_multi_host_locked(int n_mat, float *const dst[3], const void *const W
     }
     if (mode == kAdd)
         for (int m = 0; m < n_mat; m++)
-            if (n_rows[m]) HIP_TRY(hipMemcpyAsync(g.y[m].p, dst[m], (size_t)n_rows[m] * 4, hipMemcpyHostToDevice, g.stream));
+            if (n_rows[m]) { if (int rc = upload_locked(g.y[m].p, dst[m], (size_t)n_rows[m] * 4)) return rc; }
     const float *dx = (const float *)g.x.p;
     if (same && n_rows[0] > 0) {
         GemvJob job = {{dW[0], dW[1], dW[2]}, {(float *)g.y[0].p, (float *)g.y[1].p, (float *)g.y[2].p},
@@ -237,7 +290,7 @@ int matvec_multi_host_locked(int n_mat, float *const dst[3], const void *const W
     }
     const int n_out = mode == kSiluMul ? 1 : n_mat;
     for (int m = 0; m < n_out; m++)
-        if (n_rows[m]) HIP_TRY(hipMemcpyAsync(dst[m], g.y[m].p, (size_t)n_rows[m] * 4, hipMemcpyDeviceToHost, g.stream));
+        if (n_rows[m]) { if (int rc = download_locked(dst[m], g.y[m].p, (size_t)n_rows[m] * 4)) return rc; }
     return QLIN_OK;
 }
 
@@ -287,6 +340,10 @@ void qlin_shutdown(void) {
     for (auto &b : g.y) b.release();
     for (auto &b : g.tmp) b.release();
     g.x.release();
+    if (g.pinned) (void)hipHostFree(g.pinned);
+    g.pinned = nullptr;
+    g.pending.clear();
+    g.up_used = g.down_used = 0;
     (void)hipStreamDestroy(g.stream);
     g.stream = nullptr;
     g.ready = false;
@@ -333,7 +390,7 @@ int qlin_dequant_rows(uint32_t ggml_type, const void *src, float *dst, int n_row
         HIP_TRY(hipMemcpy2DAsync(dst, (size_t)n_cols * 4, g.tmp[0].p, (size_t)n_cols * 4, (size_t)whole * 4,
                                  (size_t)n_rows, hipMemcpyDeviceToHost, g.stream));
     }
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -426,7 +483,7 @@ int qlin_matvec(float *dst, const void *W, uint32_t type, int n_cols, const floa
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;
     if (int rc = matvec_host_locked(dst, W, type, n_cols, x, n_rows, 0, true)) return rc;
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -443,7 +500,7 @@ int qlin_matvec_fused2(float *dst1, const void *W1, uint32_t type1, float *dst2,
     float *dst[3] = {dst1, dst2, nullptr};
     const int rows[3] = {n_rows, n_rows, 0};
     if (int rc = matvec_multi_host_locked(2, dst, W, types, rows, n_cols, x, kStore)) return rc;
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -462,7 +519,7 @@ int qlin_matvec_qkv(float *q, const void *Wq, uint32_t type_q, int n_q, float *k
     float *dst[3] = {q, k, v};
     const int rows[3] = {n_q, n_kv, n_kv};
     if (int rc = matvec_multi_host_locked(3, dst, W, types, rows, n_cols, x, kStore)) return rc;
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -479,7 +536,7 @@ int qlin_matvec_silu_mul(float *dst, const void *Wgate, uint32_t type_gate, cons
     float *out[3] = {dst, nullptr, nullptr};
     const int rows[3] = {n_rows, n_rows, 0};
     if (int rc = matvec_multi_host_locked(2, out, W, types, rows, n_cols, x, kSiluMul)) return rc;
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -494,7 +551,7 @@ int qlin_matvec_add(float *dst, const void *W, uint32_t type, int n_cols, const 
     float *out[3] = {dst, nullptr, nullptr};
     const int rows[3] = {n_rows, 0, 0};
     if (int rc = matvec_multi_host_locked(1, out, Wm, types, rows, n_cols, x, kAdd)) return rc;
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -509,15 +566,15 @@ int qlin_matvec_argmax(int *index, float *value, float *logits, const void *W, u
     const void *dW;
     if (int rc = weights_on_device_locked(W, rb * (size_t)n_rows, g.w[0], &dW)) return rc;
     if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
-    HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_cols * 4, hipMemcpyHostToDevice, g.stream));
+    if (int rc = upload_locked(g.x.p, x, (size_t)n_cols * 4)) return rc;
     if (int rc = g.y[0].ensure((size_t)n_rows * 4 + 16)) return rc;
     if (int rc = g.tmp[0].ensure(QLIN_ARGMAX_RESULT_BYTES)) return rc;
     HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)g.y[0].p, n_rows, n_cols, g.stream));
     HIP_TRY(launch_argmax((const float *)g.y[0].p, n_rows, (float *)g.tmp[0].p, g.stream));
     float res[2];
-    HIP_TRY(hipMemcpyAsync(res, g.tmp[0].p, 8, hipMemcpyDeviceToHost, g.stream));
-    if (logits) HIP_TRY(hipMemcpyAsync(logits, g.y[0].p, (size_t)n_rows * 4, hipMemcpyDeviceToHost, g.stream));
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = download_locked(res, g.tmp[0].p, 8)) return rc;
+    if (logits) { if (int rc = download_locked(logits, g.y[0].p, (size_t)n_rows * 4)) return rc; }
+    if (int rc = finish_locked()) return rc;
     memcpy(index, &res[0], 4);
     if (value) *value = res[1];
     return QLIN_OK;
@@ -603,7 +660,7 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
     }
     HIP_TRY(hipMemcpy2DAsync(Y, (size_t)out_stride * 4, g.tmp[1].p, (size_t)n_rows * 4, (size_t)n_rows * 4,
                              (size_t)n_tok, hipMemcpyDeviceToHost, g.stream));
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
@@ -650,11 +707,11 @@ int qlin_moe_ffn_token_types(float *out, const void *gate_exps, const void *up_e
     int32_t *d_idx = (int32_t *)(t0 + off_idx);
     float *d_w = (float *)(t0 + off_w);
     HIP_TRY(hipMemcpyAsync(t0, router_logits, (size_t)n_expert * 4, hipMemcpyHostToDevice, g.stream));
-    HIP_TRY(hipMemcpyAsync(g.x.p, x, (size_t)n_embd * 4, hipMemcpyHostToDevice, g.stream));
+    if (int rc = upload_locked(g.x.p, x, (size_t)n_embd * 4)) return rc;
     HIP_TRY(launch_moe_route((const float *)t0, 1, n_expert, top_k, d_idx, d_w, g.stream));
     int32_t h_idx[64];
     HIP_TRY(hipMemcpyAsync(h_idx, d_idx, (size_t)top_k * 4, hipMemcpyDeviceToHost, g.stream));
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = finish_locked()) return rc;
     for (int k = 0; k < top_k; k++) {
         const int e = h_idx[k];
         if (e < 0 || e >= n_expert) return fail(QLIN_ERR_DEVICE, "router produced expert %d", e);
@@ -672,8 +729,8 @@ int qlin_moe_ffn_token_types(float *out, const void *gate_exps, const void *up_e
         HIP_TRY(dispatch_gemv(type_down, de, (const float *)g.tmp[1].p, (float *)g.tmp[3].p, n_embd, n_ff, g.stream));
         HIP_TRY(launch_axpy_dev_weight((float *)g.y[0].p, (const float *)g.tmp[3].p, d_w, k, n_embd, k == 0, g.stream));
     }
-    HIP_TRY(hipMemcpyAsync(out, g.y[0].p, (size_t)n_embd * 4, hipMemcpyDeviceToHost, g.stream));
-    HIP_TRY(hipStreamSynchronize(g.stream));
+    if (int rc = download_locked(out, g.y[0].p, (size_t)n_embd * 4)) return rc;
+    if (int rc = finish_locked()) return rc;
     return QLIN_OK;
 }
 
