@@ -105,6 +105,8 @@ struct State {
     size_t up_used = 0, down_used = 0;
     struct Pending { void *host; const void *staged; size_t bytes; };
     std::vector<Pending> pending;
+    bool dense_gemm_library = true; /* bf16 products by the vendor library (faster); QLIN_DENSE_GEMM=own or
+                                       qlin_set_dense_gemm_own(1): by this library's tile kernel */
     bool prefill_bf16 = false; /* qlin_gemm_tokenmajor on the matrix cores (opt-in: costs accuracy) */
 } g;
 
@@ -125,6 +127,7 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipStreamCreate(&g.stream));
     g.device = device;
     if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
+    if (const char *e = getenv("QLIN_DENSE_GEMM")) g.dense_gemm_library = e[0] != 'o';
     if (hipHostMalloc((void **)&g.pinned, 2 * kPinnedHalf, hipHostMallocDefault) != hipSuccess) {
         g.pinned = nullptr; /* transfers then go straight from and to the caller's memory */
         (void)hipGetLastError();
@@ -664,6 +667,13 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
     return QLIN_OK;
 }
 
+int qlin_set_dense_gemm_own(int enable) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    if (int rc = ensure_init_locked(0)) return rc;
+    g.dense_gemm_library = enable == 0;
+    return QLIN_OK;
+}
+
 int qlin_set_prefill_matrix_cores(int enable) {
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;
@@ -931,10 +941,23 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
         HIP_TRY(launch_dequant_bf16(type, W, (uint16_t *)workspace, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));
         Wd = (const uint16_t *)workspace;
     }
+    /* the dense product: the vendor library's kernel, or - where the library offers none for the shape, or
+     * when asked for (QLIN_DENSE_GEMM=own, qlin_set_dense_gemm_own) - this library's own tile kernel
+     * (gemm_dense_mfma.hip; K a multiple of 256) */
+    const bool own_ok = n_cols % 256 == 0 && aligned(Wd, 16);
+    if (own_ok && !g.dense_gemm_library) {
+        HIP_TRY(launch_gemm_dense_own(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        return QLIN_OK;
+    }
     void *lib_ws = (char *)workspace + dense_gemm_weight_bytes(n_rows, n_cols);
     if (const char *err = launch_gemm_dense_bf16(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, lib_ws, kDenseLibWorkspace,
-                                                 (hipStream_t)stream))
+                                                 (hipStream_t)stream)) {
+        if (own_ok) { /* a shape the library has no kernel for */
+            HIP_TRY(launch_gemm_dense_own(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+            return QLIN_OK;
+        }
         return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+    }
     return QLIN_OK;
 }
 

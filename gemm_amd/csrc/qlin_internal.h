@@ -89,6 +89,10 @@ const char *launch_gemm_dense(bool fp32_operands, const void *Wd, const void *X,
                               int n_tok, int ldx, int ldy, void *lib_ws, size_t lib_ws_bytes, hipStream_t stream);
 const char *launch_gemm_dense_bf16(const uint16_t *Wd, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                    int ldx, int ldy, void *lib_ws, size_t lib_ws_bytes, hipStream_t stream);
+/* this library's dense bf16 x bf16 tile kernel (gemm_dense_mfma.hip): n_cols % 256 == 0, Wd and X 16-byte
+ * aligned, ldx % 8 == 0 */
+hipError_t launch_gemm_dense_own(const uint16_t *Wd, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
+                                 int ldx, int ldy, hipStream_t stream);
 constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
 hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                   int ldx, int ldy, hipStream_t stream);

@@ -109,6 +109,7 @@ SIGNATURES = {
     "qlin_gguf_get_str": (C.c_char_p, [_vp, C.c_int]),
     "qlin_gguf_get_array": (C.c_int, [_vp, C.c_int, _vp, _vp, _vp]),
     "qlin_set_prefill_matrix_cores": (C.c_int, [C.c_int]),
+    "qlin_set_dense_gemm_own": (C.c_int, [C.c_int]),
     "qlin_dequant_bf16_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemm_bf16_any_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "qlin_gemm_bf16_any_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, C.c_size_t, _vp]),

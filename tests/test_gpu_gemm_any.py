@@ -32,6 +32,15 @@ def run(tid, W, Xb, n_rows, n_cols, n_tok, ldx=None, ldy=None, ws=None):
     return Y
 
 
+@pytest.fixture(params=["vendor", "own"])
+def dense_kernel(request):
+    """both dense bf16 products behind qlin_gemm_bf16_any_dev: the vendor library's (default) and this
+    library's own tile kernel"""
+    qlinear.check(qlinear.load().qlin_set_dense_gemm_own(1 if request.param == "own" else 0))
+    yield request.param
+    qlinear.check(qlinear.load().qlin_set_dense_gemm_own(0))
+
+
 def references(oracle, tid, W, Xb, n_cols):
     dec = oracle.dequant_matrix(tid, W, n_cols)
     Xf = synth.bf16_bits_to_f32(Xb).astype(np.float64)
@@ -41,7 +50,7 @@ def references(oracle, tid, W, Xb, n_cols):
 
 
 @pytest.mark.parametrize("tid", sorted(ALL), ids=lambda t: ALL[t])
-def test_every_format(oracle, tid):
+def test_every_format(oracle, tid, dense_kernel):
     n_tok, n_rows, n_cols = 72, 160, 512
     W = synth.make_weights(tid, n_rows, n_cols, seed=500 + tid)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=600 + tid, tokens=n_tok))
@@ -56,8 +65,9 @@ def test_every_format(oracle, tid):
     (synth.GGML_Q6_K, 1, 16, 256), (synth.GGML_Q6_K, 515, 1000, 1024), (synth.GGML_Q8_0, 130, 257, 96),
     (synth.GGML_Q5_K, 64, 2048, 768), (synth.GGML_IQ4_NL, 200, 130, 4096), (Q4K, 513, 384, 512),
     (Q4K, 1100, 300, 256), (Q4K, 300, 25700, 256), (synth.GGML_BF16, 33, 100, 264), (synth.GGML_F16, 300, 64, 1000),
+    (synth.GGML_BF16, 700, 3000, 1024), (synth.GGML_Q6_K, 257, 129, 2048), (synth.GGML_Q8_0, 100, 4100, 512),
 ])
-def test_shapes(oracle, tid, n_tok, n_rows, n_cols):
+def test_shapes(oracle, tid, n_tok, n_rows, n_cols, dense_kernel):
     W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + n_tok)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=n_cols + n_tok, tokens=n_tok))
     Y = run(tid, W, Xb, n_rows, n_cols, n_tok)
