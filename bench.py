@@ -37,10 +37,13 @@ BF16_PEAK_TFLOPS = 2500.0     # MI355X dense bf16 MFMA, published
 FP32_PEAK_TFLOPS = 157.3      # MI355X dense fp32 MFMA, published
 Q4K = synth.GGML_Q4_K
 
-# HBM bytes moved per Q4_K 14336x4096 matvec launch, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by what the same counters read for a device-to-device copy of known size
-# (profiles/gemv_q4k_14336x4096.md).
-MEASURED_TRAFFIC_BYTES = 33319932
+# HBM bytes moved per Q4_K 14336x4096 matvec launch. Not measured by this script: it is the figure of two
+# rocprofv3 --pmc runs of `bench.py --probe gemv` (FETCH_SIZE, then WRITE_SIZE), each scaled by what the
+# same counter reads for a device-to-device copy of known size, as recorded with its commands in
+# PROFILED_TRAFFIC_SOURCE. It changes only when the kernel's loads change and the profile is taken again;
+# tests/test_profiles.py fails when the two files disagree.
+PROFILED_TRAFFIC_BYTES = 33373986
+PROFILED_TRAFFIC_SOURCE = "profiles/gemv_q4k_14336x4096.md"
 
 
 def gemv_bytes(type_id, n_rows, n_cols):
@@ -600,6 +603,15 @@ def main():
             m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
             anyfmt["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
         extra["prefill_gemm_any_format_14336x4096_decode_to_bf16_plus_library_gemm"] = anyfmt
+        own = {}
+        qlinear.check(qlinear.load().qlin_set_dense_gemm_own(1))
+        try:
+            for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("bf16", synth.GGML_BF16, 512), ("q6_K", synth.GGML_Q6_K, 2048)):
+                m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
+                own["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
+        finally:
+            qlinear.check(qlinear.load().qlin_set_dense_gemm_own(0))
+        extra["prefill_gemm_any_format_14336x4096_decode_to_bf16_plus_own_tile_kernel"] = own
         exact = {}
         for tname, tid, M in (("q4_K", Q4K, 512), ("q6_K", synth.GGML_Q6_K, 512), ("q4_K", Q4K, 64)):
             m = time_gemm_f32_any(tid, M, 14336, 4096, max(3, args.steps // 60), 1)
@@ -649,7 +661,9 @@ def main():
                    "bytes_per_step": nbytes, "weight_copies_rotated": copies, "device": name.strip(),
                    "compute_units": n_cu},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES},
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": PROFILED_TRAFFIC_BYTES,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, scaled by a copy of "
+                                       "known size; not re-measured by this run (" + PROFILED_TRAFFIC_SOURCE + ")"},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(n_rows, n_cols)
