@@ -102,6 +102,7 @@ struct State {
     /* pinned host staging for the small per-call transfers of the host-pointer entry points (x up, y down):
      * a copy between pageable memory and the GPU is staged and waited for by the runtime one at a time */
     uint8_t *pinned = nullptr;
+    uint8_t *pinned_dev = nullptr; /* the same buffer as kernels address it; null: results come by the runtime's copy */
     size_t up_used = 0, down_used = 0;
     struct Pending { void *host; const void *staged; size_t bytes; };
     std::vector<Pending> pending;
@@ -128,8 +129,11 @@ int ensure_init_locked(int device) {
     g.device = device;
     if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
     if (const char *e = getenv("QLIN_DENSE_GEMM")) g.dense_gemm_library = e[0] != 'o';
-    if (hipHostMalloc((void **)&g.pinned, 2 * kPinnedHalf, hipHostMallocDefault) != hipSuccess) {
+    if (hipHostMalloc((void **)&g.pinned, 2 * kPinnedHalf, hipHostMallocMapped) != hipSuccess) {
         g.pinned = nullptr; /* transfers then go straight from and to the caller's memory */
+        (void)hipGetLastError();
+    } else if (hipHostGetDevicePointer((void **)&g.pinned_dev, g.pinned, 0) != hipSuccess) {
+        g.pinned_dev = nullptr;
         (void)hipGetLastError();
     }
     HIP_TRY(moe_static_scratch_setup(device)); /* address of the no-allocation entry point's scratch on this device */
@@ -176,13 +180,33 @@ int upload_locked(void *dev, const void *host, size_t bytes) {
     }
     return QLIN_OK;
 }
+/* Results go to the pinned buffer by a kernel that stores over the bus, not by the runtime's device-to-host
+ * copy: after a process has freed a few GiB of device memory that copy took 95 us instead of 9.5 us for the
+ * 57 KB of a matvec result (until another stream was created), which made a 35 us call a 130 us call. */
+__global__ void __launch_bounds__(256) store_to_host_kernel(uint8_t *__restrict__ dst, const uint8_t *__restrict__ src,
+                                                            size_t bytes) {
+    const size_t n16 = bytes >> 4;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256)
+        reinterpret_cast<uint4 *>(dst)[i] = reinterpret_cast<const uint4 *>(src)[i];
+    if (blockIdx.x == 0 && threadIdx.x < (bytes & 15)) dst[(n16 << 4) + threadIdx.x] = src[(n16 << 4) + threadIdx.x];
+}
+
 /* device -> host on the library's stream; the bytes are in `host` after finish_locked() */
 int download_locked(void *host, const void *dev, size_t bytes) {
     const size_t need = (bytes + 255) & ~(size_t)255;
+    if (bytes == 0) return QLIN_OK;
     if (g.pinned && g.down_used + need <= kPinnedHalf) {
         uint8_t *st = g.pinned + kPinnedHalf + g.down_used;
         g.down_used += need;
-        HIP_TRY(hipMemcpyAsync(st, dev, bytes, hipMemcpyDeviceToHost, g.stream));
+        if (g.pinned_dev && aligned(dev, 16)) {
+            const size_t groups = ((bytes >> 4) + 255) / 256;
+            const int grid = (int)std::min<size_t>(std::max<size_t>(groups, 1), 64);
+            store_to_host_kernel<<<grid, 256, 0, g.stream>>>(g.pinned_dev + (st - g.pinned),
+                                                             static_cast<const uint8_t *>(dev), bytes);
+            HIP_TRY(hipGetLastError());
+        } else {
+            HIP_TRY(hipMemcpyAsync(st, dev, bytes, hipMemcpyDeviceToHost, g.stream));
+        }
         g.pending.push_back({host, st, bytes});
     } else {
         HIP_TRY(hipMemcpyAsync(host, dev, bytes, hipMemcpyDeviceToHost, g.stream));
@@ -345,6 +369,7 @@ void qlin_shutdown(void) {
     g.x.release();
     if (g.pinned) (void)hipHostFree(g.pinned);
     g.pinned = nullptr;
+    g.pinned_dev = nullptr;
     g.pending.clear();
     g.up_used = g.down_used = 0;
     (void)hipStreamDestroy(g.stream);
