@@ -45,9 +45,11 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr int kQ4KBlock = 144;
+constexpr int kHeadInts = 32, kHeadTokens = 16; /* an expert's record: one 128-byte line */
 
 struct Workspace {
     int32_t *offsets;  /* [n_expert + 1] first slot of each expert */
+    int32_t *head;     /* [n_expert][32] per expert: first slot, count, 14 unused, tokens of its first 16 slots */
     int32_t *order;    /* [n_pairs] slot -> pair (t*top_k + k), grouped by expert */
     int32_t *slot_of;  /* [n_pairs] pair -> slot, -1 for an expert index out of range */
     float *w_slot;     /* [n_pairs] routing weight of the pair in each slot */
@@ -66,6 +68,7 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
     size_t off = 0;
     Workspace w;
     w.offsets = (int32_t *)(p + off); off += round256(((size_t)n_expert + 1) * 4);
+    w.head = (int32_t *)(p + off);    off += round256((size_t)n_expert * kHeadInts * 4);
     w.order = (int32_t *)(p + off);   off += round256(n_pairs * 4);
     w.slot_of = (int32_t *)(p + off); off += round256(n_pairs * 4);
     w.w_slot = (float *)(p + off);    off += round256(n_pairs * 4);
@@ -82,7 +85,7 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int32_t *__restrict__ offsets,
                  int32_t *__restrict__ order, int32_t *__restrict__ slot_of, const float *__restrict__ expert_w,
-                 float *__restrict__ w_slot) {
+                 float *__restrict__ w_slot, int32_t *__restrict__ head, int top_k) {
     extern __shared__ int32_t lds[]; /* cnt[n_expert], cur[n_expert], wave_total[16] */
     int32_t *cnt = lds, *cur = lds + n_expert;
     for (int e = threadIdx.x; e < n_expert; e += blockDim.x) cnt[e] = 0;
@@ -114,6 +117,8 @@ moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int
         for (int q = 0; q < per; q++) {
             if (e0 + q < n_expert) {
                 offsets[e0 + q] = run;
+                head[(e0 + q) * kHeadInts] = run;
+                head[(e0 + q) * kHeadInts + 1] = cnt[e0 + q];
                 cur[e0 + q] = run;
                 run += cnt[e0 + q];
             }
@@ -127,6 +132,10 @@ moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int
         if (e >= 0 && e < n_expert) {
             slot = atomicAdd(&cur[e], 1);
             order[slot] = p;
+            /* the tokens of an expert's first slots sit beside its count: the matrix kernels find them with
+             * one load instead of offsets -> order -> token */
+            const int rank = slot - offsets[e];
+            if (rank < kHeadTokens) head[e * kHeadInts + kHeadInts - kHeadTokens + rank] = p / top_k;
             w_slot[slot] = expert_w[p]; /* by slot, so that the down kernel finds it with one load */
         }
         slot_of[p] = slot;
@@ -238,24 +247,55 @@ __device__ __forceinline__ void load_acts(Acts<NA> &s, const uint16_t *const (&a
  * the matvec kernels: a 144-byte piece ends 16 bytes into a cache line whose rest belongs to the next
  * super-block, fetched a moment later by a neighbouring wave, and a second token tile of 16 walks
  * the same weights again (few-token GEMM 13.8 -> 12.9 us at 8 tokens, 26.6 -> 24.4 us at 32). */
-template <int NW>
-__device__ __forceinline__ void image_from_global(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
-                                                  int rows_per_matrix, size_t row_bytes, int sb, int lane,
-                                                  int last_row = 0x7fffffff) {
-    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
-    constexpr int kChunks = NW * 16 * 9;
+/* The per-lane part of those addresses does not depend on the super-block: byte offset of the lane's chunk
+ * inside its matrix tile, computed once per kernel. The loads then take the tile's address plus the
+ * super-block's 144 * sb as a scalar base, so fetching an image costs no vector instruction beyond the
+ * loads (the 64-bit address arithmetic per chunk was a sixth of the vector instructions of these kernels).
+ * NM = 2: the first half of the image rows comes from one matrix, the second half from another (gate, up). */
+template <int NW, int NM>
+struct ImagePlan {
+    static constexpr int kRows = NW * 16 / NM, kChunks = kRows * 9, kInstr = (kChunks + 63) / 64;
+    uint32_t off[kInstr];
+};
+
+template <int NW, int NM>
+__device__ __forceinline__ void plan_image(ImagePlan<NW, NM> &p, size_t row_bytes, int lane, int last_row = 0x7fffffff) {
 #pragma unroll
-    for (int i = 0; i < (kChunks + 63) / 64; i++) {
+    for (int i = 0; i < ImagePlan<NW, NM>::kInstr; i++) {
         const int t = 64 * i + lane;
         int R = t / 9;
         const int c9 = t - 9 * R;
+        R = R < ImagePlan<NW, NM>::kRows ? R : ImagePlan<NW, NM>::kRows - 1; /* lanes past the last chunk issue nothing */
         R = R < last_row ? R : last_row; /* a ragged last tile re-reads its last row; those results are not stored */
-        const uint8_t *src = (R < rows_per_matrix ? m0_rows + (size_t)R * row_bytes
-                                                  : m1_rows + (size_t)(R - rows_per_matrix) * row_bytes) +
-                             (size_t)sb * kQ4KBlock + 16 * c9;
-        const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
-        if (t < kChunks)
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(m0v) : "memory");
+        p.off[i] = (uint32_t)R * (uint32_t)row_bytes + 16u * (uint32_t)c9;
+    }
+}
+
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (const uint8_t *)(uintptr_t)(((uint64_t)hi << 32) | (uint64_t)lo);
+}
+
+template <int NW, int NM>
+__device__ __forceinline__ void image_from_global(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
+                                                  const ImagePlan<NW, NM> &p, int sb, int lane) {
+    using Plan = ImagePlan<NW, NM>;
+    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+        const uint8_t *base = uniform_ptr((m == 0 ? m0_rows : m1_rows) + (size_t)sb * kQ4KBlock);
+#pragma unroll
+        for (int i = 0; i < Plan::kInstr; i++) {
+            const uint32_t m0v =
+                __builtin_amdgcn_readfirstlane(img_lds + (uint32_t)(m * Plan::kRows * kQ4KBlock) + 1024u * (uint32_t)i);
+            if (64 * i + lane < Plan::kChunks)
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                             :
+                             : "v"(p.off[i]), "s"(base), "s"(m0v)
+                             : "memory");
+        }
     }
 }
 
@@ -310,21 +350,20 @@ __device__ __forceinline__ void step_math(const uint8_t *img, int j, int kg, con
  * partial sums of the waves meet in LDS: red[wave][stream][lane][4]. After the call and a barrier,
  * element (stream s, lane l, v) of the tile is the sum over waves of
  * red[(w * NW + s) * 256 + l * 4 + v], taken in wave order. */
-template <int NW, int NA>
+template <int NW, int NM, int NA>
 __device__ __forceinline__ void ksplit_tile(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
-                                            int rows_per_matrix, size_t row_bytes,
+                                            const ImagePlan<NW, NM> &plan,
                                             const uint16_t *const (&arow)[NA], int n_sb, int wv, int n_waves,
-                                            int lane, bool live, bool image_ready, float *red,
-                                            int last_row = 0x7fffffff) {
+                                            int lane, bool live, int fetched_sb, float *red) {
     const int j = lane & 15, kg = lane >> 4;
     f32x4 acc[NW];
 #pragma unroll
     for (int w = 0; w < NW; w++) acc[w] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     for (int sb = wv; sb < n_sb; sb += n_waves) {
         Acts<NA> s;
-        if (!image_ready) {
+        if (sb != fetched_sb) { /* else the image of this super-block has been requested already */
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous image have returned */
-            image_from_global<NW>(img, m0_rows, m1_rows, rows_per_matrix, row_bytes, sb, lane, last_row);
+            image_from_global(img, m0_rows, m1_rows, plan, sb, lane);
         }
         load_acts(s, arow, sb, kg, live);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* image (and activations) have landed */
@@ -332,6 +371,93 @@ __device__ __forceinline__ void ksplit_tile(uint8_t *img, const uint8_t *m0_rows
     }
 #pragma unroll
     for (int w = 0; w < NW; w++) *reinterpret_cast<f32x4 *>(red + ((wv * NW + w) * 64 + lane) * 4) = acc[w];
+}
+
+/* ---- the same sums for an expert with at most four tokens: block-diagonal activation operand ----
+ * An expert of a routed batch sees about four tokens, so twelve of the sixteen token rows of the matrix
+ * instruction above are padding, and the fp32 scale step (16 multiply-adds per lane for every two
+ * sub-blocks) is spent on them. Here the sixteen A rows are 4 sub-blocks x 4 tokens instead: row
+ * i = 4 * s + t holds token t's activations in k group s and zeros in the other three groups, and the
+ * B lanes of k group s carry codes of a sub-block of their own (2s: low nibbles, 2s + 1: high nibbles of
+ * qs[32s .. 32s + 31]). C[4s + t][j] is then the sum over that one sub-block, it lands in lane (j, s), and
+ * four instructions chained into one accumulator cover the sub-block's 32 elements: a lane applies ONE
+ * scale pair per super-block half to four token values, 16 multiply-adds per super-block instead of 128.
+ * The sums over the four k groups and over the waves are taken afterwards.
+ *
+ * The four tokens' activations of a super-block (2 KB) come into a wave-private LDS buffer by two
+ * direct-to-LDS loads (xoff[i]: the byte offset of the lane's 16-byte chunk, token row included) instead
+ * of eight register loads of which three quarters of the lanes would be idle; the operand lanes read
+ * their 16 bytes from there. K is split over the waves as in ksplit_tile. After the call and a barrier,
+ * the value for (stream s, token t, row j) is the sum over waves w of qred[((w * NW + s) * 16 + j) * 4 + t]. */
+template <int NW, int NM>
+__device__ __forceinline__ void ksplit_quad(uint8_t *img, const uint8_t *m0_rows, const uint8_t *m1_rows,
+                                            const ImagePlan<NW, NM> &plan, uint8_t *actbuf, const uint8_t *x_base,
+                                            const uint32_t (&xoff)[2], int n_sb, int wv, int n_waves, int lane,
+                                            int fetched_sb, float *qred) {
+    const int j = lane & 15, kg = lane >> 4;
+    const bool diag = (j >> 2) == kg;
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t act_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)actbuf;
+    const uint8_t *arow = actbuf + (j & 3) * 512 + 128 * kg; /* token j & 3, sub-blocks 2 * kg and 2 * kg + 1 */
+    const uint8_t *codes = img + j * kQ4KBlock + 16 + 32 * kg;
+    f32x4 acc[NW];
+#pragma unroll
+    for (int w = 0; w < NW; w++) acc[w] = zero;
+    for (int sb = wv; sb < n_sb; sb += n_waves) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous image and activations have returned */
+        if (sb != fetched_sb) image_from_global(img, m0_rows, m1_rows, plan, sb, lane);
+        const uint8_t *xb = uniform_ptr(x_base + (size_t)sb * 512);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t m0v = __builtin_amdgcn_readfirstlane(act_lds + 1024u * (uint32_t)i);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(xoff[i]), "s"(xb), "s"(m0v) : "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* image and activations have landed */
+        f32x4 S[NW][2], X0 = zero, X1 = zero;
+#pragma unroll
+        for (int w = 0; w < NW; w++) S[w][0] = S[w][1] = zero;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            u32x4 r0 = {0u, 0u, 0u, 0u}, r1 = {0u, 0u, 0u, 0u};
+            if (diag) {
+                r0 = *(const u32x4 *)(arow + 16 * c);
+                r1 = *(const u32x4 *)(arow + 64 + 16 * c);
+            }
+            const bf16x8 a0 = __builtin_bit_cast(bf16x8, r0), a1 = __builtin_bit_cast(bf16x8, r1);
+            X0 = mma(a0, ones_bf16(), X0);
+            X1 = mma(a1, ones_bf16(), X1);
+#pragma unroll
+            for (int w = 0; w < NW; w++) {
+                const u32x2 qv = *(const u32x2 *)(codes + w * 16 * kQ4KBlock + 8 * c);
+                const bf16x8 lo = codes_to_bf16(qv.x & 0x0F0F0F0Fu, qv.y & 0x0F0F0F0Fu);
+                const bf16x8 hi = codes_to_bf16((qv.x >> 4) & 0x0F0F0F0Fu, (qv.y >> 4) & 0x0F0F0F0Fu);
+                S[w][0] = mma(a0, lo, S[w][0]);
+                S[w][1] = mma(a1, hi, S[w][1]);
+            }
+        }
+#pragma unroll
+        for (int w = 0; w < NW; w++) {
+            const Scales sc = unpack_header(*(const u32x4 *)(img + (w * 16 + j) * kQ4KBlock));
+            /* the lane's two sub-blocks 2 * kg and 2 * kg + 1: bytes 2 * (kg & 1) and + 1 of the low or high word */
+            const uint32_t sh = 16u * (uint32_t)(kg & 1);
+            const uint32_t sp = (kg < 2 ? sc.sc_lo : sc.sc_hi) >> sh, mp = (kg < 2 ? sc.mn_lo : sc.mn_hi) >> sh;
+            const float dsc0 = sc.d * (float)(sp & 0xFFu), dsc1 = sc.d * (float)((sp >> 8) & 0xFFu);
+            const float dm0 = sc.dmin * (float)(mp & 0xFFu), dm1 = sc.dmin * (float)((mp >> 8) & 0xFFu);
+            apply_scales(acc[w], S[w][0], S[w][1], X0, X1, dsc0, dm0, dsc1, dm1);
+        }
+    }
+    /* a lane holds the share of its k group: add the four groups (lanes j, j + 16, j + 32, j + 48) */
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            float a = acc[w][v];
+            a += __shfl_xor(a, 16, 64);
+            a += __shfl_xor(a, 32, 64);
+            acc[w][v] = a;
+        }
+        if (kg == 0) *reinterpret_cast<f32x4 *>(qred + ((wv * NW + w) * 16 + j) * 4) = acc[w];
+    }
 }
 
 /* thread -> element of the (16 * RT)-row x 16-slot result tile, ordered so that consecutive
@@ -357,13 +483,16 @@ __device__ __forceinline__ TileElem tile_elem(int idx) {
 #ifndef MOE_DN_WAVES
 #define MOE_DN_WAVES 2
 #endif
+#ifndef MOE_GU_WG_WAVES
+#define MOE_GU_WG_WAVES 4
+#endif
 #ifndef MOE_GU_RT
 #define MOE_GU_RT 1
 #endif
 template <int RT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_GU_WAVES)))
 moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
-                   const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
+                   const uint16_t *__restrict__ X, const int32_t *__restrict__ head,
                    const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
                    int n_embd, int n_ff, int top_k) {
     constexpr int NW = 2 * RT, kRows = 16 * RT; /* streams: RT gate tiles, then RT up tiles */
@@ -372,22 +501,75 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
     const int row0 = blockIdx.x * kRows;
-    const int first = offsets[e], cnt = offsets[e + 1] - first;
-    if (cnt == 0) return;
     const int j = lane & 15;
     const int n_sb = n_embd >> 8;
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
     const size_t ebase = ((size_t)e * n_ff + row0) * row_bytes;
-    /* LDS: red [waves][NW][64][4] floats | images [waves][NW * 16 rows][144 bytes] */
+    /* LDS: red [waves][NW][64][4] floats | images [waves][NW * 16 rows][144 bytes] | qred [waves][NW][16][4] floats.
+     * The four-token form keeps a wave's activations (2 KB) in the wave's part of red and reduces through qred. */
     uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * NW * 256) + wv * (NW * 16 * kQ4KBlock);
+    float *qred = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(red + n_waves * NW * 256) + n_waves * (NW * 16 * kQ4KBlock));
     const bool one_sb = n_sb <= n_waves; /* then a wave's image is fetched once for all token tiles */
-    if (one_sb && wv < n_sb) image_from_global<NW>(img, gate + ebase, up + ebase, kRows, row_bytes, wv, lane);
+    ImagePlan<NW, 2> plan;
+    plan_image(plan, row_bytes, lane);
+    /* The expert's record and the wave's first image are requested together: the lane's token for the
+     * sixteen-token form and for the four-token form, then the image; the wait for the tokens leaves the
+     * image's loads outstanding, and the activation loads follow while the image is still on its way.
+     * (Waiting for the record first and for the token list after it cost a workgroup a quarter of its life.) */
+    const int32_t *hd = head + (size_t)e * kHeadInts;
+    const int32_t *tok_at = hd + (kHeadInts - kHeadTokens);
+    int tok16, tok_a, tok_b; /* the token of slot j; of slots lane / 32 and 2 + lane / 32 */
+    u32x2 first_cnt; /* loaded here as well: a load the compiler issues would be waited for with everything before it */
+    asm volatile("global_load_dword %0, %4, off\n\tglobal_load_dword %1, %5, off\n\tglobal_load_dword %2, %5, off offset:8\n\t"
+                 "global_load_dwordx2 %3, %6, off"
+                 : "=&v"(tok16), "=&v"(tok_a), "=&v"(tok_b), "=&v"(first_cnt)
+                 : "v"(tok_at + j), "v"(tok_at + (lane >> 5)), "v"(hd)
+                 : "memory");
+    image_from_global(img, gate + ebase, up + ebase, plan, wv, lane); /* wv < n_sb: the launch starts min(n_sb, 4) waves */
+    constexpr int kImageLoads = 2 * ImagePlan<NW, 2>::kInstr;
+    static_assert(kImageLoads <= 15, "the wait below counts outstanding loads up to 15");
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(tok16), "+v"(tok_a), "+v"(tok_b), "+v"(first_cnt) : "n"(kImageLoads) : "memory");
+    const int first = __builtin_amdgcn_readfirstlane((int)first_cnt.x), cnt = __builtin_amdgcn_readfirstlane((int)first_cnt.y);
+    if (cnt == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* nothing may arrive in LDS after the wave has ended */
+        return;
+    }
+    auto store_h = [&](float g, float u, int slot, int row) {
+        const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
+        const __bf16 hi = (__bf16)h;
+        const __bf16 lo = (__bf16)(h - (float)hi);
+        const size_t at = (size_t)slot * n_ff + row0 + row;
+        h_hi[at] = __builtin_bit_cast(uint16_t, hi);
+        h_lo[at] = __builtin_bit_cast(uint16_t, lo);
+    };
 
+    if (cnt <= 4) {
+        /* by the expert's count, not a tile's: the rounding of a token's result must not depend on its slot */
+        const int tok0 = __builtin_amdgcn_readfirstlane(tok_a); /* slot 0 exists; it stands in for the empty slots */
+        const int sa = lane >> 5, sb2 = 2 + (lane >> 5);
+        const uint32_t xoff[2] = {(uint32_t)(sa < cnt ? tok_a : tok0) * (uint32_t)n_embd * 2u + 16u * (uint32_t)(lane & 31),
+                                  (uint32_t)(sb2 < cnt ? tok_b : tok0) * (uint32_t)n_embd * 2u + 16u * (uint32_t)(lane & 31)};
+        ksplit_quad<NW, 2>(img, gate + ebase, up + ebase, plan, reinterpret_cast<uint8_t *>(red + wv * NW * 256),
+                           reinterpret_cast<const uint8_t *>(X), xoff, n_sb, wv, n_waves, lane, wv, qred);
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 64 * RT; idx += blockDim.x) {
+            /* consecutive threads: consecutive rows of one token */
+            const int jj = idx & 15, r = (idx >> 4) % RT, t = idx / (16 * RT);
+            float g = 0.0f, u = 0.0f;
+            for (int w = 0; w < n_waves; w++) {
+                g += qred[((w * NW + r) * 16 + jj) * 4 + t];
+                u += qred[((w * NW + RT + r) * 16 + jj) * 4 + t];
+            }
+            if (t < cnt) store_h(g, u, first + t, 16 * r + jj);
+        }
+        return;
+    }
     for (int t0 = 0; t0 < cnt; t0 += 16) {
+        const int fetched_sb = (t0 == 0 || one_sb) ? wv : -1;
         const bool live = t0 + j < cnt; /* as an A lane, j is the token slot */
-        const int tok = live ? order[first + t0 + j] / top_k : 0;
+        const int tok = !live ? 0 : t0 == 0 ? tok16 : order[first + t0 + j] / top_k;
         const uint16_t *const arow[1] = {X + (size_t)tok * n_embd};
-        ksplit_tile<NW, 1>(img, gate + ebase, up + ebase, kRows, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
+        ksplit_tile<NW, 2, 1>(img, gate + ebase, up + ebase, plan, arow, n_sb, wv, n_waves, lane, live, fetched_sb, red);
         __syncthreads();
         for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
             const TileElem t = tile_elem<RT>(idx);
@@ -396,14 +578,7 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
                 g += red[((w * NW + t.r) * 64 + t.lane) * 4 + t.v];
                 u += red[((w * NW + RT + t.r) * 64 + t.lane) * 4 + t.v];
             }
-            if (t0 + t.slot < cnt) {
-                const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
-                const __bf16 hi = (__bf16)h;
-                const __bf16 lo = (__bf16)(h - (float)hi);
-                const size_t at = (size_t)(first + t0 + t.slot) * n_ff + row0 + t.row;
-                h_hi[at] = __builtin_bit_cast(uint16_t, hi);
-                h_lo[at] = __builtin_bit_cast(uint16_t, lo);
-            }
+            if (t0 + t.slot < cnt) store_h(g, u, first + t0 + t.slot, t.row);
         }
         __syncthreads();
     }
@@ -434,13 +609,15 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
     /* LDS: red [waves][RT][64][4] floats | images [waves][RT * 16 rows][144 bytes] */
     uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * RT * 256) + wv * (kRows * kQ4KBlock);
     const bool one_sb = n_sb <= n_waves;
-    if (one_sb && wv < n_sb) image_from_global<RT>(img, d0, d0, kRows, row_bytes, wv, lane);
+    ImagePlan<RT, 1> plan;
+    plan_image(plan, row_bytes, lane);
+    if (one_sb && wv < n_sb) image_from_global(img, d0, d0, plan, wv, lane);
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt;
         const size_t at_a = (size_t)(first + (live ? t0 + j : 0)) * n_ff;
         const uint16_t *const arow[2] = {h_hi + at_a, h_lo + at_a};
-        ksplit_tile<RT, 2>(img, d0, d0, kRows, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red);
+        ksplit_tile<RT, 1, 2>(img, d0, d0, plan, arow, n_sb, wv, n_waves, lane, live, one_sb ? wv : -1, red);
         __syncthreads();
         for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
             const TileElem t = tile_elem<RT>(idx);
@@ -488,6 +665,8 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
     uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * kElems) + wv * (2 * kImage);
     float *wl = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(red + n_waves * kElems) + n_waves * (2 * kImage));
     const bool has_k = wv < n_sb;
+    ImagePlan<RT, 1> plan;
+    plan_image(plan, row_bytes, lane);
 
     for (int t0 = 0; t0 < cnt; t0 += 16) {
         const bool live = t0 + j < cnt;
@@ -496,7 +675,7 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
         Acts<2> s;
         if (has_k) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous token tile's images have returned */
-            image_from_global<RT>(img, d0, d0, kRows, row_bytes, wv, lane);
+            image_from_global(img, d0, d0, plan, wv, lane);
             load_acts(s, arow, wv, kg, live);
         }
         /* the tile's routing weights go to LDS once: a global load inside the walk would make the compiler
@@ -510,7 +689,7 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
                 if (rt + 1 < NT) {
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the other image has been read */
                     const uint8_t *dn = d0 + (size_t)(rt + 1) * kRows * row_bytes;
-                    image_from_global<RT>(img + ((rt + 1) & 1) * kImage, dn, dn, kRows, row_bytes, wv, lane);
+                    image_from_global(img + ((rt + 1) & 1) * kImage, dn, dn, plan, wv, lane);
                     wait_vm_at_most(kImageLoads); /* everything older than those: this group's image, the activations */
                 } else {
                     wait_vm_at_most(0);
@@ -735,12 +914,14 @@ gemm_q4k_fewtok_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict
     /* LDS: red [waves][RT][64][4] floats | images [waves][RT * 16 rows][144 bytes] */
     uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * RT * 256) + wv * (kRows * kQ4KBlock);
     const bool one_sb = n_sb <= n_waves;
-    if (one_sb && wv < n_sb) image_from_global<RT>(img, w0, w0, kRows, row_bytes, wv, lane, last_row);
+    ImagePlan<RT, 1> plan;
+    plan_image(plan, row_bytes, lane, last_row);
+    if (one_sb && wv < n_sb) image_from_global(img, w0, w0, plan, wv, lane);
 
     for (int t0 = 0; t0 < n_tok; t0 += 16) {
         const bool live = t0 + j < n_tok;
         const uint16_t *const arow[1] = {X + (size_t)(live ? t0 + j : 0) * ldx};
-        ksplit_tile<RT, 1>(img, w0, w0, kRows, row_bytes, arow, n_sb, wv, n_waves, lane, live, one_sb, red, last_row);
+        ksplit_tile<RT, 1, 1>(img, w0, w0, plan, arow, n_sb, wv, n_waves, lane, live, one_sb ? wv : -1, red);
         __syncthreads();
         for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
             const TileElem t = tile_elem<RT>(idx);
@@ -778,7 +959,7 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), ((size_t)n_expert * 2 + 16) * sizeof(int32_t), stream, idx,
-                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, w, ws.w_slot);
+                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, w, ws.w_slot, ws.head, top_k);
     static OnceFlag lds_raised;
     if (!lds_raised.is_set()) {
         hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<MOE_GU_RT>,
@@ -794,12 +975,12 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
      * super-blocks one after the other) and 8 for down. The gate/up kernel needs 138 registers, so a
      * compute unit holds 12 of its waves: three 4-wave workgroups in different phases instead of one
      * 8-wave workgroup that loads, computes and reduces with nothing beside it (75 -> 65 us). */
-    const int gu_waves = n_embd / 256 < 4 ? n_embd / 256 : 4, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
+    const int gu_waves = n_embd / 256 < MOE_GU_WG_WAVES ? n_embd / 256 : MOE_GU_WG_WAVES, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
     if (fast_gu) {
         constexpr int RT = MOE_GU_RT;
         hipLaunchKernelGGL(moe_gate_up_kernel<RT>, dim3(n_ff / (16 * RT), n_expert), dim3(64 * gu_waves),
-                           (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock), stream,
-                           (const uint8_t *)gate, (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd,
+                           (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock + 256), stream,
+                           (const uint8_t *)gate, (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd,
                            n_ff, top_k);
     } else {
         hipError_t e1 = launch_rows_any<1>(type_gate, gate, n_ff, n_embd, n_expert, ws, top_k, X, nullptr, nullptr, ws.g32, stream);
