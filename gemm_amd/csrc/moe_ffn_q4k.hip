@@ -52,10 +52,9 @@ struct Workspace {
     int32_t *head;     /* [n_expert][32] per expert: first slot, count, 14 unused, tokens of its first 16 slots */
     int32_t *order;    /* [n_pairs] slot -> pair (t*top_k + k), grouped by expert */
     int32_t *slot_of;  /* [n_pairs] pair -> slot, -1 for an expert index out of range */
-    float *w_slot;     /* [n_pairs] routing weight of the pair in each slot */
     uint16_t *h_hi;    /* [n_pairs, n_ff] bf16 head of silu(g)*u, by slot */
     uint16_t *h_lo;    /* [n_pairs, n_ff] bf16 tail */
-    float *part;       /* [n_pairs, n_embd] w * down(h), by slot */
+    float *part;       /* [n_pairs, n_embd] down(h), by slot */
     float *g32, *u32;  /* [n_pairs, n_ff] each: gate and up results of the any-format kernels, by slot */
     size_t bytes;
 };
@@ -71,7 +70,6 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
     w.head = (int32_t *)(p + off);    off += round256((size_t)n_expert * kHeadInts * 4);
     w.order = (int32_t *)(p + off);   off += round256(n_pairs * 4);
     w.slot_of = (int32_t *)(p + off); off += round256(n_pairs * 4);
-    w.w_slot = (float *)(p + off);    off += round256(n_pairs * 4);
     w.h_hi = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
     w.h_lo = (uint16_t *)(p + off);   off += round256(n_pairs * n_ff * 2);
     w.part = (float *)(p + off);      off += round256(n_pairs * n_embd * 4);
@@ -84,8 +82,7 @@ Workspace carve(void *base, int n_tok, int top_k, int n_embd, int n_ff, int n_ex
 /* ---- 1. counting sort of pairs by expert; cnt[] and cur[] live in LDS ---- */
 __global__ void __launch_bounds__(1024)
 moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int32_t *__restrict__ offsets,
-                 int32_t *__restrict__ order, int32_t *__restrict__ slot_of, const float *__restrict__ expert_w,
-                 float *__restrict__ w_slot, int32_t *__restrict__ head, int top_k) {
+                 int32_t *__restrict__ order, int32_t *__restrict__ slot_of, int32_t *__restrict__ head, int top_k) {
     extern __shared__ int32_t lds[]; /* cnt[n_expert], cur[n_expert], wave_total[16] */
     int32_t *cnt = lds, *cur = lds + n_expert;
     for (int e = threadIdx.x; e < n_expert; e += blockDim.x) cnt[e] = 0;
@@ -136,7 +133,6 @@ moe_group_kernel(const int32_t *__restrict__ idx, int n_pairs, int n_expert, int
              * one load instead of offsets -> order -> token */
             const int rank = slot - offsets[e];
             if (rank < kHeadTokens) head[e * kHeadInts + kHeadInts - kHeadTokens + rank] = p / top_k;
-            w_slot[slot] = expert_w[p]; /* by slot, so that the down kernel finds it with one load */
         }
         slot_of[p] = slot;
     }
@@ -460,21 +456,23 @@ __device__ __forceinline__ void ksplit_quad(uint8_t *img, const uint8_t *m0_rows
     }
 }
 
-/* thread -> element of the (16 * RT)-row x 16-slot result tile, ordered so that consecutive
- * threads hold consecutive rows of one token slot: idx = ((v * 4 + kg) * RT + r) * 16 + j */
+/* thread -> element of the (16 * RT)-row x 16-slot result tile, token slot by token slot with consecutive
+ * threads on consecutive rows: idx = (slot * RT + r) * 16 + j, so that a tile with n live slots is the
+ * first n * 16 * RT elements (an expert sees about four tokens; summing the empty slots' shares as well
+ * took a fifth of the down projection's time). Slot 4 * kg + v of row j is register v of lane (j, kg). */
 struct TileElem { int r, lane, v, slot, row; };
 template <int RT>
 __device__ __forceinline__ TileElem tile_elem(int idx) {
     TileElem t;
     const int j = idx & 15, q = idx >> 4;
     t.r = q % RT;
-    const int kg = (q / RT) & 3;
-    t.v = q / (4 * RT);
-    t.lane = kg * 16 + j;
-    t.slot = 4 * kg + t.v;       /* token slot inside the 16-slot tile */
+    t.slot = q / RT;
+    t.v = t.slot & 3;
+    t.lane = (t.slot >> 2) * 16 + j;
     t.row = 16 * t.r + j;        /* row inside the group */
     return t;
 }
+__device__ __forceinline__ int live_slots(int cnt, int t0) { return cnt - t0 < 16 ? cnt - t0 : 16; }
 
 /* ---- 2. gate and up for RT * 16 rows of one expert, all of its tokens ---- */
 #ifndef MOE_GU_WAVES
@@ -571,14 +569,14 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
         const uint16_t *const arow[1] = {X + (size_t)tok * n_embd};
         ksplit_tile<NW, 2, 1>(img, gate + ebase, up + ebase, plan, arow, n_sb, wv, n_waves, lane, live, fetched_sb, red);
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
+        for (int idx = threadIdx.x; idx < live_slots(cnt, t0) * 16 * RT; idx += blockDim.x) {
             const TileElem t = tile_elem<RT>(idx);
             float g = 0.0f, u = 0.0f;
             for (int w = 0; w < n_waves; w++) {
                 g += red[((w * NW + t.r) * 64 + t.lane) * 4 + t.v];
                 u += red[((w * NW + RT + t.r) * 64 + t.lane) * 4 + t.v];
             }
-            if (t0 + t.slot < cnt) store_h(g, u, first + t0 + t.slot, t.row);
+            store_h(g, u, first + t0 + t.slot, t.row);
         }
         __syncthreads();
     }
@@ -591,8 +589,7 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
 template <int RT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
-                const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
-                const float *__restrict__ w_slot, float *__restrict__ part,
+                const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets, float *__restrict__ part,
                 int n_embd, int n_ff) {
     constexpr int kRows = 16 * RT;
     extern __shared__ __attribute__((aligned(16))) float red[];
@@ -619,14 +616,11 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
         const uint16_t *const arow[2] = {h_hi + at_a, h_lo + at_a};
         ksplit_tile<RT, 1, 2>(img, d0, d0, plan, arow, n_sb, wv, n_waves, lane, live, one_sb ? wv : -1, red);
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
+        for (int idx = threadIdx.x; idx < live_slots(cnt, t0) * 16 * RT; idx += blockDim.x) {
             const TileElem t = tile_elem<RT>(idx);
             float d = 0.0f;
             for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
-            if (t0 + t.slot < cnt) {
-                const float w = w_slot[first + t0 + t.slot];
-                part[(size_t)(first + t0 + t.slot) * n_embd + row0 + t.row] = w * d; /* w * q, as out[i] += w*q does (:4116-4127) */
-            }
+            part[(size_t)(first + t0 + t.slot) * n_embd + row0 + t.row] = d; /* the routing weight goes on in the combine */
         }
         __syncthreads();
     }
@@ -645,7 +639,7 @@ template <int RT, int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
 moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                      const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
-                     const float *__restrict__ w_slot, float *__restrict__ part, int n_embd, int n_ff) {
+                     float *__restrict__ part, int n_embd, int n_ff) {
     constexpr int kRows = 16 * RT, kImage = kRows * kQ4KBlock;
     constexpr int kImageLoads = (kRows * 9 + 63) / 64; /* direct-to-LDS instructions per image and wave */
     constexpr int kElems = 256 * RT;                   /* results of one row group and token tile */
@@ -661,9 +655,8 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
     const int n_sb = n_ff >> 8; /* <= n_waves: wave wv owns super-block wv */
     const size_t row_bytes = (size_t)n_sb * kQ4KBlock;
     const uint8_t *d0 = down + ((size_t)e * n_embd + row0) * row_bytes;
-    /* LDS: red [waves][RT][64][4] floats | images [waves][2][RT * 16 rows][144 bytes] | routing weights [16] */
+    /* LDS: red [waves][RT][64][4] floats | images [waves][2][RT * 16 rows][144 bytes] */
     uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * kElems) + wv * (2 * kImage);
-    float *wl = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(red + n_waves * kElems) + n_waves * (2 * kImage));
     const bool has_k = wv < n_sb;
     ImagePlan<RT, 1> plan;
     plan_image(plan, row_bytes, lane);
@@ -678,9 +671,8 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
             image_from_global(img, d0, d0, plan, wv, lane);
             load_acts(s, arow, wv, kg, live);
         }
-        /* the tile's routing weights go to LDS once: a global load inside the walk would make the compiler
-         * wait for the image in flight as well (the first barrier of the walk publishes them) */
-        if (threadIdx.x < 16) wl[threadIdx.x] = t0 + (int)threadIdx.x < cnt ? w_slot[first + t0 + threadIdx.x] : 0.0f;
+        /* no other global load inside the walk: the compiler would wait for the image in flight with it
+         * (the pairs' routing weights are applied by the combine) */
         for (int rt = 0; rt < NT; rt++) {
             f32x4 acc[RT];
 #pragma unroll
@@ -699,12 +691,11 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
 #pragma unroll
             for (int w = 0; w < RT; w++) *reinterpret_cast<f32x4 *>(red + ((wv * RT + w) * 64 + lane) * 4) = acc[w];
             __syncthreads();
-            for (int idx = threadIdx.x; idx < kElems; idx += blockDim.x) {
+            for (int idx = threadIdx.x; idx < live_slots(cnt, t0) * 16 * RT; idx += blockDim.x) {
                 const TileElem t = tile_elem<RT>(idx);
                 float d = 0.0f;
                 for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
-                if (t0 + t.slot < cnt)
-                    part[(size_t)(first + t0 + t.slot) * n_embd + row0 + rt * kRows + t.row] = wl[t.slot] * d;
+                part[(size_t)(first + t0 + t.slot) * n_embd + row0 + rt * kRows + t.row] = d;
             }
             __syncthreads();
         }
@@ -713,8 +704,8 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
 
 /* ---- 4. out[t] = sum over k, in k order ---- */
 __global__ void __launch_bounds__(256)
-moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of, float *__restrict__ out,
-                   int n_embd, int top_k) {
+moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of,
+                   const float *__restrict__ expert_w, float *__restrict__ out, int n_embd, int top_k) {
     const int t = blockIdx.x;
     const int c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
     if (c >= n_embd) return;
@@ -722,15 +713,24 @@ moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ s
     /* eight experts at a time: their slots, then their rows, are requested together; the additions stay in k order */
     for (int k0 = 0; k0 < top_k; k0 += 8) {
         int slot[8];
+        float wq[8];
         float4 p[8];
 #pragma unroll
-        for (int q = 0; q < 8; q++) slot[q] = k0 + q < top_k ? slot_of[t * top_k + k0 + q] : -1;
+        for (int q = 0; q < 8; q++) {
+            slot[q] = k0 + q < top_k ? slot_of[t * top_k + k0 + q] : -1;
+            wq[q] = k0 + q < top_k ? expert_w[t * top_k + k0 + q] : 0.0f;
+        }
 #pragma unroll
         for (int q = 0; q < 8; q++)
             p[q] = slot[q] >= 0 ? *(const float4 *)(part + (size_t)slot[q] * n_embd + c) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
         for (int q = 0; q < 8; q++) {
-            if (slot[q] >= 0) { s.x += p[q].x; s.y += p[q].y; s.z += p[q].z; s.w += p[q].w; }
+            if (slot[q] >= 0) {
+                /* out[i] += w * q (common/transformer.h:4116-4127): product rounded, then added */
+                float4 m = make_float4(wq[q] * p[q].x, wq[q] * p[q].y, wq[q] * p[q].z, wq[q] * p[q].w);
+                asm volatile("" : "+v"(m.x), "+v"(m.y), "+v"(m.z), "+v"(m.w)); /* keeps the products out of a fused multiply-add */
+                s.x += m.x; s.y += m.y; s.z += m.z; s.w += m.w;
+            }
         }
     }
     *(float4 *)(out + (size_t)t * n_embd + c) = s;
@@ -923,11 +923,11 @@ gemm_q4k_fewtok_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict
         const uint16_t *const arow[1] = {X + (size_t)(live ? t0 + j : 0) * ldx};
         ksplit_tile<RT, 1, 1>(img, w0, w0, plan, arow, n_sb, wv, n_waves, lane, live, one_sb ? wv : -1, red);
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 256 * RT; idx += blockDim.x) {
+        for (int idx = threadIdx.x; idx < live_slots(n_tok, t0) * 16 * RT; idx += blockDim.x) {
             const TileElem t = tile_elem<RT>(idx);
             float d = 0.0f;
             for (int w = 0; w < n_waves; w++) d += red[((w * RT + t.r) * 64 + t.lane) * 4 + t.v];
-            if (t0 + t.slot < n_tok && row0 + t.row < n_rows) Y[(size_t)(t0 + t.slot) * ldy + row0 + t.row] = d;
+            if (row0 + t.row < n_rows) Y[(size_t)(t0 + t.slot) * ldy + row0 + t.row] = d;
         }
         __syncthreads();
     }
@@ -959,7 +959,7 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), ((size_t)n_expert * 2 + 16) * sizeof(int32_t), stream, idx,
-                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, w, ws.w_slot, ws.head, top_k);
+                       n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, ws.head, top_k);
     static OnceFlag lds_raised;
     if (!lds_raised.is_set()) {
         hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<MOE_GU_RT>,
@@ -1001,20 +1001,20 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
             walk_lds_raised.set();
         }
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
-                           (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock) + 64, stream,
-                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.w_slot, ws.part, n_embd, n_ff);
+                           (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock), stream,
+                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
     } else if (fast_dn) {
         constexpr int DRT = MOE_DN_RT;
         hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
-                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.w_slot, ws.part, n_embd, n_ff);
+                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
     } else {
-        hipError_t e1 = launch_rows_any<2>(type_down, down, n_embd, n_ff, n_expert, ws, top_k, ws.h_hi, ws.h_lo, ws.w_slot,
+        hipError_t e1 = launch_rows_any<2>(type_down, down, n_embd, n_ff, n_expert, ws, top_k, ws.h_hi, ws.h_lo, nullptr,
                                            ws.part, stream);
         if (e1 != hipSuccess) return e1;
     }
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tok, (n_embd / 4 + 63) / 64), dim3(64), 0, stream, ws.part,
-                       ws.slot_of, out, n_embd, top_k);
+                       ws.slot_of, w, out, n_embd, top_k);
     return hipGetLastError();
 }
 
