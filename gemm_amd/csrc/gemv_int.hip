@@ -401,11 +401,67 @@ template <> struct IntFmt<T_IQ3_S> {
     }
 };
 
+/* IQ2_XS [d][32 x (9-bit grid index, 7 sign bits)][scales 8]: d*(0.5+s)*0.25 * grid byte * sign with one
+ * 4-bit scale per 16 elements (common/ggml_dequant.h:2966-2994); 74-byte blocks */
+template <> struct IntFmt<T_IQ2_XS> {
+    static constexpr bool kSigned = true, kPer16 = true;
+    __device__ static Codes get(const uint8_t *img, int g, const Table16 &t) {
+        Codes r;
+        const int off = (g >> 3) * 74, gi = g & 7;
+        uint32_t q[2];
+        ld_dwords_at<2>(img, off + 2 + 8 * gi, q);
+        const uint32_t sc = img[off + 66 + gi];
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint32_t w = ((l < 2 ? q[0] : q[1]) >> (16 * (l & 1))) & 0xFFFFu;
+            const uint2 m = grid[w & 511u];
+            const uint2 sg = t.sign128[w >> 9];
+            r.c[2 * l] = apply_signs(m.x, sg.x);
+            r.c[2 * l + 1] = apply_signs(m.y, sg.y);
+        }
+        const float d = half_bits_fast(ld_u16(img + off));
+        r.s_lo = d * (0.5f + (float)(sc & 15u)) * 0.25f;
+        r.s_hi = d * (0.5f + (float)(sc >> 4)) * 0.25f;
+        r.o_lo = r.o_hi = 0.0f;
+        return r;
+    }
+};
+
+/* IQ2_S [d][qs 32][signs 32][qh 8][scales 8]: 10-bit grid indices (two more bits per index from qh), sign
+ * bytes stored as they are, scales as IQ2_XS (:2996-3020); 82-byte blocks */
+template <> struct IntFmt<T_IQ2_S> {
+    static constexpr bool kSigned = true, kPer16 = true;
+    __device__ static Codes get(const uint8_t *img, int g, const Table16 &t) {
+        Codes r;
+        const int off = (g >> 3) * 82, gi = g & 7;
+        uint32_t q[1], sb[1];
+        ld_dwords_at<1>(img, off + 2 + 4 * gi, q);
+        ld_dwords_at<1>(img, off + 34 + 4 * gi, sb);
+        const uint32_t qh = img[off + 66 + gi], sc = img[off + 74 + gi];
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            const uint2 m = grid[((q[0] >> (8 * l)) & 255u) | (((qh >> (2 * l)) & 3u) << 8)];
+            const uint2 sg = t.sign256[(sb[0] >> (8 * l)) & 255u];
+            r.c[2 * l] = apply_signs(m.x, sg.x);
+            r.c[2 * l + 1] = apply_signs(m.y, sg.y);
+        }
+        const float d = half_bits_fast(ld_u16(img + off));
+        r.s_lo = d * (0.5f + (float)(sc & 15u)) * 0.25f;
+        r.s_hi = d * (0.5f + (float)(sc >> 4)) * 0.25f;
+        r.o_lo = r.o_hi = 0.0f;
+        return r;
+    }
+};
+
 template <uint32_t T> constexpr bool kUsesTable = (T == T_IQ4_NL || T == T_IQ4_XS || T == T_MXFP4);
 /* codebook of the grid formats: bytes staged in LDS and their source */
 template <uint32_t T> struct IntGrid { static constexpr int kBytes = 0; __device__ static const uint32_t *src() { return nullptr; } };
 template <> struct IntGrid<T_IQ2_XXS> { static constexpr int kBytes = 2048; __device__ static const uint32_t *src() { return reinterpret_cast<const uint32_t *>(qlin_iq2xxs_grid); } };
 template <> struct IntGrid<T_IQ3_XXS> { static constexpr int kBytes = 1024; __device__ static const uint32_t *src() { return qlin_iq3xxs_grid; } };
+template <> struct IntGrid<T_IQ2_XS> { static constexpr int kBytes = 4096; __device__ static const uint32_t *src() { return reinterpret_cast<const uint32_t *>(qlin_iq2xs_grid); } };
+template <> struct IntGrid<T_IQ2_S> { static constexpr int kBytes = 8192; __device__ static const uint32_t *src() { return reinterpret_cast<const uint32_t *>(qlin_iq2s_grid); } };
 template <> struct IntGrid<T_IQ3_S> { static constexpr int kBytes = 2048; __device__ static const uint32_t *src() { return qlin_iq3s_grid; } };
 constexpr int kSignTableBytes = (256 + 128) * 8;
 template <uint32_t T> constexpr int kAuxBytes = IntGrid<T>::kBytes > 0 ? IntGrid<T>::kBytes + kSignTableBytes : 0;
@@ -413,7 +469,7 @@ template <uint32_t T> constexpr int kAuxBytes = IntGrid<T>::kBytes > 0 ? IntGrid
 /* planes and constants of one x group, as read from LDS */
 struct XGroup {
     uint32_t xt[8], xm[8], xl[8];
-    float inv, sum_lo, sum_hi;
+    float inv, sum_lo, sum_hi; /* signed codes with a scale per half: the halves' own cneg, as bit patterns */
     int cneg; /* 128 * (256 * sum of mid bytes + sum of low bytes) */
 };
 __device__ __forceinline__ XGroup load_xgroup(const uint32_t *planes, int g) {
@@ -428,7 +484,23 @@ __device__ __forceinline__ XGroup load_xgroup(const uint32_t *planes, int g) {
 
 /* one group of codes against one group of x: the group's contribution to the row's dot product */
 template <typename F> __device__ __forceinline__ float group_dot(const Codes &cd, const XGroup &x) {
-    if (F::kSigned) {
+    if (F::kSigned && F::kPer16) {
+        int at0 = 0, at1 = 0;
+        uint32_t am0 = 0, al0 = 0, am1 = 0, al1 = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t u0 = cd.c[k] ^ 0x80808080u, u1 = cd.c[4 + k] ^ 0x80808080u; /* code + 128 */
+            at0 = sdot4(cd.c[k], x.xt[k], at0);
+            am0 = udot4(u0, x.xm[k], am0);
+            al0 = udot4(u0, x.xl[k], al0);
+            at1 = sdot4(cd.c[4 + k], x.xt[4 + k], at1);
+            am1 = udot4(u1, x.xm[4 + k], am1);
+            al1 = udot4(u1, x.xl[4 + k], al1);
+        }
+        const float f0 = fmaf((float)at0, 65536.0f, (float)((int)((am0 << 8) + al0) - __float_as_int(x.sum_lo)));
+        const float f1 = fmaf((float)at1, 65536.0f, (float)((int)((am1 << 8) + al1) - __float_as_int(x.sum_hi)));
+        return (cd.s_lo * f0 + cd.s_hi * f1) * x.inv;
+    } else if (F::kSigned) {
         int at = 0;
         uint32_t am = 0, al = 0;
 #pragma unroll
@@ -573,6 +645,7 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
         uint32_t cs = (udot4(pl_mid, 0x01010101u, 0u) << 8) + udot4(pl_low, 0x01010101u, 0u);
         cs += dppu<0xB1>(cs);
         cs += dppu<0x4E>(cs);
+        const uint32_t cs_half = cs; /* over this thread's 16-element half */
         cs += dppu<0x141>(cs);
         const int grp = idx >> 3, j = idx & 7;
         uint32_t *dst = planes + grp * kGroupDw;
@@ -583,9 +656,9 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
             if (j == 0) {
                 dst[24] = __float_as_uint(inv);
                 dst[25] = cs << 7;
-                dst[26] = __float_as_uint(sum);
+                dst[26] = (F::kSigned && F::kPer16) ? cs_half << 7 : __float_as_uint(sum);
             }
-            if (j == 4) dst[27] = __float_as_uint(sum);
+            if (j == 4) dst[27] = (F::kSigned && F::kPer16) ? cs_half << 7 : __float_as_uint(sum);
         }
     }
     Table16 tab = {0, 0, 0, 0, nullptr, nullptr, nullptr};
@@ -718,6 +791,8 @@ bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_co
     case T_IQ2_XXS: return int_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err);
     case T_IQ3_XXS: return int_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err);
     case T_IQ3_S: return int_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ2_XS: return int_typed<T_IQ2_XS>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ2_S: return int_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err);
     default: return false;
     }
 }
