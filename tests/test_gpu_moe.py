@@ -241,3 +241,29 @@ def test_grouped_ffn_mixed_formats_many_tokens_per_expert_and_ragged_shapes(orac
     got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
     want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
     assert rel_l2(got, want) <= DESIGNED
+
+
+def test_experts_with_chosen_token_counts_and_repeatability(oracle):
+    """Experts that see exactly 1, 4, 5, 16, 17 and 33 tokens (and some that see none): the kernels switch form
+    at four tokens, walk tiles of sixteen, and find the first sixteen tokens of an expert in its record and the rest
+    in the sorted list. The slots inside an expert are handed out by atomics, so the call is also repeated: the
+    result may not depend on the order they came in."""
+    n_expert, n_embd, n_ff, top_k = 12, 512, 256, 2
+    counts = {0: 1, 2: 4, 3: 5, 5: 16, 6: 17, 9: 33}
+    pairs = [e for e, c in counts.items() for _ in range(c)]  # sorted by expert; no expert holds half of them
+    rng = np.random.default_rng(7)
+    n_tok = len(pairs) // top_k
+    assert n_tok * top_k == len(pairs)
+    # token t gets entries t and t + n_tok of the sorted list: two different experts, as a router would give
+    idx = np.stack([np.array(pairs[:n_tok], np.int32), np.array(pairs[n_tok:], np.int32)], axis=1)
+    idx = idx[rng.permutation(n_tok)]
+    assert np.all(idx[:, 0] != idx[:, 1])
+    w = rng.random((n_tok, top_k), dtype=np.float32) + 0.25
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=300)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=303, tokens=n_tok))
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff)
+    first = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+    assert rel_l2(first, want) <= DESIGNED
+    for _ in range(3):
+        again = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+        assert np.array_equal(first.view(np.uint32), again.view(np.uint32))
