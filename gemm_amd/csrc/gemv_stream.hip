@@ -83,6 +83,25 @@ template <uint32_t T> struct Lean {
     }
 };
 
+/* dense fp16 rows: the hardware conversion (the decoder's hand-rebuilt NaN payloads cost six instructions per
+ * element and mean nothing inside a sum) */
+template <> struct Lean<T_F16> {
+    __device__ static float dot8(const uint8_t *img, int boff, int, const float4 xa, const float4 xb, float, const Tables &) {
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        const uint4 v = *reinterpret_cast<const uint4 *>(img + boff);
+        const half2v a = __builtin_bit_cast(half2v, v.x), b = __builtin_bit_cast(half2v, v.y);
+        const half2v c = __builtin_bit_cast(half2v, v.z), d = __builtin_bit_cast(half2v, v.w);
+        float acc = (float)a[0] * xa.x;
+        acc = fmaf((float)a[1], xa.y, acc);
+        acc = fmaf((float)b[0], xa.z, acc);
+        acc = fmaf((float)b[1], xa.w, acc);
+        acc = fmaf((float)c[0], xb.x, acc);
+        acc = fmaf((float)c[1], xb.y, acc);
+        acc = fmaf((float)d[0], xb.z, acc);
+        return fmaf((float)d[1], xb.w, acc);
+    }
+};
+
 /* Q8_0 (common/ggml_dequant.h:1479-1489): d * q, q int8 = (q ^ 0x80 as unsigned) - 128 */
 template <> struct Lean<T_Q8_0> {
     __device__ static float dot8(const uint8_t *img, int boff, int k0, const float4 xa, const float4 xb, float xs8, const Tables &) {
