@@ -702,6 +702,158 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
     }
 }
 
+/* ---- 3c. down for Q6_K experts (the down projections of K-quant mixes) ----
+ * The same walk as moe_down_walk_kernel over NT groups of 16 rows, a wave per super-block of K, the next
+ * group's image in flight while this one is multiplied. What differs:
+ *   * A Q6_K block is 210 bytes, so rows and blocks start on 2-byte boundaries. A wave's image row is the 14
+ *     aligned 16-byte chunks that cover its block (the block starts `o` = 0..14 bytes into the first); LDS is
+ *     read as aligned dwords and funnel-shifted.
+ *   * A code is q = nibble + 16 * two high bits - 32 with one int8 scale per 16 elements
+ *     (common/ggml_dequant.h:1653-1686). Nibble and high bits go through the matrix instruction as two exact
+ *     bf16 operands (both below 16, so the scaled fp8 conversion applies): sum q x = S_lo + 16 S_hi - 32 X.
+ *   * One instruction spans 32 elements = two scale groups, so the token operand is block-diagonal: A row
+ *     8 s + t holds token t's activations in the k groups of scale group s (2s, 2s + 1) and zeros in the
+ *     others; C[8 s + t][j] lands in lane (j, kg) with s = kg >> 1, t = 4 (kg & 1) + v. Eight tokens per pass.
+ * The weights stay exact as in the Q4_K kernels; the intermediate arrives as bf16 head + tail. */
+constexpr int kQ6KBlock = 210, kQ6KImageRow = 224, kQ6KWalkGroups = 8;
+
+/* n dwords from byte offset off (even) of an LDS area whose base is 16-byte aligned: aligned dword reads,
+ * funnel-shifted by the two odd bytes if any */
+template <int N>
+__device__ __forceinline__ void lds_dwords_at(const uint8_t *base, int off, uint32_t (&out)[N]) {
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(base + (off & ~3));
+    const uint32_t sh = (uint32_t)(off & 3) * 8u;
+    uint32_t prev = q[0];
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        const uint32_t next = q[i + 1];
+        out[i] = __builtin_amdgcn_alignbit(next, prev, sh);
+        prev = next;
+    }
+}
+
+template <int NT>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3)))
+moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
+                         const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
+                         float *__restrict__ part, int n_embd, int n_ff) {
+    constexpr int kImage = 16 * kQ6KImageRow + 16; /* + slack for the funnel-shift read past the last row */
+    constexpr int kChunks = 16 * 14, kImageLoads = (kChunks + 63) / 64;
+    extern __shared__ __attribute__((aligned(16))) float red[];
+    const int e = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * (16 * NT);
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int j = lane & 15, kg = lane >> 4;
+    const int n_sb = n_ff >> 8; /* == n_waves: wave wv owns super-block wv */
+    const int row_bytes = n_sb * kQ6KBlock;
+    /* 16 * row_bytes is a multiple of 16, so every row group starts on a 16-byte boundary like the tensor */
+    const uint8_t *d0 = down + ((size_t)e * n_embd + row0) * row_bytes;
+    /* LDS: red [waves][8 tokens][16 rows] floats | images [waves][2][16 rows][224 bytes + slack] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 128) + wv * (2 * kImage);
+    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
+    uint32_t off[kImageLoads];
+#pragma unroll
+    for (int i = 0; i < kImageLoads; i++) {
+        const int t = 64 * i + lane;
+        int R = t / 14;
+        const int c = t - 14 * R;
+        R = R < 16 ? R : 15;
+        off[i] = (uint32_t)((R * row_bytes + wv * kQ6KBlock) & ~15) + 16u * (uint32_t)c;
+    }
+    auto request = [&](int rt, int buf) {
+        const uint8_t *base = uniform_ptr(d0 + (size_t)rt * 16 * row_bytes);
+#pragma unroll
+        for (int i = 0; i < kImageLoads; i++) {
+            const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + (uint32_t)(buf * kImage) + 1024u * (uint32_t)i);
+            if (64 * i + lane < kChunks)
+                asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off[i]), "s"(base), "s"(m0v) : "memory");
+        }
+    };
+    /* this lane's row j as a B lane: where its block starts inside its image row */
+    const int blk_at = j * kQ6KImageRow + ((j * row_bytes + wv * kQ6KBlock) & 15);
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int t0 = 0; t0 < cnt; t0 += 8) {
+        const int n_live = cnt - t0 < 8 ? cnt - t0 : 8;
+        /* A lane (i, kg): token i & 7 in the k groups of scale group i >> 3 */
+        const int tok = j & 7;
+        const bool live = (kg >> 1) == (j >> 3) && tok < n_live;
+        const size_t at_a = (size_t)(first + t0 + (tok < n_live ? tok : 0)) * n_ff + (size_t)wv * 256 + 8 * kg;
+        u32x4 a_hi[8], a_lo[8]; /* [run u]: elements 32 u + 8 kg .. + 7 of the wave's super-block */
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous pass's images have returned */
+        request(0, 0);
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            u32x4 vh = {0u, 0u, 0u, 0u}, vl = {0u, 0u, 0u, 0u};
+            if (live) {
+                vh = *(const u32x4 *)(h_hi + at_a + 32 * u);
+                vl = *(const u32x4 *)(h_lo + at_a + 32 * u);
+            }
+            a_hi[u] = vh;
+            a_lo[u] = vl;
+        }
+#pragma unroll 1
+        for (int rt = 0; rt < NT; rt++) {
+            if (rt + 1 < NT) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the other image has been read */
+                request(rt + 1, (rt + 1) & 1);
+                wait_vm_at_most(kImageLoads);
+            } else {
+                wait_vm_at_most(0);
+            }
+            const uint8_t *im = img + (rt & 1) * kImage;
+            uint32_t scw[5];
+            lds_dwords_at<5>(im, blk_at + 192, scw); /* 16 int8 scales, then d */
+            const float d = half_bits_fast(scw[4] & 0xFFFFu);
+            f32x4 acc = zero;
+#pragma unroll
+            for (int n = 0; n < 2; n++) {
+                uint32_t qa[2], qb[2], qh[2]; /* ql[64n + 8kg ..], ql[64n + 32 + 8kg ..], qh[32n + 8kg ..] */
+                lds_dwords_at<2>(im, blk_at + 64 * n + 8 * kg, qa);
+                lds_dwords_at<2>(im, blk_at + 64 * n + 32 + 8 * kg, qb);
+                lds_dwords_at<2>(im, blk_at + 128 + 32 * n + 8 * kg, qh);
+#pragma unroll
+                for (int qd = 0; qd < 4; qd++) {
+                    const int u = 4 * n + qd;
+                    const uint32_t l0 = ((qd & 1) ? qb[0] : qa[0]) >> (4 * (qd >> 1)), l1 = ((qd & 1) ? qb[1] : qa[1]) >> (4 * (qd >> 1));
+                    const bf16x8 lo = codes_to_bf16(l0 & 0x0F0F0F0Fu, l1 & 0x0F0F0F0Fu);
+                    const bf16x8 hi = codes_to_bf16((qh[0] >> (2 * qd)) & 0x03030303u, (qh[1] >> (2 * qd)) & 0x03030303u);
+                    const bf16x8 ah = __builtin_bit_cast(bf16x8, a_hi[u]), al = __builtin_bit_cast(bf16x8, a_lo[u]);
+                    f32x4 S_lo = mma(ah, lo, zero), S_hi = mma(ah, hi, zero), X = mma(ah, ones_bf16(), zero);
+                    S_lo = mma(al, lo, S_lo);
+                    S_hi = mma(al, hi, S_hi);
+                    X = mma(al, ones_bf16(), X);
+                    /* this lane's scale group of the run: byte 8n + 2qd + (kg >> 1) of the 16 scales */
+                    const int sidx = 8 * n + 2 * qd; /* + (kg >> 1) */
+                    const uint32_t w = scw[sidx >> 2] >> (8 * (sidx & 3)); /* bytes sidx, sidx + 1 at bits 0..15 */
+                    const int sc = (int)(int8_t)((kg >> 1) ? (w >> 8) : w);
+                    const float dsc = d * (float)sc;
+#pragma unroll
+                    for (int v = 0; v < 4; v++) acc[v] = fmaf(dsc, fmaf(16.0f, S_hi[v], S_lo[v]) - 32.0f * X[v], acc[v]);
+                }
+            }
+            /* the two scale groups of every run sit in lanes kg and kg ^ 2 */
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[v] += __shfl_xor(acc[v], 32, 64);
+            if (kg < 2) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) red[(wv * 8 + 4 * kg + v) * 16 + j] = acc[v];
+            }
+            __syncthreads();
+            for (int idx = threadIdx.x; idx < n_live * 16; idx += blockDim.x) {
+                const int jj = idx & 15, t = idx >> 4;
+                float dsum = 0.0f;
+                for (int w = 0; w < n_waves; w++) dsum += red[(w * 8 + t) * 16 + jj];
+                part[(size_t)(first + t0 + t) * n_embd + row0 + rt * 16 + jj] = dsum;
+            }
+            __syncthreads();
+        }
+    }
+}
+
 /* ---- 4. out[t] = sum over k, in k order ---- */
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of,
@@ -1002,6 +1154,12 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         }
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock), stream,
+                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
+    } else if (type_down == T_Q6_K && n_ff % 256 == 0 && n_ff / 256 <= 8 && n_embd % (16 * kQ6KWalkGroups) == 0 &&
+               ((uintptr_t)down & 15) == 0) {
+        const int waves = n_ff / 256;
+        hipLaunchKernelGGL(moe_down_q6k_walk_kernel<kQ6KWalkGroups>, dim3(n_embd / (16 * kQ6KWalkGroups), n_expert),
+                           dim3(64 * waves), (size_t)waves * (128 * 4 + 2 * (16 * kQ6KImageRow + 16)), stream,
                            (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
     } else if (fast_dn) {
         constexpr int DRT = MOE_DN_RT;

@@ -214,10 +214,14 @@ def test_grouped_ffn_every_block_format(oracle, type_id):
     ((Q4K, Q4K, Q4K), 256, 2304),      # 9 super-blocks of K for down: more than its 8 waves, one row group per workgroup
     ((Q8_0, Q8_0, Q4K), 160, 256),     # 160 rows of down: not a whole number of the four-group walks
     ((Q4K, Q4K, Q4K), 1024, 512),      # the walk: 8 groups of 4 x 32 rows, two super-blocks of K
-], ids=["long_k", "rows_not_multiple_of_128", "walk"])
+    ((Q4K, Q4K, Q6K), 256, 768),       # Q6_K down on the matrix cores: 630-byte rows, three waves, blocks at every even offset
+    ((Q4K, Q4K, Q6K), 1024, 512),      # 420-byte rows, two waves, eight walks per expert
+    ((Q8_0, Q8_0, Q6K), 160, 256),     # rows not a multiple of 128: the any-format kernel
+], ids=["long_k", "rows_not_multiple_of_128", "walk", "q6k_down_3_waves", "q6k_down_2_waves", "q6k_down_fallback"])
 def test_grouped_ffn_down_kernel_variants(oracle, types, n_embd, n_ff):
     """the Q4_K down projection has two kernels: one row group of 32 per workgroup, and a walk over four
-    groups with the next weight image in flight (K up to 2048, rows a multiple of 128)"""
+    groups with the next weight image in flight (K up to 2048, rows a multiple of 128); Q6_K down has a walk of
+    its own (eight tokens per pass: 21 tokens over 3 experts give it several) and the any-format kernel"""
     n_expert, k, n_tok = 3, 2, 21
     gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=950, types=types)
     Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=951, tokens=n_tok))
