@@ -732,6 +732,46 @@ __device__ __forceinline__ void lds_dwords_at(const uint8_t *base, int off, uint
     }
 }
 
+/* One Q6_K block of this lane's weight row (at byte blk_at of the image im) against NA activation operands
+ * (a[p][u]: elements 32 u + 8 kg .. + 7 of the block, block-diagonal as described above): adds, for the
+ * lane's scale groups kg >> 1 of the eight runs, d * sc * (S_lo + 16 S_hi - 32 X) to acc[v], token 4 (kg & 1) + v */
+template <int NA>
+__device__ __forceinline__ void q6k_block_math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t scw[5];
+    lds_dwords_at<5>(im, blk_at + 192, scw); /* 16 int8 scales, then d */
+    const float d = half_bits_fast(scw[4] & 0xFFFFu);
+#pragma unroll
+    for (int n = 0; n < 2; n++) {
+        uint32_t qa[2], qb[2], qh[2]; /* ql[64n + 8kg ..], ql[64n + 32 + 8kg ..], qh[32n + 8kg ..] */
+        lds_dwords_at<2>(im, blk_at + 64 * n + 8 * kg, qa);
+        lds_dwords_at<2>(im, blk_at + 64 * n + 32 + 8 * kg, qb);
+        lds_dwords_at<2>(im, blk_at + 128 + 32 * n + 8 * kg, qh);
+#pragma unroll
+        for (int qd = 0; qd < 4; qd++) {
+            const int u = 4 * n + qd;
+            const uint32_t l0 = ((qd & 1) ? qb[0] : qa[0]) >> (4 * (qd >> 1)), l1 = ((qd & 1) ? qb[1] : qa[1]) >> (4 * (qd >> 1));
+            const bf16x8 lo = codes_to_bf16(l0 & 0x0F0F0F0Fu, l1 & 0x0F0F0F0Fu);
+            const bf16x8 hi = codes_to_bf16((qh[0] >> (2 * qd)) & 0x03030303u, (qh[1] >> (2 * qd)) & 0x03030303u);
+            f32x4 S_lo = zero, S_hi = zero, X = zero;
+#pragma unroll
+            for (int p = 0; p < NA; p++) {
+                const bf16x8 av = __builtin_bit_cast(bf16x8, a[p][u]);
+                S_lo = mma(av, lo, S_lo);
+                S_hi = mma(av, hi, S_hi);
+                X = mma(av, ones_bf16(), X);
+            }
+            /* this lane's scale group of the run: byte 8n + 2qd + (kg >> 1) of the 16 scales */
+            const int sidx = 8 * n + 2 * qd;
+            const uint32_t w = scw[sidx >> 2] >> (8 * (sidx & 3)); /* bytes sidx, sidx + 1 at bits 0..15 */
+            const int sc = (int)(int8_t)((kg >> 1) ? (w >> 8) : w);
+            const float dsc = d * (float)sc;
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[v] = fmaf(dsc, fmaf(16.0f, S_hi[v], S_lo[v]) - 32.0f * X[v], acc[v]);
+        }
+    }
+}
+
 template <int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3)))
 moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
@@ -805,36 +845,9 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
                 wait_vm_at_most(0);
             }
             const uint8_t *im = img + (rt & 1) * kImage;
-            uint32_t scw[5];
-            lds_dwords_at<5>(im, blk_at + 192, scw); /* 16 int8 scales, then d */
-            const float d = half_bits_fast(scw[4] & 0xFFFFu);
             f32x4 acc = zero;
-#pragma unroll
-            for (int n = 0; n < 2; n++) {
-                uint32_t qa[2], qb[2], qh[2]; /* ql[64n + 8kg ..], ql[64n + 32 + 8kg ..], qh[32n + 8kg ..] */
-                lds_dwords_at<2>(im, blk_at + 64 * n + 8 * kg, qa);
-                lds_dwords_at<2>(im, blk_at + 64 * n + 32 + 8 * kg, qb);
-                lds_dwords_at<2>(im, blk_at + 128 + 32 * n + 8 * kg, qh);
-#pragma unroll
-                for (int qd = 0; qd < 4; qd++) {
-                    const int u = 4 * n + qd;
-                    const uint32_t l0 = ((qd & 1) ? qb[0] : qa[0]) >> (4 * (qd >> 1)), l1 = ((qd & 1) ? qb[1] : qa[1]) >> (4 * (qd >> 1));
-                    const bf16x8 lo = codes_to_bf16(l0 & 0x0F0F0F0Fu, l1 & 0x0F0F0F0Fu);
-                    const bf16x8 hi = codes_to_bf16((qh[0] >> (2 * qd)) & 0x03030303u, (qh[1] >> (2 * qd)) & 0x03030303u);
-                    const bf16x8 ah = __builtin_bit_cast(bf16x8, a_hi[u]), al = __builtin_bit_cast(bf16x8, a_lo[u]);
-                    f32x4 S_lo = mma(ah, lo, zero), S_hi = mma(ah, hi, zero), X = mma(ah, ones_bf16(), zero);
-                    S_lo = mma(al, lo, S_lo);
-                    S_hi = mma(al, hi, S_hi);
-                    X = mma(al, ones_bf16(), X);
-                    /* this lane's scale group of the run: byte 8n + 2qd + (kg >> 1) of the 16 scales */
-                    const int sidx = 8 * n + 2 * qd; /* + (kg >> 1) */
-                    const uint32_t w = scw[sidx >> 2] >> (8 * (sidx & 3)); /* bytes sidx, sidx + 1 at bits 0..15 */
-                    const int sc = (int)(int8_t)((kg >> 1) ? (w >> 8) : w);
-                    const float dsc = d * (float)sc;
-#pragma unroll
-                    for (int v = 0; v < 4; v++) acc[v] = fmaf(dsc, fmaf(16.0f, S_hi[v], S_lo[v]) - 32.0f * X[v], acc[v]);
-                }
-            }
+            const u32x4 *const aa[2] = {a_hi, a_lo};
+            q6k_block_math<2>(im, blk_at, kg, aa, acc);
             /* the two scale groups of every run sit in lanes kg and kg ^ 2 */
 #pragma unroll
             for (int v = 0; v < 4; v++) acc[v] += __shfl_xor(acc[v], 32, 64);
@@ -851,6 +864,99 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
             }
             __syncthreads();
         }
+    }
+}
+
+/* ---- 2c. gate and up for Q6_K experts: 16 rows of each per workgroup, K split over at most four waves (a wave
+ * takes super-blocks wv, wv + 4, ...), eight tokens per pass, the arithmetic of the Q6_K down kernel ---- */
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4)))
+moe_gate_up_q6k_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
+                       const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
+                       const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
+                       int n_embd, int n_ff, int top_k) {
+    constexpr int kImage = 16 * kQ6KImageRow + 16;
+    constexpr int kChunks = 16 * 14, kImageLoads = (kChunks + 63) / 64;
+    extern __shared__ __attribute__((aligned(16))) float red[];
+    const int e = blockIdx.y;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * 16;
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int j = lane & 15, kg = lane >> 4;
+    const int n_sb = n_embd >> 8;
+    const int row_bytes = n_sb * kQ6KBlock;
+    const size_t ebase = ((size_t)e * n_ff + row0) * row_bytes; /* a multiple of 16: row0 is */
+    /* LDS: red [waves][gate, up][8 tokens][16 rows] floats | images [waves][gate, up][16 rows][224 bytes + slack] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 256) + wv * (2 * kImage);
+    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int t0 = 0; t0 < cnt; t0 += 8) {
+        const int n_live = cnt - t0 < 8 ? cnt - t0 : 8;
+        const int tslot = j & 7;
+        const bool live = (kg >> 1) == (j >> 3) && tslot < n_live;
+        const int tok = order[first + t0 + (tslot < n_live ? tslot : 0)] / top_k;
+        const uint16_t *xrow = X + (size_t)tok * n_embd + 8 * kg;
+        f32x4 acc_g = zero, acc_u = zero;
+        for (int sb = wv; sb < n_sb; sb += n_waves) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous images have returned */
+            const uint8_t *gb = uniform_ptr(gate + ebase), *ub = uniform_ptr(up + ebase);
+#pragma unroll
+            for (int i = 0; i < kImageLoads; i++) {
+                const int t = 64 * i + lane;
+                int R = t / 14;
+                const int c = t - 14 * R;
+                R = R < 16 ? R : 15;
+                const uint32_t off = (uint32_t)((R * row_bytes + sb * kQ6KBlock) & ~15) + 16u * (uint32_t)c;
+                const uint32_t m0g = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
+                const uint32_t m0u = __builtin_amdgcn_readfirstlane(img_lds + (uint32_t)kImage + 1024u * (uint32_t)i);
+                if (t < kChunks) {
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(gb), "s"(m0g) : "memory");
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(ub), "s"(m0u) : "memory");
+                }
+            }
+            u32x4 a[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if (live) v = *(const u32x4 *)(xrow + sb * 256 + 32 * u);
+                a[u] = v;
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* images and activations have landed */
+            const int blk_at = j * kQ6KImageRow + ((j * row_bytes + sb * kQ6KBlock) & 15);
+            const u32x4 *const aa[1] = {a};
+            q6k_block_math<1>(img, blk_at, kg, aa, acc_g);
+            q6k_block_math<1>(img + kImage, blk_at, kg, aa, acc_u);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            acc_g[v] += __shfl_xor(acc_g[v], 32, 64);
+            acc_u[v] += __shfl_xor(acc_u[v], 32, 64);
+        }
+        if (kg < 2) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                red[(wv * 2 + 0) * 128 + (4 * kg + v) * 16 + j] = acc_g[v];
+                red[(wv * 2 + 1) * 128 + (4 * kg + v) * 16 + j] = acc_u[v];
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < n_live * 16; idx += blockDim.x) {
+            const int jj = idx & 15, t = idx >> 4;
+            float g = 0.0f, u = 0.0f;
+            for (int w = 0; w < n_waves; w++) {
+                g += red[(w * 2 + 0) * 128 + t * 16 + jj];
+                u += red[(w * 2 + 1) * 128 + t * 16 + jj];
+            }
+            const float h = g / (1.0f + expf(-g)) * u; /* tf_silu_mul, common/transformer.h:4679-4694 */
+            const __bf16 hh = (__bf16)h;
+            const __bf16 hl = (__bf16)(h - (float)hh);
+            const size_t at = (size_t)(first + t0 + t) * n_ff + row0 + jj;
+            h_hi[at] = __builtin_bit_cast(uint16_t, hh);
+            h_lo[at] = __builtin_bit_cast(uint16_t, hl);
+        }
+        __syncthreads();
     }
 }
 
@@ -1134,6 +1240,12 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                            (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock + 256), stream,
                            (const uint8_t *)gate, (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd,
                            n_ff, top_k);
+    } else if (type_gate == T_Q6_K && type_up == T_Q6_K && n_embd % 256 == 0 && n_ff % 16 == 0 &&
+               (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
+        const int waves = n_embd / 256 < 4 ? n_embd / 256 : 4;
+        hipLaunchKernelGGL(moe_gate_up_q6k_kernel, dim3(n_ff / 16, n_expert), dim3(64 * waves),
+                           (size_t)waves * (256 * 4 + 2 * (16 * kQ6KImageRow + 16)), stream, (const uint8_t *)gate,
+                           (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
     } else {
         hipError_t e1 = launch_rows_any<1>(type_gate, gate, n_ff, n_embd, n_expert, ws, top_k, X, nullptr, nullptr, ws.g32, stream);
         if (e1 != hipSuccess) return e1;
