@@ -702,7 +702,7 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
     }
 }
 
-/* ---- 3c. down for Q6_K experts (the down projections of K-quant mixes) ----
+/* ---- 3c. down for Q6_K and Q5_K experts (what K-quant mixes store beside or instead of Q4_K) ----
  * The same walk as moe_down_walk_kernel over NT groups of 16 rows, a wave per super-block of K, the next
  * group's image in flight while this one is multiplied. What differs:
  *   * A Q6_K block is 210 bytes, so rows and blocks start on 2-byte boundaries. A wave's image row is the 14
@@ -715,7 +715,7 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
  *     8 s + t holds token t's activations in the k groups of scale group s (2s, 2s + 1) and zeros in the
  *     others; C[8 s + t][j] lands in lane (j, kg) with s = kg >> 1, t = 4 (kg & 1) + v. Eight tokens per pass.
  * The weights stay exact as in the Q4_K kernels; the intermediate arrives as bf16 head + tail. */
-constexpr int kQ6KBlock = 210, kQ6KImageRow = 224, kQ6KWalkGroups = 8;
+constexpr int kQ6KBlock = 210, kKqWalkGroups = 8;
 
 /* n dwords from byte offset off (even) of an LDS area whose base is 16-byte aligned: aligned dword reads,
  * funnel-shifted by the two odd bytes if any */
@@ -772,13 +772,60 @@ __device__ __forceinline__ void q6k_block_math(const uint8_t *im, int blk_at, in
     }
 }
 
-template <int NT>
+/* The same for a Q5_K block (176 bytes, 16-byte aligned): code = nibble + 16 * high bit, one 6-bit scale and min
+ * per 32 elements (common/ggml_dequant.h:1620-1651): (d sc) (S_lo + 16 S_hi) - (dmin m) X. Both scale groups
+ * of a run share the sub-block's scale, so the block-diagonal operand only costs its eight-token passes. */
+template <int NA>
+__device__ __forceinline__ void q5k_block_math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const Scales sc = unpack_header(*(const u32x4 *)(im + blk_at));
+    const u32x2 qh = *(const u32x2 *)(im + blk_at + 16 + 8 * kg); /* bit s of byte l: high bit of element l of sub-block s */
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const u32x2 qs = *(const u32x2 *)(im + blk_at + 48 + 32 * c + 8 * kg); /* sub-blocks 2c (low nibbles), 2c + 1 */
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int u = 2 * c + h;
+            const bf16x8 lo = codes_to_bf16((qs.x >> (4 * h)) & 0x0F0F0F0Fu, (qs.y >> (4 * h)) & 0x0F0F0F0Fu);
+            const bf16x8 hi = codes_to_bf16((qh.x >> u) & 0x01010101u, (qh.y >> u) & 0x01010101u);
+            f32x4 S_lo = zero, S_hi = zero, X = zero;
+#pragma unroll
+            for (int p = 0; p < NA; p++) {
+                const bf16x8 av = __builtin_bit_cast(bf16x8, a[p][u]);
+                S_lo = mma(av, lo, S_lo);
+                S_hi = mma(av, hi, S_hi);
+                X = mma(av, ones_bf16(), X);
+            }
+            const uint32_t scw = (u < 4 ? sc.sc_lo : sc.sc_hi) >> (8 * (u & 3)), mnw = (u < 4 ? sc.mn_lo : sc.mn_hi) >> (8 * (u & 3));
+            const float dsc = sc.d * (float)(scw & 0xFFu), dm = sc.dmin * (float)(mnw & 0xFFu);
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[v] = fmaf(dsc, fmaf(16.0f, S_hi[v], S_lo[v]), fmaf(-dm, X[v], acc[v]));
+        }
+    }
+}
+
+/* what the two kernels below need to know about a format */
+struct KqQ6K {
+    static constexpr int kBlock = kQ6KBlock, kRowChunks = 14;
+    template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+        q6k_block_math<NA>(im, blk_at, kg, a, acc);
+    }
+};
+struct KqQ5K {
+    static constexpr int kBlock = 176, kRowChunks = 11;
+    template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+        q5k_block_math<NA>(im, blk_at, kg, a, acc);
+    }
+};
+
+template <typename F, int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3)))
-moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
+moe_down_kq_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                          const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
                          float *__restrict__ part, int n_embd, int n_ff) {
-    constexpr int kImage = 16 * kQ6KImageRow + 16; /* + slack for the funnel-shift read past the last row */
-    constexpr int kChunks = 16 * 14, kImageLoads = (kChunks + 63) / 64;
+    constexpr int kImageRow = 16 * F::kRowChunks;
+    constexpr int kImage = 16 * kImageRow + 16; /* + slack for the funnel-shift read past the last row */
+    constexpr int kChunks = 16 * F::kRowChunks, kImageLoads = (kChunks + 63) / 64;
     extern __shared__ __attribute__((aligned(16))) float red[];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63;
@@ -788,7 +835,7 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
     if (cnt == 0) return;
     const int j = lane & 15, kg = lane >> 4;
     const int n_sb = n_ff >> 8; /* == n_waves: wave wv owns super-block wv */
-    const int row_bytes = n_sb * kQ6KBlock;
+    const int row_bytes = n_sb * F::kBlock;
     /* 16 * row_bytes is a multiple of 16, so every row group starts on a 16-byte boundary like the tensor */
     const uint8_t *d0 = down + ((size_t)e * n_embd + row0) * row_bytes;
     /* LDS: red [waves][8 tokens][16 rows] floats | images [waves][2][16 rows][224 bytes + slack] */
@@ -798,10 +845,10 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
 #pragma unroll
     for (int i = 0; i < kImageLoads; i++) {
         const int t = 64 * i + lane;
-        int R = t / 14;
-        const int c = t - 14 * R;
+        int R = t / F::kRowChunks;
+        const int c = t - F::kRowChunks * R;
         R = R < 16 ? R : 15;
-        off[i] = (uint32_t)((R * row_bytes + wv * kQ6KBlock) & ~15) + 16u * (uint32_t)c;
+        off[i] = (uint32_t)((R * row_bytes + wv * F::kBlock) & ~15) + 16u * (uint32_t)c;
     }
     auto request = [&](int rt, int buf) {
         const uint8_t *base = uniform_ptr(d0 + (size_t)rt * 16 * row_bytes);
@@ -813,7 +860,7 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
         }
     };
     /* this lane's row j as a B lane: where its block starts inside its image row */
-    const int blk_at = j * kQ6KImageRow + ((j * row_bytes + wv * kQ6KBlock) & 15);
+    const int blk_at = j * kImageRow + ((j * row_bytes + wv * F::kBlock) & 15);
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
 
     for (int t0 = 0; t0 < cnt; t0 += 8) {
@@ -847,7 +894,7 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
             const uint8_t *im = img + (rt & 1) * kImage;
             f32x4 acc = zero;
             const u32x4 *const aa[2] = {a_hi, a_lo};
-            q6k_block_math<2>(im, blk_at, kg, aa, acc);
+            F::template math<2>(im, blk_at, kg, aa, acc);
             /* the two scale groups of every run sit in lanes kg and kg ^ 2 */
 #pragma unroll
             for (int v = 0; v < 4; v++) acc[v] += __shfl_xor(acc[v], 32, 64);
@@ -869,13 +916,15 @@ moe_down_q6k_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__res
 
 /* ---- 2c. gate and up for Q6_K experts: 16 rows of each per workgroup, K split over at most four waves (a wave
  * takes super-blocks wv, wv + 4, ...), eight tokens per pass, the arithmetic of the Q6_K down kernel ---- */
+template <typename F>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4)))
-moe_gate_up_q6k_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
+moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
                        const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
                        const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
                        int n_embd, int n_ff, int top_k) {
-    constexpr int kImage = 16 * kQ6KImageRow + 16;
-    constexpr int kChunks = 16 * 14, kImageLoads = (kChunks + 63) / 64;
+    constexpr int kImageRow = 16 * F::kRowChunks;
+    constexpr int kImage = 16 * kImageRow + 16;
+    constexpr int kChunks = 16 * F::kRowChunks, kImageLoads = (kChunks + 63) / 64;
     extern __shared__ __attribute__((aligned(16))) float red[];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63;
@@ -885,7 +934,7 @@ moe_gate_up_q6k_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restri
     if (cnt == 0) return;
     const int j = lane & 15, kg = lane >> 4;
     const int n_sb = n_embd >> 8;
-    const int row_bytes = n_sb * kQ6KBlock;
+    const int row_bytes = n_sb * F::kBlock;
     const size_t ebase = ((size_t)e * n_ff + row0) * row_bytes; /* a multiple of 16: row0 is */
     /* LDS: red [waves][gate, up][8 tokens][16 rows] floats | images [waves][gate, up][16 rows][224 bytes + slack] */
     uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 256) + wv * (2 * kImage);
@@ -905,10 +954,10 @@ moe_gate_up_q6k_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restri
 #pragma unroll
             for (int i = 0; i < kImageLoads; i++) {
                 const int t = 64 * i + lane;
-                int R = t / 14;
-                const int c = t - 14 * R;
+                int R = t / F::kRowChunks;
+                const int c = t - F::kRowChunks * R;
                 R = R < 16 ? R : 15;
-                const uint32_t off = (uint32_t)((R * row_bytes + sb * kQ6KBlock) & ~15) + 16u * (uint32_t)c;
+                const uint32_t off = (uint32_t)((R * row_bytes + sb * F::kBlock) & ~15) + 16u * (uint32_t)c;
                 const uint32_t m0g = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
                 const uint32_t m0u = __builtin_amdgcn_readfirstlane(img_lds + (uint32_t)kImage + 1024u * (uint32_t)i);
                 if (t < kChunks) {
@@ -924,10 +973,10 @@ moe_gate_up_q6k_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restri
                 a[u] = v;
             }
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* images and activations have landed */
-            const int blk_at = j * kQ6KImageRow + ((j * row_bytes + sb * kQ6KBlock) & 15);
+            const int blk_at = j * kImageRow + ((j * row_bytes + sb * F::kBlock) & 15);
             const u32x4 *const aa[1] = {a};
-            q6k_block_math<1>(img, blk_at, kg, aa, acc_g);
-            q6k_block_math<1>(img + kImage, blk_at, kg, aa, acc_u);
+            F::template math<1>(img, blk_at, kg, aa, acc_g);
+            F::template math<1>(img + kImage, blk_at, kg, aa, acc_u);
         }
 #pragma unroll
         for (int v = 0; v < 4; v++) {
@@ -1240,12 +1289,17 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                            (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock + 256), stream,
                            (const uint8_t *)gate, (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd,
                            n_ff, top_k);
-    } else if (type_gate == T_Q6_K && type_up == T_Q6_K && n_embd % 256 == 0 && n_ff % 16 == 0 &&
+    } else if (type_gate == type_up && (type_gate == T_Q6_K || type_gate == T_Q5_K) && n_embd % 256 == 0 && n_ff % 16 == 0 &&
                (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
         const int waves = n_embd / 256 < 4 ? n_embd / 256 : 4;
-        hipLaunchKernelGGL(moe_gate_up_q6k_kernel, dim3(n_ff / 16, n_expert), dim3(64 * waves),
-                           (size_t)waves * (256 * 4 + 2 * (16 * kQ6KImageRow + 16)), stream, (const uint8_t *)gate,
-                           (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
+        if (type_gate == T_Q6_K)
+            hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ6K>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
+                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ6K::kRowChunks + 16)), stream, (const uint8_t *)gate,
+                               (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
+        else
+            hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ5K>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
+                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ5K::kRowChunks + 16)), stream, (const uint8_t *)gate,
+                               (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
     } else {
         hipError_t e1 = launch_rows_any<1>(type_gate, gate, n_ff, n_embd, n_expert, ws, top_k, X, nullptr, nullptr, ws.g32, stream);
         if (e1 != hipSuccess) return e1;
@@ -1267,12 +1321,18 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock), stream,
                            (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
-    } else if (type_down == T_Q6_K && n_ff % 256 == 0 && n_ff / 256 <= 8 && n_embd % (16 * kQ6KWalkGroups) == 0 &&
-               ((uintptr_t)down & 15) == 0) {
+    } else if ((type_down == T_Q6_K || type_down == T_Q5_K) && n_ff % 256 == 0 && n_ff / 256 <= 8 &&
+               n_embd % (16 * kKqWalkGroups) == 0 && ((uintptr_t)down & 15) == 0) {
         const int waves = n_ff / 256;
-        hipLaunchKernelGGL(moe_down_q6k_walk_kernel<kQ6KWalkGroups>, dim3(n_embd / (16 * kQ6KWalkGroups), n_expert),
-                           dim3(64 * waves), (size_t)waves * (128 * 4 + 2 * (16 * kQ6KImageRow + 16)), stream,
-                           (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
+        const dim3 grid(n_embd / (16 * kKqWalkGroups), n_expert);
+        if (type_down == T_Q6_K)
+            hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ6K, kKqWalkGroups>), grid, dim3(64 * waves),
+                               (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ6K::kRowChunks + 16)), stream,
+                               (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
+        else
+            hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ5K, kKqWalkGroups>), grid, dim3(64 * waves),
+                               (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ5K::kRowChunks + 16)), stream,
+                               (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
     } else if (fast_dn) {
         constexpr int DRT = MOE_DN_RT;
         hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),
