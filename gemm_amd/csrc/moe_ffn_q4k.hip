@@ -804,11 +804,43 @@ __device__ __forceinline__ void q5k_block_math(const uint8_t *im, int blk_at, in
     }
 }
 
+/* The same for eight Q8_0 blocks (256 elements, 8 x 34 = 272 bytes: a 16-byte multiple, but the codes of a
+ * block start 2 bytes in): an int8 code is low nibble + 16 * (high nibble ^ 8) - 128 (the high nibble read as
+ * signed, shifted to 0..15), one fp16 scale per 32 elements (common/ggml_dequant.h:1479-1489). */
+template <int NA>
+__device__ __forceinline__ void q8_0_block_math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        uint32_t q[2];
+        lds_dwords_at<2>(im, blk_at + 34 * u + 2 + 8 * kg, q);
+        const float d = half_bits_fast(*reinterpret_cast<const uint16_t *>(im + blk_at + 34 * u));
+        const bf16x8 lo = codes_to_bf16(q[0] & 0x0F0F0F0Fu, q[1] & 0x0F0F0F0Fu);
+        const bf16x8 hi = codes_to_bf16(((q[0] >> 4) & 0x0F0F0F0Fu) ^ 0x08080808u, ((q[1] >> 4) & 0x0F0F0F0Fu) ^ 0x08080808u);
+        f32x4 S_lo = zero, S_hi = zero, X = zero;
+#pragma unroll
+        for (int p = 0; p < NA; p++) {
+            const bf16x8 av = __builtin_bit_cast(bf16x8, a[p][u]);
+            S_lo = mma(av, lo, S_lo);
+            S_hi = mma(av, hi, S_hi);
+            X = mma(av, ones_bf16(), X);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[v] = fmaf(d, fmaf(16.0f, S_hi[v], S_lo[v]) - 128.0f * X[v], acc[v]);
+    }
+}
+
 /* what the two kernels below need to know about a format */
 struct KqQ6K {
     static constexpr int kBlock = kQ6KBlock, kRowChunks = 14;
     template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
         q6k_block_math<NA>(im, blk_at, kg, a, acc);
+    }
+};
+struct KqQ8_0 {
+    static constexpr int kBlock = 272, kRowChunks = 17;
+    template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+        q8_0_block_math<NA>(im, blk_at, kg, a, acc);
     }
 };
 struct KqQ5K {
@@ -1289,10 +1321,14 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                            (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock + 256), stream,
                            (const uint8_t *)gate, (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd,
                            n_ff, top_k);
-    } else if (type_gate == type_up && (type_gate == T_Q6_K || type_gate == T_Q5_K) && n_embd % 256 == 0 && n_ff % 16 == 0 &&
-               (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
+    } else if (type_gate == type_up && (type_gate == T_Q6_K || type_gate == T_Q5_K || type_gate == T_Q8_0) &&
+               n_embd % 256 == 0 && n_ff % 16 == 0 && (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
         const int waves = n_embd / 256 < 4 ? n_embd / 256 : 4;
-        if (type_gate == T_Q6_K)
+        if (type_gate == T_Q8_0)
+            hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ8_0>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
+                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ8_0::kRowChunks + 16)), stream, (const uint8_t *)gate,
+                               (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
+        else if (type_gate == T_Q6_K)
             hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ6K>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
                                (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ6K::kRowChunks + 16)), stream, (const uint8_t *)gate,
                                (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
@@ -1321,11 +1357,15 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock), stream,
                            (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
-    } else if ((type_down == T_Q6_K || type_down == T_Q5_K) && n_ff % 256 == 0 && n_ff / 256 <= 8 &&
+    } else if ((type_down == T_Q6_K || type_down == T_Q5_K || type_down == T_Q8_0) && n_ff % 256 == 0 && n_ff / 256 <= 8 &&
                n_embd % (16 * kKqWalkGroups) == 0 && ((uintptr_t)down & 15) == 0) {
         const int waves = n_ff / 256;
         const dim3 grid(n_embd / (16 * kKqWalkGroups), n_expert);
-        if (type_down == T_Q6_K)
+        if (type_down == T_Q8_0)
+            hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ8_0, kKqWalkGroups>), grid, dim3(64 * waves),
+                               (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ8_0::kRowChunks + 16)), stream,
+                               (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
+        else if (type_down == T_Q6_K)
             hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ6K, kKqWalkGroups>), grid, dim3(64 * waves),
                                (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ6K::kRowChunks + 16)), stream,
                                (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
