@@ -716,6 +716,7 @@ moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restric
  *     others; C[8 s + t][j] lands in lane (j, kg) with s = kg >> 1, t = 4 (kg & 1) + v. Eight tokens per pass.
  * The weights stay exact as in the Q4_K kernels; the intermediate arrives as bf16 head + tail. */
 constexpr int kQ6KBlock = 210, kKqWalkGroups = 8;
+constexpr uint32_t kNoChunk = 0xFFFFFFFFu;
 
 /* n dwords from byte offset off (even) of an LDS area whose base is 16-byte aligned: aligned dword reads,
  * funnel-shifted by the two odd bytes if any */
@@ -830,11 +831,100 @@ __device__ __forceinline__ void q8_0_block_math(const uint8_t *im, int blk_at, i
     }
 }
 
+/* byte `i` (lane-variable, 0..11) of three dwords */
+__device__ __forceinline__ uint32_t byte_of3(const uint32_t (&w)[3], int i) {
+    const uint32_t d = i < 4 ? w[0] : i < 8 ? w[1] : w[2];
+    return (d >> (8 * (i & 3))) & 255u;
+}
+
+/* Q2_K (84 bytes, 4-byte aligned): 2-bit codes, per 16 elements a 4-bit scale and a 4-bit min in one byte:
+ * (d sc) q - dmin m (common/ggml_dequant.h:1495-1534) */
+template <int NA>
+__device__ __forceinline__ void q2k_block_math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t scw[4], dd[1];
+    lds_dwords_at<4>(im, blk_at, scw);       /* 16 scale/min bytes */
+    lds_dwords_at<1>(im, blk_at + 80, dd);   /* d, dmin */
+    const float d = half_bits_fast(dd[0] & 0xFFFFu), dmin = half_bits_fast(dd[0] >> 16);
+#pragma unroll
+    for (int n = 0; n < 2; n++) {
+        uint32_t q[2]; /* qs[32 n + 8 kg ..]: two bits per run j of the half */
+        lds_dwords_at<2>(im, blk_at + 16 + 32 * n + 8 * kg, q);
+#pragma unroll
+        for (int jr = 0; jr < 4; jr++) {
+            const int u = 4 * n + jr;
+            const bf16x8 lo = codes_to_bf16((q[0] >> (2 * jr)) & 0x03030303u, (q[1] >> (2 * jr)) & 0x03030303u);
+            f32x4 S = zero, X = zero;
+#pragma unroll
+            for (int p = 0; p < NA; p++) {
+                const bf16x8 av = __builtin_bit_cast(bf16x8, a[p][u]);
+                S = mma(av, lo, S);
+                X = mma(av, ones_bf16(), X);
+            }
+            const int sidx = 8 * n + 2 * jr; /* + (kg >> 1): bytes sidx, sidx + 1 of the dword sidx / 4 */
+            const uint32_t w = scw[sidx >> 2] >> (8 * (sidx & 3));
+            const uint32_t sb = ((kg >> 1) ? (w >> 8) : w) & 255u;
+            const float dl = d * (float)(sb & 15u), ml = dmin * (float)(sb >> 4);
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[v] = fmaf(dl, S[v], fmaf(-ml, X[v], acc[v]));
+        }
+    }
+}
+
+/* Q3_K (110 bytes): q = 2 low bits + 4 * mask bit - 4, a 6-bit scale (minus 32) per 16 elements packed into
+ * 12 bytes (common/ggml_dequant.h:1536-1580): (d (sc - 32)) (S_lo + 4 S_hb - 4 X) */
+template <int NA>
+__device__ __forceinline__ void q3k_block_math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint32_t scw4[4], hm[2];
+    lds_dwords_at<4>(im, blk_at + 96, scw4); /* 12 scale bytes, d, two bytes beyond the block */
+    const uint32_t scw[3] = {scw4[0], scw4[1], scw4[2]};
+    const float d = half_bits_fast(scw4[3] & 0xFFFFu);
+    lds_dwords_at<2>(im, blk_at + 8 * kg, hm); /* bit u of byte l: mask bit of element l of run u */
+#pragma unroll
+    for (int n = 0; n < 2; n++) {
+        uint32_t q[2];
+        lds_dwords_at<2>(im, blk_at + 32 + 32 * n + 8 * kg, q);
+#pragma unroll
+        for (int jr = 0; jr < 4; jr++) {
+            const int u = 4 * n + jr;
+            const bf16x8 lo = codes_to_bf16((q[0] >> (2 * jr)) & 0x03030303u, (q[1] >> (2 * jr)) & 0x03030303u);
+            const bf16x8 hb = codes_to_bf16((hm[0] >> u) & 0x01010101u, (hm[1] >> u) & 0x01010101u);
+            f32x4 S_lo = zero, S_hb = zero, X = zero;
+#pragma unroll
+            for (int p = 0; p < NA; p++) {
+                const bf16x8 av = __builtin_bit_cast(bf16x8, a[p][u]);
+                S_lo = mma(av, lo, S_lo);
+                S_hb = mma(av, hb, S_hb);
+                X = mma(av, ones_bf16(), X);
+            }
+            const int is = 2 * u + (kg >> 1);
+            const uint32_t lo4 = (byte_of3(scw, is & 7) >> (4 * (is >> 3))) & 15u;
+            const uint32_t hi2 = (byte_of3(scw, 8 + (is & 3)) >> (2 * (is >> 2))) & 3u;
+            const float dl = d * (float)((int)(lo4 | (hi2 << 4)) - 32);
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[v] = fmaf(dl, fmaf(4.0f, S_hb[v], S_lo[v]) - 4.0f * X[v], acc[v]);
+        }
+    }
+}
+
 /* what the two kernels below need to know about a format */
 struct KqQ6K {
     static constexpr int kBlock = kQ6KBlock, kRowChunks = 14;
     template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
         q6k_block_math<NA>(im, blk_at, kg, a, acc);
+    }
+};
+struct KqQ2K {
+    static constexpr int kBlock = 84, kRowChunks = 6;
+    template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+        q2k_block_math<NA>(im, blk_at, kg, a, acc);
+    }
+};
+struct KqQ3K {
+    static constexpr int kBlock = 110, kRowChunks = 8;
+    template <int NA> __device__ static void math(const uint8_t *im, int blk_at, int kg, const u32x4 *const (&a)[NA], f32x4 &acc) {
+        q3k_block_math<NA>(im, blk_at, kg, a, acc);
     }
 };
 struct KqQ8_0 {
@@ -880,14 +970,16 @@ moe_down_kq_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__rest
         int R = t / F::kRowChunks;
         const int c = t - F::kRowChunks * R;
         R = R < 16 ? R : 15;
-        off[i] = (uint32_t)((R * row_bytes + wv * F::kBlock) & ~15) + 16u * (uint32_t)c;
+        const int at = R * row_bytes + wv * F::kBlock;
+        /* a chunk that lies wholly behind the block is not read: behind the tensor's last block there may be nothing */
+        off[i] = (t < kChunks && 16 * c < (at & 15) + F::kBlock) ? (uint32_t)(at & ~15) + 16u * (uint32_t)c : kNoChunk;
     }
     auto request = [&](int rt, int buf) {
         const uint8_t *base = uniform_ptr(d0 + (size_t)rt * 16 * row_bytes);
 #pragma unroll
         for (int i = 0; i < kImageLoads; i++) {
             const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + (uint32_t)(buf * kImage) + 1024u * (uint32_t)i);
-            if (64 * i + lane < kChunks)
+            if (off[i] != kNoChunk)
                 asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off[i]), "s"(base), "s"(m0v) : "memory");
         }
     };
@@ -989,10 +1081,12 @@ moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restric
                 int R = t / F::kRowChunks;
                 const int c = t - F::kRowChunks * R;
                 R = R < 16 ? R : 15;
-                const uint32_t off = (uint32_t)((R * row_bytes + sb * F::kBlock) & ~15) + 16u * (uint32_t)c;
+                const int at = R * row_bytes + sb * F::kBlock;
+                const uint32_t off = (uint32_t)(at & ~15) + 16u * (uint32_t)c;
+                const bool wanted = t < kChunks && 16 * c < (at & 15) + F::kBlock; /* not the chunk behind the block */
                 const uint32_t m0g = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
                 const uint32_t m0u = __builtin_amdgcn_readfirstlane(img_lds + (uint32_t)kImage + 1024u * (uint32_t)i);
-                if (t < kChunks) {
+                if (wanted) {
                     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(gb), "s"(m0g) : "memory");
                     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(ub), "s"(m0u) : "memory");
                 }
@@ -1288,6 +1382,9 @@ hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, in
     return hipGetLastError();
 }
 
+/* formats whose experts run on the matrix cores through moe_gate_up_kq_kernel / moe_down_kq_walk_kernel */
+static bool kq_type(uint32_t t) { return t == T_Q6_K || t == T_Q5_K || t == T_Q3_K || t == T_Q2_K || t == T_Q8_0; }
+
 size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
     return carve(nullptr, n_tok, top_k, n_embd, n_ff, n_expert).bytes;
 }
@@ -1321,21 +1418,22 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                            (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock + 256), stream,
                            (const uint8_t *)gate, (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd,
                            n_ff, top_k);
-    } else if (type_gate == type_up && (type_gate == T_Q6_K || type_gate == T_Q5_K || type_gate == T_Q8_0) &&
-               n_embd % 256 == 0 && n_ff % 16 == 0 && (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
+    } else if (type_gate == type_up && kq_type(type_gate) && n_embd % 256 == 0 && n_ff % 16 == 0 &&
+               (((uintptr_t)gate | (uintptr_t)up) & 15) == 0) {
         const int waves = n_embd / 256 < 4 ? n_embd / 256 : 4;
-        if (type_gate == T_Q8_0)
-            hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ8_0>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
-                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ8_0::kRowChunks + 16)), stream, (const uint8_t *)gate,
+        auto go = [&](auto tag) {
+            using F = decltype(tag);
+            hipLaunchKernelGGL(moe_gate_up_kq_kernel<F>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
+                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * F::kRowChunks + 16)), stream, (const uint8_t *)gate,
                                (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
-        else if (type_gate == T_Q6_K)
-            hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ6K>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
-                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ6K::kRowChunks + 16)), stream, (const uint8_t *)gate,
-                               (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
-        else
-            hipLaunchKernelGGL(moe_gate_up_kq_kernel<KqQ5K>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
-                               (size_t)waves * (256 * 4 + 2 * (16 * 16 * KqQ5K::kRowChunks + 16)), stream, (const uint8_t *)gate,
-                               (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
+        };
+        switch (type_gate) {
+        case T_Q6_K: go(KqQ6K()); break;
+        case T_Q5_K: go(KqQ5K()); break;
+        case T_Q3_K: go(KqQ3K()); break;
+        case T_Q2_K: go(KqQ2K()); break;
+        default: go(KqQ8_0()); break;
+        }
     } else {
         hipError_t e1 = launch_rows_any<1>(type_gate, gate, n_ff, n_embd, n_expert, ws, top_k, X, nullptr, nullptr, ws.g32, stream);
         if (e1 != hipSuccess) return e1;
@@ -1357,22 +1455,22 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), n_expert), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock), stream,
                            (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
-    } else if ((type_down == T_Q6_K || type_down == T_Q5_K || type_down == T_Q8_0) && n_ff % 256 == 0 && n_ff / 256 <= 8 &&
-               n_embd % (16 * kKqWalkGroups) == 0 && ((uintptr_t)down & 15) == 0) {
+    } else if (kq_type(type_down) && n_ff % 256 == 0 && n_ff / 256 <= 8 && n_embd % (16 * kKqWalkGroups) == 0 &&
+               ((uintptr_t)down & 15) == 0) {
         const int waves = n_ff / 256;
-        const dim3 grid(n_embd / (16 * kKqWalkGroups), n_expert);
-        if (type_down == T_Q8_0)
-            hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ8_0, kKqWalkGroups>), grid, dim3(64 * waves),
-                               (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ8_0::kRowChunks + 16)), stream,
+        auto go = [&](auto tag) {
+            using F = decltype(tag);
+            hipLaunchKernelGGL((moe_down_kq_walk_kernel<F, kKqWalkGroups>), dim3(n_embd / (16 * kKqWalkGroups), n_expert),
+                               dim3(64 * waves), (size_t)waves * (128 * 4 + 2 * (16 * 16 * F::kRowChunks + 16)), stream,
                                (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
-        else if (type_down == T_Q6_K)
-            hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ6K, kKqWalkGroups>), grid, dim3(64 * waves),
-                               (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ6K::kRowChunks + 16)), stream,
-                               (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
-        else
-            hipLaunchKernelGGL((moe_down_kq_walk_kernel<KqQ5K, kKqWalkGroups>), grid, dim3(64 * waves),
-                               (size_t)waves * (128 * 4 + 2 * (16 * 16 * KqQ5K::kRowChunks + 16)), stream,
-                               (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff);
+        };
+        switch (type_down) {
+        case T_Q6_K: go(KqQ6K()); break;
+        case T_Q5_K: go(KqQ5K()); break;
+        case T_Q3_K: go(KqQ3K()); break;
+        case T_Q2_K: go(KqQ2K()); break;
+        default: go(KqQ8_0()); break;
+        }
     } else if (fast_dn) {
         constexpr int DRT = MOE_DN_RT;
         hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), n_expert), dim3(64 * dn_waves),

@@ -222,8 +222,12 @@ def test_grouped_ffn_every_block_format(oracle, type_id):
     ((synth.GGML_Q5_K, synth.GGML_Q5_K, Q6K), 1024, 768),   # what the 5-bit K-quant mixes store
     ((synth.GGML_Q5_K, synth.GGML_Q5_K, synth.GGML_Q5_K), 2048, 512),
     ((Q8_0, Q8_0, Q8_0), 1024, 768),
+    ((synth.GGML_Q3_K, synth.GGML_Q3_K, Q4K), 1024, 512),   # the 3-bit mixes
+    ((synth.GGML_Q3_K, synth.GGML_Q3_K, synth.GGML_Q3_K), 768, 768),
+    ((synth.GGML_Q2_K, synth.GGML_Q2_K, synth.GGML_Q3_K), 1024, 512),
+    ((synth.GGML_Q2_K, synth.GGML_Q2_K, synth.GGML_Q2_K), 768, 768),
 ], ids=["long_k", "rows_not_multiple_of_128", "walk", "q6k_down_3_waves", "q6k_down_2_waves", "q6k_down_fallback",
-        "q6k_gate_up_4_waves", "q6k_gate_up_3_waves", "q5k_q5k_q6k", "q5k", "q8_0"])
+        "q6k_gate_up_4_waves", "q6k_gate_up_3_waves", "q5k_q5k_q6k", "q5k", "q8_0", "q3k_q3k_q4k", "q3k", "q2k_q2k_q3k", "q2k"])
 def test_grouped_ffn_down_kernel_variants(oracle, types, n_embd, n_ff):
     """the Q4_K down projection has two kernels: one row group of 32 per workgroup, and a walk over four
     groups with the next weight image in flight (K up to 2048, rows a multiple of 128); Q6_K down has a walk of
