@@ -645,7 +645,8 @@ def main():
         Q6K = synth.GGML_Q6_K
         Q5K = synth.GGML_Q5_K
         for label, tys in (("q4k_q4k_q6k", (Q4K, Q4K, Q6K)), ("q6k", (Q6K, Q6K, Q6K)), ("q5k_q5k_q6k", (Q5K, Q5K, Q6K)),
-                           ("q5k", (Q5K, Q5K, Q5K)), ("q8_0", (synth.GGML_Q8_0,) * 3)):
+                           ("q5k", (Q5K, Q5K, Q5K)), ("q8_0", (synth.GGML_Q8_0,) * 3), ("q3k", (synth.GGML_Q3_K,) * 3),
+                           ("q2k", (synth.GGML_Q2_K,) * 3)):
             mm, bb, _, _ = time_moe(max(5, args.steps // 40), 2, types=tys)
             extra["moe_ffn_128x(768x2048)_64tok_top8_%s" % label] = {
                 "us": round(mm * 1e3, 1), "bytes": bb, "GB/s": round(bb / (mm * 1e-3) / 1e9, 1),
