@@ -1043,7 +1043,7 @@ moe_down_kq_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__rest
 template <typename F>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4)))
 moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
-                       const uint16_t *__restrict__ X, const int32_t *__restrict__ offsets,
+                       const uint16_t *__restrict__ X, const int32_t *__restrict__ head,
                        const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
                        int n_embd, int n_ff, int top_k) {
     constexpr int kImageRow = 16 * F::kRowChunks;
@@ -1054,7 +1054,8 @@ moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restric
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
     const int row0 = blockIdx.x * 16;
-    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    const int32_t *hd = head + (size_t)e * kHeadInts; /* first slot, count and the first 16 tokens in one line */
+    const int first = hd[0], cnt = hd[1];
     if (cnt == 0) return;
     const int j = lane & 15, kg = lane >> 4;
     const int n_sb = n_embd >> 8;
@@ -1069,7 +1070,8 @@ moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restric
         const int n_live = cnt - t0 < 8 ? cnt - t0 : 8;
         const int tslot = j & 7;
         const bool live = (kg >> 1) == (j >> 3) && tslot < n_live;
-        const int tok = order[first + t0 + (tslot < n_live ? tslot : 0)] / top_k;
+        const int ts = t0 + (tslot < n_live ? tslot : 0);
+        const int tok = ts < kHeadTokens ? hd[kHeadInts - kHeadTokens + ts] : order[first + ts] / top_k;
         const uint16_t *xrow = X + (size_t)tok * n_embd + 8 * kg;
         f32x4 acc_g = zero, acc_u = zero;
         for (int sb = wv; sb < n_sb; sb += n_waves) {
@@ -1425,7 +1427,7 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
             using F = decltype(tag);
             hipLaunchKernelGGL(moe_gate_up_kq_kernel<F>, dim3(n_ff / 16, n_expert), dim3(64 * waves),
                                (size_t)waves * (256 * 4 + 2 * (16 * 16 * F::kRowChunks + 16)), stream, (const uint8_t *)gate,
-                               (const uint8_t *)up, X, ws.offsets, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
+                               (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd, n_ff, top_k);
         };
         switch (type_gate) {
         case T_Q6_K: go(KqQ6K()); break;
