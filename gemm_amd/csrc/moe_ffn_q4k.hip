@@ -1137,6 +1137,101 @@ moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restric
     }
 }
 
+/* ---- 5b. dense GEMM for a handful of tokens in the formats of the kernels above ----
+ * Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k] for 16 rows per workgroup, K split over at most four waves,
+ * eight tokens per pass, the weights exact: what a small batch of decode steps needs for a Q6_K, Q5_K, Q3_K, Q2_K
+ * or Q8_0 tensor (decoding the whole tensor to bf16 for the library's GEMM costs more than streaming it a few
+ * times). Rows past n_rows repeat the last row and are not stored. */
+template <typename F, int NQ>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NQ == 1 ? 4 : 2)))
+gemm_kq_fewtok_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y, int n_rows,
+                      int n_sb, int n_tok, int ldx, int ldy) {
+    constexpr int kImageRow = 16 * F::kRowChunks;
+    constexpr int kImage = 16 * kImageRow + 16;
+    constexpr int kChunks = 16 * F::kRowChunks, kImageLoads = (kChunks + 63) / 64;
+    constexpr int kPass = 8 * NQ; /* tokens per pass over the weights */
+    extern __shared__ __attribute__((aligned(16))) float red[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * 16;
+    const int j = lane & 15, kg = lane >> 4;
+    const int row_bytes = n_sb * F::kBlock;
+    const int last = n_rows - 1 - row0; /* >= 0: the grid covers n_rows */
+    /* LDS: red [waves][8 NQ tokens][16 rows] floats | images [waves][16 rows][chunks + slack] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * (16 * kPass)) + wv * kImage;
+    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
+    const uint8_t *w0 = uniform_ptr(W + (size_t)row0 * row_bytes); /* 16-byte aligned: row0 is a multiple of 16 */
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int jrow = j < last ? j : last;
+    const int tslot = j & 7;
+    const bool mine = (kg >> 1) == (j >> 3); /* the block-diagonal operand: scale group kg >> 1 in rows 8 (kg >> 1) .. + 7 */
+
+    for (int t0 = 0; t0 < n_tok; t0 += kPass) {
+        const int n_live = n_tok - t0 < kPass ? n_tok - t0 : kPass;
+        const uint16_t *xrow[NQ];
+        bool live[NQ];
+        f32x4 acc[NQ];
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            live[q] = mine && 8 * q + tslot < n_live;
+            xrow[q] = X + (size_t)(t0 + (8 * q + tslot < n_live ? 8 * q + tslot : 0)) * ldx + 8 * kg;
+            acc[q] = zero;
+        }
+        for (int sb = wv; sb < n_sb; sb += n_waves) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous image have returned */
+#pragma unroll
+            for (int i = 0; i < kImageLoads; i++) {
+                const int t = 64 * i + lane;
+                int R = t / F::kRowChunks;
+                const int c = t - F::kRowChunks * R;
+                R = R < 16 ? R : 15;
+                R = R < last ? R : last;
+                const int at = R * row_bytes + sb * F::kBlock;
+                const uint32_t off = (uint32_t)(at & ~15) + 16u * (uint32_t)c;
+                const bool wanted = t < kChunks && 16 * c < (at & 15) + F::kBlock;
+                const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
+                if (wanted)
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(w0), "s"(m0v) : "memory");
+            }
+            u32x4 a[NQ][8];
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    u32x4 v = {0u, 0u, 0u, 0u};
+                    if (live[q]) v = *(const u32x4 *)(xrow[q] + sb * 256 + 32 * u);
+                    a[q][u] = v;
+                }
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* image and activations have landed */
+            const int blk_at = j * kImageRow + ((jrow * row_bytes + sb * F::kBlock) & 15);
+            /* one call per token group: the decode of the block is common to them */
+#pragma unroll
+            for (int q = 0; q < NQ; q++) {
+                const u32x4 *const aa[1] = {a[q]};
+                F::template math<1>(img, blk_at, kg, aa, acc[q]);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[q][v] += __shfl_xor(acc[q][v], 32, 64);
+            if (kg < 2) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) red[(wv * kPass + 8 * q + 4 * kg + v) * 16 + j] = acc[q][v];
+            }
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < n_live * 16; idx += blockDim.x) {
+            const int jj = idx & 15, t = idx >> 4;
+            float d = 0.0f;
+            for (int w = 0; w < n_waves; w++) d += red[(w * kPass + t) * 16 + jj];
+            if (row0 + jj < n_rows) Y[(size_t)(t0 + t) * ldy + row0 + jj] = d;
+        }
+        __syncthreads();
+    }
+}
+
 /* ---- 4. out[t] = sum over k, in k order ---- */
 __global__ void __launch_bounds__(256)
 moe_combine_kernel(const float *__restrict__ part, const int32_t *__restrict__ slot_of,
@@ -1386,6 +1481,39 @@ hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, in
 
 /* formats whose experts run on the matrix cores through moe_gate_up_kq_kernel / moe_down_kq_walk_kernel */
 static bool kq_type(uint32_t t) { return t == T_Q6_K || t == T_Q5_K || t == T_Q3_K || t == T_Q2_K || t == T_Q8_0; }
+
+bool launch_gemm_kq_fewtok(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
+                           int ldx, int ldy, hipStream_t stream, hipError_t *err) {
+    *err = hipSuccess;
+    if (!kq_type(type) || n_cols % 256 != 0 || n_tok > kKqFewTokens || ((uintptr_t)W & 15) || ((uintptr_t)X & 15) || (ldx & 7))
+        return false;
+    const int n_sb = n_cols / 256;
+    const int waves = n_sb < 4 ? n_sb : 4;
+    auto go = [&](auto tag) {
+        using F = decltype(tag);
+        /* the tensor has to end on a 16-byte boundary: the image of its last block is whole chunks */
+        if (((size_t)n_rows * n_sb * F::kBlock) & 15) return false;
+        const dim3 grid((n_rows + 15) / 16), block(64 * waves);
+        const size_t image = (size_t)waves * (16 * 16 * F::kRowChunks + 16);
+        const uint8_t *Wb = (const uint8_t *)W;
+        /* 8, 16 or 24 tokens per pass over the weights */
+        if (n_tok <= 8)
+            hipLaunchKernelGGL((gemm_kq_fewtok_kernel<F, 1>), grid, block, waves * 512 + image, stream, Wb, X, Y, n_rows, n_sb, n_tok, ldx, ldy);
+        else if (n_tok <= 16)
+            hipLaunchKernelGGL((gemm_kq_fewtok_kernel<F, 2>), grid, block, waves * 1024 + image, stream, Wb, X, Y, n_rows, n_sb, n_tok, ldx, ldy);
+        else
+            hipLaunchKernelGGL((gemm_kq_fewtok_kernel<F, 3>), grid, block, waves * 1536 + image, stream, Wb, X, Y, n_rows, n_sb, n_tok, ldx, ldy);
+        *err = hipGetLastError();
+        return true;
+    };
+    switch (type) {
+    case T_Q6_K: return go(KqQ6K());
+    case T_Q5_K: return go(KqQ5K());
+    case T_Q3_K: return go(KqQ3K());
+    case T_Q2_K: return go(KqQ2K());
+    default: return go(KqQ8_0());
+    }
+}
 
 size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert) {
     return carve(nullptr, n_tok, top_k, n_embd, n_ff, n_expert).bytes;

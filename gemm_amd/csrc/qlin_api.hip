@@ -955,6 +955,15 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
         if (n_tok <= kFewTokens || (n_tok <= 512 && tiles >= 200))
             return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     }
+    /* a few tokens of a Q6_K, Q5_K, Q3_K, Q2_K or Q8_0 tensor: streamed once per eight tokens with exact codes
+     * (14336 x 4096 Q6_K, 8 tokens: decode + library GEMM about 75 us) */
+    {
+        hipError_t e = hipSuccess;
+        if (launch_gemm_kq_fewtok(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream, &e)) {
+            if (e != hipSuccess) return fail(QLIN_ERR_DEVICE, "few-token GEMM launch failed: %s", hipGetErrorString(e));
+            return QLIN_OK;
+        }
+    }
     if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols))
         return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes");
     {

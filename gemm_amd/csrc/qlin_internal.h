@@ -93,6 +93,11 @@ const char *launch_gemm_dense_bf16(const uint16_t *Wd, const uint16_t *X, float 
  * aligned, ldx % 8 == 0 */
 hipError_t launch_gemm_dense_own(const uint16_t *Wd, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                  int ldx, int ldy, hipStream_t stream);
+constexpr int kKqFewTokens = 24; /* up to this many tokens Q6_K, Q5_K, Q3_K, Q2_K and Q8_0 tensors are streamed once per
+                                    eight tokens with exact codes instead of decoded to bf16 for the library's GEMM */
+/* false: not a shape for this kernel (the caller takes another route); true: launched, *err says how it went */
+bool launch_gemm_kq_fewtok(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
+                           int ldx, int ldy, hipStream_t stream, hipError_t *err);
 constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
 hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                   int ldx, int ldy, hipStream_t stream);

@@ -41,6 +41,14 @@ def dense_kernel(request):
     qlinear.check(qlinear.load().qlin_set_dense_gemm_own(0))
 
 
+KQ = {synth.GGML_Q6_K, synth.GGML_Q5_K, synth.GGML_Q3_K, synth.GGML_Q2_K, synth.GGML_Q8_0}
+
+
+def streams_exact_weights(tid, n_tok, n_rows, n_cols):
+    """few tokens of these formats go through a kernel that multiplies the unrounded weights"""
+    return tid in KQ and n_tok <= 24 and n_cols % 256 == 0 and n_rows * synth.row_bytes(tid, n_cols) % 16 == 0
+
+
 def references(oracle, tid, W, Xb, n_cols):
     dec = oracle.dequant_matrix(tid, W, n_cols)
     Xf = synth.bf16_bits_to_f32(Xb).astype(np.float64)
@@ -72,8 +80,39 @@ def test_shapes(oracle, tid, n_tok, n_rows, n_cols, dense_kernel):
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=n_cols + n_tok, tokens=n_tok))
     Y = run(tid, W, Xb, n_rows, n_cols, n_tok)
     exact, designed = references(oracle, tid, W, Xb, n_cols)
-    assert rel_l2(Y, designed) <= 2e-5, (ALL[tid], n_tok, n_rows, n_cols)
+    assert rel_l2(Y, exact if streams_exact_weights(tid, n_tok, n_rows, n_cols) else designed) <= 2e-5, (ALL[tid], n_tok, n_rows, n_cols)
     assert rel_l2(Y, exact) <= 3e-3
+
+
+@pytest.mark.parametrize("n_tok", [1, 8, 9, 24, 25])
+@pytest.mark.parametrize("tid", sorted(KQ), ids=lambda t: ALL[t])
+def test_few_tokens_of_a_k_quant_or_q8_0_tensor(oracle, tid, n_tok):
+    """up to 24 tokens: one kernel, unrounded weights, no workspace, rows and padding of any count; 25 tokens: the
+    decode + dense route, which needs the workspace"""
+    # 5 super-blocks over 4 waves, a last row tile of 8 rows; the kernel wants the tensor to end on a 16-byte
+    # boundary (210-, 110- and 84-byte blocks: a row count that is a multiple of 8)
+    n_rows, n_cols = 296, 1280
+    W = synth.make_weights(tid, n_rows, n_cols, seed=40 + tid)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=41 + n_tok, tokens=n_tok))
+    ldx, ldy = n_cols + 8, n_rows + 3
+    Xpad = np.zeros((n_tok, ldx), np.uint16)
+    Xpad[:, :n_cols] = Xb
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xpad)
+    dY = qlinear.DevBuf.from_numpy(np.full((n_tok, ldy), -3.0, np.float32))
+    exact, designed = references(oracle, tid, W, Xb, n_cols)
+    if n_tok <= 24:
+        qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, None)
+        want = exact
+    else:
+        with pytest.raises(qlinear.QlinError):
+            qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, None)
+        ws = qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+        qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, ws)
+        want = designed
+    qlinear.sync()
+    Y = dY.to_numpy(np.float32, (n_tok, ldy))
+    assert rel_l2(Y[:, :n_rows], want) <= 2e-5, (ALL[tid], n_tok)
+    assert np.all(Y[:, n_rows:] == -3.0)
 
 
 def test_q4k_few_tokens_is_the_fused_path_and_needs_no_workspace(oracle):
@@ -127,9 +166,10 @@ def test_argument_checks():
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 300, 4, 304, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ragged K
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 260, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ldx % 8
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 100, ws.ptr, need, None) == qlinear.ERR_ARG      # ldy < rows
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, None, 0, None) == 0  # few tokens: no workspace needed
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 0, 256, 4, 256, 128, None, 0, None) == 0
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 0, 256, 128, None, 0, None) == 0
     assert lib.qlin_gemm_bf16_any_workspace_bytes(0, 256) == 0
