@@ -1,0 +1,514 @@
+/*
+ * gemv_grid.hip - batch-1 matvec for the codebook ("grid") formats IQ2_XXS, IQ3_XXS and IQ3_S on gfx950: the
+ * inner products run on the 8-bit integer matrix instruction, the codebook and sign-mask lookups in LDS.
+ *
+ * y[r] = sum over 32-element groups of scale(r, group) * (signed grid bytes . x_group)
+ * (the decoders of common/ggml_dequant.h:2793-2816, :2916-2940 and :3022-3058 dotted with x).
+ *
+ *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
+ *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
+ *     2^-23 of that largest |x| per element.
+ *  2. v_mfma_i32_16x16x64_i8: 16 weight rows (B operand: one signed grid byte per element) against 16
+ *     "x rows" (A operand). Lane group g = lane/16 of a wave owns groups 2g and 2g+1 of the wave's
+ *     super-block: instruction s = 0..3 of the super-block takes from lane group g the 16 elements
+ *     [16 (s & 1), +16) of group 2g + (s >> 1). The A operand is block-diagonal to match: x row 4g + digit
+ *     (digit 0..2; row 4g+3 stays zero) holds that digit plane of lane group g's 16 elements at lane group g's k positions and zeros elsewhere,
+ *     so after two instructions result register v of lane (n, g) is digit plane v of group 2g (then 2g+1)
+ *     for weight row n. Which k position carries which element is free as long as both operands agree.
+ *  3. Wave w of the 16-wave workgroup owns super-block w (w+16, ...) of every row of the workgroup, prepares
+ *     only its own 256 elements of x, and reads its bytes of a block straight from HBM: lane (n, g) takes
+ *     the bytes of groups 2g, 2g+1 of row n (blocks are 2-byte aligned: dword-aligned loads, a 16-bit
+ *     tail and a funnel shift). The waves' shares of a row meet in LDS at the end.
+ *
+ * What a lane spends per element is one table lookup per 4-8 elements for the grid, one per 8 for the sign
+ * mask, two vector instructions per 4 elements to apply the signs and a sixteenth of a matrix instruction;
+ * the v_dot4 formulation (gemv_int.hip) spends an instruction per element on the products alone.
+ *
+ * A non-finite x makes every output NaN (the fixed-point form cannot carry Inf).
+ */
+#include "qlin_codebooks.h"
+#include "qlin_codebooks_ext.h"
+#include "qlin_device.h"
+#include "qlin_internal.h"
+#include <type_traits>
+
+namespace qlin {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+
+constexpr int kWaves = 16;        /* wavefronts per workgroup */
+constexpr int kMaxKc = 4;         /* super-blocks per wave: K <= 16384 */
+constexpr int kMaxRowsPerWg = 128;
+constexpr int kXScratch = 1088;   /* per wave: 3 digit planes x 256 B, 64 zero bytes, (at 1024) 8 x 2^(e-22) */
+
+/* x operand of one super-block: A[s] for instruction s; scale[h] = 2^(e-22) of group 2 (lane/16) + h */
+struct XOperand {
+    v4i A[4];
+    float scale[2];
+};
+
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_movu(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+
+/* sixteen bytes at p (2-byte aligned, inside a block that starts at least two bytes before p): the aligned
+ * dwords around them and, where p sits in the middle of a dword, the two bytes behind the last full one */
+struct Raw16 {
+    u32x4_a4 q;
+    uint32_t tail;
+};
+__device__ __forceinline__ Raw16 load16(const uint8_t *p) {
+    Raw16 r;
+    const uint32_t odd = (uint32_t)(uintptr_t)p & 2u;
+    r.q = *reinterpret_cast<const u32x4_a4 *>(p - odd);
+    r.tail = 0;
+    if (odd) r.tail = *reinterpret_cast<const uint16_t *>(p + 14);
+    return r;
+}
+__device__ __forceinline__ void bytes16(const Raw16 &r, uint32_t sh, uint32_t (&w)[4]) { /* sh = 0 or 16 */
+    w[0] = __builtin_amdgcn_alignbit(r.q.y, r.q.x, sh);
+    w[1] = __builtin_amdgcn_alignbit(r.q.z, r.q.y, sh);
+    w[2] = __builtin_amdgcn_alignbit(r.q.w, r.q.z, sh);
+    w[3] = __builtin_amdgcn_alignbit(r.tail, r.q.w, sh);
+}
+struct Raw8 {
+    u32x2_a4 q;
+    uint32_t tail;
+};
+__device__ __forceinline__ Raw8 load8(const uint8_t *p) {
+    Raw8 r;
+    const uint32_t odd = (uint32_t)(uintptr_t)p & 2u;
+    r.q = *reinterpret_cast<const u32x2_a4 *>(p - odd);
+    r.tail = 0;
+    if (odd) r.tail = *reinterpret_cast<const uint16_t *>(p + 6);
+    return r;
+}
+__device__ __forceinline__ void bytes8(const Raw8 &r, uint32_t sh, uint32_t (&w)[2]) {
+    w[0] = __builtin_amdgcn_alignbit(r.q.y, r.q.x, sh);
+    w[1] = __builtin_amdgcn_alignbit(r.tail, r.q.y, sh);
+}
+
+/* the tables in LDS: the format's grid, and the sign masks (0xFF per negative element, two dwords per sign
+ * byte): 256 entries by sign byte, then 128 by the seven stored bits of the formats that keep a parity bit */
+struct Tables {
+    const uint32_t *grid;
+    const uint2 *sign256, *sign128;
+};
+
+/* magnitudes m (four bytes, each 1..127: no grid of these formats holds a zero) with the signs of mask s
+ * (0xFF = negative) -> signed bytes: (m ^ s) + (s & 1) per byte; a nonzero m keeps the +1 inside its byte */
+__device__ __forceinline__ int apply_signs(uint32_t m, uint32_t s) { return (int)((m ^ s) + (s & 0x01010101u)); }
+__device__ __forceinline__ uint32_t spread4(uint32_t v) { return ((v & 15u) * 0x00204081u) & 0x01010101u; }
+
+/* digit sums of one group (top, middle, low) -> the group's integer inner product as a float */
+__device__ __forceinline__ float join_digits(v4i c) {
+    return fmaf((float)c.x, 65536.0f, (float)((c.y << 8) + c.z));
+}
+
+template <uint32_t T> struct GridFmt;
+
+/* IQ2_XXS [d][8 x (4 grid indices, 4 x 7 sign bits + 4-bit scale)]: d*(0.5+s)*0.25 * grid byte * sign, an
+ * eight-byte grid entry per index (common/ggml_dequant.h:2793-2816); 66-byte blocks */
+template <> struct GridFmt<T_IQ2_XXS> {
+    static constexpr int kBlock = 66, kGridBytes = 2048, kDepth = 4;
+    __device__ static const uint32_t *grid_src() { return reinterpret_cast<const uint32_t *>(qlin_iq2xxs_grid); }
+    struct Raw {
+        Raw16 a; /* groups 2g, 2g+1: [indices, signs + scale] each */
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.a = load16(blk + 2 + 16 * g);
+        r.d = *reinterpret_cast<const uint16_t *>(blk);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t) {
+        uint32_t w[4];
+        bytes16(r.a, sh, w);
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+        const float d = half_bits_fast(r.d) * 0.25f;
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t a0 = w[2 * h], a1 = w[2 * h + 1];
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const uint2 m0 = grid[(a0 >> (16 * q)) & 255u], m1 = grid[(a0 >> (16 * q + 8)) & 255u];
+                const uint2 s0 = t.sign128[(a1 >> (14 * q)) & 127u], s1 = t.sign128[(a1 >> (14 * q + 7)) & 127u];
+                const v4i b = {apply_signs(m0.x, s0.x), apply_signs(m0.y, s0.y), apply_signs(m1.x, s1.x), apply_signs(m1.y, s1.y)};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2 * h + q], b, c, 0, 0, 0);
+            }
+            acc = fmaf(join_digits(c) * xo.scale[h], 0.5f + (float)(a1 >> 28), acc);
+        }
+        return d * acc;
+    }
+};
+
+/* IQ3_XXS [d][qs 64][8 x (4 x 7 sign bits + 4-bit scale)]: d*(0.5+s)*0.5 * grid byte * sign, a four-byte
+ * grid entry per index byte (:2916-2940); 98-byte blocks */
+template <> struct GridFmt<T_IQ3_XXS> {
+    static constexpr int kBlock = 98, kGridBytes = 1024, kDepth = 2;
+    __device__ static const uint32_t *grid_src() { return qlin_iq3xxs_grid; }
+    struct Raw {
+        Raw16 qs; /* index bytes of groups 2g, 2g+1 */
+        Raw8 sc;  /* their sign + scale words */
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load16(blk + 2 + 16 * g);
+        r.sc = load8(blk + 66 + 8 * g);
+        r.d = *reinterpret_cast<const uint16_t *>(blk);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t) {
+        uint32_t qs[4], sc[2];
+        bytes16(r.qs, sh, qs);
+        bytes8(r.sc, sh, sc);
+        const float d = half_bits_fast(r.d) * 0.5f;
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint32_t a1 = sc[h];
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const uint32_t ix = qs[2 * h + q];
+                const uint2 s0 = t.sign128[(a1 >> (14 * q)) & 127u], s1 = t.sign128[(a1 >> (14 * q + 7)) & 127u];
+                const v4i b = {apply_signs(t.grid[ix & 255u], s0.x), apply_signs(t.grid[(ix >> 8) & 255u], s0.y),
+                               apply_signs(t.grid[(ix >> 16) & 255u], s1.x), apply_signs(t.grid[ix >> 24], s1.y)};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2 * h + q], b, c, 0, 0, 0);
+            }
+            acc = fmaf(join_digits(c) * xo.scale[h], 0.5f + (float)(a1 >> 28), acc);
+        }
+        return d * acc;
+    }
+};
+
+/* IQ3_S [d][qs 64][qh 8][signs 32][scales 4]: d*(1+2s) * grid byte * sign, 9-bit grid indices (:3022-3058);
+ * 110-byte blocks */
+template <> struct GridFmt<T_IQ3_S> {
+    static constexpr int kBlock = 110, kGridBytes = 2048, kDepth = 2;
+    __device__ static const uint32_t *grid_src() { return qlin_iq3s_grid; }
+    struct Raw {
+        Raw16 qs;  /* low index bytes of groups 2g, 2g+1 */
+        Raw8 sg;   /* their sign bytes */
+        uint32_t qh, scales, d; /* the ninth index bits (a byte per group), the byte with both 4-bit scales */
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load16(blk + 2 + 16 * g);
+        r.sg = load8(blk + 74 + 8 * g);
+        r.qh = *reinterpret_cast<const uint16_t *>(blk + 66 + 2 * g);
+        r.scales = blk[106 + g];
+        r.d = *reinterpret_cast<const uint16_t *>(blk);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t) {
+        uint32_t qs[4], sg[2];
+        bytes16(r.qs, sh, qs);
+        bytes8(r.sg, sh, sg);
+        const float d = half_bits_fast(r.d);
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const uint32_t ix = qs[2 * h + q];
+                const uint32_t hb = r.qh >> (8 * h + 4 * q); /* bits 0..3: the ninth bits of these four indices */
+                const uint2 s0 = t.sign256[(sg[h] >> (16 * q)) & 255u], s1 = t.sign256[(sg[h] >> (16 * q + 8)) & 255u];
+                const uint32_t i0 = (ix & 255u) | ((hb & 1u) << 8), i1 = ((ix >> 8) & 255u) | ((hb & 2u) << 7);
+                const uint32_t i2 = ((ix >> 16) & 255u) | ((hb & 4u) << 6), i3 = (ix >> 24) | ((hb & 8u) << 5);
+                const v4i b = {apply_signs(t.grid[i0], s0.x), apply_signs(t.grid[i1], s0.y),
+                               apply_signs(t.grid[i2], s1.x), apply_signs(t.grid[i3], s1.y)};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2 * h + q], b, c, 0, 0, 0);
+            }
+            const uint32_t nib = (r.scales >> (4 * h)) & 15u;
+            acc = fmaf(join_digits(c) * xo.scale[h], (float)(1u + 2u * nib), acc);
+        }
+        return d * acc;
+    }
+};
+
+}  // namespace
+
+template <uint32_t T, int NKC>
+__global__ void __launch_bounds__(kWaves * 64)
+gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg) {
+    using F = GridFmt<T>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15, g = lane >> 4;
+
+    /* a workgroup owns rows_per_wg rows: of the concatenated matrices, or, where two results are
+     * combined (mode 2), the same rows of both matrices (local rows: first matrix, then second) */
+    const bool paired = job.mode == 2;
+    const int n_mats_here = paired ? 2 : 1;
+    const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
+    const int row0 = blockIdx.x * rows_per_wg;
+    int rows_here = n_rows - row0;
+    if (rows_here > rows_per_wg) rows_here = rows_per_wg;
+    const int n_lrows = rows_here * n_mats_here;
+    const int n_rg = (n_lrows + 15) >> 4;
+    const size_t row_bytes = (size_t)n_sb * F::kBlock;
+    const int n_kc = wv < n_sb ? ((n_sb - wv + 15) >> 4) : 0; /* this wave's super-blocks: wv, wv+16, ... */
+
+    /* LDS: x scratch per wave, the grid and the sign masks at addresses the compiler knows (a lookup is then a
+     * shift, a mask and a read with a constant offset); the partial sums [rows][kWaves] behind them */
+    __shared__ __attribute__((aligned(16))) uint8_t xs_all[kWaves * kXScratch];
+    __shared__ __attribute__((aligned(16))) uint32_t grid_lds[F::kGridBytes / 4];
+    __shared__ __attribute__((aligned(16))) uint2 sign_lds[256 + 128];
+    uint8_t *xs = xs_all + wv * kXScratch;
+    float *partial = reinterpret_cast<float *>(lds);
+    const Tables tab = {grid_lds, sign_lds, sign_lds + 256};
+
+    auto locate = [&](int lr, const uint8_t *&Wm, float *&ym, int &r) {
+        if (paired) {
+            const bool second = lr >= rows_here;
+            Wm = second ? job.W1 : job.W0;
+            ym = job.y0;
+            r = row0 + (second ? lr - rows_here : lr);
+        } else {
+            job_locate(job, row0 + lr, Wm, ym, r);
+        }
+    };
+    auto row_pointer = [&](int rg) { /* this lane's row of row group rg (rows past the end: the last one, never stored) */
+        int lr = 16 * rg + n;
+        if (lr >= n_lrows) lr = n_lrows - 1;
+        /* matrix and row by selects, not branches: the lanes of a row group may sit in different matrices */
+        const int v = row0 + lr;
+        const bool in1 = paired ? lr >= rows_here : v >= job.n0, in2 = !paired && v >= job.n0 + job.n1;
+        const uint8_t *Wm = in2 ? job.W2 : in1 ? job.W1 : job.W0;
+        const int r = paired ? (in1 ? v - rows_here : v) : v - (in2 ? job.n0 + job.n1 : in1 ? job.n0 : 0);
+        return Wm + (size_t)r * row_bytes + (size_t)wv * F::kBlock;
+    };
+
+    v4f xr[NKC];
+#pragma unroll
+    for (int kc = 0; kc < NKC; kc++) {
+        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (kc < n_kc) v = *reinterpret_cast<const v4f *>(x + (16 * kc + wv) * 256 + 4 * lane);
+        xr[kc] = v;
+    }
+
+    /* x -> signed digit planes -> A operands, wave-private */
+    auto prepare = [&](v4f v, XOperand &xo) {
+        /* the largest |x| of the group as a bit pattern: an integer maximum keeps a NaN or an Inf on top */
+        constexpr uint32_t kAbs = 0x7FFFFFFFu;
+        uint32_t amax = max(max(__float_as_uint(v.x) & kAbs, __float_as_uint(v.y) & kAbs),
+                            max(__float_as_uint(v.z) & kAbs, __float_as_uint(v.w) & kAbs));
+        /* 8 consecutive lanes share one 32-element group */
+        amax = max(amax, dpp_movu<0xB1>(amax));
+        amax = max(amax, dpp_movu<0x4E>(amax));
+        amax = max(amax, dpp_movu<0x141>(amax));
+        int e = (int)(amax >> 23) - 126; /* amax in [2^(e-1), 2^e) */
+        if (e < -96) e = -96;            /* zero and tiny groups */
+        const float up = __uint_as_float((uint32_t)(127 + 22 - e) << 23);
+        float down = __uint_as_float((uint32_t)(127 - 22 + e) << 23);
+        if (amax >= 0x7F800000u) down = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
+        const int X[4] = {__float2int_rn(v.x * up), __float2int_rn(v.y * up), __float2int_rn(v.z * up),
+                          __float2int_rn(v.w * up)};
+        int X1[4], X2[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            X1[k] = (X[k] + 128) >> 8;  /* X = 256*X1 + d0, d0 = (int8)X */
+            X2[k] = (X1[k] + 128) >> 8; /* X1 = 256*X2 + d1; d2 = X2 in [-64, 64] */
+        }
+        /* byte 0 of four values -> one dword (selector 0-3: second operand, 4-7: first, 0x0c: zero) */
+        auto pack = [](const int (&a)[4]) {
+            const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)a[1], (uint32_t)a[0], 0x0c0c0400u);
+            const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)a[3], (uint32_t)a[2], 0x0c0c0400u);
+            return __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+        };
+        uint32_t *pl = reinterpret_cast<uint32_t *>(xs);
+        pl[lane] = pack(X2);       /* digit 2 (top) */
+        pl[64 + lane] = pack(X1);  /* digit 1 */
+        pl[128 + lane] = pack(X);  /* digit 0 */
+        if ((lane & 7) == 0) reinterpret_cast<float *>(xs + 1024)[lane >> 3] = down;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        /* A operand: x row i = lane%16 = 4*g' + plane (plane 3 unused) is live in lane group g' only; its four
+         * instructions take the 64 elements of groups 2g', 2g'+1 in order. Every other lane reads zeros. */
+        const int plane = n & 3;
+        const bool live = (n >> 2) == g && plane < 3;
+        const uint4 *src = reinterpret_cast<const uint4 *>(xs + (live ? plane * 256 + 64 * g : 768));
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const uint4 d = src[s];
+            const v4i a = {(int)d.x, (int)d.y, (int)d.z, (int)d.w};
+            xo.A[s] = a;
+        }
+        const float2 m = reinterpret_cast<const float2 *>(xs + 1024)[g];
+        xo.scale[0] = m.x;
+        xo.scale[1] = m.y;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    auto store_partial = [&](int rg, float v, bool add) { /* the four lane groups hold four shares of the same row */
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        const int lr = 16 * rg + n;
+        if (lane < 16 && lr < n_lrows) {
+            float *p = partial + lr * kWaves + wv;
+            *p = add ? *p + v : v;
+        }
+    };
+
+    /* every piece of a block that a lane reads starts 2 (mod 4) bytes into the block: the funnel shift of its bytes */
+    auto shift_of = [](const uint8_t *blk) { return (((uint32_t)(uintptr_t)blk + 2u) & 2u) * 8u; };
+
+    /* the first blocks are requested before the tables are built and x is prepared: the wave's first two
+     * super-blocks of a lone row group (long rows), else its first super-block of the first row groups */
+    const bool long_rows = NKC > 1 && n_rg < 2;
+    constexpr int D = F::kDepth; /* row groups of a super-block column in flight per wave */
+    typename F::Raw first[D];
+    uint32_t first_sh[D];
+    if (n_kc > 0) {
+#pragma unroll
+        for (int q = 0; q < D; q++) {
+            if (long_rows && q >= 2) break;
+            const uint8_t *blk = long_rows ? row_pointer(0) + (size_t)(q < n_kc ? q : 0) * (16 * F::kBlock)
+                                           : row_pointer(q < n_rg ? q : 0);
+            first[q] = F::load(blk, g);
+            first_sh[q] = shift_of(blk);
+        }
+    }
+    if (lane < 16) reinterpret_cast<uint32_t *>(xs + 768)[lane] = 0u; /* what the dead lanes of the x operand read */
+    for (int t = threadIdx.x; t < F::kGridBytes / 4; t += kWaves * 64) grid_lds[t] = F::grid_src()[t];
+    if (threadIdx.x < 384) {
+        const uint32_t i = threadIdx.x, sb = i < 256 ? i : iq_sign_byte(i - 256);
+        sign_lds[i] = make_uint2(spread4(sb) * 0xFFu, spread4(sb >> 4) * 0xFFu);
+    }
+    __syncthreads();
+
+    XOperand xo;
+    if (n_kc == 0) { /* a wave without a super-block (K < 4096) contributes zeros */
+        for (int rg = 0; rg < n_rg; rg++) store_partial(rg, 0.0f, false);
+    } else if (long_rows) {
+        /* one row group: the wave's super-blocks of it, two requested ahead of the one being multiplied */
+        float acc = 0.0f;
+        const uint8_t *blk0 = row_pointer(0);
+#pragma unroll
+        for (int kc = 0; kc < NKC; kc++) {
+            typename F::Raw nxt = first[1];
+            uint32_t nxt_sh = first_sh[1];
+            if (kc + 2 < n_kc) {
+                const uint8_t *blk = blk0 + (size_t)(kc + 2) * (16 * F::kBlock);
+                nxt = F::load(blk, g);
+                nxt_sh = shift_of(blk);
+            }
+            if (kc < n_kc) {
+                prepare(xr[kc], xo);
+                acc += F::item(xo, first[0], first_sh[0], tab);
+            }
+            first[0] = first[1];
+            first_sh[0] = first_sh[1];
+            first[1] = nxt;
+            first_sh[1] = nxt_sh;
+        }
+        store_partial(0, acc, false);
+    } else {
+        for (int kc = 0; kc < n_kc; kc++) {
+            v4f v = xr[0];
+#pragma unroll
+            for (int kk = 1; kk < NKC; kk++) v = kc == kk ? xr[kk] : v;
+            prepare(v, xo);
+            /* D row groups in flight: a group's registers are refilled as soon as it has been multiplied */
+            if (kc > 0) {
+#pragma unroll
+                for (int q = 0; q < D; q++) {
+                    const uint8_t *blk = row_pointer(q < n_rg ? q : 0) + (size_t)kc * (16 * F::kBlock);
+                    first[q] = F::load(blk, g);
+                    first_sh[q] = shift_of(blk);
+                }
+            }
+            for (int rg = 0; rg < n_rg; rg += D) {
+#pragma unroll
+                for (int q = 0; q < D; q++) {
+                    if (rg + q < n_rg) store_partial(rg + q, F::item(xo, first[q], first_sh[q], tab), kc > 0);
+                    if (rg + q + D < n_rg) {
+                        const uint8_t *blk = row_pointer(rg + q + D) + (size_t)kc * (16 * F::kBlock);
+                        first[q] = F::load(blk, g);
+                        first_sh[q] = shift_of(blk);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    /* sum the waves' shares of each row and store */
+    auto row_total = [&](int lr) {
+        const float4 *p = reinterpret_cast<const float4 *>(partial + lr * kWaves);
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kWaves / 4; k++) {
+            const float4 v = p[k];
+            s += (v.x + v.y) + (v.z + v.w);
+        }
+        return s;
+    };
+    if (paired) {
+        for (int lr = threadIdx.x; lr < rows_here; lr += kWaves * 64)
+            job.y0[row0 + lr] = silu_times(row_total(lr), row_total(rows_here + lr));
+    } else {
+        for (int lr = threadIdx.x; lr < n_lrows; lr += kWaves * 64) {
+            const uint8_t *Wm;
+            float *ym;
+            int r;
+            locate(lr, Wm, ym, r);
+            const float s = row_total(lr);
+            ym[r] = job.mode == 1 ? ym[r] + s : s;
+        }
+    }
+}
+
+namespace {
+
+template <uint32_t T>
+bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err) {
+    const int n_sb = n_cols / 256;
+    /* rows of more than 4096 elements: up to there the v_dot4 kernel (gemv_int.hip) measured faster (both wait
+     * for the table lookups; this one saves its vector instructions where x has to be prepared for few rows) */
+    if (n_cols % 256 != 0 || n_sb <= 16 || n_sb > 16 * kMaxKc || ((uintptr_t)x & 15)) return false;
+    /* rows start on even addresses (even block sizes); the loads want the matrices dword-aligned at least */
+    for (int m = 0; m < job.n_mat; m++)
+        if ((uintptr_t)job.W[m] & 3) return false;
+    const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
+    const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
+    if (n_rows == 0) return false;
+    int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
+    rows_per_wg = (rows_per_wg + 15) & ~15; /* whole row groups: a matrix instruction wants 16 rows anyway */
+    if (rows_per_wg * n_mats_here > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / n_mats_here;
+    const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
+    const size_t lds_bytes = (size_t)rows_per_wg * n_mats_here * kWaves * 4; /* the partial sums; the rest is static */
+    const JobView view = job_view(job);
+    hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg);
+    *err = hipGetLastError();
+    return true;
+}
+
+}  // namespace
+
+bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
+                      hipError_t *err) {
+    *err = hipSuccess;
+    switch (type) {
+    case T_IQ2_XXS: return grid_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ3_XXS: return grid_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ3_S: return grid_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err);
+    default: return false;
+    }
+}
+
+}  // namespace qlin

@@ -248,6 +248,7 @@ hipError_t dispatch_gemv_job(uint32_t type, const GemvJob &job, const float *x, 
     if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && w_aligned && aligned(x, 16))
         return launch_gemv_q4k(job, x, n_cols, s, g.n_cu);
     hipError_t err;
+    if (launch_gemv_grid(type, job, x, n_cols, g.n_cu, s, &err)) return err;
     if (launch_gemv_int(type, job, x, n_cols, g.n_cu, s, &err)) return err;
     if (launch_gemv_stream(type, job, x, n_cols, g.n_cu, s, &err)) return err;
     return launch_gemv_generic(type, job, x, n_cols, s);

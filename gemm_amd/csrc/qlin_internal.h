@@ -70,6 +70,10 @@ bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n
 /* integer-dot matvec (gemv_int.hip) for the formats it covers; same contract as launch_gemv_stream */
 bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
                      hipStream_t stream, hipError_t *err);
+/* matrix-instruction matvec for the codebook formats IQ2_XXS, IQ3_XXS and IQ3_S (gemv_grid.hip): n_cols % 256 == 0,
+ * n_cols <= 16384; same contract as launch_gemv_stream */
+bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
+                      hipStream_t stream, hipError_t *err);
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu);
 

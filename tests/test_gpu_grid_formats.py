@@ -1,0 +1,114 @@
+"""GPU parity of the matrix-instruction matvec for the codebook formats (IQ2_XXS, IQ3_XXS, IQ3_S; rows longer
+than 4096 elements take it) against the CPU oracle, through the C ABI: plain, ragged row counts, several
+matrices in one launch, gate+up+SiLU, projection+residual, non-finite x. Relative L2 <= 1e-5."""
+import numpy as np
+import pytest
+
+from gemm_amd import qlinear
+import synth
+from tests.conftest import rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+GRID = {synth.GGML_IQ2_XXS: "iq2_xxs", synth.GGML_IQ3_XXS: "iq3_xxs", synth.GGML_IQ3_S: "iq3_s"}
+
+
+# 17 super-blocks (one wave with two), 43 (ragged over the 16 waves), 56 and 64 (the most a wave takes);
+# one row, a ragged last row group, several row groups per workgroup, more rows than compute units x 16
+@pytest.mark.parametrize("n_rows,n_cols", [(1, 4352), (16, 4352), (37, 11008), (300, 8192), (4096, 14336), (130, 16384),
+                                           (5000, 4608)])
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_matvec(oracle, tid, n_rows, n_cols):
+    W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + tid)
+    x = synth.make_activation(n_cols, seed=n_cols + tid)
+    dW, dx, dy = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(x), qlinear.DevBuf(n_rows * 4)
+    qlinear.gemv_dev(tid, dW, dx, dy, n_rows, n_cols)
+    qlinear.sync()
+    got = dy.to_numpy(np.float32, (n_rows,))
+    rows = np.arange(n_rows) if n_rows <= 400 else np.r_[0:60, n_rows // 2:n_rows // 2 + 60, n_rows - 60:n_rows]
+    want = oracle.gemv_f64(tid, W[rows], x, n_cols)
+    if n_rows >= 16:
+        assert rel_l2(got[rows], want) <= TOL
+    assert np.allclose(got[rows], want, rtol=2e-4, atol=2e-6 * np.abs(want).max())
+
+
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_outlier_and_tiny_activations(oracle, tid):
+    """an element 1e5 times its neighbours, a group of zeros and a group of denormal-sized values"""
+    n_rows, n_cols = 48, 8192
+    W = synth.make_weights(tid, n_rows, n_cols, seed=7)
+    x = synth.make_activation(n_cols, seed=8)
+    x[1000] = 1.0e5
+    x[2048:2080] = 0.0
+    x[4096:4128] = 1.0e-39
+    dW, dx, dy = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(x), qlinear.DevBuf(n_rows * 4)
+    qlinear.gemv_dev(tid, dW, dx, dy, n_rows, n_cols)
+    qlinear.sync()
+    assert rel_l2(dy.to_numpy(np.float32, (n_rows,)), oracle.gemv_f64(tid, W, x, n_cols)) <= TOL
+
+
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_gate_up_silu(oracle, tid):
+    n_rows, n_cols = 203, 8192
+    Wg = synth.make_weights(tid, n_rows, n_cols, seed=11)
+    Wu = synth.make_weights(tid, n_rows, n_cols, seed=12)
+    x = synth.make_activation(n_cols, seed=13) * np.float32(0.02)
+    got = qlinear.matvec_silu_mul(tid, Wg, tid, Wu, x, n_cols)
+    g, u = oracle.gemv_f64(tid, Wg, x, n_cols), oracle.gemv_f64(tid, Wu, x, n_cols)
+    assert rel_l2(got, g / (1.0 + np.exp(-g)) * u) <= TOL
+
+
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_projection_plus_residual_twice(oracle, tid):
+    n_rows, n_cols = 77, 14336
+    W = synth.make_weights(tid, n_rows, n_cols, seed=31)
+    x = synth.make_activation(n_cols, seed=32)
+    res = synth.make_activation(n_rows, seed=33)
+    dW, dx, dy = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(x), qlinear.DevBuf.from_numpy(res)
+    qlinear.gemv_add_dev(tid, dW, dx, dy, n_rows, n_cols)
+    qlinear.gemv_add_dev(tid, dW, dx, dy, n_rows, n_cols)
+    qlinear.sync()
+    want = res.astype(np.float64) + 2.0 * oracle.gemv_f64(tid, W, x, n_cols)
+    assert rel_l2(dy.to_numpy(np.float32, (n_rows,)), want) <= TOL
+
+
+# row counts that put the matrices' borders inside a row group and inside a workgroup
+@pytest.mark.parametrize("rows", [(40, 9, 9), (16, 16, 0), (300, 7, 100)])
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_several_matrices_one_launch(oracle, tid, rows):
+    n_cols = 5120
+    Ws = [synth.make_weights(tid, max(r, 1), n_cols, seed=41 + i) for i, r in enumerate(rows)]
+    x = synth.make_activation(n_cols, seed=44)
+    dWs = [qlinear.DevBuf.from_numpy(W) for W in Ws]
+    dys = [qlinear.DevBuf(max(r, 1) * 4) for r in rows]
+    dx = qlinear.DevBuf.from_numpy(x)
+    qlinear.gemv_multi_dev(tid, dWs, dys, list(rows), dx, n_cols)
+    qlinear.sync()
+    for W, dy, r in zip(Ws, dys, rows):
+        if r:
+            assert rel_l2(dy.to_numpy(np.float32, (r,)), oracle.gemv_f64(tid, W[:r], x, n_cols)) <= TOL
+
+
+@pytest.mark.parametrize("bad", [np.nan, np.inf, -np.inf])
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_non_finite_x_poisons_every_row(tid, bad):
+    n_rows, n_cols = 33, 8192
+    W = synth.make_weights(tid, n_rows, n_cols, seed=3)
+    x = synth.make_activation(n_cols, seed=4)
+    x[5000] = bad
+    y = qlinear.matvec(tid, W, x, n_cols)
+    assert np.all(np.isnan(y))
+
+
+@pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
+def test_repeatable_bits(tid):
+    n_rows, n_cols = 512, 14336
+    W = synth.make_weights(tid, n_rows, n_cols, seed=5)
+    x = synth.make_activation(n_cols, seed=6)
+    dW, dx, dy = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(x), qlinear.DevBuf(n_rows * 4)
+    outs = []
+    for _ in range(3):
+        qlinear.gemv_dev(tid, dW, dx, dy, n_rows, n_cols)
+        qlinear.sync()
+        outs.append(dy.to_numpy(np.float32, (n_rows,)).copy())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
