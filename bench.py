@@ -581,7 +581,10 @@ def main():
         shapes = [("q4_K", Q4K, 4096, 4096), ("q4_K", Q4K, 4096, 14336), ("q8_0", synth.GGML_Q8_0, 4096, 4096),
                   ("q5_K", synth.GGML_Q5_K, 4096, 4096), ("iq4_nl", synth.GGML_IQ4_NL, 14336, 4096),
                   ("iq2_xxs", synth.GGML_IQ2_XXS, 4096, 14336), ("iq3_s", synth.GGML_IQ3_S, 4096, 14336),
-                  ("q6_K", synth.GGML_Q6_K, 151936, 4096)]
+                  ("q6_K", synth.GGML_Q6_K, 151936, 4096),
+                  # down projections whose rows run as column ranges or start off the 16-byte grid
+                  ("q6_K", synth.GGML_Q6_K, 4096, 14336), ("q6_K", synth.GGML_Q6_K, 4096, 11008),
+                  ("q4_K", Q4K, 8192, 28672), ("q5_K", synth.GGML_Q5_K, 3584, 18944)]
         gemv = {}
         for tname, tid, r, c in shapes:
             st = max(20, args.steps // 8)

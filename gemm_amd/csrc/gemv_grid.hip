@@ -241,7 +241,7 @@ template <> struct GridFmt<T_IQ3_S> {
 
 template <uint32_t T, int NKC>
 __global__ void __launch_bounds__(kWaves * 64)
-gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg) {
+gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes) {
     using F = GridFmt<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
@@ -258,7 +258,6 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
     if (rows_here > rows_per_wg) rows_here = rows_per_wg;
     const int n_lrows = rows_here * n_mats_here;
     const int n_rg = (n_lrows + 15) >> 4;
-    const size_t row_bytes = (size_t)n_sb * F::kBlock;
     const int n_kc = wv < n_sb ? ((n_sb - wv + 15) >> 4) : 0; /* this wave's super-blocks: wv, wv+16, ... */
 
     /* LDS: x scratch per wave, the grid and the sign masks at addresses the compiler knows (a lookup is then a
@@ -476,14 +475,16 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
 namespace {
 
 template <uint32_t T>
-bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err) {
+bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err,
+                size_t row_stride) {
     const int n_sb = n_cols / 256;
     /* rows of more than 4096 elements: up to there the v_dot4 kernel (gemv_int.hip) measured faster (both wait
      * for the table lookups; this one saves its vector instructions where x has to be prepared for few rows) */
     if (n_cols % 256 != 0 || n_sb <= 16 || n_sb > 16 * kMaxKc || ((uintptr_t)x & 15)) return false;
-    /* rows start on even addresses (even block sizes); the loads want the matrices dword-aligned at least */
+    /* the loads want even addresses (block sizes are even) */
     for (int m = 0; m < job.n_mat; m++)
-        if ((uintptr_t)job.W[m] & 3) return false;
+        if ((uintptr_t)job.W[m] & 1) return false;
+    if (row_stride & 1) return false;
     const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     if (n_rows == 0) return false;
@@ -493,7 +494,8 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = (size_t)rows_per_wg * n_mats_here * kWaves * 4; /* the partial sums; the rest is static */
     const JobView view = job_view(job);
-    hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg);
+    hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg,
+                       row_stride ? row_stride : (size_t)n_sb * GridFmt<T>::kBlock);
     *err = hipGetLastError();
     return true;
 }
@@ -501,12 +503,12 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 }  // namespace
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
-                      hipError_t *err) {
+                      hipError_t *err, size_t row_stride) {
     *err = hipSuccess;
     switch (type) {
-    case T_IQ2_XXS: return grid_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ3_XXS: return grid_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ3_S: return grid_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err);
+    case T_IQ2_XXS: return grid_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ3_XXS: return grid_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ3_S: return grid_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }

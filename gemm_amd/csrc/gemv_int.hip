@@ -41,11 +41,13 @@ template <int CTRL> __device__ __forceinline__ uint32_t dppu(uint32_t v) {
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) { return __builtin_amdgcn_sdot4((int)a, (int)b, c, false); }
 __device__ __forceinline__ uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_udot4(a, b, c, false); }
 
-/* n dwords starting at any byte offset of a 16-byte aligned LDS image, read as aligned dwords and
- * funnel-shifted (misaligned LDS reads stall the LDS pipeline); touches up to 4 bytes past the end */
+/* n dwords starting at any byte of an LDS image (img itself may sit at any byte too), read as aligned dwords
+ * and funnel-shifted (misaligned LDS reads stall the LDS pipeline); touches up to 4 bytes past the end */
 template <int N> __device__ __forceinline__ void ld_dwords_at(const uint8_t *img, int off, uint32_t (&out)[N]) {
-    const uint32_t *q = reinterpret_cast<const uint32_t *>(img + (off & ~3));
-    const uint32_t sh = (uint32_t)(off & 3) * 8u;
+    const uint8_t *p = img + off;
+    const uint32_t mis = (uint32_t)(uintptr_t)p & 3u;
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(p - mis);
+    const uint32_t sh = mis * 8u;
     uint32_t prev = q[0];
 #pragma unroll
     for (int i = 0; i < N; i++) {
@@ -545,11 +547,14 @@ template <typename F> __device__ __forceinline__ float group_dot(const Codes &cd
  * for all rows; NG == 0: any row length, the planes are read from LDS for every row */
 template <uint32_t T, int NG>
 __global__ void __launch_bounds__(NG > 2 ? 512 : 1024)
-gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int row_bytes, int depth, int rows_per_wg) {
+gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int row_bytes, int n_chunks, size_t row_stride,
+                int depth, int rows_per_wg) {
     using F = IntFmt<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     /* LDS map: x groups [n_cols/32][28 dwords] | raw x [n_cols] floats | codebook and sign masks of the grid
-     * formats | row images [waves][depth][row_bytes] */
+     * formats | row images [waves][depth][16 n_chunks]. A row (row_bytes bytes from any even address) is copied as
+     * the n_chunks aligned 16-byte pieces from the one that holds its first byte on; its image starts that many
+     * bytes into the copy */
     const int n_groups = n_cols >> 5;
     uint32_t *planes = reinterpret_cast<uint32_t *>(lds);
     const float4 *xraw = reinterpret_cast<const float4 *>(planes + n_groups * kGroupDw);
@@ -574,25 +579,33 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
             job_locate(job, row0 + wv + i * n_waves, Wm, ym, r);
         }
     };
-    const int n_chunks = row_bytes >> 4;
+    const int image_bytes = n_chunks << 4;
     const int loads_per_row = (n_chunks + 63) >> 6;
-    uint8_t *my_images = images + (size_t)wv * depth * row_bytes;
+    uint8_t *my_images = images + (size_t)wv * depth * image_bytes;
     const uint32_t my_images_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)my_images;
-    /* Row i of this wave -> image i % depth; data goes HBM -> LDS at M0 + 16*lane. The loads are
-     * written as instructions and waited for by hand (the compiler would wait for all of them
-     * before any LDS access). Nothing else in this kernel uses M0. */
-    auto issue = [&](int i) {
+    auto row_address = [&](int i) {
         const uint8_t *Wm;
         float *ym;
         int r;
         locate(i, Wm, ym, r);
-        const uint4 *gp = reinterpret_cast<const uint4 *>(Wm + (size_t)r * row_bytes);
-        const uint32_t img = my_images_lds + (uint32_t)((i % depth) * row_bytes);
+        return Wm + (size_t)r * row_stride;
+    };
+    /* Row i of this wave -> image i % depth; data goes HBM -> LDS at M0 + 16*lane. The loads are
+     * written as instructions and waited for by hand (the compiler would wait for all of them
+     * before any LDS access). Nothing else in this kernel uses M0. Every row takes the same number of
+     * instructions: lanes past the row's last piece fetch that piece again (their LDS slots lie behind the row). */
+    auto issue = [&](int i) {
+        const uint8_t *row = row_address(i);
+        const uint32_t delta = (uint32_t)(uintptr_t)row & 15u;
+        const uint4 *gp = reinterpret_cast<const uint4 *>(row - delta);
+        const int last_piece = (int)((delta + (uint32_t)row_bytes + 15u) >> 4) - 1;
+        const uint32_t img = my_images_lds + (uint32_t)((i % depth) * image_bytes);
         for (int c0 = 0; c0 < n_chunks; c0 += 64) {
             const uint32_t m0v = __builtin_amdgcn_readfirstlane(img + 16u * (uint32_t)c0);
+            const int piece = c0 + lane < last_piece ? c0 + lane : last_piece;
             if (c0 + lane < n_chunks)
                 asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt"
-                             : : "v"(gp + c0 + lane), "s"(m0v) : "memory");
+                             : : "v"(gp + piece), "s"(m0v) : "memory");
         }
     };
 
@@ -691,7 +704,7 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
     float gate_value = 0.0f;
     for (int i = 0; i < my_rows; i++) {
         wait_vm_at_most((issued - i - 1) * loads_per_row);
-        const uint8_t *img = my_images + (size_t)(i % depth) * row_bytes;
+        const uint8_t *img = my_images + (size_t)(i % depth) * image_bytes + ((uint32_t)(uintptr_t)row_address(i) & 15u);
         float acc = 0.0f;
         if (NG > 0) {
 #pragma unroll
@@ -727,13 +740,23 @@ gemv_int_kernel(const JobView job, const float *__restrict__ x, int n_cols, int 
 }
 
 template <uint32_t T>
-bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err) {
+bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err, size_t row_stride) {
     int be, bb;
     type_geometry(T, &be, &bb);
     const size_t row_bytes = (size_t)(n_cols / be) * bb;
-    if (n_cols > 16384 || (n_cols & 31) || (n_cols % be) || (row_bytes & 15) || row_bytes > 8192) return false;
-    for (int m = 0; m < job.n_mat; m++)
-        if ((uintptr_t)job.W[m] & 15) return false;
+    if (n_cols > 16384 || (n_cols & 31) || (n_cols % be) || row_bytes > 8192) return false;
+    if (row_stride == 0) row_stride = row_bytes; /* rows that are a column range of longer ones keep those rows' pitch */
+    /* rows on 16-byte boundaries are copied as they are; rows at other (even) addresses with the 16-byte piece
+     * that holds their first byte and the one that holds their last */
+    bool on16 = (row_stride & 15) == 0 && (row_bytes & 15) == 0;
+    for (int m = 0; m < job.n_mat; m++) on16 = on16 && ((uintptr_t)job.W[m] & 15) == 0;
+    if (!on16) {
+        if ((bb & 1) || (row_stride & 1)) return false; /* the 16-bit fields want even addresses */
+        for (int m = 0; m < job.n_mat; m++)
+            if ((uintptr_t)job.W[m] & 1) return false;
+    }
+    const int n_chunks = (int)((row_bytes + (on16 ? 0 : 14) + 15) >> 4);
+    const size_t image_bytes = (size_t)n_chunks * 16;
     if ((uintptr_t)x & 15) return false;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     const size_t x_bytes = (size_t)(n_cols >> 5) * kGroupDw * 4 + (size_t)n_cols * 4 + (size_t)kAuxBytes<T>;
@@ -743,15 +766,15 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
      * seven groups for all its rows (read from LDS for every row they are what the kernel waits for) */
     const bool wide = IntGrid<T>::kBytes > 0 && n_groups > 128 && n_groups <= 448;
     int waves = wide ? 8 : 16, depth = 2;
-    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) depth = 1;
-    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) { waves = 8; depth = 2; }
-    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) depth = 1;
-    if (x_bytes + (size_t)waves * depth * row_bytes > lds_cap) return false;
-    if ((size_t)((row_bytes >> 4) + 63) / 64 * depth > 15) return false; /* the hand-placed waits count to 15 */
+    if (x_bytes + (size_t)waves * depth * image_bytes > lds_cap) depth = 1;
+    if (x_bytes + (size_t)waves * depth * image_bytes > lds_cap) { waves = 8; depth = 2; }
+    if (x_bytes + (size_t)waves * depth * image_bytes > lds_cap) depth = 1;
+    if (x_bytes + (size_t)waves * depth * image_bytes > lds_cap) return false;
+    if ((size_t)(n_chunks + 63) / 64 * depth > 15) return false; /* the hand-placed waits count to 15 */
     int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
     if (rows_per_wg < 1) rows_per_wg = 1;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
-    const size_t lds_bytes = x_bytes + (size_t)waves * depth * row_bytes + 16; /* + slack for the funnel-shift reads */
+    const size_t lds_bytes = x_bytes + (size_t)waves * depth * image_bytes + 16; /* + slack for the funnel-shift reads */
     auto launch = [&](auto kernel, OnceFlag &raised) {
         if (!raised.is_set()) {
             *err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -759,7 +782,7 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
             raised.set();
         }
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds_bytes, stream, job_view(job), x, n_cols,
-                           (int)row_bytes, depth, rows_per_wg);
+                           (int)row_bytes, n_chunks, row_stride, depth, rows_per_wg);
         *err = hipGetLastError();
     };
     static OnceFlag raised[4];
@@ -772,27 +795,36 @@ bool int_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStre
 
 }  // namespace
 
+bool gemv_int_takes_any_even_address(uint32_t type) {
+    switch (type) {
+    case T_Q8_0: case T_Q4_0: case T_Q4_1: case T_Q5_0: case T_Q5_1: case T_Q5_K: case T_Q6_K: case T_Q2_K: case T_Q3_K:
+    case T_IQ4_NL: case T_IQ4_XS: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: case T_IQ2_XS: case T_IQ2_S:
+        return true;
+    default: return false; /* MXFP4 (17-byte blocks) and the formats of the other kernels */
+    }
+}
+
 bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
-                     hipError_t *err) {
+                     hipError_t *err, size_t row_stride) {
     *err = hipSuccess;
     switch (type) {
-    case T_Q8_0: return int_typed<T_Q8_0>(job, x, n_cols, n_cu, stream, err);
-    case T_Q4_0: return int_typed<T_Q4_0>(job, x, n_cols, n_cu, stream, err);
-    case T_Q4_1: return int_typed<T_Q4_1>(job, x, n_cols, n_cu, stream, err);
-    case T_Q5_0: return int_typed<T_Q5_0>(job, x, n_cols, n_cu, stream, err);
-    case T_Q5_1: return int_typed<T_Q5_1>(job, x, n_cols, n_cu, stream, err);
-    case T_Q5_K: return int_typed<T_Q5_K>(job, x, n_cols, n_cu, stream, err);
-    case T_Q6_K: return int_typed<T_Q6_K>(job, x, n_cols, n_cu, stream, err);
-    case T_Q2_K: return int_typed<T_Q2_K>(job, x, n_cols, n_cu, stream, err);
-    case T_Q3_K: return int_typed<T_Q3_K>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ4_NL: return int_typed<T_IQ4_NL>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ4_XS: return int_typed<T_IQ4_XS>(job, x, n_cols, n_cu, stream, err);
-    case T_MXFP4: return int_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ2_XXS: return int_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ3_XXS: return int_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ3_S: return int_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ2_XS: return int_typed<T_IQ2_XS>(job, x, n_cols, n_cu, stream, err);
-    case T_IQ2_S: return int_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err);
+    case T_Q8_0: return int_typed<T_Q8_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q4_0: return int_typed<T_Q4_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q4_1: return int_typed<T_Q4_1>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q5_0: return int_typed<T_Q5_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q5_1: return int_typed<T_Q5_1>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q5_K: return int_typed<T_Q5_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q6_K: return int_typed<T_Q6_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q2_K: return int_typed<T_Q2_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q3_K: return int_typed<T_Q3_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ4_NL: return int_typed<T_IQ4_NL>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ4_XS: return int_typed<T_IQ4_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_MXFP4: return int_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ2_XXS: return int_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ3_XXS: return int_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ3_S: return int_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ2_XS: return int_typed<T_IQ2_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ2_S: return int_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }

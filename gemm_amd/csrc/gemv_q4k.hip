@@ -67,7 +67,7 @@ struct XOperand {
 
 template <int NKC>
 __global__ void __launch_bounds__(kWaves * 64)
-gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg) {
+gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -83,7 +83,6 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
     if (rows_here > rows_per_wg) rows_here = rows_per_wg;
     const int n_lrows = rows_here * n_mats_here;
     const int n_rg = (n_lrows + 15) >> 4;
-    const size_t row_bytes = (size_t)n_sb * 144;
     const int n_kc = wv < n_sb ? ((n_sb - wv + 15) >> 4) : 0; /* this wave's super-blocks: wv, wv+16, ... */
 
     /* LDS map: x scratch [kWaves][kXScratch] | partial sums [rows][kWaves] */
@@ -305,7 +304,7 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
     }
 }
 
-hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu) {
+hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu, size_t row_stride) {
     const int n_sb = n_cols / 256;
     if (n_sb > 16 * kMaxKc || n_sb < 1) return hipErrorInvalidValue;
     const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
@@ -317,12 +316,13 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = (size_t)kWaves * kXScratch + (size_t)rows_per_wg * n_mats_here * kWaves * 4;
     const JobView view = job_view(job);
+    if (row_stride == 0) row_stride = (size_t)n_sb * 144; /* rows that are a column range of longer ones keep those rows' pitch */
     if (n_sb <= 16)
         hipLaunchKernelGGL(gemv_q4k_kernel<1>, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb,
-                           rows_per_wg);
+                           rows_per_wg, row_stride);
     else
         hipLaunchKernelGGL(gemv_q4k_kernel<kMaxKc>, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb,
-                           rows_per_wg);
+                           rows_per_wg, row_stride);
     return hipGetLastError();
 }
 

@@ -442,7 +442,7 @@ QLIN_GRID(T_IQ1_M, qlin_iq1s_grid, true)
 template <uint32_t T>
 __global__ void __launch_bounds__(1024)
 gemv_stream_kernel(const JobView job, const float *__restrict__ x, int n_cols, int row_bytes, int image_bytes,
-                   int depth, int rows_per_wg) {
+                   size_t row_stride, int depth, int rows_per_wg) {
     using C = Codec<T>;
     constexpr int GPB = C::BE / 8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -487,7 +487,7 @@ gemv_stream_kernel(const JobView job, const float *__restrict__ x, int n_cols, i
         float *ym;
         int r;
         locate(i, Wm, ym, r);
-        const uint4 *g = reinterpret_cast<const uint4 *>(Wm + (size_t)r * row_bytes);
+        const uint4 *g = reinterpret_cast<const uint4 *>(Wm + (size_t)r * row_stride);
         const uint32_t img = my_images_lds + (uint32_t)((i % depth) * image_bytes);
         for (int c0 = 0; c0 < n_chunks; c0 += 64) {
             const uint32_t m0v = __builtin_amdgcn_readfirstlane(img + 16u * (uint32_t)c0);
@@ -579,9 +579,12 @@ gemv_stream_kernel(const JobView job, const float *__restrict__ x, int n_cols, i
 }
 
 template <uint32_t T>
-bool stream_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err) {
+bool stream_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err,
+                  size_t row_stride) {
     const size_t row_bytes = (size_t)(n_cols / Codec<T>::BE) * Codec<T>::BB;
     if (n_cols > 16384 || (n_cols & 31) || (row_bytes & 15) || row_bytes > 8192) return false;
+    if (row_stride == 0) row_stride = row_bytes; /* rows that are a column range of longer ones keep those rows' pitch */
+    if (row_stride & 15) return false;
     for (int m = 0; m < job.n_mat; m++)
         if ((uintptr_t)job.W[m] & 15) return false;
     if ((uintptr_t)x & 15) return false;
@@ -608,7 +611,7 @@ bool stream_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipS
     }
     const JobView view = job_view(job);
     hipLaunchKernelGGL((gemv_stream_kernel<T>), dim3(grid), dim3(waves * 64), lds_bytes, stream, view, x, n_cols,
-                       (int)row_bytes, (int)row_bytes, depth, rows_per_wg);
+                       (int)row_bytes, (int)row_bytes, row_stride, depth, rows_per_wg);
     *err = hipGetLastError();
     return true;
 }
@@ -616,10 +619,10 @@ bool stream_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipS
 }  // namespace
 
 bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
-                        hipStream_t stream, hipError_t *err) {
+                        hipStream_t stream, hipError_t *err, size_t row_stride) {
     *err = hipSuccess;
     switch (type) {
-#define QLIN_CASE(TT) case TT: return stream_typed<TT>(job, x, n_cols, n_cu, stream, err);
+#define QLIN_CASE(TT) case TT: return stream_typed<TT>(job, x, n_cols, n_cu, stream, err, row_stride);
     QLIN_FOR_EACH_BLOCK_TYPE(QLIN_CASE)
     QLIN_FOR_EACH_DENSE_TYPE(QLIN_CASE)
 #undef QLIN_CASE

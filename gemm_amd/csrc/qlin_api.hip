@@ -236,21 +236,74 @@ int weights_on_device_locked(const void *host, size_t bytes, DevBuf &buf, const 
     return QLIN_OK;
 }
 
-/* matvec dispatch: the tuned Q4_K kernel where its shape rules hold, else the integer-dot kernel
- * (formats with small integer codes), else the streaming float kernel, else (ragged or oversized
- * shapes, unaligned pointers) the plain kernel */
+/* the tuned kernels, on packed rows (row_stride 0) or on a column range of longer rows; false: none takes the shape */
+static bool launch_gemv_tuned(uint32_t type, const GemvJob &job, const float *x, int n_cols, size_t row_stride,
+                              hipStream_t s, hipError_t *err) {
+    bool w_aligned = true;
+    for (int m = 0; m < job.n_mat; m++) w_aligned = w_aligned && aligned(job.W[m], 16);
+    if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && w_aligned && aligned(x, 16)) {
+        *err = launch_gemv_q4k(job, x, n_cols, s, g.n_cu, row_stride);
+        return true;
+    }
+    if (launch_gemv_grid(type, job, x, n_cols, g.n_cu, s, err, row_stride)) return true;
+    if (launch_gemv_int(type, job, x, n_cols, g.n_cu, s, err, row_stride)) return true;
+    return launch_gemv_stream(type, job, x, n_cols, g.n_cu, s, err, row_stride);
+}
+
+/* Rows too long for the tuned kernels (more than 16384 elements or 8 KB) as column ranges of at most `cap`
+ * elements, each a launch of its own over the full rows' pitch: the first with the job's mode, the others adding
+ * to y in stream order. 0: the type or the shape does not split that way. */
+static int column_range(uint32_t type, int n_cols) {
+    int be, bb;
+    type_geometry(type, &be, &bb);
+    /* a range is whole 256-element groups; for the kernels that want rows on 16-byte boundaries also so many
+     * blocks that their bytes are a multiple of 16 */
+    const bool any_address = gemv_int_takes_any_even_address(type);
+    int granule = be;
+    while (granule % 256 != 0 || (!any_address && ((size_t)(granule / be) * bb) % 16 != 0)) granule += be;
+    if (n_cols % granule != 0) return 0;
+    /* Q4_K: what its kernel takes; the others: the longest range whose x stays in the lanes' registers */
+    const int cap = type == T_Q4_K ? 16384 : 4096;
+    int range = cap / granule * granule;
+    while (range > 0 && (size_t)(range / be) * bb > 8192) range -= granule;
+    if (range <= 0) return 0;
+    const int n_ranges = (n_cols + range - 1) / range;
+    range = ((n_cols + n_ranges - 1) / n_ranges + granule - 1) / granule * granule; /* ranges of about equal length */
+    return range;
+}
+
+/* shape-based choice: tuned Q4_K kernel, else the matrix-instruction kernel for long rows of the codebook formats,
+ * else the integer-dot kernel (formats with small integer codes), else the streaming float kernel, else - rows
+ * too long for those - the same kernels over column ranges, else (ragged shapes, unaligned pointers) the plain kernel */
 hipError_t dispatch_gemv_job(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t s) {
     if ((job.mode == kSiluMul ? job.n_rows[0] : job.total_rows()) == 0) return hipSuccess;
     bool w_aligned = true;
     for (int m = 0; m < job.n_mat; m++) w_aligned = w_aligned && aligned(job.W[m], 16);
     if ((type == T_F16 || type == T_BF16 || type == T_F32) && (n_cols % 8 != 0 || !w_aligned))
         return launch_gemv_dense_ragged(type, job, x, n_cols, s); /* rows that are not whole 16-byte groups */
-    if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && w_aligned && aligned(x, 16))
-        return launch_gemv_q4k(job, x, n_cols, s, g.n_cu);
     hipError_t err;
-    if (launch_gemv_grid(type, job, x, n_cols, g.n_cu, s, &err)) return err;
-    if (launch_gemv_int(type, job, x, n_cols, g.n_cu, s, &err)) return err;
-    if (launch_gemv_stream(type, job, x, n_cols, g.n_cu, s, &err)) return err;
+    if (launch_gemv_tuned(type, job, x, n_cols, 0, s, &err)) return err;
+    int be, bb;
+    type_geometry(type, &be, &bb);
+    const size_t row_bytes = (size_t)(n_cols / be) * bb;
+    const int range = (job.mode != kSiluMul && w_aligned && aligned(x, 16) && n_cols % be == 0 &&
+                       (row_bytes % 16 == 0 || gemv_int_takes_any_even_address(type)))
+                          ? column_range(type, n_cols) : 0;
+    if (range > 0 && range < n_cols) {
+        for (int c0 = 0; c0 < n_cols; c0 += range) {
+            GemvJob part = job;
+            for (int m = 0; m < job.n_mat; m++) part.W[m] = (const uint8_t *)job.W[m] + (size_t)(c0 / be) * bb;
+            if (c0 > 0) part.mode = kAdd;
+            const int cols = n_cols - c0 < range ? n_cols - c0 : range;
+            if (!launch_gemv_tuned(type, part, x + c0, cols, row_bytes, s, &err)) {
+                /* every range has the shape of the first or is shorter: cannot happen once the first was taken */
+                if (c0 == 0) return launch_gemv_generic(type, job, x, n_cols, s);
+                return hipErrorInvalidValue;
+            }
+            if (err != hipSuccess) return err;
+        }
+        return hipSuccess;
+    }
     return launch_gemv_generic(type, job, x, n_cols, s);
 }
 hipError_t dispatch_gemv(uint32_t type, const void *W, const float *x, float *y, int n_rows,

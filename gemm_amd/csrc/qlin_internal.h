@@ -65,17 +65,22 @@ hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x
 hipError_t launch_gemv_dense_ragged(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t stream);
 /* streaming matvec for every type; returns false if the shape rules of gemv_stream.hip do not
  * hold (nothing was launched), else true with the launch status in *err */
+/* row_stride (all four kernels below): bytes between the rows of a matrix; 0 = the rows are packed. Anything else
+ * runs the kernel over a column range of longer rows (W then points at the range's first block of row 0). */
 bool launch_gemv_stream(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
-                        hipStream_t stream, hipError_t *err);
+                        hipStream_t stream, hipError_t *err, size_t row_stride = 0);
 /* integer-dot matvec (gemv_int.hip) for the formats it covers; same contract as launch_gemv_stream */
 bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
-                     hipStream_t stream, hipError_t *err);
+                     hipStream_t stream, hipError_t *err, size_t row_stride = 0);
+/* the formats whose rows launch_gemv_int reads from any even address (the others want 16-byte boundaries) */
+bool gemv_int_takes_any_even_address(uint32_t type);
 /* matrix-instruction matvec for the codebook formats IQ2_XXS, IQ3_XXS and IQ3_S (gemv_grid.hip): n_cols % 256 == 0,
  * n_cols <= 16384; same contract as launch_gemv_stream */
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
-                      hipStream_t stream, hipError_t *err);
+                      hipStream_t stream, hipError_t *err, size_t row_stride = 0);
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
-hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu);
+hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu,
+                           size_t row_stride = 0);
 
 /* Y[t*ldy + r] = dot(W[r,:], X[t*ldx..]) in fp32 */
 hipError_t launch_gemm_f32(uint32_t type, const void *W, const float *X, float *Y, int n_rows,
