@@ -243,6 +243,28 @@ def test_grouped_ffn_down_kernel_variants(oracle, types, n_embd, n_ff):
         assert rel_l2(got[t], want[t]) <= 10 * DESIGNED, t
 
 
+@pytest.mark.parametrize("types", [(Q4K, Q4K, Q4K), (Q4K, Q4K, Q6K), (Q6K, Q6K, Q6K), (Q8_0, Q8_0, Q8_0)],
+                         ids=["q4k", "q4k_q4k_q6k", "q6k", "q8_0"])
+@pytest.mark.parametrize("n_tok", [1, 2, 7, 8, 9, 17])
+def test_grouped_ffn_fewer_pairs_than_experts(oracle, types, n_tok):
+    """32 experts, top-4: up to two pairs per expert (16 tokens) the expert kernels look their expert up in the list
+    of routed ones and the launch covers no more experts than pairs; 17 tokens take the launch over all experts.
+    One and two tokens also take the 32-row down kernel instead of the walk."""
+    n_expert, n_embd, n_ff, k = 32, 512, 256, 4
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=970, types=types)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=971 + n_tok, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=972 + n_tok), k)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
+    assert rel_l2(got, want) <= DESIGNED
+    for t in range(n_tok):
+        assert rel_l2(got[t], want[t]) <= 10 * DESIGNED, t
+    # the highest and the lowest expert routed, everything between unused
+    idx2 = np.tile(np.array([[n_expert - 1, 0, 5, 6]], np.int32), (n_tok, 1))
+    got2 = run_ffn(gate, up, down, Xb, idx2, w, n_embd, n_ff, n_expert, types=types)
+    assert rel_l2(got2, numpy_ffn(oracle, gate, up, down, Xb, idx2, w, n_embd, n_ff, types=types)) <= DESIGNED
+
+
 def test_grouped_ffn_mixed_formats_many_tokens_per_expert_and_ragged_shapes(oracle):
     """two experts, 50 tokens: 8-token passes of the any-format kernel with a ragged tail; n_ff = 96 is not a
     multiple of the matrix-core tiles, so Q4_K gate/up cannot be used and Q8_0 (32-element blocks) is"""
