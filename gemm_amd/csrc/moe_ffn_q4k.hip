@@ -1072,6 +1072,90 @@ moe_down_kq_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__rest
     }
 }
 
+/* ---- 3c. down for experts in those formats when K is longer than the walk's eight super-blocks (n_ff above 2048):
+ * 16 rows per workgroup, K split over at most four waves (a wave takes super-blocks wv, wv + 4, ...), eight tokens
+ * per pass, one image per wave ---- */
+template <typename F>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3)))
+moe_down_kq_long_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
+                        const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
+                        float *__restrict__ part, int n_embd, int n_ff, const int32_t *__restrict__ routed) {
+    constexpr int kImageRow = 16 * F::kRowChunks;
+    constexpr int kImage = 16 * kImageRow + 16;
+    constexpr int kChunks = 16 * F::kRowChunks, kImageLoads = (kChunks + 63) / 64;
+    extern __shared__ __attribute__((aligned(16))) float red[];
+    const int e = block_expert(routed);
+    if (e < 0) return;
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int row0 = blockIdx.x * 16;
+    const int first = offsets[e], cnt = offsets[e + 1] - first;
+    if (cnt == 0) return;
+    const int j = lane & 15, kg = lane >> 4;
+    const int n_sb = n_ff >> 8;
+    const int row_bytes = n_sb * F::kBlock;
+    /* 16 * row_bytes is a multiple of 16, so every row group starts on a 16-byte boundary like the tensor */
+    const uint8_t *w0 = uniform_ptr(down + ((size_t)e * n_embd + row0) * row_bytes);
+    /* LDS: red [waves][8 tokens][16 rows] floats | images [waves][16 rows][chunks + slack] */
+    uint8_t *img = reinterpret_cast<uint8_t *>(red + n_waves * 128) + wv * kImage;
+    const uint32_t img_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void *)img;
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int t0 = 0; t0 < cnt; t0 += 8) {
+        const int n_live = cnt - t0 < 8 ? cnt - t0 : 8;
+        const int tok = j & 7;
+        const bool live = (kg >> 1) == (j >> 3) && tok < n_live;
+        const size_t at_a = (size_t)(first + t0 + (tok < n_live ? tok : 0)) * n_ff + 8 * kg;
+        f32x4 acc = zero;
+        for (int sb = wv; sb < n_sb; sb += n_waves) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* reads of the previous image have returned */
+#pragma unroll
+            for (int i = 0; i < kImageLoads; i++) {
+                const int t = 64 * i + lane;
+                int R = t / F::kRowChunks;
+                const int c = t - F::kRowChunks * R;
+                R = R < 16 ? R : 15;
+                const int at = R * row_bytes + sb * F::kBlock;
+                const uint32_t off = (uint32_t)(at & ~15) + 16u * (uint32_t)c;
+                /* a chunk that lies wholly behind the block is not read: behind the tensor's last block there may be nothing */
+                const bool wanted = t < kChunks && 16 * c < (at & 15) + F::kBlock;
+                const uint32_t m0v = __builtin_amdgcn_readfirstlane(img_lds + 1024u * (uint32_t)i);
+                if (wanted)
+                    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(w0), "s"(m0v) : "memory");
+            }
+            u32x4 a_hi[8], a_lo[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                u32x4 vh = {0u, 0u, 0u, 0u}, vl = {0u, 0u, 0u, 0u};
+                if (live) {
+                    vh = *(const u32x4 *)(h_hi + at_a + (size_t)sb * 256 + 32 * u);
+                    vl = *(const u32x4 *)(h_lo + at_a + (size_t)sb * 256 + 32 * u);
+                }
+                a_hi[u] = vh;
+                a_lo[u] = vl;
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* image and activations have landed */
+            const int blk_at = j * kImageRow + ((j * row_bytes + sb * F::kBlock) & 15);
+            const u32x4 *const aa[2] = {a_hi, a_lo};
+            F::template math<2>(img, blk_at, kg, aa, acc);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[v] += __shfl_xor(acc[v], 32, 64);
+        if (kg < 2) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[(wv * 8 + 4 * kg + v) * 16 + j] = acc[v];
+        }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < n_live * 16; idx += blockDim.x) {
+            const int jj = idx & 15, t = idx >> 4;
+            float dsum = 0.0f;
+            for (int w = 0; w < n_waves; w++) dsum += red[(w * 8 + t) * 16 + jj];
+            part[(size_t)(first + t0 + t) * n_embd + row0 + jj] = dsum;
+        }
+        __syncthreads();
+    }
+}
+
 /* ---- 2c. gate and up for Q6_K experts: 16 rows of each per workgroup, K split over at most four waves (a wave
  * takes super-blocks wv, wv + 4, ...), eight tokens per pass, the arithmetic of the Q6_K down kernel ---- */
 template <typename F>
@@ -1629,14 +1713,29 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         hipLaunchKernelGGL((moe_down_walk_kernel<DRT, DNT>), dim3(n_embd / (16 * DRT * DNT), grid_y), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 2 * 16 * kQ4KBlock), stream,
                            (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff, routed);
-    } else if (!fast_dn && kq_type(type_down) && n_ff % 256 == 0 && n_ff / 256 <= 8 && n_embd % (16 * kKqWalkGroups) == 0 &&
-               ((uintptr_t)down & 15) == 0) {
+    } else if (!fast_dn && !few_tiles && kq_type(type_down) && n_ff % 256 == 0 && n_ff / 256 <= 8 &&
+               n_embd % (16 * kKqWalkGroups) == 0 && ((uintptr_t)down & 15) == 0) {
         const int waves = n_ff / 256;
         auto go = [&](auto tag) {
             using F = decltype(tag);
             hipLaunchKernelGGL((moe_down_kq_walk_kernel<F, kKqWalkGroups>), dim3(n_embd / (16 * kKqWalkGroups), grid_y),
                                dim3(64 * waves), (size_t)waves * (128 * 4 + 2 * (16 * 16 * F::kRowChunks + 16)), stream,
                                (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff, routed);
+        };
+        switch (type_down) {
+        case T_Q6_K: go(KqQ6K()); break;
+        case T_Q5_K: go(KqQ5K()); break;
+        case T_Q3_K: go(KqQ3K()); break;
+        case T_Q2_K: go(KqQ2K()); break;
+        default: go(KqQ8_0()); break;
+        }
+    } else if (!fast_dn && kq_type(type_down) && n_ff % 256 == 0 && n_embd % 16 == 0 && ((uintptr_t)down & 15) == 0) {
+        const int waves = n_ff / 256 < 4 ? n_ff / 256 : 4;
+        auto go = [&](auto tag) {
+            using F = decltype(tag);
+            hipLaunchKernelGGL((moe_down_kq_long_kernel<F>), dim3(n_embd / 16, grid_y), dim3(64 * waves),
+                               (size_t)waves * (128 * 4 + 16 * 16 * F::kRowChunks + 16), stream, (const uint8_t *)down, ws.h_hi,
+                               ws.h_lo, ws.offsets, ws.part, n_embd, n_ff, routed);
         };
         switch (type_down) {
         case T_Q6_K: go(KqQ6K()); break;

@@ -226,8 +226,14 @@ def test_grouped_ffn_every_block_format(oracle, type_id):
     ((synth.GGML_Q3_K, synth.GGML_Q3_K, synth.GGML_Q3_K), 768, 768),
     ((synth.GGML_Q2_K, synth.GGML_Q2_K, synth.GGML_Q3_K), 1024, 512),
     ((synth.GGML_Q2_K, synth.GGML_Q2_K, synth.GGML_Q2_K), 768, 768),
+    ((Q4K, Q4K, Q6K), 256, 2304),      # Q6_K down with nine super-blocks of K: the 16-row kernel that loops over K
+    ((Q8_0, Q8_0, Q8_0), 256, 4096),   # sixteen super-blocks over four waves
+    ((synth.GGML_Q5_K, synth.GGML_Q5_K, synth.GGML_Q5_K), 512, 2560),
+    ((synth.GGML_Q3_K, synth.GGML_Q3_K, synth.GGML_Q3_K), 256, 2304),
+    ((synth.GGML_Q2_K, synth.GGML_Q2_K, synth.GGML_Q2_K), 256, 2816),
 ], ids=["long_k", "rows_not_multiple_of_128", "walk", "q6k_down_3_waves", "q6k_down_2_waves", "q6k_down_fallback",
-        "q6k_gate_up_4_waves", "q6k_gate_up_3_waves", "q5k_q5k_q6k", "q5k", "q8_0", "q3k_q3k_q4k", "q3k", "q2k_q2k_q3k", "q2k"])
+        "q6k_gate_up_4_waves", "q6k_gate_up_3_waves", "q5k_q5k_q6k", "q5k", "q8_0", "q3k_q3k_q4k", "q3k", "q2k_q2k_q3k", "q2k",
+        "q6k_down_long_k", "q8_0_long_k", "q5k_long_k", "q3k_long_k", "q2k_long_k"])
 def test_grouped_ffn_down_kernel_variants(oracle, types, n_embd, n_ff):
     """the Q4_K down projection has two kernels: one row group of 32 per workgroup, and a walk over four
     groups with the next weight image in flight (K up to 2048, rows a multiple of 128); Q6_K down has a walk of
