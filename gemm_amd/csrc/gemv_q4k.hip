@@ -125,24 +125,20 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
         if (!(amax <= 3.0e38f)) down = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
         const int X[4] = {__float2int_rn(v.x * up), __float2int_rn(v.y * up), __float2int_rn(v.z * up),
                           __float2int_rn(v.w * up)};
-        int X1[4], X2[4], X3[4];
+        /* The four signed base-256 digits of X (X = 256*X1 + d0 with d0 = (int8)X, X1 = 256*X2 + d1, ...;
+         * the top one in [-64, 64]) are the bytes of (X + 0x00808080) ^ 0x00808080: adding 128 at a byte makes its
+         * digit unsigned and carries exactly when the digit is negative, the xor takes the 128 off again. */
+        uint32_t Z[4];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            X1[k] = (X[k] + 128) >> 8;  /* X = 256*X1 + d0, d0 = (int8)X */
-            X2[k] = (X1[k] + 128) >> 8; /* X1 = 256*X2 + d1 */
-            X3[k] = (X2[k] + 128) >> 8; /* X2 = 256*X3 + d2; d3 = X3 in [-64, 64] */
-        }
-        /* byte 0 of four values -> one dword (selector 0-3: second operand, 4-7: first, 0x0c: zero) */
-        auto pack = [](const int (&a)[4]) {
-            const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)a[1], (uint32_t)a[0], 0x0c0c0400u);
-            const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)a[3], (uint32_t)a[2], 0x0c0c0400u);
-            return __builtin_amdgcn_perm(p23, p01, 0x05040100u);
-        };
+        for (int k = 0; k < 4; k++) Z[k] = ((uint32_t)X[k] + 0x00808080u) ^ 0x00808080u;
+        /* byte transpose: plane j = byte j of Z[0..3] (selector 0-3: second operand, 4-7: first) */
+        const uint32_t lo01 = __builtin_amdgcn_perm(Z[1], Z[0], 0x05010400u), lo23 = __builtin_amdgcn_perm(Z[3], Z[2], 0x05010400u);
+        const uint32_t hi01 = __builtin_amdgcn_perm(Z[1], Z[0], 0x07030602u), hi23 = __builtin_amdgcn_perm(Z[3], Z[2], 0x07030602u);
         uint32_t *pl = reinterpret_cast<uint32_t *>(xs);
-        pl[lane] = pack(X3);       /* digit 3 (top) */
-        pl[64 + lane] = pack(X2);  /* digit 2 */
-        pl[128 + lane] = pack(X1); /* digit 1 */
-        pl[192 + lane] = pack(X);  /* digit 0 */
+        pl[lane] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);       /* digit 3 (top) */
+        pl[64 + lane] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  /* digit 2 */
+        pl[128 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u); /* digit 1 */
+        pl[192 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); /* digit 0 */
         if ((lane & 7) == 0) reinterpret_cast<float2 *>(xs + 1024)[lane >> 3] = make_float2(down, sum);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -236,8 +232,7 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
         }
         if (rg0 == 0) { /* x is prepared while the first blocks are on their way */
             v4f v = xr[0];
-#pragma unroll
-            for (int kk = 1; kk < NKC; kk++) v = kc == kk ? xr[kk] : v;
+            if (NKC > 1 && kc > 0) v = *reinterpret_cast<const v4f *>(x + (size_t)(16 * kc + wv) * 256 + 4 * lane);
             prepare(v, xo);
         }
 #pragma unroll
