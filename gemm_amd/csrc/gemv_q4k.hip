@@ -233,6 +233,10 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
         if (rg0 == 0) { /* x is prepared while the first blocks are on their way */
             v4f v = xr[0];
             if (NKC > 1 && kc > 0) v = *reinterpret_cast<const v4f *>(x + (size_t)(16 * kc + wv) * 256 + 4 * lane);
+            /* x is not looked at before this point: left alone, the compiler moves the first steps of the
+             * preparation (they do not change from one pass of the loops to the next) in front of the loops, and
+             * every wave then waits for x before it requests its first weights */
+            asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w) : : "memory");
             prepare(v, xo);
         }
 #pragma unroll
