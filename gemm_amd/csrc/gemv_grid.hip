@@ -282,11 +282,12 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
     auto row_pointer = [&](int rg) { /* this lane's row of row group rg (rows past the end: the last one, never stored) */
         int lr = 16 * rg + n;
         if (lr >= n_lrows) lr = n_lrows - 1;
-        /* matrix and row by selects, not branches: the lanes of a row group may sit in different matrices */
-        const int v = row0 + lr;
-        const bool in1 = paired ? lr >= rows_here : v >= job.n0, in2 = !paired && v >= job.n0 + job.n1;
-        const uint8_t *Wm = in2 ? job.W2 : in1 ? job.W1 : job.W0;
-        const int r = paired ? (in1 ? v - rows_here : v) : v - (in2 ? job.n0 + job.n1 : in1 ? job.n0 : 0);
+        /* by branches: a choice between the three matrix arguments by selects becomes a load from the argument
+         * block, with a full wait, in front of every weight request */
+        const uint8_t *Wm;
+        float *ym;
+        int r;
+        locate(lr, Wm, ym, r);
         return Wm + (size_t)r * row_bytes + (size_t)wv * F::kBlock;
     };
 
