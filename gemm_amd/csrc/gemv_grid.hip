@@ -1,6 +1,8 @@
 /*
- * gemv_grid.hip - batch-1 matvec for the codebook ("grid") formats IQ2_XXS, IQ3_XXS and IQ3_S on gfx950: the
- * inner products run on the 8-bit integer matrix instruction, the codebook and sign-mask lookups in LDS.
+ * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements on gfx950, for the codebook ("grid") formats
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K and Q8_0: the inner products run on the 8-bit integer matrix
+ * instruction; the grid formats look their codebook and sign masks up in LDS, the others build their codes in
+ * registers and read the x operand from LDS for every item.
  *
  * y[r] = sum over 32-element groups of scale(r, group) * (signed grid bytes . x_group)
  * (the decoders of common/ggml_dequant.h:2793-2816, :2916-2940 and :3022-3058 dotted with x).
@@ -44,12 +46,15 @@ typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 constexpr int kWaves = 16;        /* wavefronts per workgroup */
 constexpr int kMaxKc = 4;         /* super-blocks per wave: K <= 16384 */
 constexpr int kMaxRowsPerWg = 128;
-constexpr int kXScratch = 1088;   /* per wave: 3 digit planes x 256 B, 64 zero bytes, (at 1024) 8 x 2^(e-22) */
+constexpr int kXScratch = 1152;   /* per wave: 3 digit planes x 256 B, 128 zero bytes, (at 1024) 8 x 2^(e-22), (at 1056) 16 sums of 16 x */
 
-/* x operand of one super-block: A[s] for instruction s; scale[h] = 2^(e-22) of group 2 (lane/16) + h */
+/* x operand of one super-block: A[s] for instruction s. The other two things an item needs stay in the wave's
+ * scratch until the next super-block is prepared: meta[G] = 2^(e-22) of 32-element group G, meta[8 + S] = the sum
+ * of x over 16-element group S (formats with a constant offset per code). */
 struct XOperand {
-    v4i A[4];
-    float scale[2];
+    v4i A[4];             /* formats whose items keep LDS busy with table lookups hold the operand in registers */
+    const uint8_t *arows; /* the others read it per item: instruction s at arows + F::kStep * s (zeros for a dead lane) */
+    const float *meta;
 };
 
 template <int CTRL> __device__ __forceinline__ uint32_t dpp_movu(uint32_t v) {
@@ -116,6 +121,13 @@ template <uint32_t T> struct GridFmt;
  * eight-byte grid entry per index (common/ggml_dequant.h:2793-2816); 66-byte blocks */
 template <> struct GridFmt<T_IQ2_XXS> {
     static constexpr int kBlock = 66, kGridBytes = 2048, kDepth = 4;
+    static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
+    static constexpr int kStep = 16; /* bytes between the x rows of consecutive instructions */
+    static constexpr bool kAInRegs = true;
+    static constexpr int kPiece = 2; /* every piece a lane reads starts 2 (mod 4) bytes into the block */
+    static constexpr bool kSums = false;
+    /* lane group g takes elements [64 g, 64 g + 64) in order, 16 per instruction */
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
     __device__ static const uint32_t *grid_src() { return reinterpret_cast<const uint32_t *>(qlin_iq2xxs_grid); }
     struct Raw {
         Raw16 a; /* groups 2g, 2g+1: [indices, signs + scale] each */
@@ -127,7 +139,7 @@ template <> struct GridFmt<T_IQ2_XXS> {
         r.d = *reinterpret_cast<const uint16_t *>(blk);
         return r;
     }
-    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t) {
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t, int g) {
         uint32_t w[4];
         bytes16(r.a, sh, w);
         const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
@@ -144,7 +156,7 @@ template <> struct GridFmt<T_IQ2_XXS> {
                 const v4i b = {apply_signs(m0.x, s0.x), apply_signs(m0.y, s0.y), apply_signs(m1.x, s1.x), apply_signs(m1.y, s1.y)};
                 c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2 * h + q], b, c, 0, 0, 0);
             }
-            acc = fmaf(join_digits(c) * xo.scale[h], 0.5f + (float)(a1 >> 28), acc);
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + h], 0.5f + (float)(a1 >> 28), acc);
         }
         return d * acc;
     }
@@ -154,6 +166,13 @@ template <> struct GridFmt<T_IQ2_XXS> {
  * grid entry per index byte (:2916-2940); 98-byte blocks */
 template <> struct GridFmt<T_IQ3_XXS> {
     static constexpr int kBlock = 98, kGridBytes = 1024, kDepth = 2;
+    static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
+    static constexpr int kStep = 16; /* bytes between the x rows of consecutive instructions */
+    static constexpr bool kAInRegs = true;
+    static constexpr int kPiece = 2; /* every piece a lane reads starts 2 (mod 4) bytes into the block */
+    static constexpr bool kSums = false;
+    /* lane group g takes elements [64 g, 64 g + 64) in order, 16 per instruction */
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
     __device__ static const uint32_t *grid_src() { return qlin_iq3xxs_grid; }
     struct Raw {
         Raw16 qs; /* index bytes of groups 2g, 2g+1 */
@@ -167,7 +186,7 @@ template <> struct GridFmt<T_IQ3_XXS> {
         r.d = *reinterpret_cast<const uint16_t *>(blk);
         return r;
     }
-    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t) {
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t, int g) {
         uint32_t qs[4], sc[2];
         bytes16(r.qs, sh, qs);
         bytes8(r.sc, sh, sc);
@@ -185,7 +204,7 @@ template <> struct GridFmt<T_IQ3_XXS> {
                                apply_signs(t.grid[(ix >> 16) & 255u], s1.x), apply_signs(t.grid[ix >> 24], s1.y)};
                 c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2 * h + q], b, c, 0, 0, 0);
             }
-            acc = fmaf(join_digits(c) * xo.scale[h], 0.5f + (float)(a1 >> 28), acc);
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + h], 0.5f + (float)(a1 >> 28), acc);
         }
         return d * acc;
     }
@@ -195,6 +214,13 @@ template <> struct GridFmt<T_IQ3_XXS> {
  * 110-byte blocks */
 template <> struct GridFmt<T_IQ3_S> {
     static constexpr int kBlock = 110, kGridBytes = 2048, kDepth = 2;
+    static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
+    static constexpr int kStep = 16; /* bytes between the x rows of consecutive instructions */
+    static constexpr bool kAInRegs = true;
+    static constexpr int kPiece = 2; /* every piece a lane reads starts 2 (mod 4) bytes into the block */
+    static constexpr bool kSums = false;
+    /* lane group g takes elements [64 g, 64 g + 64) in order, 16 per instruction */
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
     __device__ static const uint32_t *grid_src() { return qlin_iq3s_grid; }
     struct Raw {
         Raw16 qs;  /* low index bytes of groups 2g, 2g+1 */
@@ -210,7 +236,7 @@ template <> struct GridFmt<T_IQ3_S> {
         r.d = *reinterpret_cast<const uint16_t *>(blk);
         return r;
     }
-    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t) {
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t, int g) {
         uint32_t qs[4], sg[2];
         bytes16(r.qs, sh, qs);
         bytes8(r.sg, sh, sg);
@@ -231,9 +257,173 @@ template <> struct GridFmt<T_IQ3_S> {
                 c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2 * h + q], b, c, 0, 0, 0);
             }
             const uint32_t nib = (r.scales >> (4 * h)) & 15u;
-            acc = fmaf(join_digits(c) * xo.scale[h], (float)(1u + 2u * nib), acc);
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + h], (float)(1u + 2u * nib), acc);
         }
         return d * acc;
+    }
+};
+
+/* Q6_K [ql 128][qh 64][16 int8 scales][d]: d * sc * (q - 32), q = low nibble | two high bits << 4, one scale per
+ * 16 elements (common/ggml_dequant.h:1653-1687); 210-byte blocks. Element 128 h + 32 q + l (h = half, q = 0..3,
+ * l < 32) has its nibble in ql[64 h + 32 (q & 1) + l] (the high one for q >= 2) and its high bits in
+ * qh[32 h + l] >> 2 q. Lane group g = (h, p) takes l in [16 p, 16 p + 16) of all four q: instruction q, sixteen
+ * elements of one scale. The codes stay unsigned (0..63); the -32 goes onto the sum of x. */
+template <> struct GridFmt<T_Q6_K> {
+    static constexpr int kBlock = 210, kGridBytes = 0, kDepth = 1;
+    static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
+    static constexpr int kStep = 32;
+    static constexpr bool kAInRegs = false; /* no table lookups: LDS has time to deliver the x operand per item */
+    static constexpr int kPiece = 0;
+    static constexpr bool kSums = true;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 128 * (g >> 1) + 32 * st + 16 * (g & 1); }
+    struct Raw {
+        Raw16 qa, qb, qh; /* ql[64 h + 16 p ..], ql[64 h + 32 + 16 p ..], qh[32 h + 16 p ..] */
+        Raw8 sc;          /* the eight scales of the half */
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const int h = g >> 1, p = g & 1;
+        r.qa = load16(blk + 64 * h + 16 * p);
+        r.qb = load16(blk + 64 * h + 32 + 16 * p);
+        r.qh = load16(blk + 128 + 32 * h + 16 * p);
+        r.sc = load8(blk + 192 + 8 * h);
+        r.d = *reinterpret_cast<const uint16_t *>(blk + 208);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &, int g) {
+        uint32_t qa[4], qb[4], qh[4], sc[2];
+        bytes16(r.qa, sh, qa);
+        bytes16(r.qb, sh, qb);
+        bytes16(r.qh, sh, qh);
+        bytes8(r.sc, sh, sc);
+        const uint32_t scp = (g & 1) ? (sc[0] >> 8) | (sc[1] << 24) : sc[0]; /* byte 2 q (q < 2): scale of (q, p) */
+        const uint32_t scq = (g & 1) ? sc[1] >> 8 : sc[1];                  /* byte 2 (q - 2) for q >= 2 */
+        float acc = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t(&ql)[4] = (q & 1) ? qb : qa;
+            v4i b;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t lo = (ql[i] >> (4 * (q >> 1))) & 0x0F0F0F0Fu;
+                const uint32_t hi = ((qh[i] >> (2 * q)) & 0x03030303u) << 4;
+                b[i] = (int)(lo | hi);
+            }
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * q);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+            const uint32_t w = q < 2 ? scp >> (16 * q) : scq >> (16 * (q - 2));
+            const float scale = (float)(int)(int8_t)(w & 0xFFu);
+            const int e0 = elem0(g, q);
+            acc = fmaf(scale, fmaf(join_digits(c), xo.meta[e0 >> 5], -32.0f * xo.meta[8 + (e0 >> 4)]), acc);
+        }
+        return half_bits_fast(r.d) * acc;
+    }
+};
+
+/* Q8_0 [d][32 x int8] x 8 per 256 elements (common/ggml_dequant.h:1479-1489): 272 bytes, so a row of whole
+ * 256-element groups keeps the alignment of the matrix. Lane group g takes blocks 2g, 2g+1: 68 bytes, 17 dwords. */
+template <> struct GridFmt<T_Q8_0> {
+    static constexpr int kBlock = 272, kGridBytes = 0, kDepth = 1;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = false, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        u32x4_a4 a, b, c, d;
+        uint32_t e;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const uint8_t *p = blk + 68 * g;
+        r.a = *reinterpret_cast<const u32x4_a4 *>(p);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        r.c = *reinterpret_cast<const u32x4_a4 *>(p + 32);
+        r.d = *reinterpret_cast<const u32x4_a4 *>(p + 48);
+        r.e = *reinterpret_cast<const uint32_t *>(p + 64);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t w[17] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c.x,
+                                r.c.y, r.c.z, r.c.w, r.d.x, r.d.y, r.d.z, r.d.w, r.e};
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                v4i b;
+#pragma unroll
+                for (int i = 0; i < 4; i++) /* block 0: the codes start 2 bytes into dword 0; block 1: at dword 9 */
+                    b[i] = h == 0 ? (int)__builtin_amdgcn_alignbit(w[4 * q + i + 1], w[4 * q + i], 16) : (int)w[9 + 4 * q + i];
+                const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * (2 * h + q));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+            }
+            const float d = half_bits_fast(h == 0 ? w[0] & 0xFFFFu : w[8] >> 16);
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + h], d, acc);
+        }
+        return acc;
+    }
+};
+
+/* Q5_K [d][dmin][12 bytes of 6-bit scales and mins][qh 32][qs 128] (:1620-1651), 176 bytes: element 64 j + 32 u + l
+ * has its nibble in qs[32 j + l] (the high one for u = 1) and its fifth bit in qh[l] >> (2 j + u); (d sc) q - dmin m
+ * with one scale and min per 32 elements. Lane group g takes j = g: low nibbles, then high nibbles. */
+template <> struct GridFmt<T_Q5_K> {
+    static constexpr int kBlock = 176, kGridBytes = 0, kDepth = 1;
+    static constexpr int kPiece = 0, kAlign = 16;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        uint4 hd, qh0, qh1, qs0, qs1;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.hd = *reinterpret_cast<const uint4 *>(blk);
+        r.qh0 = *reinterpret_cast<const uint4 *>(blk + 16);
+        r.qh1 = *reinterpret_cast<const uint4 *>(blk + 32);
+        r.qs0 = *reinterpret_cast<const uint4 *>(blk + 48 + 32 * g);
+        r.qs1 = *reinterpret_cast<const uint4 *>(blk + 64 + 32 * g);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t qs[8] = {r.qs0.x, r.qs0.y, r.qs0.z, r.qs0.w, r.qs1.x, r.qs1.y, r.qs1.z, r.qs1.w};
+        const uint32_t qh[8] = {r.qh0.x, r.qh0.y, r.qh0.z, r.qh0.w, r.qh1.x, r.qh1.y, r.qh1.z, r.qh1.w};
+        float dots = 0.0f, mins = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int hf = 0; hf < 2; hf++) {
+                v4i b;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t lo = (qs[4 * hf + i] >> (4 * u)) & 0x0F0F0F0Fu;
+                    const uint32_t hi = ((qh[4 * hf + i] >> (2 * g + u)) & 0x01010101u) << 4;
+                    b[i] = (int)(lo | hi);
+                }
+                const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * (2 * u + hf));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+            }
+            /* get_scale_min_k4 (:1582-1590) for sub-block j = 2g + u, from the header's registers */
+            const int j = 2 * g + u;
+            const uint32_t at = 8u * (uint32_t)(j & 3);
+            const uint32_t yb = __builtin_amdgcn_ubfe(r.hd.y, at, 8), zb = __builtin_amdgcn_ubfe(r.hd.z, at, 8);
+            const uint32_t wb = __builtin_amdgcn_ubfe(r.hd.w, at, 8);
+            const uint32_t sc = j < 4 ? yb & 63u : (wb & 15u) | ((yb >> 6) << 4);
+            const uint32_t mn = j < 4 ? zb & 63u : (wb >> 4) | ((zb >> 6) << 4);
+            dots = fmaf((float)sc, join_digits(c) * xo.meta[j], dots);
+            mins = fmaf((float)mn, xo.meta[8 + 2 * j] + xo.meta[8 + 2 * j + 1], mins);
+        }
+        return half_bits_fast(r.hd.x & 0xFFFFu) * dots - half_bits_fast(r.hd.x >> 16) * mins;
     }
 };
 
@@ -263,11 +453,11 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
     /* LDS: x scratch per wave, the grid and the sign masks at addresses the compiler knows (a lookup is then a
      * shift, a mask and a read with a constant offset); the partial sums [rows][kWaves] behind them */
     __shared__ __attribute__((aligned(16))) uint8_t xs_all[kWaves * kXScratch];
-    __shared__ __attribute__((aligned(16))) uint32_t grid_lds[F::kGridBytes / 4];
-    __shared__ __attribute__((aligned(16))) uint2 sign_lds[256 + 128];
+    __shared__ __attribute__((aligned(16))) uint32_t grid_lds[F::kGridBytes > 0 ? F::kGridBytes / 4 : 4];
+    __shared__ __attribute__((aligned(16))) uint2 sign_lds[F::kGridBytes > 0 ? 256 + 128 : 2];
     uint8_t *xs = xs_all + wv * kXScratch;
     float *partial = reinterpret_cast<float *>(lds);
-    const Tables tab = {grid_lds, sign_lds, sign_lds + 256};
+    const Tables tab = {grid_lds, sign_lds, sign_lds + (F::kGridBytes > 0 ? 256 : 0)};
 
     auto locate = [&](int lr, const uint8_t *&Wm, float *&ym, int &r) {
         if (paired) {
@@ -291,13 +481,10 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
         return Wm + (size_t)r * row_bytes + (size_t)wv * F::kBlock;
     };
 
-    v4f xr[NKC];
-#pragma unroll
-    for (int kc = 0; kc < NKC; kc++) {
-        v4f v = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (kc < n_kc) v = *reinterpret_cast<const v4f *>(x + (16 * kc + wv) * 256 + 4 * lane);
-        xr[kc] = v;
-    }
+    /* the wave's first super-block of x; later ones are fetched where they are used */
+    auto load_x = [&](int kc) { return *reinterpret_cast<const v4f *>(x + (size_t)(16 * kc + wv) * 256 + 4 * lane); };
+    v4f xq = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (n_kc > 0) xq = load_x(0);
 
     /* x -> signed digit planes -> A operands, wave-private */
     auto prepare = [&](v4f v, XOperand &xo) {
@@ -330,23 +517,29 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
         pl[64 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);  /* digit 1 */
         pl[128 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); /* digit 0 */
         if ((lane & 7) == 0) reinterpret_cast<float *>(xs + 1024)[lane >> 3] = down;
+        if (F::kSums) { /* the sum of x over each 16 elements: four lanes */
+            float sum = (v.x + v.y) + (v.z + v.w);
+            sum += dpp_mov<0xB1>(sum);
+            sum += dpp_mov<0x4E>(sum);
+            if ((lane & 3) == 0) reinterpret_cast<float *>(xs + 1056)[lane >> 2] = sum;
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        /* A operand: x row i = lane%16 = 4*g' + plane (plane 3 unused) is live in lane group g' only; its four
-         * instructions take the 64 elements of groups 2g', 2g'+1 in order. Every other lane reads zeros. */
+        /* A operand: x row i = lane%16 = 4*g' + plane (plane 3 unused) is live in lane group g' only and holds,
+         * for instruction s, the digits of the 16 elements from F::elem0(g', s) on. Every other lane reads zeros. */
         const int plane = n & 3;
         const bool live = (n >> 2) == g && plane < 3;
-        const uint4 *src = reinterpret_cast<const uint4 *>(xs + (live ? plane * 256 + 64 * g : 768));
+        xo.arows = xs + (live ? plane * 256 + F::elem0(g, 0) : 768);
+        if (F::kAInRegs) {
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            const uint4 d = src[s];
-            const v4i a = {(int)d.x, (int)d.y, (int)d.z, (int)d.w};
-            xo.A[s] = a;
+            for (int st = 0; st < 4; st++) {
+                const uint4 d = *reinterpret_cast<const uint4 *>(xo.arows + F::kStep * st);
+                const v4i a = {(int)d.x, (int)d.y, (int)d.z, (int)d.w};
+                xo.A[st] = a;
+            }
         }
-        const float2 m = reinterpret_cast<const float2 *>(xs + 1024)[g];
-        xo.scale[0] = m.x;
-        xo.scale[1] = m.y;
+        xo.meta = reinterpret_cast<const float *>(xs + 1024);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
     };
@@ -361,28 +554,29 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
         }
     };
 
-    /* every piece of a block that a lane reads starts 2 (mod 4) bytes into the block: the funnel shift of its bytes */
-    auto shift_of = [](const uint8_t *blk) { return (((uint32_t)(uintptr_t)blk + 2u) & 2u) * 8u; };
+    /* every piece of a block that a lane reads starts F::kPiece (mod 4) bytes into the block: the funnel shift of its bytes */
+    auto shift_of = [](const uint8_t *blk) { return (((uint32_t)(uintptr_t)blk + (uint32_t)F::kPiece) & 2u) * 8u; };
 
     /* the first blocks are requested before the tables are built and x is prepared: the wave's first two
      * super-blocks of a lone row group (long rows), else its first super-block of the first row groups */
     const bool long_rows = NKC > 1 && n_rg < 2;
     constexpr int D = F::kDepth; /* row groups of a super-block column in flight per wave */
-    typename F::Raw first[D];
-    uint32_t first_sh[D];
+    constexpr int NF = D > 2 ? D : 2; /* the long-rows path keeps two */
+    typename F::Raw first[NF];
+    uint32_t first_sh[NF];
     if (n_kc > 0) {
 #pragma unroll
-        for (int q = 0; q < D; q++) {
-            if (long_rows && q >= 2) break;
+        for (int q = 0; q < NF; q++) {
+            if (long_rows ? q >= 2 : q >= D) break;
             const uint8_t *blk = long_rows ? row_pointer(0) + (size_t)(q < n_kc ? q : 0) * (16 * F::kBlock)
                                            : row_pointer(q < n_rg ? q : 0);
             first[q] = F::load(blk, g);
             first_sh[q] = shift_of(blk);
         }
     }
-    if (lane < 16) reinterpret_cast<uint32_t *>(xs + 768)[lane] = 0u; /* what the dead lanes of the x operand read */
+    if (lane < 32) reinterpret_cast<uint32_t *>(xs + 768)[lane] = 0u; /* what the dead lanes of the x operand read */
     for (int t = threadIdx.x; t < F::kGridBytes / 4; t += kWaves * 64) grid_lds[t] = F::grid_src()[t];
-    if (threadIdx.x < 384) {
+    if (F::kGridBytes > 0 && threadIdx.x < 384) {
         const uint32_t i = threadIdx.x, sb = i < 256 ? i : iq_sign_byte(i - 256);
         sign_lds[i] = make_uint2(spread4(sb) * 0xFFu, spread4(sb >> 4) * 0xFFu);
     }
@@ -397,28 +591,23 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
         const uint8_t *blk0 = row_pointer(0);
 #pragma unroll
         for (int kc = 0; kc < NKC; kc++) {
-            typename F::Raw nxt = first[1];
-            uint32_t nxt_sh = first_sh[1];
-            if (kc + 2 < n_kc) {
-                const uint8_t *blk = blk0 + (size_t)(kc + 2) * (16 * F::kBlock);
-                nxt = F::load(blk, g);
-                nxt_sh = shift_of(blk);
-            }
             if (kc < n_kc) {
-                prepare(xr[kc], xo);
-                acc += F::item(xo, first[0], first_sh[0], tab);
+                prepare(xq, xo);
+                if (kc + 1 < n_kc) xq = load_x(kc + 1); /* on its way while this super-block is multiplied */
+                acc += F::item(xo, first[kc & 1], first_sh[kc & 1], tab, g);
             }
-            first[0] = first[1];
-            first_sh[0] = first_sh[1];
-            first[1] = nxt;
-            first_sh[1] = nxt_sh;
+            if (kc + 2 < n_kc) { /* into the registers just used */
+                const uint8_t *blk = blk0 + (size_t)(kc + 2) * (16 * F::kBlock);
+                first[kc & 1] = F::load(blk, g);
+                first_sh[kc & 1] = shift_of(blk);
+            }
+            __builtin_amdgcn_sched_barrier(0); /* one super-block at a time: interleaving them costs registers */
         }
         store_partial(0, acc, false);
     } else {
         for (int kc = 0; kc < n_kc; kc++) {
-            v4f v = xr[0];
-#pragma unroll
-            for (int kk = 1; kk < NKC; kk++) v = kc == kk ? xr[kk] : v;
+            v4f v = xq;
+            if (kc > 0) v = load_x(kc);
             prepare(v, xo);
             /* D row groups in flight: a group's registers are refilled as soon as it has been multiplied */
             if (kc > 0) {
@@ -432,7 +621,7 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
             for (int rg = 0; rg < n_rg; rg += D) {
 #pragma unroll
                 for (int q = 0; q < D; q++) {
-                    if (rg + q < n_rg) store_partial(rg + q, F::item(xo, first[q], first_sh[q], tab), kc > 0);
+                    if (rg + q < n_rg) store_partial(rg + q, F::item(xo, first[q], first_sh[q], tab, g), kc > 0);
                     if (rg + q + D < n_rg) {
                         const uint8_t *blk = row_pointer(rg + q + D) + (size_t)kc * (16 * F::kBlock);
                         first[q] = F::load(blk, g);
@@ -476,13 +665,16 @@ template <uint32_t T>
 bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err,
                 size_t row_stride) {
     const int n_sb = n_cols / 256;
-    /* rows of more than 4096 elements: up to there the v_dot4 kernel (gemv_int.hip) measured faster (both wait
-     * for the table lookups; this one saves its vector instructions where x has to be prepared for few rows) */
+    /* rows of more than 4096 elements: up to there the v_dot4 kernel (gemv_int.hip) measured faster for every format
+     * here (14336 x 4096: Q6_K 14.4 against 15.3 us, Q8_0 12.7 against 14.5; the grid formats wait for the same table
+     * lookups in both); this one saves its vector instructions where x has to be prepared for few rows, and it
+     * has no limit on a row's bytes */
     if (n_cols % 256 != 0 || n_sb <= 16 || n_sb > 16 * kMaxKc || ((uintptr_t)x & 15)) return false;
-    /* the loads want even addresses (block sizes are even) */
+    /* what the format's loads want of the addresses (block sizes are even; the formats whose 256 elements fill a
+     * multiple of 4 or 16 bytes read whole dwords or 16-byte groups) */
     for (int m = 0; m < job.n_mat; m++)
-        if ((uintptr_t)job.W[m] & 1) return false;
-    if (row_stride & 1) return false;
+        if ((uintptr_t)job.W[m] % GridFmt<T>::kAlign) return false;
+    if (row_stride % GridFmt<T>::kAlign) return false;
     const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     if (n_rows == 0) return false;
@@ -500,6 +692,10 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 
 }  // namespace
 
+bool gemv_grid_covers(uint32_t type) {
+    return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0;
+}
+
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
                       hipError_t *err, size_t row_stride) {
     *err = hipSuccess;
@@ -507,6 +703,9 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_IQ2_XXS: return grid_typed<T_IQ2_XXS>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ3_XXS: return grid_typed<T_IQ3_XXS>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ3_S: return grid_typed<T_IQ3_S>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q6_K: return grid_typed<T_Q6_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q5_K: return grid_typed<T_Q5_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q8_0: return grid_typed<T_Q8_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }

@@ -263,9 +263,9 @@ static int column_range(uint32_t type, int n_cols) {
     while (granule % 256 != 0 || (!any_address && ((size_t)(granule / be) * bb) % 16 != 0)) granule += be;
     if (n_cols % granule != 0) return 0;
     /* Q4_K: what its kernel takes; the others: the longest range whose x stays in the lanes' registers */
-    const int cap = type == T_Q4_K ? 16384 : 4096;
+    const int cap = (type == T_Q4_K || gemv_grid_covers(type)) ? 16384 : 4096; /* the matrix-instruction kernels' limit */
     int range = cap / granule * granule;
-    while (range > 0 && (size_t)(range / be) * bb > 8192) range -= granule;
+    while (cap == 4096 && range > 0 && (size_t)(range / be) * bb > 8192) range -= granule; /* those kernels' row images */
     if (range <= 0) return 0;
     const int n_ranges = (n_cols + range - 1) / range;
     range = ((n_cols + n_ranges - 1) / n_ranges + granule - 1) / granule * granule; /* ranges of about equal length */

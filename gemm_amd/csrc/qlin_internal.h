@@ -78,6 +78,7 @@ bool gemv_int_takes_any_even_address(uint32_t type);
  * n_cols <= 16384; same contract as launch_gemv_stream */
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
                       hipStream_t stream, hipError_t *err, size_t row_stride = 0);
+bool gemv_grid_covers(uint32_t type); /* the formats it has an item for */
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu,
                            size_t row_stride = 0);
