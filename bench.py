@@ -119,10 +119,12 @@ def time_fused(steps):
     return out
 
 
-def time_decode_step_linear(n_layers=32, steps=5):
+def time_decode_step_linear(n_layers=32, steps=5, mix=False):
     """The block-quantized linear operators of one decode step of a Llama-3-8B-shaped model (hidden
     4096, FFN 14336, 32 query / 8 KV heads of 128, vocabulary 128256), all Q4_K except a Q6_K output
-    projection, each layer with its own weights (3.6 GB in all), as 4 launches per layer + 2:
+    projection (mix=True: V and down projections in Q6_K in the layers where the usual 4-bit K-quant mix puts
+    them - the first and last eighth and every third layer between; V then takes a launch of its own),
+    each layer with its own weights (3.6 GB in all), as 4 launches per layer + 2:
     Q/K/V in one launch, attention output + residual, gate+up+SiLU, down + residual; then the output
     projection with the greedy pick. Attention, norms and RoPE are outside this library and not run.
     -> dict"""
@@ -136,7 +138,13 @@ def time_decode_step_linear(n_layers=32, steps=5):
     hq, hk, hv = (synth.make_weights(Q4K, r, K, seed=61 + i) for i, r in enumerate((K, KV, KV)))
     ho, hg, hu = (synth.make_weights(Q4K, r, K, seed=64 + i) for i, r in enumerate((K, FF, FF)))
     hd = synth.make_weights(Q4K, K, FF, seed=67)
-    layers = [[qlinear.DevBuf.from_numpy(h) for h in (hq, hk, hv, ho, hg, hu, hd)] for _ in range(n_layers)]
+    hv6, hd6 = synth.make_weights(Q6K, KV, K, seed=69), synth.make_weights(Q6K, K, FF, seed=70)
+
+    def more_bits(i):
+        return mix and (i < n_layers // 8 or i >= 7 * n_layers // 8 or (i - n_layers // 8) % 3 == 2)
+
+    layers = [[qlinear.DevBuf.from_numpy(h) for h in (hq, hk, hv6 if more_bits(i) else hv, ho, hg, hu,
+                                                       hd6 if more_bits(i) else hd)] for i in range(n_layers)]
     Wout = dev(Q6K, V, K, 68)
     x = qlinear.DevBuf.from_numpy(synth.make_activation(K, seed=5) * np.float32(0.05))
     q, k, v = qlinear.DevBuf(K * 4), qlinear.DevBuf(KV * 4), qlinear.DevBuf(KV * 4)
@@ -144,11 +152,15 @@ def time_decode_step_linear(n_layers=32, steps=5):
     logits, pick = qlinear.DevBuf(V * 4), qlinear.DevBuf(qlinear.ARGMAX_RESULT_BYTES)
 
     def step(stream=None):
-        for Wq, Wk, Wv, Wo, Wg, Wu, Wd in layers:
-            qlinear.gemv_multi_dev(Q4K, [Wq, Wk, Wv], [q, k, v], [K, KV, KV], x, K, stream)
+        for i, (Wq, Wk, Wv, Wo, Wg, Wu, Wd) in enumerate(layers):
+            if more_bits(i):
+                qlinear.gemv_multi_dev(Q4K, [Wq, Wk], [q, k], [K, KV], x, K, stream)
+                qlinear.gemv_dev(Q6K, Wv, x, v, KV, K, stream)
+            else:
+                qlinear.gemv_multi_dev(Q4K, [Wq, Wk, Wv], [q, k, v], [K, KV, KV], x, K, stream)
             qlinear.gemv_add_dev(Q4K, Wo, q, x, K, K, stream)     # attention output (stand-in input: q) + residual
             qlinear.gemv_silu_mul_dev(Q4K, Wg, Wu, x, h, FF, K, stream)
-            qlinear.gemv_add_dev(Q4K, Wd, h, x, K, FF, stream)
+            qlinear.gemv_add_dev(Q6K if more_bits(i) else Q4K, Wd, h, x, K, FF, stream)
         qlinear.gemv_argmax_dev(Q6K, Wout, x, logits, pick, V, K, stream)
 
     step()
@@ -159,7 +171,9 @@ def time_decode_step_linear(n_layers=32, steps=5):
         step()
     host_ms = (time.time() - t_host) * 1e3 / steps  # time to enqueue one step from Python
     ms = qlinear.timer_end() / steps
-    weight_bytes = n_layers * sum(a.nbytes for a in (hq, hk, hv, ho, hg, hu, hd)) + V * synth.row_bytes(Q6K, K)
+    n_more = sum(more_bits(i) for i in range(n_layers))
+    weight_bytes = (n_layers * sum(a.nbytes for a in (hq, hk, hv, ho, hg, hu, hd)) + V * synth.row_bytes(Q6K, K) +
+                    n_more * (hv6.nbytes + hd6.nbytes - hv.nbytes - hd.nbytes))
     # the same step captured once into a HIP graph and replayed (the entry points only enqueue kernels)
     hip = ctypes.CDLL("libamdhip64.so")
     stream, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
@@ -187,7 +201,8 @@ def time_decode_step_linear(n_layers=32, steps=5):
     for d in (Wout, x, q, k, v, h, logits, pick):
         d.free()
     return {"ms_per_token": round(ms, 4), "host_enqueue_ms": round(host_ms, 4),
-            "ms_per_token_graph_replay": None if graph_ms is None else round(graph_ms, 4), "launches": 4 * n_layers + 3,
+            "ms_per_token_graph_replay": None if graph_ms is None else round(graph_ms, 4),
+            "launches": 4 * n_layers + n_more + 3, "layers_with_q6_K_v_and_down": n_more,
             "weight_bytes": weight_bytes,
             "GB/s": round(weight_bytes / (ms * 1e-3) / 1e9, 1),
             "hbm_frac": round(weight_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
@@ -639,6 +654,7 @@ def main():
         extra["q4k_fused_decode_shapes"] = time_fused(max(20, args.steps // 8))
 
         extra["q4k_llama8b_shaped_decode_step_linear_ops"] = time_decode_step_linear()
+        extra["q4k_q6k_mix_llama8b_shaped_decode_step_linear_ops"] = time_decode_step_linear(mix=True)
         extra["q4k_llama8b_shaped_prefill_512tok_linear_ops"] = time_prefill_chunk_linear()
 
         hb = time_host_boundary(n_rows, n_cols)
