@@ -197,7 +197,9 @@ int qlin_embed_rows_dev(uint32_t ggml_type, const void *table, int n_table_rows,
                         int n_ids, float *out, int n_cols, void *stream);
 /* y[n_rows] = W . x, x fp32. Besides the block formats W may be dense F16, BF16 or F32 rows
  * (n_cols a multiple of 8, W 16-byte aligned): the fp32 dot of the widened row with x, as
- * tf_qmatvec does for these types (common/transformer.h:1051-1075). */
+ * tf_qmatvec does for these types (common/transformer.h:1051-1075). Rows of any length in whole blocks: rows
+ * of more than 16384 elements run as several launches over column ranges, the later ones adding to y (still one
+ * call, ordered on `stream`). */
 int qlin_gemv_dev(uint32_t ggml_type, const void *W, const float *x, float *y, int n_rows,
                   int n_cols, void *stream);
 /* The fused call shapes of the decode loop, one launch each (all matrices of one ggml type):
@@ -263,8 +265,8 @@ int qlin_gemm_f32_any_dev(uint32_t ggml_type, const void *W, const float *X, flo
  *   X bf16 [n_tok, n_embd]; expert_idx int32 [n_tok, top_k]; expert_w fp32 [n_tok, top_k];
  *   gate/up: [n_expert][n_ff][n_embd] blocks, down: [n_expert][n_embd][n_ff] blocks;
  *   out fp32 [n_tok, n_embd] (overwritten). workspace: qlin_moe_workspace_bytes() bytes.
- * Q4_K matrices run on the matrix cores with unrounded codes; every other format (block-quantized or dense)
- * runs through the bit-exact decoder in fp32, several times slower. qlin_moe_ffn_types_dev takes one format
+ * Q4_K, Q5_K, Q6_K, Q3_K, Q2_K and Q8_0 matrices run on the matrix cores with unrounded codes; every other format
+ * (block-quantized or dense) runs through the bit-exact decoder in fp32, several times slower. qlin_moe_ffn_types_dev takes one format
  * per tensor: K-quant mixes store part of the down projections as Q6_K beside Q4_K gate and up. */
 size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
 int qlin_moe_route_dev(const float *router_logits, int n_tok, int n_expert, int top_k,
