@@ -545,8 +545,7 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
     };
 
     auto store_partial = [&](int rg, float v, bool add) { /* the four lane groups hold four shares of the same row */
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
+        v = sum_lane_groups(v);
         const int lr = 16 * rg + n;
         if (lane < 16 && lr < n_lrows) {
             float *p = partial + lr * kWaves + wv;

@@ -65,7 +65,9 @@ struct XOperand {
 
 }  // namespace
 
-template <int NKC>
+/* ONE: the job is one matrix, stored or added to y (the matrix and row of a local row then need no searching:
+ * found by branches, they cost each weight request some forty instructions before it could go out) */
+template <int NKC, bool ONE>
 __global__ void __launch_bounds__(kWaves * 64)
 gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -75,9 +77,9 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
 
     /* a workgroup owns rows_per_wg rows: of the concatenated matrices, or, where two results are
      * combined (mode 2), the same rows of both matrices (local rows: first matrix, then second) */
-    const bool paired = job.mode == 2;
+    const bool paired = !ONE && job.mode == 2;
     const int n_mats_here = paired ? 2 : 1;
-    const int n_rows = paired ? job.n0 : job.n0 + job.n1 + job.n2;
+    const int n_rows = ONE ? job.n0 : paired ? job.n0 : job.n0 + job.n1 + job.n2;
     const int row0 = blockIdx.x * rows_per_wg;
     int rows_here = n_rows - row0;
     if (rows_here > rows_per_wg) rows_here = rows_per_wg;
@@ -90,7 +92,11 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
     float *partial = reinterpret_cast<float *>(lds + kWaves * kXScratch);
 
     auto locate = [&](int lr, const uint8_t *&Wm, float *&ym, int &r) {
-        if (paired) {
+        if (ONE) {
+            Wm = job.W0;
+            ym = job.y0;
+            r = row0 + lr;
+        } else if (paired) {
             const bool second = lr >= rows_here;
             Wm = second ? job.W1 : job.W0;
             ym = job.y0;
@@ -210,8 +216,7 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
         return Wm + (size_t)r * row_bytes + (size_t)wv * 144;
     };
     auto store_partial = [&](int rg, float v, bool add) { /* the four lane groups hold four sub-blocks' shares of the same row */
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
+        v = sum_lane_groups(v);
         const int lr = 16 * rg + n;
         if (lane < 16 && lr < n_lrows) {
             float *p = partial + lr * kWaves + wv;
@@ -316,12 +321,17 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
     const size_t lds_bytes = (size_t)kWaves * kXScratch + (size_t)rows_per_wg * n_mats_here * kWaves * 4;
     const JobView view = job_view(job);
     if (row_stride == 0) row_stride = (size_t)n_sb * 144; /* rows that are a column range of longer ones keep those rows' pitch */
-    if (n_sb <= 16)
-        hipLaunchKernelGGL(gemv_q4k_kernel<1>, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb,
-                           rows_per_wg, row_stride);
-    else
-        hipLaunchKernelGGL(gemv_q4k_kernel<kMaxKc>, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb,
-                           rows_per_wg, row_stride);
+    const bool one = job.n_mat == 1 && job.mode != kSiluMul;
+    auto launch = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, row_stride);
+    };
+    if (n_sb <= 16) {
+        if (one) launch(gemv_q4k_kernel<1, true>);
+        else launch(gemv_q4k_kernel<1, false>);
+    } else {
+        if (one) launch(gemv_q4k_kernel<kMaxKc, true>);
+        else launch(gemv_q4k_kernel<kMaxKc, false>);
+    }
     return hipGetLastError();
 }
 

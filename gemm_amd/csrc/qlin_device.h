@@ -348,6 +348,18 @@ __device__ __forceinline__ void job_locate(const JobView &j, int v, const uint8_
 }
 __device__ __forceinline__ float silu_times(float g, float u) { return g / (1.0f + expf(-g)) * u; }
 
+/* v + the value 32 lanes away, and the sum of v over lanes n, n + 16, n + 32, n + 48 (in every one of them), by
+ * gfx950's lane swaps: vector instructions, where a shuffle is a trip through LDS */
+__device__ __forceinline__ float add_lane32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_lane_groups(float v) {
+    v = add_lane32(v);
+    const auto q = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+
 /* wave64 sum: every lane ends up with the total */
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
