@@ -459,8 +459,13 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
     float *partial = reinterpret_cast<float *>(lds);
     const Tables tab = {grid_lds, sign_lds, sign_lds + (F::kGridBytes > 0 ? 256 : 0)};
 
+    const bool one_matrix = !paired && job.n1 == 0 && job.n2 == 0; /* a scalar test: no search by row then */
     auto locate = [&](int lr, const uint8_t *&Wm, float *&ym, int &r) {
-        if (paired) {
+        if (one_matrix) {
+            Wm = job.W0;
+            ym = job.y0;
+            r = row0 + lr;
+        } else if (paired) {
             const bool second = lr >= rows_here;
             Wm = second ? job.W1 : job.W0;
             ym = job.y0;
