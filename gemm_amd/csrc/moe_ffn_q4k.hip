@@ -478,8 +478,7 @@ __device__ __forceinline__ void ksplit_quad(uint8_t *img, const uint8_t *m0_rows
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             float a = acc[w][v];
-            a += __shfl_xor(a, 16, 64);
-            a += __shfl_xor(a, 32, 64);
+            a = sum_lane_groups(a);
             acc[w][v] = a;
         }
         if (kg == 0) *reinterpret_cast<f32x4 *>(qred + ((wv * NW + w) * 16 + j) * 4) = acc[w];
@@ -1055,7 +1054,7 @@ moe_down_kq_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__rest
             F::template math<2>(im, blk_at, kg, aa, acc);
             /* the two scale groups of every run sit in lanes kg and kg ^ 2 */
 #pragma unroll
-            for (int v = 0; v < 4; v++) acc[v] += __shfl_xor(acc[v], 32, 64);
+            for (int v = 0; v < 4; v++) acc[v] = add_lane32(acc[v]);
             if (kg < 2) {
 #pragma unroll
                 for (int v = 0; v < 4; v++) red[(wv * 8 + 4 * kg + v) * 16 + j] = acc[v];
@@ -1140,7 +1139,7 @@ moe_down_kq_long_kernel(const uint8_t *__restrict__ down, const uint16_t *__rest
             F::template math<2>(img, blk_at, kg, aa, acc);
         }
 #pragma unroll
-        for (int v = 0; v < 4; v++) acc[v] += __shfl_xor(acc[v], 32, 64);
+        for (int v = 0; v < 4; v++) acc[v] = add_lane32(acc[v]);
         if (kg < 2) {
 #pragma unroll
             for (int v = 0; v < 4; v++) red[(wv * 8 + 4 * kg + v) * 16 + j] = acc[v];
@@ -1227,8 +1226,8 @@ moe_gate_up_kq_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restric
         }
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            acc_g[v] += __shfl_xor(acc_g[v], 32, 64);
-            acc_u[v] += __shfl_xor(acc_u[v], 32, 64);
+            acc_g[v] = add_lane32(acc_g[v]);
+            acc_u[v] = add_lane32(acc_u[v]);
         }
         if (kg < 2) {
 #pragma unroll
@@ -1334,7 +1333,7 @@ gemm_kq_fewtok_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict_
 #pragma unroll
         for (int q = 0; q < NQ; q++) {
 #pragma unroll
-            for (int v = 0; v < 4; v++) acc[q][v] += __shfl_xor(acc[q][v], 32, 64);
+            for (int v = 0; v < 4; v++) acc[q][v] = add_lane32(acc[q][v]);
             if (kg < 2) {
 #pragma unroll
                 for (int v = 0; v < 4; v++) red[(wv * kPass + 8 * q + 4 * kg + v) * 16 + j] = acc[q][v];
