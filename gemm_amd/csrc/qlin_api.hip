@@ -168,22 +168,10 @@ const void *lookup_locked(const void *host, size_t need) {
 }
 
 /* host -> device on the library's stream; small transfers go through the pinned buffer */
-int upload_locked(void *dev, const void *host, size_t bytes) {
-    const size_t need = (bytes + 255) & ~(size_t)255;
-    if (g.pinned && g.up_used + need <= kPinnedHalf) {
-        uint8_t *st = g.pinned + g.up_used;
-        g.up_used += need;
-        memcpy(st, host, bytes);
-        HIP_TRY(hipMemcpyAsync(dev, st, bytes, hipMemcpyHostToDevice, g.stream));
-    } else {
-        HIP_TRY(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, g.stream));
-    }
-    return QLIN_OK;
-}
 /* Results go to the pinned buffer by a kernel that stores over the bus, not by the runtime's device-to-host
  * copy: after a process has freed a few GiB of device memory that copy took 95 us instead of 9.5 us for the
  * 57 KB of a matvec result (until another stream was created), which made a 35 us call a 130 us call. */
-__global__ void __launch_bounds__(256) store_to_host_kernel(uint8_t *__restrict__ dst, const uint8_t *__restrict__ src,
+__global__ void __launch_bounds__(256) copy16_kernel(uint8_t *__restrict__ dst, const uint8_t *__restrict__ src,
                                                             size_t bytes) {
     const size_t n16 = bytes >> 4;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256)
@@ -191,6 +179,27 @@ __global__ void __launch_bounds__(256) store_to_host_kernel(uint8_t *__restrict_
     if (blockIdx.x == 0 && threadIdx.x < (bytes & 15)) dst[(n16 << 4) + threadIdx.x] = src[(n16 << 4) + threadIdx.x];
 }
 
+int upload_locked(void *dev, const void *host, size_t bytes) {
+    const size_t need = (bytes + 255) & ~(size_t)255;
+    if (g.pinned && g.up_used + need <= kPinnedHalf) {
+        uint8_t *st = g.pinned + g.up_used;
+        g.up_used += need;
+        memcpy(st, host, bytes);
+        if (g.pinned_dev && aligned(dev, 16) && bytes <= (1u << 20)) {
+            /* small inputs (an activation vector): a kernel that reads the staging buffer over the bus, for the
+             * reason given at copy16_kernel and because it starts sooner than the runtime's copy */
+            const size_t groups = ((bytes >> 4) + 255) / 256;
+            const int grid = (int)std::min<size_t>(std::max<size_t>(groups, 1), 64);
+            copy16_kernel<<<grid, 256, 0, g.stream>>>(static_cast<uint8_t *>(dev), g.pinned_dev + (st - g.pinned), bytes);
+            HIP_TRY(hipGetLastError());
+        } else {
+            HIP_TRY(hipMemcpyAsync(dev, st, bytes, hipMemcpyHostToDevice, g.stream));
+        }
+    } else {
+        HIP_TRY(hipMemcpyAsync(dev, host, bytes, hipMemcpyHostToDevice, g.stream));
+    }
+    return QLIN_OK;
+}
 /* device -> host on the library's stream; the bytes are in `host` after finish_locked() */
 int download_locked(void *host, const void *dev, size_t bytes) {
     const size_t need = (bytes + 255) & ~(size_t)255;
@@ -201,7 +210,7 @@ int download_locked(void *host, const void *dev, size_t bytes) {
         if (g.pinned_dev && aligned(dev, 16)) {
             const size_t groups = ((bytes >> 4) + 255) / 256;
             const int grid = (int)std::min<size_t>(std::max<size_t>(groups, 1), 64);
-            store_to_host_kernel<<<grid, 256, 0, g.stream>>>(g.pinned_dev + (st - g.pinned),
+            copy16_kernel<<<grid, 256, 0, g.stream>>>(g.pinned_dev + (st - g.pinned),
                                                              static_cast<const uint8_t *>(dev), bytes);
             HIP_TRY(hipGetLastError());
         } else {
@@ -332,9 +341,20 @@ int matvec_host_locked(float *dst, const void *W, uint32_t type, int n_cols, con
         if (int rc = g.x.ensure((size_t)n_cols * 4)) return rc;
         if (int rc = upload_locked(g.x.p, x, (size_t)n_cols * 4)) return rc;
     }
-    if (int rc = g.y[slot].ensure((size_t)n_rows * 4 + 16)) return rc;
+    /* the tuned Q4_K kernel stores a workgroup's results as one run of consecutive floats: it can write them
+     * straight into the pinned result buffer over the bus, which saves the copy kernel behind it */
+    const size_t y_bytes = (size_t)n_rows * 4, y_need = (y_bytes + 255) & ~(size_t)255;
+    if (type == T_Q4_K && n_cols % 256 == 0 && n_cols <= 16384 && aligned(dW, 16) && g.pinned_dev &&
+        g.down_used + y_need <= kPinnedHalf) {
+        uint8_t *st = g.pinned + kPinnedHalf + g.down_used;
+        g.down_used += y_need;
+        HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)(g.pinned_dev + (st - g.pinned)), n_rows, n_cols, g.stream));
+        g.pending.push_back({dst, st, y_bytes});
+        return QLIN_OK;
+    }
+    if (int rc = g.y[slot].ensure(y_bytes + 16)) return rc;
     HIP_TRY(dispatch_gemv(type, dW, (const float *)g.x.p, (float *)g.y[slot].p, n_rows, n_cols, g.stream));
-    if (int rc = download_locked(dst, g.y[slot].p, (size_t)n_rows * 4)) return rc;
+    if (int rc = download_locked(dst, g.y[slot].p, y_bytes)) return rc;
     return QLIN_OK;
 }
 
