@@ -4,27 +4,28 @@
  * instruction; the grid formats look their codebook and sign masks up in LDS, the others build their codes in
  * registers and read the x operand from LDS for every item.
  *
- * y[r] = sum over 32-element groups of scale(r, group) * (signed grid bytes . x_group)
- * (the decoders of common/ggml_dequant.h:2793-2816, :2916-2940 and :3022-3058 dotted with x).
+ * y[r] = sum over 16- or 32-element groups of scale(r, group) * (codes . x_group) (- offset * sum of x_group), with
+ * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
+ * :1620-1651 (Q5_K) and :1479-1489 (Q8_0).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
  *     2^-23 of that largest |x| per element.
- *  2. v_mfma_i32_16x16x64_i8: 16 weight rows (B operand: one signed grid byte per element) against 16
- *     "x rows" (A operand). Lane group g = lane/16 of a wave owns groups 2g and 2g+1 of the wave's
- *     super-block: instruction s = 0..3 of the super-block takes from lane group g the 16 elements
- *     [16 (s & 1), +16) of group 2g + (s >> 1). The A operand is block-diagonal to match: x row 4g + digit
- *     (digit 0..2; row 4g+3 stays zero) holds that digit plane of lane group g's 16 elements at lane group g's k positions and zeros elsewhere,
- *     so after two instructions result register v of lane (n, g) is digit plane v of group 2g (then 2g+1)
- *     for weight row n. Which k position carries which element is free as long as both operands agree.
+ *  2. v_mfma_i32_16x16x64_i8: 16 weight rows (B operand: one code byte per element) against 16 "x rows"
+ *     (A operand). Lane group g = lane/16 of a wave owns 64 elements of the wave's super-block, 16 per
+ *     instruction s = 0..3 (F::elem0(g, s): elements [64 g + 16 s, +16) for most formats; Q6_K takes the 16
+ *     elements of one scale). The A operand is block-diagonal to match: x row 4g + digit (digit 0..2; row 4g+3
+ *     stays zero) holds that digit plane of lane group g's 16 elements at lane group g's k positions and zeros
+ *     elsewhere, so result register v of lane (n, g) is digit plane v of lane group g's elements for weight
+ *     row n. Which k position carries which element is free as long as both operands agree.
  *  3. Wave w of the 16-wave workgroup owns super-block w (w+16, ...) of every row of the workgroup, prepares
  *     only its own 256 elements of x, and reads its bytes of a block straight from HBM: lane (n, g) takes
- *     the bytes of groups 2g, 2g+1 of row n (blocks are 2-byte aligned: dword-aligned loads, a 16-bit
- *     tail and a funnel shift). The waves' shares of a row meet in LDS at the end.
+ *     the bytes of its 64 elements of row n (blocks of the grid formats and Q6_K are 2-byte aligned:
+ *     dword-aligned loads, a 16-bit tail and a funnel shift). The waves' shares of a row meet in LDS at the end.
  *
- * What a lane spends per element is one table lookup per 4-8 elements for the grid, one per 8 for the sign
- * mask, two vector instructions per 4 elements to apply the signs and a sixteenth of a matrix instruction;
- * the v_dot4 formulation (gemv_int.hip) spends an instruction per element on the products alone.
+ * What a lane of a grid format spends per element is one table lookup per 4-8 elements for the grid, one per 8
+ * for the sign mask, two vector instructions per 4 elements to apply the signs and a sixteenth of a matrix
+ * instruction; the v_dot4 formulation (gemv_int.hip) spends an instruction per element on the products alone.
  *
  * A non-finite x makes every output NaN (the fixed-point form cannot carry Inf).
  */
