@@ -1,12 +1,12 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K and Q8_0: the inner products run on the 8-bit integer matrix
- * instruction; the grid formats look their codebook and sign masks up in LDS, the others build their codes in
- * registers and read the x operand from LDS for every item.
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, IQ4_NL and IQ4_XS: the inner products run on the 8-bit
+ * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
+ * codes in registers and read the x operand from LDS for every item.
  *
  * y[r] = sum over 16- or 32-element groups of scale(r, group) * (codes . x_group) (- offset * sum of x_group), with
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
- * :1620-1651 (Q5_K) and :1479-1489 (Q8_0).
+ * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL) and :2956-2973 (IQ4_XS).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -428,6 +428,124 @@ template <> struct GridFmt<T_Q5_K> {
     }
 };
 
+/* the sixteen signed bytes of the IQ4 codebook (common/ggml_dequant.h:2942-2954) in four registers, and its
+ * lookup for four nibbles at once: two byte permutes and a select by the nibbles' top bits */
+struct Table16 {
+    uint32_t t0, t1, t2, t3;
+};
+__device__ __forceinline__ Table16 iq4_table() {
+    const uint4 v = *reinterpret_cast<const uint4 *>(qlin_iq4nl_values);
+    const Table16 t = {v.x, v.y, v.z, v.w};
+    return t;
+}
+__device__ __forceinline__ int look4(uint32_t n, const Table16 &t) {
+    const uint32_t sel = n & 0x07070707u;
+    const uint32_t lo = __builtin_amdgcn_perm(t.t1, t.t0, sel), hi = __builtin_amdgcn_perm(t.t3, t.t2, sel);
+    const uint32_t m = ((n >> 3) & 0x01010101u) * 0xFFu;
+    return (int)((hi & m) | (lo & ~m));
+}
+
+/* IQ4_NL [d][16 bytes of nibbles] x 8 per 256 elements (:2942-2954): d * table[nibble]; element l of a block is the
+ * low nibble of byte l, element 16 + l the high one. 144 bytes per 256 elements; lane group g takes blocks 2g, 2g+1:
+ * 36 bytes, nine dwords. Q4_0 (:2850-2862) has the same layout with d * (nibble - 8): its codes stay unsigned and
+ * the -8 goes onto the sum of x. */
+template <uint32_t T> struct Nibble18 {
+    static constexpr int kBlock = 144, kGridBytes = 0, kDepth = 2;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = T == T_Q4_0, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        u32x4_a4 a, b;
+        uint32_t c;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const uint8_t *p = blk + 36 * g;
+        r.a = *reinterpret_cast<const u32x4_a4 *>(p);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        r.c = *reinterpret_cast<const uint32_t *>(p + 32);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t w[9] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c};
+        const Table16 tab = iq4_table();
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint32_t qs[4]; /* block 0: the nibble bytes start 2 bytes into dword 0; block 1: at dword 5 */
+#pragma unroll
+            for (int i = 0; i < 4; i++) qs[i] = h == 0 ? __builtin_amdgcn_alignbit(w[i + 1], w[i], 16) : w[5 + i];
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                v4i b;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint32_t nib = (qs[i] >> (4 * u)) & 0x0F0F0F0Fu;
+                    b[i] = T == T_Q4_0 ? (int)nib : look4(nib, tab);
+                }
+                const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * (2 * h + u));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+            }
+            const float d = half_bits_fast(h == 0 ? w[0] & 0xFFFFu : w[4] >> 16);
+            const int G = 2 * g + h;
+            float dot = join_digits(c) * xo.meta[G];
+            if (T == T_Q4_0) dot = fmaf(-8.0f, xo.meta[8 + 2 * G] + xo.meta[8 + 2 * G + 1], dot);
+            acc = fmaf(dot, d, acc);
+        }
+        return acc;
+    }
+};
+template <> struct GridFmt<T_IQ4_NL> : Nibble18<T_IQ4_NL> {};
+template <> struct GridFmt<T_Q4_0> : Nibble18<T_Q4_0> {};
+
+/* IQ4_XS [d][scales_h 2][scales_l 4][qs 128] (:2956-2973), 136 bytes: group j of 32 elements has its nibbles in
+ * qs[16 j ..] (low nibbles first, as IQ4_NL) and a 6-bit scale - 32. Lane group g takes groups 2g, 2g+1. */
+template <> struct GridFmt<T_IQ4_XS> {
+    static constexpr int kBlock = 136, kGridBytes = 0, kDepth = 2;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = false, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        u32x4_a4 a, b;
+        u32x2_a4 hd;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.hd = *reinterpret_cast<const u32x2_a4 *>(blk);
+        r.a = *reinterpret_cast<const u32x4_a4 *>(blk + 8 + 32 * g);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(blk + 24 + 32 * g);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t qs[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
+        const Table16 tab = iq4_table();
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                v4i b;
+#pragma unroll
+                for (int i = 0; i < 4; i++) b[i] = look4((qs[4 * h + i] >> (4 * u)) & 0x0F0F0F0Fu, tab);
+                const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * (2 * h + u));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+            }
+            const int j = 2 * g + h;
+            const uint32_t ls = ((r.hd.y >> (4 * j)) & 15u) | ((((r.hd.x >> 16) >> (2 * j)) & 3u) << 4);
+            acc = fmaf(join_digits(c) * xo.meta[j], (float)((int)ls - 32), acc);
+        }
+        return half_bits_fast(r.hd.x & 0xFFFFu) * acc;
+    }
+};
+
 }  // namespace
 
 template <uint32_t T, int NKC>
@@ -698,7 +816,8 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 }  // namespace
 
 bool gemv_grid_covers(uint32_t type) {
-    return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0;
+    return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
+           type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -711,6 +830,9 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_Q6_K: return grid_typed<T_Q6_K>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q5_K: return grid_typed<T_Q5_K>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q8_0: return grid_typed<T_Q8_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ4_NL: return grid_typed<T_IQ4_NL>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ4_XS: return grid_typed<T_IQ4_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q4_0: return grid_typed<T_Q4_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
