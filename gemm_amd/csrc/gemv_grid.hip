@@ -1,12 +1,13 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, IQ4_NL and IQ4_XS: the inner products run on the 8-bit
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, IQ4_NL, IQ4_XS, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
  * y[r] = sum over 16- or 32-element groups of scale(r, group) * (codes . x_group) (- offset * sum of x_group), with
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
- * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL) and :2956-2973 (IQ4_XS).
+ * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
+ * :1505-1534 (Q2_K) and :1536-1580 (Q3_K).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -428,6 +429,122 @@ template <> struct GridFmt<T_Q5_K> {
     }
 };
 
+/* Q2_K [16 scale bytes][qs 64][d][dmin] (common/ggml_dequant.h:1505-1534), 84 bytes: element 128 h + 32 j + l
+ * (l < 32) is bits 2j, 2j+1 of qs[32 h + l], scaled by d * (low nibble) and offset by -dmin * (high nibble) of
+ * scale byte 8 h + 2 j + l / 16. Lane group g = (h, p) takes l in [16 p, 16 p + 16) of all four j, as Q6_K. */
+template <> struct GridFmt<T_Q2_K> {
+    static constexpr int kBlock = 84, kGridBytes = 0, kDepth = 2;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 32;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 128 * (g >> 1) + 32 * st + 16 * (g & 1); }
+    struct Raw {
+        u32x4_a4 qs;
+        u32x2_a4 sc; /* the eight scale bytes of the half */
+        uint32_t dd;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = *reinterpret_cast<const u32x4_a4 *>(blk + 16 + 16 * g);
+        r.sc = *reinterpret_cast<const u32x2_a4 *>(blk + 8 * (g >> 1));
+        r.dd = *reinterpret_cast<const uint32_t *>(blk + 80);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t qs[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+        const uint32_t scp = (g & 1) ? (r.sc.x >> 8) | (r.sc.y << 24) : r.sc.x; /* byte 2 j (j < 2): scale of (j, p) */
+        const uint32_t scq = (g & 1) ? r.sc.y >> 8 : r.sc.y;                    /* byte 2 (j - 2) for j >= 2 */
+        float dots = 0.0f, mins = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v4i b;
+#pragma unroll
+            for (int i = 0; i < 4; i++) b[i] = (int)((qs[i] >> (2 * j)) & 0x03030303u);
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * j);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+            const uint32_t w = (j < 2 ? scp >> (16 * j) : scq >> (16 * (j - 2))) & 0xFFu;
+            const int e0 = elem0(g, j);
+            dots = fmaf((float)(w & 15u), join_digits(c) * xo.meta[e0 >> 5], dots);
+            mins = fmaf((float)(w >> 4), xo.meta[8 + (e0 >> 4)], mins);
+        }
+        return half_bits_fast(r.dd & 0xFFFFu) * dots - half_bits_fast(r.dd >> 16) * mins;
+    }
+};
+
+/* four bytes at p (2-byte aligned, at least two bytes into a block) */
+struct Raw4 {
+    uint32_t q, tail;
+};
+__device__ __forceinline__ Raw4 load4(const uint8_t *p) {
+    Raw4 r;
+    const uint32_t odd = (uint32_t)(uintptr_t)p & 2u;
+    r.q = *reinterpret_cast<const uint32_t *>(p - odd);
+    r.tail = 0;
+    if (odd) r.tail = *reinterpret_cast<const uint16_t *>(p + 2);
+    return r;
+}
+
+/* Q3_K [hmask 32][qs 64][12 packed scale bytes][d] (:1536-1580), 110 bytes: element 128 h + 32 j + l (l < 32) is
+ * bits 2j, 2j+1 of qs[32 h + l], minus 4 unless bit 4 h + j of hmask[l] is set, times d * (6-bit scale - 32) of
+ * index 8 h + 2 j + l / 16: low nibbles in bytes 0..7 (index & 7, the high nibble for indices 8..15), the two high
+ * bits of index i in byte 8 + (i & 3) at bit 2 (i >> 2). Lane group g = (h, p) as Q6_K; the codes stay unsigned
+ * (0..7) and the -4 goes onto the sum of x. */
+template <> struct GridFmt<T_Q3_K> {
+    static constexpr int kBlock = 110, kGridBytes = 0, kDepth = 1;
+    static constexpr int kPiece = 0, kAlign = 2;
+    static constexpr int kStep = 32;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 128 * (g >> 1) + 32 * st + 16 * (g & 1); }
+    struct Raw {
+        Raw16 qs, hm;
+        Raw8 lo; /* scale bytes 0..7 */
+        Raw4 hi; /* scale bytes 8..11 */
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load16(blk + 32 + 16 * g);
+        r.hm = load16(blk + 16 * (g & 1));
+        r.lo = load8(blk + 96);
+        r.hi = load4(blk + 104);
+        r.d = *reinterpret_cast<const uint16_t *>(blk + 108);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &, int g) {
+        uint32_t qs[4], hm[4], lo[2];
+        bytes16(r.qs, sh, qs);
+        bytes16(r.hm, sh, hm);
+        bytes8(r.lo, sh, lo);
+        const uint32_t hi = __builtin_amdgcn_alignbit(r.hi.tail, r.hi.q, sh);
+        const int h = g >> 1, p = g & 1;
+        const uint32_t scp = p ? (lo[0] >> 8) | (lo[1] << 24) : lo[0]; /* byte 2 j (j < 2) */
+        const uint32_t scq = p ? lo[1] >> 8 : lo[1];                   /* byte 2 (j - 2) for j >= 2 */
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v4i b;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                b[i] = (int)(((qs[i] >> (2 * j)) & 0x03030303u) | (((hm[i] >> (4 * h + j)) & 0x01010101u) << 2));
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * j);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+            const uint32_t w = j < 2 ? scp >> (16 * j) : scq >> (16 * (j - 2));
+            const uint32_t low = (w >> (4 * h)) & 15u;
+            const uint32_t high = (hi >> (8 * (2 * (j & 1) + p) + 2 * (2 * h + (j >> 1)))) & 3u;
+            const float scale = (float)((int)(low | (high << 4)) - 32);
+            const int e0 = elem0(g, j);
+            acc = fmaf(scale, fmaf(join_digits(c), xo.meta[e0 >> 5], -4.0f * xo.meta[8 + (e0 >> 4)]), acc);
+        }
+        return half_bits_fast(r.d) * acc;
+    }
+};
+
 /* the sixteen signed bytes of the IQ4 codebook (common/ggml_dequant.h:2942-2954) in four registers, and its
  * lookup for four nibbles at once: two byte permutes and a select by the nibbles' top bits */
 struct Table16 {
@@ -817,7 +934,7 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
-           type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0;
+           type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -833,6 +950,8 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_IQ4_NL: return grid_typed<T_IQ4_NL>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ4_XS: return grid_typed<T_IQ4_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q4_0: return grid_typed<T_Q4_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q2_K: return grid_typed<T_Q2_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q3_K: return grid_typed<T_Q3_K>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
