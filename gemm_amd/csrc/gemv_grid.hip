@@ -1,5 +1,6 @@
 /*
- * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements on gfx950, for the codebook ("grid") formats
+ * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
+ * 4096) on gfx950, for the codebook ("grid") formats
  * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, IQ4_NL, IQ4_XS, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
@@ -122,7 +123,7 @@ template <uint32_t T> struct GridFmt;
 /* IQ2_XXS [d][8 x (4 grid indices, 4 x 7 sign bits + 4-bit scale)]: d*(0.5+s)*0.25 * grid byte * sign, an
  * eight-byte grid entry per index (common/ggml_dequant.h:2793-2816); 66-byte blocks */
 template <> struct GridFmt<T_IQ2_XXS> {
-    static constexpr int kBlock = 66, kGridBytes = 2048, kDepth = 4;
+    static constexpr int kBlock = 66, kGridBytes = 2048;
     static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
     static constexpr int kStep = 16; /* bytes between the x rows of consecutive instructions */
     static constexpr bool kAInRegs = true;
@@ -167,7 +168,7 @@ template <> struct GridFmt<T_IQ2_XXS> {
 /* IQ3_XXS [d][qs 64][8 x (4 x 7 sign bits + 4-bit scale)]: d*(0.5+s)*0.5 * grid byte * sign, a four-byte
  * grid entry per index byte (:2916-2940); 98-byte blocks */
 template <> struct GridFmt<T_IQ3_XXS> {
-    static constexpr int kBlock = 98, kGridBytes = 1024, kDepth = 2;
+    static constexpr int kBlock = 98, kGridBytes = 1024;
     static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
     static constexpr int kStep = 16; /* bytes between the x rows of consecutive instructions */
     static constexpr bool kAInRegs = true;
@@ -215,7 +216,7 @@ template <> struct GridFmt<T_IQ3_XXS> {
 /* IQ3_S [d][qs 64][qh 8][signs 32][scales 4]: d*(1+2s) * grid byte * sign, 9-bit grid indices (:3022-3058);
  * 110-byte blocks */
 template <> struct GridFmt<T_IQ3_S> {
-    static constexpr int kBlock = 110, kGridBytes = 2048, kDepth = 2;
+    static constexpr int kBlock = 110, kGridBytes = 2048;
     static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
     static constexpr int kStep = 16; /* bytes between the x rows of consecutive instructions */
     static constexpr bool kAInRegs = true;
@@ -271,7 +272,7 @@ template <> struct GridFmt<T_IQ3_S> {
  * qh[32 h + l] >> 2 q. Lane group g = (h, p) takes l in [16 p, 16 p + 16) of all four q: instruction q, sixteen
  * elements of one scale. The codes stay unsigned (0..63); the -32 goes onto the sum of x. */
 template <> struct GridFmt<T_Q6_K> {
-    static constexpr int kBlock = 210, kGridBytes = 0, kDepth = 1;
+    static constexpr int kBlock = 210, kGridBytes = 0;
     static constexpr int kAlign = 2; /* what the loads want of the matrix address and the row pitch */
     static constexpr int kStep = 32;
     static constexpr bool kAInRegs = false; /* no table lookups: LDS has time to deliver the x operand per item */
@@ -329,7 +330,7 @@ template <> struct GridFmt<T_Q6_K> {
 /* Q8_0 [d][32 x int8] x 8 per 256 elements (common/ggml_dequant.h:1479-1489): 272 bytes, so a row of whole
  * 256-element groups keeps the alignment of the matrix. Lane group g takes blocks 2g, 2g+1: 68 bytes, 17 dwords. */
 template <> struct GridFmt<T_Q8_0> {
-    static constexpr int kBlock = 272, kGridBytes = 0, kDepth = 1;
+    static constexpr int kBlock = 272, kGridBytes = 0;
     static constexpr int kPiece = 0, kAlign = 4;
     static constexpr int kStep = 16;
     static constexpr bool kSums = false, kAInRegs = false;
@@ -377,7 +378,7 @@ template <> struct GridFmt<T_Q8_0> {
  * has its nibble in qs[32 j + l] (the high one for u = 1) and its fifth bit in qh[l] >> (2 j + u); (d sc) q - dmin m
  * with one scale and min per 32 elements. Lane group g takes j = g: low nibbles, then high nibbles. */
 template <> struct GridFmt<T_Q5_K> {
-    static constexpr int kBlock = 176, kGridBytes = 0, kDepth = 1;
+    static constexpr int kBlock = 176, kGridBytes = 0;
     static constexpr int kPiece = 0, kAlign = 16;
     static constexpr int kStep = 16;
     static constexpr bool kSums = true, kAInRegs = false;
@@ -433,7 +434,7 @@ template <> struct GridFmt<T_Q5_K> {
  * (l < 32) is bits 2j, 2j+1 of qs[32 h + l], scaled by d * (low nibble) and offset by -dmin * (high nibble) of
  * scale byte 8 h + 2 j + l / 16. Lane group g = (h, p) takes l in [16 p, 16 p + 16) of all four j, as Q6_K. */
 template <> struct GridFmt<T_Q2_K> {
-    static constexpr int kBlock = 84, kGridBytes = 0, kDepth = 2;
+    static constexpr int kBlock = 84, kGridBytes = 0;
     static constexpr int kPiece = 0, kAlign = 4;
     static constexpr int kStep = 32;
     static constexpr bool kSums = true, kAInRegs = false;
@@ -493,7 +494,7 @@ __device__ __forceinline__ Raw4 load4(const uint8_t *p) {
  * bits of index i in byte 8 + (i & 3) at bit 2 (i >> 2). Lane group g = (h, p) as Q6_K; the codes stay unsigned
  * (0..7) and the -4 goes onto the sum of x. */
 template <> struct GridFmt<T_Q3_K> {
-    static constexpr int kBlock = 110, kGridBytes = 0, kDepth = 1;
+    static constexpr int kBlock = 110, kGridBytes = 0;
     static constexpr int kPiece = 0, kAlign = 2;
     static constexpr int kStep = 32;
     static constexpr bool kSums = true, kAInRegs = false;
@@ -567,7 +568,7 @@ __device__ __forceinline__ int look4(uint32_t n, const Table16 &t) {
  * 36 bytes, nine dwords. Q4_0 (:2850-2862) has the same layout with d * (nibble - 8): its codes stay unsigned and
  * the -8 goes onto the sum of x. */
 template <uint32_t T> struct Nibble18 {
-    static constexpr int kBlock = 144, kGridBytes = 0, kDepth = 2;
+    static constexpr int kBlock = 144, kGridBytes = 0;
     static constexpr int kPiece = 0, kAlign = 4;
     static constexpr int kStep = 16;
     static constexpr bool kSums = T == T_Q4_0, kAInRegs = false;
@@ -622,7 +623,7 @@ template <> struct GridFmt<T_Q4_0> : Nibble18<T_Q4_0> {};
 /* IQ4_XS [d][scales_h 2][scales_l 4][qs 128] (:2956-2973), 136 bytes: group j of 32 elements has its nibbles in
  * qs[16 j ..] (low nibbles first, as IQ4_NL) and a 6-bit scale - 32. Lane group g takes groups 2g, 2g+1. */
 template <> struct GridFmt<T_IQ4_XS> {
-    static constexpr int kBlock = 136, kGridBytes = 0, kDepth = 2;
+    static constexpr int kBlock = 136, kGridBytes = 0;
     static constexpr int kPiece = 0, kAlign = 4;
     static constexpr int kStep = 16;
     static constexpr bool kSums = false, kAInRegs = false;
@@ -800,8 +801,10 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
     /* the first blocks are requested before the tables are built and x is prepared: the wave's first two
      * super-blocks of a lone row group (long rows), else its first super-block of the first row groups */
     const bool long_rows = NKC > 1 && n_rg < 2;
-    constexpr int D = F::kDepth; /* row groups of a super-block column in flight per wave */
-    constexpr int NF = D > 2 ? D : 2; /* the long-rows path keeps two */
+    /* row groups of a super-block column in flight per wave: with sixteen waves per compute unit one is enough, and
+     * two or four measured slower for every format (IQ2_XXS 8192 x 28672: 38.8 us with four, 29.6 with one) */
+    constexpr int D = 1;
+    constexpr int NF = (NKC > 1 && D < 2) ? 2 : D; /* the long-rows path keeps two */
     typename F::Raw first[NF];
     uint32_t first_sh[NF];
     if (n_kc > 0) {
@@ -901,15 +904,30 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
 
 namespace {
 
+/* Rows of up to 4096 elements, one super-block per wave and one row group per wave in flight (two and four measured
+ * slower for every format): where this kernel measured faster than the v_dot4 kernel (gemv_int.hip) over 1024 to
+ * 151936 rows of 2048 to 4096 elements. 14336 x 4096, us: IQ4_NL 13.3 -> 10.3, IQ4_XS 12.8 -> 10.6, Q4_0 10.4 -> 8.7,
+ * Q2_K 10.0 -> 8.0, IQ2_XXS 11.0 -> 9.0, Q3_K 13.8 -> 12.8, IQ3_S 13.3 -> 12.5, Q5_K 12.8 -> 12.5; 151936 x 4096:
+ * IQ2_XXS 82 -> 51, Q2_K 74 -> 54, IQ4_NL 100 -> 79, but Q5_K 90 -> 112, Q6_K 103 -> 141, Q8_0 103 -> 132 (and
+ * Q6_K, Q8_0 no faster at 14336 rows: they stay with the other kernel). With fewer than eight super-blocks more
+ * than half of the waves would have nothing to do. Two workgroups per compute unit (the instances of 64 registers
+ * or fewer would fit) measured slower for every format. */
+bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
+    if (n_sb < 8) return false;
+    switch (type) {
+    case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
+    case T_Q3_K: return n_rows >= 4096;
+    case T_Q5_K: return n_rows <= 16384;
+    default: return false;
+    }
+}
+
 template <uint32_t T>
 bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream, hipError_t *err,
                 size_t row_stride) {
     const int n_sb = n_cols / 256;
-    /* rows of more than 4096 elements: up to there the v_dot4 kernel (gemv_int.hip) measured faster for every format
-     * here (14336 x 4096: Q6_K 14.4 against 15.3 us, Q8_0 12.7 against 14.5; the grid formats wait for the same table
-     * lookups in both); this one saves its vector instructions where x has to be prepared for few rows, and it
-     * has no limit on a row's bytes */
-    if (n_cols % 256 != 0 || n_sb <= 16 || n_sb > 16 * kMaxKc || ((uintptr_t)x & 15)) return false;
+    const bool short_rows = n_sb <= 16;
+    if (n_cols % 256 != 0 || n_sb > 16 * kMaxKc || ((uintptr_t)x & 15)) return false;
     /* what the format's loads want of the addresses (block sizes are even; the formats whose 256 elements fill a
      * multiple of 4 or 16 bytes read whole dwords or 16-byte groups) */
     for (int m = 0; m < job.n_mat; m++)
@@ -919,13 +937,19 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     if (n_rows == 0) return false;
     int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
-    rows_per_wg = (rows_per_wg + 15) & ~15; /* whole row groups: a matrix instruction wants 16 rows anyway */
+    if (short_rows && !short_rows_pay(T, n_sb, n_rows * n_mats_here)) return false;
+    /* long rows: whole row groups, a matrix instruction wants 16 rows anyway; short ones: a workgroup on every
+     * compute unit counts for more (14336 rows: 56 each) */
+    if (!short_rows) rows_per_wg = (rows_per_wg + 15) & ~15;
     if (rows_per_wg * n_mats_here > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / n_mats_here;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = (size_t)rows_per_wg * n_mats_here * kWaves * 4; /* the partial sums; the rest is static */
     const JobView view = job_view(job);
-    hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg,
-                       row_stride ? row_stride : (size_t)n_sb * GridFmt<T>::kBlock);
+    const size_t pitch = row_stride ? row_stride : (size_t)n_sb * GridFmt<T>::kBlock;
+    if (short_rows)
+        hipLaunchKernelGGL((gemv_grid_kernel<T, 1>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch);
+    else
+        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch);
     *err = hipGetLastError();
     return true;
 }

@@ -1,5 +1,5 @@
 """GPU parity of the matrix-instruction matvec for the codebook formats IQ2_XXS, IQ3_XXS, IQ3_S and for Q6_K, Q5_K,
-Q8_0, Q4_0, IQ4_NL, IQ4_XS, Q2_K, Q3_K (rows longer than 4096 elements take it) against the CPU oracle, through the C ABI: plain, ragged row counts, several
+Q8_0, Q4_0, IQ4_NL, IQ4_XS, Q2_K, Q3_K (rows longer than 4096 elements take it, and most of these formats' rows from 2048 elements) against the CPU oracle, through the C ABI: plain, ragged row counts, several
 matrices in one launch, gate+up+SiLU, projection+residual, non-finite x. Relative L2 <= 1e-5."""
 import numpy as np
 import pytest
@@ -16,9 +16,10 @@ GRID = {synth.GGML_IQ2_XXS: "iq2_xxs", synth.GGML_IQ3_XXS: "iq3_xxs", synth.GGML
 
 
 # 17 super-blocks (one wave with two), 43 (ragged over the 16 waves), 56 and 64 (the most a wave takes);
-# one row, a ragged last row group, several row groups per workgroup, more rows than compute units x 16
+# one row, a ragged last row group, several row groups per workgroup, more rows than compute units x 16; rows of
+# 2048 to 4096 elements (one super-block or none per wave): 56 rows per workgroup, ragged row counts, many row groups
 @pytest.mark.parametrize("n_rows,n_cols", [(1, 4352), (16, 4352), (37, 11008), (300, 8192), (4096, 14336), (130, 16384),
-                                           (5000, 4608)])
+                                           (5000, 4608), (14336, 4096), (4113, 2048), (9, 4096), (40001, 3072)])
 @pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
 def test_matvec(oracle, tid, n_rows, n_cols):
     W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + tid)
