@@ -35,7 +35,6 @@
 #include "qlin_codebooks_ext.h"
 #include "qlin_device.h"
 #include "qlin_internal.h"
-#include <type_traits>
 
 namespace qlin {
 

@@ -43,7 +43,6 @@
  */
 #include "qlin_device.h"
 #include "qlin_internal.h"
-#include <type_traits>
 
 namespace qlin {
 
@@ -224,18 +223,16 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
         }
     };
     XOperand xo;
-    /* NG row groups of column chunk kc: every block is requested before the first is used */
-    auto run_group = [&](int rg0, int kc, auto ng_tag) {
-        constexpr int NG = decltype(ng_tag)::value;
-        uint4 h[NG], q0[NG], q1[NG];
-#pragma unroll
-        for (int q = 0; q < NG; q++) {
-            const uint8_t *blk = row_pointer(rg0 + q) + (size_t)kc * (16 * 144);
-            h[q] = *reinterpret_cast<const uint4 *>(blk);
-            q0[q] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
-            q1[q] = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
-        }
-        if (rg0 == 0) { /* x is prepared while the first blocks are on their way */
+    /* one row group of column chunk kc at a time: the sixteen waves of a compute unit keep enough requests going
+     * between them, and a wave that requested two to four row groups together before using the first measured slower
+     * wherever a workgroup has more than one (14336 x 4096: 9.1 -> 8.7 us, gate+up+SiLU of that shape 15.6 -> 13.5,
+     * 151936 x 4096: 80 -> 68, 8192 x 28672: 37 -> 32) */
+    auto run_group = [&](int rg, int kc) {
+        const uint8_t *blk = row_pointer(rg) + (size_t)kc * (16 * 144);
+        const uint4 h = *reinterpret_cast<const uint4 *>(blk);
+        const uint4 q0 = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+        const uint4 q1 = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
+        if (rg == 0) { /* x is prepared while the first blocks are on their way */
             v4f v = xr[0];
             if (NKC > 1 && kc > 0) v = *reinterpret_cast<const v4f *>(x + (size_t)(16 * kc + wv) * 256 + 4 * lane);
             /* x is not looked at before this point: left alone, the compiler moves the first steps of the
@@ -244,21 +241,13 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
             asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w) : : "memory");
             prepare(v, xo);
         }
-#pragma unroll
-        for (int q = 0; q < NG; q++) store_partial(rg0 + q, item(xo, h[q], q0[q], q1[q]), kc > 0);
+        store_partial(rg, item(xo, h, q0, q1), kc > 0);
     };
     if (n_kc == 0) { /* a wave without a super-block (K < 4096) contributes zeros */
         for (int rg = 0; rg < n_rg; rg++) store_partial(rg, 0.0f, false);
     } else if (NKC == 1 || n_rg >= 2) {
-        for (int kc = 0; kc < n_kc; kc++) {
-            int rg0 = 0;
-            for (; rg0 + 4 <= n_rg; rg0 += 4) run_group(rg0, kc, std::integral_constant<int, 4>());
-            if (rg0 + 2 <= n_rg) {
-                run_group(rg0, kc, std::integral_constant<int, 2>());
-                rg0 += 2;
-            }
-            if (rg0 < n_rg) run_group(rg0, kc, std::integral_constant<int, 1>());
-        }
+        for (int kc = 0; kc < n_kc; kc++)
+            for (int rg = 0; rg < n_rg; rg++) run_group(rg, kc);
     } else {
         /* long rows, one row group: the wave's up to NKC super-blocks of the row are requested together */
         const uint8_t *blk0 = row_pointer(0);
