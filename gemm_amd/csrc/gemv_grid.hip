@@ -47,7 +47,7 @@ typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
 
 constexpr int kWaves = 16;        /* wavefronts per workgroup */
 constexpr int kMaxKc = 4;         /* super-blocks per wave: K <= 16384 */
-constexpr int kMaxRowsPerWg = 128;
+constexpr int kMaxRowsPerWg = 640; /* local rows (both matrices of a gate+up pair): 40 KB of partial sums, 63 KB in all */
 constexpr int kXScratch = 1152;   /* per wave: 3 digit planes x 256 B, 128 zero bytes, (at 1024) 8 x 2^(e-22), (at 1056) 16 sums of 16 x */
 
 /* x operand of one super-block: A[s] for instruction s. The other two things an item needs stay in the wave's
@@ -935,12 +935,18 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
     const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     if (n_rows == 0) return false;
-    int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
     if (short_rows && !short_rows_pay(T, n_sb, n_rows * n_mats_here)) return false;
+    /* one workgroup per compute unit where its partial sums fit in LDS (with the lookup tables: in 128 rows' worth,
+     * more measured slower for those formats), else so many equal rounds of workgroups that they do (Q2_K 151936 x
+     * 4096: 55 -> 48 us, 49152 rows 22.3 -> 17.4) */
+    constexpr int max_rows = GridFmt<T>::kGridBytes > 0 ? 128 : kMaxRowsPerWg;
+    const int rows_per_cu = (n_rows + n_cu - 1) / n_cu;
+    const int rounds = (rows_per_cu * n_mats_here + max_rows - 1) / max_rows;
+    int rows_per_wg = (n_rows + n_cu * rounds - 1) / (n_cu * rounds);
     /* long rows: whole row groups, a matrix instruction wants 16 rows anyway; short ones: a workgroup on every
      * compute unit counts for more (14336 rows: 56 each) */
     if (!short_rows) rows_per_wg = (rows_per_wg + 15) & ~15;
-    if (rows_per_wg * n_mats_here > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / n_mats_here;
+    if (rows_per_wg * n_mats_here > max_rows) rows_per_wg = max_rows / n_mats_here;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
     const size_t lds_bytes = (size_t)rows_per_wg * n_mats_here * kWaves * 4; /* the partial sums; the rest is static */
     const JobView view = job_view(job);

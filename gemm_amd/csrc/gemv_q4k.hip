@@ -53,7 +53,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 16;             /* wavefronts per workgroup */
 constexpr int kMaxKc = 4;               /* 16-super-block column chunks: K <= 16384 */
-constexpr int kMaxRowsPerWg = 128;
+constexpr int kMaxRowsPerWg = 640; /* local rows (both matrices of a gate+up pair): 40 KB of partial sums */
 constexpr int kXScratch = 1088;         /* per wave: 4 digit planes x 256 B + 8 x (2^(e-30), sum) */
 /* x operand of one super-block: A[2p+h] for chain p, instruction h; scale[p] = 2^(e-30) and
  * sum[p] = sum of x for sub-block 4p + lane/16 */
@@ -68,7 +68,7 @@ struct XOperand {
  * found by branches, they cost each weight request some forty instructions before it could go out) */
 template <int NKC, bool ONE>
 __global__ void __launch_bounds__(kWaves * 64)
-gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes) {
+gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes, int lone_ahead) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -245,28 +245,34 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
     };
     if (n_kc == 0) { /* a wave without a super-block (K < 4096) contributes zeros */
         for (int rg = 0; rg < n_rg; rg++) store_partial(rg, 0.0f, false);
-    } else if (NKC == 1 || n_rg >= 2) {
+    } else if (NKC == 1 || n_rg >= 2 || !lone_ahead) {
         for (int kc = 0; kc < n_kc; kc++)
             for (int rg = 0; rg < n_rg; rg++) run_group(rg, kc);
     } else {
-        /* long rows, one row group: the wave's up to NKC super-blocks of the row are requested together */
+        /* long rows, one row group, workgroups for part of the compute units only: two of the wave's super-blocks
+         * of the row are requested ahead of the one being multiplied (2048 x 16384: 7.9 us, 9.1 one at a time, 8.5
+         * with all four requested together). With a workgroup on every compute unit the loop above, one super-block
+         * at a time, is the faster one (4096 x 14336: 9.5 against 9.9 us, 4096 x 11008: 7.6 against 7.9). */
         const uint8_t *blk0 = row_pointer(0);
-        uint4 h[NKC], q0[NKC], q1[NKC];
-#pragma unroll
-        for (int kc = 0; kc < NKC; kc++)
-            if (kc < n_kc) {
-                const uint8_t *blk = blk0 + (size_t)kc * (16 * 144);
-                h[kc] = *reinterpret_cast<const uint4 *>(blk);
-                q0[kc] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
-                q1[kc] = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
-            }
+        uint4 h[2], q0[2], q1[2];
+        auto request = [&](int slot, int kc) {
+            const uint8_t *blk = blk0 + (size_t)kc * (16 * 144);
+            h[slot] = *reinterpret_cast<const uint4 *>(blk);
+            q0[slot] = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+            q1[slot] = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
+        };
+        request(0, 0);
+        request(1, n_kc > 1 ? 1 : 0);
         float acc = 0.0f;
 #pragma unroll
-        for (int kc = 0; kc < NKC; kc++)
+        for (int kc = 0; kc < NKC; kc++) {
             if (kc < n_kc) {
                 prepare(xr[kc], xo);
-                acc += item(xo, h[kc], q0[kc], q1[kc]);
+                acc += item(xo, h[kc & 1], q0[kc & 1], q1[kc & 1]);
             }
+            if (kc + 2 < n_kc) request(kc & 1, kc + 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         store_partial(0, acc, false);
     }
     __syncthreads();
@@ -303,7 +309,12 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
     const int n_mats_here = job.mode == kSiluMul ? 2 : 1;
     const int n_rows = job.mode == kSiluMul ? job.n_rows[0] : job.total_rows();
     if (n_rows == 0) return hipSuccess;
-    int rows_per_wg = (n_rows + n_cu - 1) / n_cu;
+    /* one workgroup per compute unit where its partial sums fit in LDS, else so many equal rounds of workgroups
+     * that they do (151936 rows: 594 each; with 128-row workgroups the 1187 of them left a fifth round a third full:
+     * 66.5 -> 60.5 us, 49152 rows 26.8 -> 21.3) */
+    const int rows_per_cu = (n_rows + n_cu - 1) / n_cu;
+    const int rounds = (rows_per_cu * n_mats_here + kMaxRowsPerWg - 1) / kMaxRowsPerWg;
+    int rows_per_wg = (n_rows + n_cu * rounds - 1) / (n_cu * rounds);
     if (rows_per_wg < 1) rows_per_wg = 1;
     if (rows_per_wg * n_mats_here > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / n_mats_here;
     const int grid = (n_rows + rows_per_wg - 1) / rows_per_wg;
@@ -312,7 +323,8 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
     if (row_stride == 0) row_stride = (size_t)n_sb * 144; /* rows that are a column range of longer ones keep those rows' pitch */
     const bool one = job.n_mat == 1 && job.mode != kSiluMul;
     auto launch = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, row_stride);
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, row_stride,
+                           grid < n_cu ? 1 : 0);
     };
     if (n_sb <= 16) {
         if (one) launch(gemv_q4k_kernel<1, true>);

@@ -73,6 +73,10 @@ FULL = [
     (synth.GGML_Q8_0, 4096, 4096), (synth.GGML_Q4_K, 4096, 4096), (synth.GGML_Q4_K, 14336, 4096),
     (synth.GGML_Q4_K, 4096, 14336), (synth.GGML_Q5_K, 4096, 4096), (synth.GGML_IQ4_NL, 14336, 4096),
     (synth.GGML_IQ2_XXS, 4096, 14336), (synth.GGML_IQ3_S, 4096, 14336), (synth.GGML_Q6_K, 151936, 4096),
+    # vocabulary-sized projections in the formats of the matrix-instruction kernels: one workgroup of several hundred
+    # rows per compute unit, or several equal rounds of them
+    (synth.GGML_Q4_K, 151936, 4096), (synth.GGML_Q4_K, 200003, 2048), (synth.GGML_IQ4_NL, 151936, 4096),
+    (synth.GGML_Q2_K, 170001, 2048), (synth.GGML_IQ2_XXS, 151936, 4096), (synth.GGML_Q4_0, 49152, 4096),
 ]
 
 
