@@ -22,10 +22,12 @@
  * super-block: d, dmin and the packed scales of the thread's row are unpacked once per super-block.
  * When 128-row tiles would leave compute units
  * without a workgroup (few tokens, or few rows) the same kernel runs with BN = 64: 4 x 2 waves
- * of 64 tokens x 32 rows, eight 4-byte weight parts per row (M = 128: 66 -> 55 us). When even those
+ * of 64 tokens x 32 rows, eight 4-byte weight parts per row. When even those
  * tiles number 128 or fewer (4096 rows at 512 tokens), K is cut in two halves that add their results to
  * a zeroed Y (4096 x 14336 at 512 tokens: 166 -> 108 us; two addends onto zero commute, so the result
- * does not depend on which half arrives first).
+ * does not depend on which half arrives first). Up to 128 tokens the tile is 128 tokens x 64 rows on four waves
+ * (2 x 2 of 64 x 32, four 8-byte weight parts per row), two workgroups to a compute unit, K cut in two while the
+ * tiles number a chip's worth or fewer (M = 128 at 14336 x 4096: 51.7 -> 39.5 us).
  *
  * Measured on MI355X at M=512, N=14336, K=4096: 76-77 us, 0.79 PFLOP/s on 224 of 256 compute
  * units. Cycle stamps (s_memtime) around the parts of one tile show a tile of about 1920 cycles
@@ -103,14 +105,18 @@ __device__ __forceinline__ uint2 decode4(uint32_t n0, float dl, float ml) {
 }  // namespace
 
 /* NB = 2: 128 weight rows per workgroup (wave tile 64 tokens x 64 rows); NB = 1: 64 weight rows (wave
- * tile 64 x 32) and twice as many workgroups, for shapes whose grid would not fill the chip */
+ * tile 64 x 32) and twice as many workgroups, for shapes whose grid would not fill the chip. WM = 4: 256 tokens
+ * per workgroup, eight waves; WM = 2: 128 tokens, four waves (with NB = 1 only) */
 template <int WM, int NB>
 __global__ void __launch_bounds__(128 * WM)
 gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y,
                      int n_rows, int n_sb, int n_tok, int ldx, int ldy, int m_tiles, int k_split) {
     constexpr int BM = 64 * WM, NT = 128 * WM;
-    static_assert(NT == 512, "one weight-row part per thread: 512 threads");
     constexpr int BN = 64 * NB;
+    /* one part of a weight row's 32 nibble bytes per thread: four parts of 8 bytes or eight of 4 */
+    constexpr bool kPart8 = BN * 4 == NT;
+    static_assert(kPart8 || BN * 8 == NT, "one weight-row part per thread");
+    constexpr int kARows = NT / 8; /* token rows that one pass of the threads' 16-byte activation chunks covers */
     constexpr int kATile = BM * kRow, kBTile = BN * kRow;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     uint8_t *As = lds;                      /* [kStages][BM][kRow]  */
@@ -130,11 +136,11 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     const size_t row_bytes = (size_t)n_sb * 144;
     /* B-tile role: weight row br, part bp of the 32 nibble bytes of a sub-block pair (NB = 2: four
      * 8-byte parts per row, NB = 1: eight 4-byte parts) */
-    const int br = NB == 2 ? tid >> 2 : tid >> 3, bp = NB == 2 ? tid & 3 : tid & 7;
+    const int br = kPart8 ? tid >> 2 : tid >> 3, bp = kPart8 ? tid & 3 : tid & 7;
     int w_row = tile_n * BN + br;
     if (w_row >= n_rows) w_row = n_rows - 1;
     const uint8_t *w_ptr = W + (size_t)w_row * row_bytes;
-    /* A-tile role: chunks (token row ar + 64j, 16-byte column ac), j = 0..3 */
+    /* A-tile role: chunks (token row ar + kARows j, 16-byte column ac), j = 0..3 */
     const int ar = tid >> 3, ac = tid & 7;
     /* blockIdx.y = which part of K (k_split parts of equal, even length); with more than one part the
      * results are added to a zeroed Y */
@@ -151,14 +157,14 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     auto x_chunk = [&](int j, int step) {
         /* token rows past the end re-read row 0: their products land in accumulator rows that
          * are never stored */
-        const int m = tile_m * BM + ar + 64 * j;
+        const int m = tile_m * BM + ar + kARows * j;
         return *reinterpret_cast<const uint4 *>(X + (size_t)(m < n_tok ? m : 0) * ldx + (size_t)step * kBK + 8 * ac);
     };
     auto fetch = [&](StepRegs &r, int step) {
         if (step >= n_steps) step = n_steps - 1; /* harmless re-read past the end */
         const int sb = step >> 2, c = step & 3;
         const uint8_t *blk = w_ptr + (size_t)sb * 144;
-        if (NB == 2) r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * bp);
+        if (kPart8) r.qs = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * c + 8 * bp);
         else r.qs = make_uint2(*reinterpret_cast<const uint32_t *>(blk + 16 + 32 * c + 4 * bp), 0u);
         r.x0 = x_chunk(0, step); r.x1 = x_chunk(1, step); r.x2 = x_chunk(2, step); r.x3 = x_chunk(3, step);
     };
@@ -185,7 +191,7 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
         const float ml_a = sc.dmin * (float)(mn2 & 0xFFu), ml_b = sc.dmin * (float)((mn2 >> 8) & 0xFFu);
         uint8_t *bt = Bs + st * kBTile;
         /* sub-block 2c (low nibbles) -> k 0..31 = chunks 0..3, sub-block 2c+1 -> chunks 4..7 */
-        if (NB == 2) {
+        if (kPart8) {
             *reinterpret_cast<uint4 *>(bt + swz(br, bp)) = decode8(r.qs.x & 0x0F0F0F0Fu, r.qs.y & 0x0F0F0F0Fu, dl_a, ml_a);
             *reinterpret_cast<uint4 *>(bt + swz(br, 4 + bp)) =
                 decode8((r.qs.x >> 4) & 0x0F0F0F0Fu, (r.qs.y >> 4) & 0x0F0F0F0Fu, dl_b, ml_b);
@@ -198,9 +204,9 @@ gemm_q4k_bf16_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__
     auto stage_acts = [&](const StepRegs &r, int st) {
         uint8_t *at = As + st * kATile;
         *reinterpret_cast<uint4 *>(at + swz(ar, ac)) = r.x0;
-        *reinterpret_cast<uint4 *>(at + swz(ar + 64, ac)) = r.x1;
-        *reinterpret_cast<uint4 *>(at + swz(ar + 128, ac)) = r.x2;
-        *reinterpret_cast<uint4 *>(at + swz(ar + 192, ac)) = r.x3;
+        *reinterpret_cast<uint4 *>(at + swz(ar + kARows, ac)) = r.x1;
+        *reinterpret_cast<uint4 *>(at + swz(ar + 2 * kARows, ac)) = r.x2;
+        *reinterpret_cast<uint4 *>(at + swz(ar + 3 * kARows, ac)) = r.x3;
     };
 
     floatx16 acc00, acc01, acc10, acc11;
@@ -330,11 +336,11 @@ __global__ void __launch_bounds__(256) zero_rows_kernel(float *__restrict__ Y, i
     if (n < n_rows) Y[(size_t)blockIdx.y * ldy + n] = 0.0f;
 }
 
-template <int NB>
+template <int WM, int NB>
 hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok, int ldx,
                         int ldy, hipStream_t stream) {
     static OnceFlag lds_raised;
-    constexpr int WM = 4, BM = 64 * WM, BN = 64 * NB;
+    constexpr int BM = 64 * WM, BN = 64 * NB;
     const int n_sb = n_cols / 256;
     const int m_tiles = (n_tok + BM - 1) / BM;
     const int n_tiles = (n_rows + BN - 1) / BN;
@@ -345,7 +351,8 @@ hipError_t launch_tiled(const void *W, const uint16_t *X, float *Y, int n_rows, 
     /* half a chip's worth of tiles or less (4096 rows at 512 tokens: 128): each tile's K range is cut in
      * two halves that add their results to a zeroed Y; a + b onto zero is the same in either order, so
      * the result stays deterministic (three or more parts would not) */
-    const int k_split = (NB == 1 && n_tiles * m_tiles <= 128 && n_sb >= 4 && n_sb % 2 == 0) ? 2 : 1;
+    /* (128-token tiles: two workgroups fit a compute unit, so up to a chip's worth of tiles is cut) */
+    const int k_split = (NB == 1 && n_tiles * m_tiles <= (WM == 2 ? 256 : 128) && n_sb >= 4 && n_sb % 2 == 0) ? 2 : 1;
     if (k_split > 1) {
         hipLaunchKernelGGL(zero_rows_kernel, dim3((n_rows + 255) / 256, n_tok), dim3(256), 0, stream, Y, n_rows, ldy);
     }
@@ -369,8 +376,11 @@ hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int 
     if (n_tok <= kFewTokens) return launch_gemm_q4k_fewtok(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     /* 128-row tiles unless they would leave compute units without a workgroup */
     const int m_tiles = (n_tok + 255) / 256, n_tiles_128 = (n_rows + 127) / 128;
-    if (m_tiles * n_tiles_128 < 200) return launch_tiled<1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    return launch_tiled<2>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    /* up to 128 tokens: 128-token x 64-row tiles of four waves, two workgroups per compute unit, instead of
+     * half-empty 256-token tiles (128 tokens at 14336 x 4096: 51.7 -> 39.5 us, 64 tokens: 50.7 -> 34.4) */
+    if (n_tok <= 128) return launch_tiled<2, 1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    if (m_tiles * n_tiles_128 < 200) return launch_tiled<4, 1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    return launch_tiled<4, 2>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
 }
 
 }  // namespace qlin

@@ -47,6 +47,8 @@ def references(oracle, W, Xb, n_cols):
     (300, 257, 2048), (512, 1024, 4096), (33, 1000, 768), (16, 14336, 256), (17, 48, 512), (48, 100, 256),
     (49, 100, 256), (3, 16, 2560),
     (260, 12805, 256), (1030, 5130, 512),  # enough tiles for the 128-row variant of the kernel
+    # 49..128 tokens: 128-token tiles; more than a chip's worth of them (K stays whole), an odd super-block count
+    (128, 16500, 1024), (100, 20000, 512), (90, 130, 768), (65, 70, 2048),
 ])
 def test_gemm_bf16_shapes(oracle, n_tok, n_rows, n_cols):
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=n_rows + n_tok)
