@@ -1,14 +1,14 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, IQ4_NL, IQ4_XS, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
  * y[r] = sum over 16- or 32-element groups of scale(r, group) * (codes . x_group) (- offset * sum of x_group), with
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
- * :1505-1534 (Q2_K) and :1536-1580 (Q3_K).
+ * :1505-1534 (Q2_K), :1536-1580 (Q3_K) and :2864-2915 (Q4_1, Q5_0, Q5_1).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -619,6 +619,87 @@ template <uint32_t T> struct Nibble18 {
 template <> struct GridFmt<T_IQ4_NL> : Nibble18<T_IQ4_NL> {};
 template <> struct GridFmt<T_Q4_0> : Nibble18<T_Q4_0> {};
 
+/* Q4_1 [d][m][16 nibble bytes] (common/ggml_dequant.h:2864-2877), Q5_0 [d][qh 4][16] (:2879-2895) and Q5_1
+ * [d][m][qh 4][16] (:2897-2915): blocks of 32 elements in 20, 22 and 24 bytes; element l < 16 is the low nibble of
+ * byte l (+ 16 x bit l of qh), element 16 + l the high nibble (+ 16 x bit 16 + l); Q4_1 and Q5_1 add m, Q5_0
+ * subtracts 16. Lane group g takes blocks 2g and 2g + 1 as 10, 11 or 12 dwords; the codes stay unsigned and m or
+ * -16 d goes onto the sum of x. */
+template <uint32_t T> struct Legacy32 {
+    static constexpr int kBytes = T == T_Q4_1 ? 20 : T == T_Q5_0 ? 22 : 24;
+    static constexpr int kDw = kBytes / 2; /* dwords of two blocks */
+    static constexpr bool kHigh = T != T_Q4_1, kMin = T != T_Q5_0;
+    static constexpr int kBlock = 8 * kBytes, kGridBytes = 0;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        uint32_t w[kDw];
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const uint8_t *p = blk + 2 * kBytes * g;
+#pragma unroll
+        for (int i = 0; i + 4 <= kDw; i += 4) {
+            const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(p + 4 * i);
+            r.w[i] = v.x; r.w[i + 1] = v.y; r.w[i + 2] = v.z; r.w[i + 3] = v.w;
+        }
+        if (kDw % 4 >= 2) {
+            const u32x2_a4 v = *reinterpret_cast<const u32x2_a4 *>(p + 4 * (kDw & ~3));
+            r.w[kDw & ~3] = v.x; r.w[(kDw & ~3) + 1] = v.y;
+        }
+        if (kDw % 2) r.w[kDw - 1] = *reinterpret_cast<const uint32_t *>(p + 4 * (kDw - 1));
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t(&w)[kDw] = r.w;
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint32_t dm, qh = 0, qs[4];
+            if (T == T_Q5_0) { /* the second block starts in the middle of dword 5 */
+                dm = h == 0 ? w[0] & 0xFFFFu : w[5] >> 16;
+                qh = h == 0 ? __builtin_amdgcn_alignbit(w[1], w[0], 16) : w[6];
+#pragma unroll
+                for (int i = 0; i < 4; i++) qs[i] = h == 0 ? __builtin_amdgcn_alignbit(w[i + 2], w[i + 1], 16) : w[7 + i];
+            } else {
+                constexpr int kHead = kHigh ? 2 : 1;
+                const int b = (kDw / 2) * h;
+                dm = w[b];
+                if (kHigh) qh = w[b + 1];
+#pragma unroll
+                for (int i = 0; i < 4; i++) qs[i] = w[b + kHead + i];
+            }
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                v4i b;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t code = (qs[i] >> (4 * u)) & 0x0F0F0F0Fu;
+                    if (kHigh) code |= spread4(qh >> (16 * u + 4 * i)) << 4;
+                    b[i] = (int)code;
+                }
+                const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * (2 * h + u));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+            }
+            const int G = 2 * g + h;
+            const float sum = xo.meta[8 + 2 * G] + xo.meta[8 + 2 * G + 1];
+            const float d = half_bits_fast(dm & 0xFFFFu);
+            float dot = join_digits(c) * xo.meta[G];
+            if (!kMin) dot = fmaf(-16.0f, sum, dot);
+            acc = fmaf(dot, d, acc);
+            if (kMin) acc = fmaf(half_bits_fast(dm >> 16), sum, acc);
+        }
+        return acc;
+    }
+};
+template <> struct GridFmt<T_Q4_1> : Legacy32<T_Q4_1> {};
+template <> struct GridFmt<T_Q5_0> : Legacy32<T_Q5_0> {};
+template <> struct GridFmt<T_Q5_1> : Legacy32<T_Q5_1> {};
+
 /* IQ4_XS [d][scales_h 2][scales_l 4][qs 128] (:2956-2973), 136 bytes: group j of 32 elements has its nibbles in
  * qs[16 j ..] (low nibbles first, as IQ4_NL) and a 6-bit scale - 32. Lane group g takes groups 2g, 2g+1. */
 template <> struct GridFmt<T_IQ4_XS> {
@@ -908,7 +989,8 @@ namespace {
  * 151936 rows of 2048 to 4096 elements. 14336 x 4096, us: IQ4_NL 13.3 -> 10.3, IQ4_XS 12.8 -> 10.6, Q4_0 10.4 -> 8.7,
  * Q2_K 10.0 -> 8.0, IQ2_XXS 11.0 -> 9.0, Q3_K 13.8 -> 12.8, IQ3_S 13.3 -> 12.5, Q5_K 12.8 -> 12.5; 151936 x 4096:
  * IQ2_XXS 82 -> 51, Q2_K 74 -> 54, IQ4_NL 100 -> 79, but Q5_K 90 -> 112, Q6_K 103 -> 141, Q8_0 103 -> 132 (and
- * Q6_K, Q8_0 no faster at 14336 rows: they stay with the other kernel). With fewer than eight super-blocks more
+ * Q6_K, Q8_0 no faster at 14336 rows or below 4096: they come here for 4096 to 8192 rows only, 4096 x 4096:
+ * Q8_0 6.9 -> 6.0, Q6_K 7.1 -> 6.8; 8192 x 4096: 9.3 -> 8.7, 11.1 -> 10.0). With fewer than eight super-blocks more
  * than half of the waves would have nothing to do. Two workgroups per compute unit (the instances of 64 registers
  * or fewer would fit) measured slower for every format. */
 bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
@@ -917,6 +999,8 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
+    case T_Q4_1: case T_Q5_0: case T_Q5_1: return n_rows <= 32768; /* 14336: 10.5 -> 9.3, 12.1 -> 10.0, 12.0 -> 10.3; 151936: 67 -> 88 */
+    case T_Q6_K: case T_Q8_0: return n_rows >= 4096 && n_rows <= 8192;
     default: return false;
     }
 }
@@ -963,7 +1047,8 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
-           type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K;
+           type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -981,6 +1066,9 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_Q4_0: return grid_typed<T_Q4_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q2_K: return grid_typed<T_Q2_K>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q3_K: return grid_typed<T_Q3_K>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q4_1: return grid_typed<T_Q4_1>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q5_0: return grid_typed<T_Q5_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q5_1: return grid_typed<T_Q5_1>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
