@@ -254,6 +254,7 @@ static bool launch_gemv_tuned(uint32_t type, const GemvJob &job, const float *x,
         *err = launch_gemv_q4k(job, x, n_cols, s, g.n_cu, row_stride);
         return true;
     }
+    if (launch_gemv_dense_long(type, job, x, n_cols, g.n_cu, s, err, row_stride)) return true;
     if (launch_gemv_grid(type, job, x, n_cols, g.n_cu, s, err, row_stride)) return true;
     if (launch_gemv_int(type, job, x, n_cols, g.n_cu, s, err, row_stride)) return true;
     return launch_gemv_stream(type, job, x, n_cols, g.n_cu, s, err, row_stride);
@@ -272,7 +273,8 @@ static int column_range(uint32_t type, int n_cols) {
     while (granule % 256 != 0 || (!any_address && ((size_t)(granule / be) * bb) % 16 != 0)) granule += be;
     if (n_cols % granule != 0) return 0;
     /* Q4_K: what its kernel takes; the others: the longest range whose x stays in the lanes' registers */
-    const int cap = (type == T_Q4_K || gemv_grid_covers(type)) ? 16384 : 4096; /* the matrix-instruction kernels' limit */
+    const bool dense = type == T_F32 || type == T_F16 || type == T_BF16;
+    const int cap = (type == T_Q4_K || gemv_grid_covers(type) || dense) ? 16384 : 4096; /* the long-row kernels' limit */
     int range = cap / granule * granule;
     while (cap == 4096 && range > 0 && (size_t)(range / be) * bb > 8192) range -= granule; /* those kernels' row images */
     if (range <= 0) return 0;

@@ -63,6 +63,9 @@ inline JobView job_view(const GemvJob &job) {
 hipError_t launch_gemv_generic(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t stream);
 /* dense F32/F16/BF16 rows of any length and element alignment, one element per lane and step */
 hipError_t launch_gemv_dense_ragged(uint32_t type, const GemvJob &job, const float *x, int n_cols, hipStream_t stream);
+/* dense rows of 4097..16384 elements in one launch; false: not this kernel's shape */
+bool launch_gemv_dense_long(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
+                            hipError_t *err, size_t row_stride = 0);
 /* streaming matvec for every type; returns false if the shape rules of gemv_stream.hip do not
  * hold (nothing was launched), else true with the launch status in *err */
 /* row_stride (all four kernels below): bytes between the rows of a matrix; 0 = the rows are packed. Anything else
