@@ -52,6 +52,31 @@ def test_residual_add_and_several_matrices(oracle, tid, name):
         assert rel_l2(d.to_numpy(np.float32, (r,)), oracle.gemv_f64(tid, W, x, n_cols)) <= TOL, name
 
 
+# dense rows of 4097..16384 elements take one launch of their own kernel: the longest it takes (64 KB of x in LDS), the
+# shortest, many rows per workgroup; then a residual add and three matrices in one launch
+@pytest.mark.parametrize("n_rows,n_cols", [(130, 16384), (70, 4104), (5000, 8192), (3, 6000)])
+@pytest.mark.parametrize("tid,name", list(synth.DENSE_TYPES.items()))
+def test_dense_long_rows(oracle, tid, name, n_rows, n_cols):
+    W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + tid)
+    x = synth.make_activation(n_cols, seed=n_cols + tid)
+    res = synth.make_activation(n_rows, seed=3)
+    dW, dx, dy = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(x), qlinear.DevBuf.from_numpy(res)
+    qlinear.gemv_add_dev(tid, dW, dx, dy, n_rows, n_cols)
+    qlinear.sync()
+    rows = np.arange(n_rows) if n_rows <= 400 else np.r_[0:50, n_rows - 50:n_rows]
+    want = res[rows].astype(np.float64) + oracle.gemv_f64(tid, np.ascontiguousarray(W[rows]), x, n_cols)
+    assert rel_l2(dy.to_numpy(np.float32, (n_rows,))[rows], want) <= TOL, (name, n_rows, n_cols)
+    if n_rows == 130:
+        parts = (60, 1, 69)
+        dys = [qlinear.DevBuf(r * 4) for r in parts]
+        offs = np.cumsum((0,) + parts)
+        dWs = [qlinear.DevBuf.from_numpy(np.ascontiguousarray(W[offs[i]:offs[i + 1]])) for i in range(3)]
+        qlinear.gemv_multi_dev(tid, dWs, dys, list(parts), dx, n_cols)
+        qlinear.sync()
+        got = np.concatenate([d.to_numpy(np.float32, (r,)) for d, r in zip(dys, parts)])
+        assert rel_l2(got, oracle.gemv_f64(tid, W, x, n_cols)) <= TOL, name
+
+
 @pytest.mark.parametrize("tid", [synth.GGML_Q6_K, synth.GGML_Q3_K, synth.GGML_IQ2_XXS, synth.GGML_Q8_0])
 def test_gate_up_silu_on_rows_off_the_16_byte_grid(oracle, tid):
     n_rows, n_cols = 45, 11008
