@@ -26,9 +26,11 @@
  *     (2 shift-adds, 2 converts, 4 multiply-adds per sub-block and row). About 60 vector instructions per
  *     (16 rows x super-block) instead of the ~150 per row of a v_dot4 formulation.
  *  3. Lane (n, g) loads the header and its two 16-byte code chunks of row 16*rg + n directly from HBM:
- *     per instruction 16 rows x 64 contiguous bytes. Four row groups (12 loads) are in flight per
- *     wave before the first is used; waves never wait for each other until the final sum over the 16
- *     super-block shares of a row, which meets in LDS.
+ *     per instruction 16 rows x 64 contiguous bytes. One row group (3 loads) is in flight per wave - the
+ *     sixteen waves of a compute unit keep the requests coming, and a wave that requested several row groups
+ *     together measured slower; waves never wait for each other until the final sum over the 16
+ *     super-block shares of a row, which meets in LDS. A workgroup takes up to 640 rows (one workgroup per
+ *     compute unit up to 163840 rows, equal rounds of them beyond).
  *
  * Measured alternatives on this part (14336x4096, period per launch; a bare read of the same bytes with
  * contiguous 1 KB-per-instruction loads is 6.2 us, with this kernel's access pattern 7.3 us): rows copied
@@ -36,7 +38,7 @@
  * 10.3-11.2 us (waves stuck in issue reach the barrier late, and LDS instructions of other waves slow
  * the incoming copy stream); dedicated copying waves that publish their progress in LDS 10.4 us; each
  * wave gathering its own 144-byte blocks into LDS 16 us (a gather of short runs costs one access per
- * lane); a v_dot4 kernel with one row per wave in LDS 8.3-8.6 us, the same as this one, which needs a
+ * lane); a v_dot4 kernel with one row per wave in LDS 8.3-8.6 us, against 7.9-8.4 us for this one, which needs a
  * third of the vector instructions and no LDS for the weights.
  *
  * A non-finite x makes every output NaN (the fixed-point form cannot carry Inf).
@@ -53,7 +55,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 16;             /* wavefronts per workgroup */
 constexpr int kMaxKc = 4;               /* 16-super-block column chunks: K <= 16384 */
-constexpr int kMaxRowsPerWg = 640; /* local rows (both matrices of a gate+up pair): 40 KB of partial sums */
+constexpr int kMaxRowsPerWg = 640;      /* local rows (both matrices of a gate+up pair): 40 KB of partial sums */
 constexpr int kXScratch = 1088;         /* per wave: 4 digit planes x 256 B + 8 x (2^(e-30), sum) */
 /* x operand of one super-block: A[2p+h] for chain p, instruction h; scale[p] = 2^(e-30) and
  * sum[p] = sum of x for sub-block 4p + lane/16 */
