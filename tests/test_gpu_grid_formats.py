@@ -51,9 +51,9 @@ def test_outlier_and_tiny_activations(oracle, tid):
     assert rel_l2(dy.to_numpy(np.float32, (n_rows,)), oracle.gemv_f64(tid, W, x, n_cols)) <= TOL
 
 
+@pytest.mark.parametrize("n_rows,n_cols", [(203, 8192), (203, 4096), (9000, 2048)])
 @pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
-def test_gate_up_silu(oracle, tid):
-    n_rows, n_cols = 203, 8192
+def test_gate_up_silu(oracle, tid, n_rows, n_cols):
     Wg = synth.make_weights(tid, n_rows, n_cols, seed=11)
     Wu = synth.make_weights(tid, n_rows, n_cols, seed=12)
     x = synth.make_activation(n_cols, seed=13) * np.float32(0.02)
@@ -77,10 +77,10 @@ def test_projection_plus_residual_twice(oracle, tid):
 
 
 # row counts that put the matrices' borders inside a row group and inside a workgroup
-@pytest.mark.parametrize("rows", [(40, 9, 9), (16, 16, 0), (300, 7, 100)])
+@pytest.mark.parametrize("rows,n_cols", [((40, 9, 9), 5120), ((16, 16, 0), 5120), ((300, 7, 100), 5120),
+                                         ((4096, 1024, 1024), 4096), ((5000, 3, 700), 3072)])
 @pytest.mark.parametrize("tid", sorted(GRID), ids=lambda t: GRID[t])
-def test_several_matrices_one_launch(oracle, tid, rows):
-    n_cols = 5120
+def test_several_matrices_one_launch(oracle, tid, rows, n_cols):
     Ws = [synth.make_weights(tid, max(r, 1), n_cols, seed=41 + i) for i, r in enumerate(rows)]
     x = synth.make_activation(n_cols, seed=44)
     dWs = [qlinear.DevBuf.from_numpy(W) for W in Ws]
