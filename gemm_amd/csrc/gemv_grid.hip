@@ -1,14 +1,14 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
  * y[r] = sum over 16- or 32-element groups of scale(r, group) * (codes . x_group) (- offset * sum of x_group), with
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
- * :1505-1534 (Q2_K), :1536-1580 (Q3_K) and :2864-2915 (Q4_1, Q5_0, Q5_1).
+ * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1) and :2818-2830 (MXFP4).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -550,8 +550,8 @@ template <> struct GridFmt<T_Q3_K> {
 struct Table16 {
     uint32_t t0, t1, t2, t3;
 };
-__device__ __forceinline__ Table16 iq4_table() {
-    const uint4 v = *reinterpret_cast<const uint4 *>(qlin_iq4nl_values);
+__device__ __forceinline__ Table16 table16(const int8_t *values) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(values);
     const Table16 t = {v.x, v.y, v.z, v.w};
     return t;
 }
@@ -587,7 +587,7 @@ template <uint32_t T> struct Nibble18 {
     }
     __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
         const uint32_t w[9] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c};
-        const Table16 tab = iq4_table();
+        const Table16 tab = table16(qlin_iq4nl_values);
         float acc = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -618,6 +618,58 @@ template <uint32_t T> struct Nibble18 {
 };
 template <> struct GridFmt<T_IQ4_NL> : Nibble18<T_IQ4_NL> {};
 template <> struct GridFmt<T_Q4_0> : Nibble18<T_Q4_0> {};
+
+/* MXFP4 [e][16 nibble bytes] (common/ggml_dequant.h:2818-2830), 17 bytes: table[nibble] * 2^(e - 127) / 2, low
+ * nibbles first as in IQ4_NL; 136 bytes per 256 elements. Lane group g takes blocks 2g and 2g + 1, the 34 bytes from
+ * byte 34 g - which is 2 (mod 4) for odd g: nine aligned dwords from two bytes earlier there, and byte shifts. */
+template <> struct GridFmt<T_MXFP4> {
+    static constexpr int kBlock = 136, kGridBytes = 0;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = false, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        u32x4_a4 a, b;
+        uint32_t c;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const uint8_t *p = blk + 34 * g - 2 * (g & 1);
+        r.a = *reinterpret_cast<const u32x4_a4 *>(p);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        r.c = *reinterpret_cast<const uint32_t *>(p + 32);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t w[9] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c};
+        const Table16 tab = table16(qlin_mxfp4_values);
+        const uint32_t odd = (uint32_t)g & 1u; /* the piece starts two bytes into w */
+        float acc = 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint32_t qs[4]; /* block 0: the nibble bytes start 1 (3) bytes into dword 0; block 1: 2 bytes into dword 4 (at dword 5) */
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (h == 0) qs[i] = __builtin_amdgcn_alignbit(w[i + 1], w[i], 8u + 16u * odd);
+                else qs[i] = odd ? w[5 + i] : __builtin_amdgcn_alignbit(w[5 + i], w[4 + i], 16);
+            }
+            v4i c = {0, 0, 0, 0};
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                v4i b;
+#pragma unroll
+                for (int i = 0; i < 4; i++) b[i] = look4((qs[i] >> (4 * u)) & 0x0F0F0F0Fu, tab);
+                const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * (2 * h + u));
+                const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+                c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+            }
+            const uint32_t e = (h == 0 ? w[0] >> (16u * odd) : w[4] >> (8u + 16u * odd)) & 0xFFu;
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + h], e8m0_half(e), acc);
+        }
+        return acc;
+    }
+};
 
 /* Q4_1 [d][m][16 nibble bytes] (common/ggml_dequant.h:2864-2877), Q5_0 [d][qh 4][16] (:2879-2895) and Q5_1
  * [d][m][qh 4][16] (:2897-2915): blocks of 32 elements in 20, 22 and 24 bytes; element l < 16 is the low nibble of
@@ -722,7 +774,7 @@ template <> struct GridFmt<T_IQ4_XS> {
     }
     __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
         const uint32_t qs[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
-        const Table16 tab = iq4_table();
+        const Table16 tab = table16(qlin_iq4nl_values);
         float acc = 0.0f;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -997,6 +1049,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     if (n_sb < 8) return false;
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
+    case T_MXFP4: return true; /* 14336: 13.4 -> 11.2, 151936: 98 -> 74 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
     case T_Q4_1: case T_Q5_0: case T_Q5_1: return n_rows <= 32768; /* 14336: 10.5 -> 9.3, 12.1 -> 10.0, 12.0 -> 10.3; 151936: 67 -> 88 */
@@ -1048,7 +1101,7 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1069,6 +1122,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_Q4_1: return grid_typed<T_Q4_1>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q5_0: return grid_typed<T_Q5_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q5_1: return grid_typed<T_Q5_1>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_MXFP4: return grid_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
