@@ -1,14 +1,15 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
  * y[r] = sum over 16- or 32-element groups of scale(r, group) * (codes . x_group) (- offset * sum of x_group), with
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
- * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1) and :2818-2830 (MXFP4).
+ * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
+ * :2832-2848 (NVFP4).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -671,6 +672,47 @@ template <> struct GridFmt<T_MXFP4> {
     }
 };
 
+/* NVFP4 [4 x ue4m3 scale][32 nibble bytes] per 64 elements (common/ggml_dequant.h:2832-2848), 36 bytes: sub-block s
+ * of 16 elements is table[nibble] * scale_s over bytes 8 s .. 8 s + 7, low nibbles first. Lane group g takes block g
+ * of the 256 elements, nine dwords; an instruction is one sub-block. */
+template <> struct GridFmt<T_NVFP4> {
+    static constexpr int kBlock = 144, kGridBytes = 0;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = false, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        u32x4_a4 a, b;
+        uint32_t c;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const uint8_t *p = blk + 36 * g;
+        r.a = *reinterpret_cast<const u32x4_a4 *>(p);
+        r.b = *reinterpret_cast<const u32x4_a4 *>(p + 16);
+        r.c = *reinterpret_cast<const uint32_t *>(p + 32);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t w[9] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w, r.c};
+        const Table16 tab = table16(qlin_mxfp4_values);
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const uint32_t q0 = w[1 + 2 * st], q1 = w[2 + 2 * st];
+            const v4i b = {look4(q0 & 0x0F0F0F0Fu, tab), look4(q1 & 0x0F0F0F0Fu, tab), look4((q0 >> 4) & 0x0F0F0F0Fu, tab),
+                           look4((q1 >> 4) & 0x0F0F0F0Fu, tab)};
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * st);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + (st >> 1)], ue4m3_half((w[0] >> (8 * st)) & 0xFFu), acc);
+        }
+        return acc;
+    }
+};
+
 /* Q4_1 [d][m][16 nibble bytes] (common/ggml_dequant.h:2864-2877), Q5_0 [d][qh 4][16] (:2879-2895) and Q5_1
  * [d][m][qh 4][16] (:2897-2915): blocks of 32 elements in 20, 22 and 24 bytes; element l < 16 is the low nibble of
  * byte l (+ 16 x bit l of qh), element 16 + l the high nibble (+ 16 x bit 16 + l); Q4_1 and Q5_1 add m, Q5_0
@@ -1049,7 +1091,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     if (n_sb < 8) return false;
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
-    case T_MXFP4: return true; /* 14336: 13.4 -> 11.2, 151936: 98 -> 74 */
+    case T_MXFP4: case T_NVFP4: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5; 151936: 98 -> 74, 162 -> 88 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
     case T_Q4_1: case T_Q5_0: case T_Q5_1: return n_rows <= 32768; /* 14336: 10.5 -> 9.3, 12.1 -> 10.0, 12.0 -> 10.3; 151936: 67 -> 88 */
@@ -1101,7 +1143,7 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1123,6 +1165,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_Q5_0: return grid_typed<T_Q5_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q5_1: return grid_typed<T_Q5_1>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_MXFP4: return grid_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_NVFP4: return grid_typed<T_NVFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
