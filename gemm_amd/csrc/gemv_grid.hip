@@ -1,7 +1,7 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
@@ -9,7 +9,7 @@
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
  * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
- * :2832-2848 (NVFP4).
+ * :2832-2848 (NVFP4), :3161-3176 (TQ2_0).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -472,6 +472,46 @@ template <> struct GridFmt<T_Q2_K> {
             mins = fmaf((float)(w >> 4), xo.meta[8 + (e0 >> 4)], mins);
         }
         return half_bits_fast(r.dd & 0xFFFFu) * dots - half_bits_fast(r.dd >> 16) * mins;
+    }
+};
+
+/* TQ2_0 [qs 64][d] (common/ggml_dequant.h:3161-3176), 66 bytes: element 128 h + 32 l + m (m < 32) is bits 2l, 2l+1
+ * of qs[32 h + m], minus 1, times d. Lane group g = (h, p) takes m in [16 p, 16 p + 16) of all four l, as Q6_K; the
+ * codes stay unsigned (0..2) and the -1 goes onto the sum of x. */
+template <> struct GridFmt<T_TQ2_0> {
+    static constexpr int kBlock = 66, kGridBytes = 0;
+    static constexpr int kPiece = 0, kAlign = 2;
+    static constexpr int kStep = 32;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 128 * (g >> 1) + 32 * st + 16 * (g & 1); }
+    struct Raw {
+        Raw16 qs;
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load16(blk + 16 * g);
+        r.d = *reinterpret_cast<const uint16_t *>(blk + 64);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &, int g) {
+        uint32_t qs[4];
+        bytes16(r.qs, sh, qs);
+        float acc = 0.0f;
+#pragma unroll
+        for (int l = 0; l < 4; l++) {
+            v4i b;
+#pragma unroll
+            for (int i = 0; i < 4; i++) b[i] = (int)((qs[i] >> (2 * l)) & 0x03030303u);
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * l);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+            const int e0 = elem0(g, l);
+            acc += fmaf(join_digits(c), xo.meta[e0 >> 5], -xo.meta[8 + (e0 >> 4)]);
+        }
+        return half_bits_fast(r.d) * acc;
     }
 };
 
@@ -1091,7 +1131,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     if (n_sb < 8) return false;
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
-    case T_MXFP4: case T_NVFP4: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5; 151936: 98 -> 74, 162 -> 88 */
+    case T_MXFP4: case T_NVFP4: case T_TQ2_0: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5, 11.7 -> 7.4; 151936: 98 -> 74, 162 -> 88, 93 -> 43 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
     case T_Q4_1: case T_Q5_0: case T_Q5_1: return n_rows <= 32768; /* 14336: 10.5 -> 9.3, 12.1 -> 10.0, 12.0 -> 10.3; 151936: 67 -> 88 */
@@ -1143,7 +1183,7 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1166,6 +1206,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_Q5_1: return grid_typed<T_Q5_1>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_MXFP4: return grid_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_NVFP4: return grid_typed<T_NVFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_TQ2_0: return grid_typed<T_TQ2_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
