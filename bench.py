@@ -681,6 +681,13 @@ def main():
             extra["moe_ffn_128x(768x2048)_64tok_top8_%s" % label] = {
                 "us": round(mm * 1e3, 1), "bytes": bb, "GB/s": round(bb / (mm * 1e-3) / 1e9, 1),
                 "hbm_frac": round(bb / (mm * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        # decode: one token (the reference's own MoE block) and a few, each token's eight experts read for it alone
+        few = {}
+        for nt in (1, 2, 4, 8, 16):
+            mm, bb, _, rr = time_moe(max(10, args.steps // 10), 3, n_tok=nt)
+            few["%d_tok" % nt] = {"us": round(mm * 1e3, 1), "routed_experts": rr,
+                                  "GB/s_of_routed_expert_bytes": round(bb / (mm * 1e-3) / 1e9, 1)}
+        extra["q4k_moe_ffn_128x(768x2048)_top8_few_tokens"] = few
         extra["q4k_moe_ffn_128x(768x2048)_64tok_top8"] = {
             "us": round(m * 1e3, 1), "routed_experts": routed, "bytes": b, "GB/s": round(b / (m * 1e-3) / 1e9, 1),
             "hbm_frac": round(b / (m * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "TFLOP/s": round(fl / (m * 1e-3) / 1e12, 1)}

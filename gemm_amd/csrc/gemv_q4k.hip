@@ -64,6 +64,100 @@ struct XOperand {
     float scale[2], sum[2];
 };
 
+/* x -> signed digit planes -> A operands, wave-private (xs: the wave's kXScratch bytes of LDS) */
+__device__ __forceinline__ void q4k_prepare(v4f v, XOperand &xo, uint8_t *xs, int lane) {
+    const int n = lane & 15, g = lane >> 4;
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    float sum = (v.x + v.y) + (v.z + v.w);
+    /* 8 consecutive lanes share one 32-element sub-block */
+    amax = fmaxf(amax, dpp_mov<0xB1>(amax));
+    amax = fmaxf(amax, dpp_mov<0x4E>(amax));
+    amax = fmaxf(amax, dpp_mov<0x141>(amax));
+    sum += dpp_mov<0xB1>(sum);
+    sum += dpp_mov<0x4E>(sum);
+    sum += dpp_mov<0x141>(sum);
+    int e = (int)(__float_as_uint(amax) >> 23) - 126; /* amax in [2^(e-1), 2^e) */
+    if (e < -96) e = -96;                              /* zero and tiny sub-blocks */
+    const float up = __uint_as_float((uint32_t)(127 + 30 - e) << 23);
+    float down = __uint_as_float((uint32_t)(127 - 30 + e) << 23);
+    if (!(amax <= 3.0e38f)) down = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
+    const int X[4] = {__float2int_rn(v.x * up), __float2int_rn(v.y * up), __float2int_rn(v.z * up),
+                      __float2int_rn(v.w * up)};
+    /* The four signed base-256 digits of X (X = 256*X1 + d0 with d0 = (int8)X, X1 = 256*X2 + d1, ...;
+     * the top one in [-64, 64]) are the bytes of (X + 0x00808080) ^ 0x00808080: adding 128 at a byte makes its
+     * digit unsigned and carries exactly when the digit is negative, the xor takes the 128 off again. */
+    uint32_t Z[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) Z[k] = ((uint32_t)X[k] + 0x00808080u) ^ 0x00808080u;
+    /* byte transpose: plane j = byte j of Z[0..3] (selector 0-3: second operand, 4-7: first) */
+    const uint32_t lo01 = __builtin_amdgcn_perm(Z[1], Z[0], 0x05010400u), lo23 = __builtin_amdgcn_perm(Z[3], Z[2], 0x05010400u);
+    const uint32_t hi01 = __builtin_amdgcn_perm(Z[1], Z[0], 0x07030602u), hi23 = __builtin_amdgcn_perm(Z[3], Z[2], 0x07030602u);
+    uint32_t *pl = reinterpret_cast<uint32_t *>(xs);
+    pl[lane] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);       /* digit 3 (top) */
+    pl[64 + lane] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  /* digit 2 */
+    pl[128 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u); /* digit 1 */
+    pl[192 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); /* digit 0 */
+    if ((lane & 7) == 0) reinterpret_cast<float2 *>(xs + 1024)[lane >> 3] = make_float2(down, sum);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    /* A operand: x-row i = lane%16 = 4*s' + plane; k group lane/16 carries sub-blocks 2*(g>>1)
+     * (registers 0-1) and 2*(g>>1)+1 (registers 2-3) of the chain, elements 16*(g&1) + 8h .. +7 */
+    const int sq = n >> 2, plane = n & 3;
+    const bool live = (g >> 1) == (sq >> 1);
+    const uint8_t *src = xs + plane * 256 + 32 * sq + 16 * (g & 1);
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const uint2 d = *reinterpret_cast<const uint2 *>(src + 128 * p + 8 * h);
+            const bool lo = live && !(sq & 1), hi = live && (sq & 1);
+            v4i a;
+            a.x = lo ? (int)d.x : 0;
+            a.y = lo ? (int)d.y : 0;
+            a.z = hi ? (int)d.x : 0;
+            a.w = hi ? (int)d.y : 0;
+            xo.A[2 * p + h] = a;
+        }
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const float2 m = reinterpret_cast<const float2 *>(xs + 1024)[4 * p + g];
+        xo.scale[p] = m.x;
+        xo.sum[p] = m.y;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+/* one super-block of 16 rows: header hh, code bytes qa (chain 0) and qb (chain 1) of this lane; g = lane / 16 */
+__device__ __forceinline__ float q4k_item(const XOperand &xo, const uint4 hh, const uint4 qa, const uint4 qb, int g) {
+    constexpr uint32_t M = 0x0F0F0F0Fu;
+    v4i c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
+    v4i b;
+    b.x = (int)(qa.x & M); b.y = (int)(qa.y & M); b.z = (int)((qa.x >> 4) & M); b.w = (int)((qa.y >> 4) & M);
+    c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[0], b, c0, 0, 0, 0);
+    b.x = (int)(qb.x & M); b.y = (int)(qb.y & M); b.z = (int)((qb.x >> 4) & M); b.w = (int)((qb.y >> 4) & M);
+    c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2], b, c1, 0, 0, 0);
+    b.x = (int)(qa.z & M); b.y = (int)(qa.w & M); b.z = (int)((qa.z >> 4) & M); b.w = (int)((qa.w >> 4) & M);
+    c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[1], b, c0, 0, 0, 0);
+    b.x = (int)(qb.z & M); b.y = (int)(qb.w & M); b.z = (int)((qb.z >> 4) & M); b.w = (int)((qb.w >> 4) & M);
+    c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[3], b, c1, 0, 0, 0);
+    /* 6-bit scale and min of sub-blocks g (chain 0) and 4+g (chain 1) */
+    const uint32_t sh = 8u * (uint32_t)g;
+    const uint32_t sc0 = __builtin_amdgcn_ubfe(hh.y, sh, 6), mn0 = __builtin_amdgcn_ubfe(hh.z, sh, 6);
+    const uint32_t sc1 = __builtin_amdgcn_ubfe(hh.w, sh, 4) | (__builtin_amdgcn_ubfe(hh.y, sh + 6, 2) << 4);
+    const uint32_t mn1 = __builtin_amdgcn_ubfe(hh.w, sh + 4, 4) | (__builtin_amdgcn_ubfe(hh.z, sh + 6, 2) << 4);
+    const float d = half_bits_fast(hh.x & 0xFFFFu), dmin = half_bits_fast(hh.x >> 16);
+    /* digit sums: |top| <= 32*15*64, the others <= 32*15*128, so each pair below is an integer of less
+     * than 24 bits and its conversion is exact; one rounding in the multiply-add that joins them */
+    const float s0 = fmaf((float)((c0.x << 8) + c0.y), 65536.0f, (float)((c0.z << 8) + c0.w));
+    const float s1 = fmaf((float)((c1.x << 8) + c1.y), 65536.0f, (float)((c1.z << 8) + c1.w));
+    const float z0 = s0 * xo.scale[0], z1 = s1 * xo.scale[1];
+    const float dots = (float)sc0 * z0 + (float)sc1 * z1;
+    const float mins = (float)mn0 * xo.sum[0] + (float)mn1 * xo.sum[1];
+    return d * dots - dmin * mins;
+}
+
 }  // namespace
 
 /* ONE: the job is one matrix, stored or added to y (the matrix and row of a local row then need no searching:
@@ -114,99 +208,8 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
         if (kc < n_kc) v = *reinterpret_cast<const v4f *>(x + (16 * kc + wv) * 256 + 4 * lane);
         xr[kc] = v;
     }
-        /* x -> signed digit planes -> A operands, wave-private */
-    auto prepare = [&](v4f v, XOperand &xo) {
-        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        float sum = (v.x + v.y) + (v.z + v.w);
-        /* 8 consecutive lanes share one 32-element sub-block */
-        amax = fmaxf(amax, dpp_mov<0xB1>(amax));
-        amax = fmaxf(amax, dpp_mov<0x4E>(amax));
-        amax = fmaxf(amax, dpp_mov<0x141>(amax));
-        sum += dpp_mov<0xB1>(sum);
-        sum += dpp_mov<0x4E>(sum);
-        sum += dpp_mov<0x141>(sum);
-        int e = (int)(__float_as_uint(amax) >> 23) - 126; /* amax in [2^(e-1), 2^e) */
-        if (e < -96) e = -96;                              /* zero and tiny sub-blocks */
-        const float up = __uint_as_float((uint32_t)(127 + 30 - e) << 23);
-        float down = __uint_as_float((uint32_t)(127 - 30 + e) << 23);
-        if (!(amax <= 3.0e38f)) down = __uint_as_float(0x7FC00000u); /* Inf/NaN in x: poison every row */
-        const int X[4] = {__float2int_rn(v.x * up), __float2int_rn(v.y * up), __float2int_rn(v.z * up),
-                          __float2int_rn(v.w * up)};
-        /* The four signed base-256 digits of X (X = 256*X1 + d0 with d0 = (int8)X, X1 = 256*X2 + d1, ...;
-         * the top one in [-64, 64]) are the bytes of (X + 0x00808080) ^ 0x00808080: adding 128 at a byte makes its
-         * digit unsigned and carries exactly when the digit is negative, the xor takes the 128 off again. */
-        uint32_t Z[4];
-#pragma unroll
-        for (int k = 0; k < 4; k++) Z[k] = ((uint32_t)X[k] + 0x00808080u) ^ 0x00808080u;
-        /* byte transpose: plane j = byte j of Z[0..3] (selector 0-3: second operand, 4-7: first) */
-        const uint32_t lo01 = __builtin_amdgcn_perm(Z[1], Z[0], 0x05010400u), lo23 = __builtin_amdgcn_perm(Z[3], Z[2], 0x05010400u);
-        const uint32_t hi01 = __builtin_amdgcn_perm(Z[1], Z[0], 0x07030602u), hi23 = __builtin_amdgcn_perm(Z[3], Z[2], 0x07030602u);
-        uint32_t *pl = reinterpret_cast<uint32_t *>(xs);
-        pl[lane] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);       /* digit 3 (top) */
-        pl[64 + lane] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);  /* digit 2 */
-        pl[128 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u); /* digit 1 */
-        pl[192 + lane] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u); /* digit 0 */
-        if ((lane & 7) == 0) reinterpret_cast<float2 *>(xs + 1024)[lane >> 3] = make_float2(down, sum);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        /* A operand: x-row i = lane%16 = 4*s' + plane; k group lane/16 carries sub-blocks 2*(g>>1)
-         * (registers 0-1) and 2*(g>>1)+1 (registers 2-3) of the chain, elements 16*(g&1) + 8h .. +7 */
-        const int sq = n >> 2, plane = n & 3;
-        const bool live = (g >> 1) == (sq >> 1);
-        const uint8_t *src = xs + plane * 256 + 32 * sq + 16 * (g & 1);
-#pragma unroll
-        for (int p = 0; p < 2; p++)
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const uint2 d = *reinterpret_cast<const uint2 *>(src + 128 * p + 8 * h);
-                const bool lo = live && !(sq & 1), hi = live && (sq & 1);
-                v4i a;
-                a.x = lo ? (int)d.x : 0;
-                a.y = lo ? (int)d.y : 0;
-                a.z = hi ? (int)d.x : 0;
-                a.w = hi ? (int)d.y : 0;
-                xo.A[2 * p + h] = a;
-            }
-#pragma unroll
-        for (int p = 0; p < 2; p++) {
-            const float2 m = reinterpret_cast<const float2 *>(xs + 1024)[4 * p + g];
-            xo.scale[p] = m.x;
-            xo.sum[p] = m.y;
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-    };
-
-
-    /* one super-block of 16 rows: header h, code bytes q0 (chain 0) and q1 (chain 1) of this lane */
-    auto item = [&](const XOperand &xo, const uint4 hh, const uint4 qa, const uint4 qb) {
-        constexpr uint32_t M = 0x0F0F0F0Fu;
-        v4i c0 = {0, 0, 0, 0}, c1 = {0, 0, 0, 0};
-        v4i b;
-        b.x = (int)(qa.x & M); b.y = (int)(qa.y & M); b.z = (int)((qa.x >> 4) & M); b.w = (int)((qa.y >> 4) & M);
-        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[0], b, c0, 0, 0, 0);
-        b.x = (int)(qb.x & M); b.y = (int)(qb.y & M); b.z = (int)((qb.x >> 4) & M); b.w = (int)((qb.y >> 4) & M);
-        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[2], b, c1, 0, 0, 0);
-        b.x = (int)(qa.z & M); b.y = (int)(qa.w & M); b.z = (int)((qa.z >> 4) & M); b.w = (int)((qa.w >> 4) & M);
-        c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[1], b, c0, 0, 0, 0);
-        b.x = (int)(qb.z & M); b.y = (int)(qb.w & M); b.z = (int)((qb.z >> 4) & M); b.w = (int)((qb.w >> 4) & M);
-        c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[3], b, c1, 0, 0, 0);
-        /* 6-bit scale and min of sub-blocks g (chain 0) and 4+g (chain 1) */
-        const uint32_t sh = 8u * (uint32_t)g;
-        const uint32_t sc0 = __builtin_amdgcn_ubfe(hh.y, sh, 6), mn0 = __builtin_amdgcn_ubfe(hh.z, sh, 6);
-        const uint32_t sc1 = __builtin_amdgcn_ubfe(hh.w, sh, 4) | (__builtin_amdgcn_ubfe(hh.y, sh + 6, 2) << 4);
-        const uint32_t mn1 = __builtin_amdgcn_ubfe(hh.w, sh + 4, 4) | (__builtin_amdgcn_ubfe(hh.z, sh + 6, 2) << 4);
-        const float d = half_bits_fast(hh.x & 0xFFFFu), dmin = half_bits_fast(hh.x >> 16);
-        /* digit sums: |top| <= 32*15*64, the others <= 32*15*128, so each pair below is an integer of less
-         * than 24 bits and its conversion is exact; one rounding in the multiply-add that joins them */
-        const float s0 = fmaf((float)((c0.x << 8) + c0.y), 65536.0f, (float)((c0.z << 8) + c0.w));
-        const float s1 = fmaf((float)((c1.x << 8) + c1.y), 65536.0f, (float)((c1.z << 8) + c1.w));
-        const float z0 = s0 * xo.scale[0], z1 = s1 * xo.scale[1];
-        const float dots = (float)sc0 * z0 + (float)sc1 * z1;
-        const float mins = (float)mn0 * xo.sum[0] + (float)mn1 * xo.sum[1];
-        return d * dots - dmin * mins;
-    };
+    auto prepare = [&](v4f v, XOperand &xo) { q4k_prepare(v, xo, xs, lane); };
+    auto item = [&](const XOperand &xo, const uint4 hh, const uint4 qa, const uint4 qb) { return q4k_item(xo, hh, qa, qb, g); };
     auto row_pointer = [&](int rg) { /* this lane's row of row group rg (rows past the end: the last one, never stored) */
         int lr = 16 * rg + n;
         if (lr >= n_lrows) lr = n_lrows - 1;
@@ -303,6 +306,134 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
             ym[r] = job.mode == 1 ? ym[r] + s : s;
         }
     }
+}
+
+/* A token (or a few, each on its own) through its top_k routed experts, Q4_K expert tensors (the reference's MoE block for a token,
+ * common/transformer.h:4045-4131: sum_j w_j * down_e(silu(gate_e x) * up_e x), e = idx[j]), as two launches of the
+ * matvec above:
+ *   DOWN = false  h[j][r] = silu(gate_e[r,:] . x) * (up_e[r,:] . x), r < rows_per_expert (n_ff); grid (row tiles, tokens x top_k);
+ *                 x is the token's bf16 activations, sb_per_expert = n_embd / 256
+ *   DOWN = true   y[r] = sum_j w_j * (down_e[r,:] . h[j]), r < rows_per_expert (n_embd), grid (row tiles, tokens): ONE matvec over a row of
+ *                 top_k * n_ff elements whose super-blocks sit in different experts, the routing weight folded into
+ *                 its x; sb_per_expert = n_ff / 256. The sum runs in a fixed order.
+ * An expert index outside [0, n_expert) contributes nothing. Wave w owns super-blocks w, w + waves, ... */
+template <bool DOWN>
+__global__ void __launch_bounds__(kWaves * 64)
+moe1_q4k_kernel(const uint8_t *__restrict__ Wa, const uint8_t *__restrict__ Wb, const void *xin,
+                const int32_t *idx, const float *wts, float *y, int top_k,
+                int n_expert, int rows_per_expert, int sb_per_expert, int rows_per_wg, int ldx) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
+    const int n = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * rows_per_wg;
+    int rows_here = rows_per_expert - row0;
+    if (rows_here > rows_per_wg) rows_here = rows_per_wg;
+    const int n_lrows = DOWN ? rows_here : 2 * rows_here; /* gate rows, then up rows */
+    const int n_rg = (n_lrows + 15) >> 4;
+    const size_t row_bytes = (size_t)sb_per_expert * 144, expert_bytes = (size_t)rows_per_expert * row_bytes;
+    const int n_sb = DOWN ? top_k * sb_per_expert : sb_per_expert;
+    const int pair = DOWN ? 0 : (int)blockIdx.y; /* token * top_k + k */
+    if (DOWN) { /* blockIdx.y = token */
+        idx += (size_t)blockIdx.y * top_k;
+        wts += (size_t)blockIdx.y * top_k;
+        xin = static_cast<const float *>(xin) + (size_t)blockIdx.y * top_k * (sb_per_expert * 256);
+        y += (size_t)blockIdx.y * rows_per_expert;
+    } else {
+        xin = static_cast<const uint16_t *>(xin) + (size_t)(pair / top_k) * ldx;
+    }
+    int e_up = 0;
+    if (!DOWN) {
+        e_up = idx[pair];
+        if (e_up < 0 || e_up >= n_expert) return; /* uniform over the workgroup */
+    }
+    uint8_t *xs = lds + wv * kXScratch;
+    float *partial = reinterpret_cast<float *>(lds + n_waves * kXScratch); /* [local row][wave] */
+    for (int lr = lane; lr < n_lrows; lr += 64) partial[lr * n_waves + wv] = 0.0f;
+
+    XOperand xo;
+    for (int sb = wv; sb < n_sb; sb += n_waves) {
+        /* the expert and the super-block inside its rows that this (virtual) super-block is, and its x */
+        int e = e_up, sbi = sb, j = pair;
+        if (DOWN) {
+            j = sb / sb_per_expert;
+            sbi = sb - j * sb_per_expert;
+            e = idx[j];
+            if (e < 0 || e >= n_expert) continue; /* uniform over the wave */
+        }
+        const uint8_t *base_a = Wa + (size_t)e * expert_bytes + (size_t)sbi * 144;
+        const uint8_t *base_b = DOWN ? base_a : Wb + (size_t)e * expert_bytes + (size_t)sbi * 144;
+        for (int rg = 0; rg < n_rg; rg++) {
+            int lr = 16 * rg + n;
+            if (lr >= n_lrows) lr = n_lrows - 1; /* rows past the end: the last one, never stored */
+            const bool second = !DOWN && lr >= rows_here;
+            const uint8_t *blk = (second ? base_b : base_a) + (size_t)(row0 + (second ? lr - rows_here : lr)) * row_bytes;
+            const uint4 h = *reinterpret_cast<const uint4 *>(blk);
+            const uint4 q0 = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+            const uint4 q1 = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
+            if (rg == 0) { /* x is prepared while the first blocks are on their way */
+                v4f v;
+                if (DOWN) {
+                    const float wj = wts[j];
+                    v = *reinterpret_cast<const v4f *>(static_cast<const float *>(xin) + (size_t)j * (sb_per_expert * 256) + sbi * 256 + 4 * lane);
+                    v.x *= wj; v.y *= wj; v.z *= wj; v.w *= wj;
+                } else {
+                    const uint2 b = *reinterpret_cast<const uint2 *>(static_cast<const uint16_t *>(xin) + sbi * 256 + 4 * lane);
+                    v.x = __uint_as_float(b.x << 16); v.y = __uint_as_float(b.x & 0xFFFF0000u);
+                    v.z = __uint_as_float(b.y << 16); v.w = __uint_as_float(b.y & 0xFFFF0000u);
+                }
+                asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w) : : "memory");
+                q4k_prepare(v, xo, xs, lane);
+            }
+            const float part = sum_lane_groups(q4k_item(xo, h, q0, q1, g));
+            const int slr = 16 * rg + n;
+            if (lane < 16 && slr < n_lrows) partial[slr * n_waves + wv] += part;
+        }
+    }
+    __syncthreads();
+    auto row_total = [&](int lr) {
+        const float4 *p = reinterpret_cast<const float4 *>(partial + lr * n_waves);
+        float s = 0.0f;
+        for (int k = 0; k < n_waves / 4; k++) {
+            const float4 v = p[k];
+            s += (v.x + v.y) + (v.z + v.w);
+        }
+        return s;
+    };
+    for (int lr = threadIdx.x; lr < rows_here; lr += blockDim.x) {
+        if (DOWN) y[row0 + lr] = row_total(lr);
+        else y[(size_t)pair * rows_per_expert + row0 + lr] = silu_times(row_total(lr), row_total(rows_here + lr));
+    }
+}
+
+/* false: not a shape for the two launches above (the caller takes its general path) */
+bool launch_moe1_q4k(const void *gate, const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
+                     float *out, float *h, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream,
+                     hipError_t *err) {
+    *err = hipSuccess;
+    if (n_embd % 256 != 0 || n_ff % 256 != 0 || top_k < 1 || n_tok < 1 || n_cu < 1) return false;
+    if ((((uintptr_t)gate | (uintptr_t)up | (uintptr_t)down | (uintptr_t)h) & 15) || ((uintptr_t)X & 7)) return false;
+    auto lds_of = [](int waves, int local_rows) { return (size_t)waves * kXScratch + (size_t)local_rows * waves * 4; };
+    {   /* gate, up, SiLU: top_k experts x n_ff row pairs over the compute units */
+        const int n_pairs = n_tok * top_k;
+        const int tiles = n_cu / n_pairs > 0 ? n_cu / n_pairs : 1;
+        int rows_per_wg = (n_ff + tiles - 1) / tiles;
+        if (2 * rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / 2;
+        const int waves = n_embd / 256 <= 8 ? 8 : kWaves;
+        hipLaunchKernelGGL(moe1_q4k_kernel<false>, dim3((n_ff + rows_per_wg - 1) / rows_per_wg, n_pairs), dim3(waves * 64),
+                           lds_of(waves, 2 * rows_per_wg), stream, (const uint8_t *)gate, (const uint8_t *)up, (const void *)X, idx,
+                           w, h, top_k, n_expert, n_ff, n_embd / 256, rows_per_wg, n_embd);
+    }
+    {
+        const int tiles = n_cu / n_tok > 0 ? n_cu / n_tok : 1;
+        int rows_per_wg = (n_embd + tiles - 1) / tiles;
+        if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
+        hipLaunchKernelGGL(moe1_q4k_kernel<true>, dim3((n_embd + rows_per_wg - 1) / rows_per_wg, n_tok), dim3(kWaves * 64),
+                           lds_of(kWaves, rows_per_wg), stream, (const uint8_t *)down, (const uint8_t *)down, (const void *)h, idx, w,
+                           out, top_k, n_expert, n_embd, n_ff / 256, rows_per_wg, 0);
+    }
+    *err = hipGetLastError();
+    return true;
 }
 
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu, size_t row_stride) {

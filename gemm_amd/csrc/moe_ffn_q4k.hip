@@ -1642,6 +1642,21 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                           int top_k, int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream) {
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
+    /* One token (the reference's own case), or up to eight that will mostly meet different experts (two pairs or
+     * fewer per four experts): each token on its own through two launches of the Q4_K matvec, no grouping and no
+     * combine. 128 experts of 768 x 2048, top-8, us: 1 token 19.9 -> 10.6, 2: 24.3 -> 13.5, 4: 33.5 -> 19.2,
+     * 8: 49.1 -> 37.6; at 12 tokens (76.9 against 61.0) the experts that tokens share are read once per token too often. */
+    if ((n_tok == 1 || (n_tok <= 8 && 2 * n_pairs <= n_expert)) && type_gate == T_Q4_K && type_up == T_Q4_K &&
+        type_down == T_Q4_K) {
+        static int n_cu = 0;
+        if (n_cu == 0) {
+            int dev = 0, v = 0;
+            if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n_cu = v;
+            else n_cu = 256;
+        }
+        hipError_t e1;
+        if (launch_moe1_q4k(gate, up, down, X, idx, w, out, ws.g32, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, &e1)) return e1;
+    }
     /* few pairs per expert: the matrix kernels look their expert up in the list of those that have tokens, and
      * the launch covers no more experts than there are pairs */
     /* up to two pairs per expert (a third or more of the experts unused at random routing): measured faster or equal

@@ -97,6 +97,32 @@ def test_grouped_ffn_small(oracle, n_tok):
     assert rel_l2(numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff), want) <= 1e-6
 
 
+@pytest.mark.parametrize("n_tok", [1, 2, 3, 8, 9])
+def test_few_tokens_many_experts(oracle, n_tok):
+    """one to eight tokens over 64 experts, top-4: each token goes through the matvec kernels on its own (nine tokens:
+    the grouped kernels); one expert twice in a token, an index out of range, and the same bits on a second run"""
+    n_expert, n_embd, n_ff, k = 64, 512, 768, 4
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=900)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=910 + n_tok, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=920 + n_tok), k)
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert)
+    want = oracle_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff)
+    for t in range(n_tok):
+        assert rel_l2(got[t], want[t]) <= DESIGNED, t
+    assert np.array_equal(run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert), got)
+    idx2, w2 = idx.copy(), w.copy()
+    idx2[0, 1] = idx2[0, 0]  # the same expert twice: its output counts with both weights
+    idx2[-1, 2] = n_expert + 5  # out of range: contributes nothing
+    got2 = run_ffn(gate, up, down, Xb, idx2, w2, n_embd, n_ff, n_expert)
+    w3 = w2.copy()
+    w3[-1, 2] = 0.0
+    idx3 = idx2.copy()
+    idx3[-1, 2] = 0
+    want2 = oracle_ffn(oracle, gate, up, down, Xb, idx3, w3, n_embd, n_ff)
+    for t in range(n_tok):
+        assert rel_l2(got2[t], want2[t]) <= DESIGNED, t
+
+
 def test_grouped_ffn_all_tokens_one_expert(oracle):
     """37 tokens on one expert: three passes of 16 token slots, the last one ragged."""
     n_expert, n_embd, n_ff, k, n_tok = 8, 256, 256, 2, 37
