@@ -880,10 +880,39 @@ template <> struct GridFmt<T_IQ4_XS> {
 
 }  // namespace
 
-template <uint32_t T, int NKC>
+/* MOE = 0: the matvec. MOE = 1, 2: a token's routed experts (the reference's MoE block for a token,
+ * common/transformer.h:4045-4131) on the same kernel, as moe1_q4k_kernel (gemv_q4k.hip) does for Q4_K:
+ *   1  gate + up + SiLU of pair blockIdx.y = token * top_k + k: the job's two matrices moved to expert idx[pair], the
+ *      result to h[pair], x the token's bf16 activations;
+ *   2  down of token blockIdx.y: one matvec over a row of top_k * n_ff elements whose super-blocks sit in different
+ *      experts, x = h scaled by the routing weight of the super-block's expert (nothing for an index out of range). */
+struct MoeArgs {
+    const int32_t *idx;
+    const float *wts;
+    int top_k, n_expert, sb_per_expert, ldx; /* ldx: elements between two tokens' activations (MOE = 1) */
+    size_t expert_bytes;
+};
+
+template <uint32_t T, int NKC, int MOE = 0>
 __global__ void __launch_bounds__(kWaves * 64)
-gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes) {
+gemv_grid_kernel(const JobView job_in, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes, const MoeArgs moe) {
     using F = GridFmt<T>;
+    JobView job = job_in;
+    const int32_t *idx = moe.idx;
+    const float *wts = moe.wts;
+    if (MOE == 1) {
+        const int pair = blockIdx.y, e = idx[pair];
+        if (e < 0 || e >= moe.n_expert) return; /* uniform over the workgroup */
+        job.W0 += (size_t)e * moe.expert_bytes;
+        job.W1 += (size_t)e * moe.expert_bytes;
+        job.y0 += (size_t)pair * job.n0;
+        x = reinterpret_cast<const float *>(reinterpret_cast<const uint16_t *>(x) + (size_t)(pair / moe.top_k) * moe.ldx);
+    } else if (MOE == 2) {
+        idx += (size_t)blockIdx.y * moe.top_k;
+        wts += (size_t)blockIdx.y * moe.top_k;
+        x += (size_t)blockIdx.y * n_sb * 256;
+        job.y0 += (size_t)blockIdx.y * job.n0;
+    }
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int lane = threadIdx.x & 63;
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -934,11 +963,39 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
         float *ym;
         int r;
         locate(lr, Wm, ym, r);
-        return Wm + (size_t)r * row_bytes + (size_t)wv * F::kBlock;
+        return Wm + (size_t)r * row_bytes;
+    };
+    /* where in its row the wave's super-block kc sits (MOE = 2: in which expert's copy of the row, too; an index
+     * out of range reads expert 0 and gets zeros for x) */
+    auto sb_off = [&](int kc) {
+        const int s = wv + 16 * kc;
+        if (MOE == 2) {
+            const int j = s / moe.sb_per_expert, e = idx[j];
+            const bool valid = e >= 0 && e < moe.n_expert;
+            return (size_t)(valid ? e : 0) * moe.expert_bytes + (size_t)(s - j * moe.sb_per_expert) * F::kBlock;
+        }
+        return (size_t)s * F::kBlock;
+    };
+    auto moe_x = [&](v4f v, int kc) { /* MOE = 2: the routing weight of the super-block's expert goes onto x */
+        if (MOE == 2) {
+            const int j = (wv + 16 * kc) / moe.sb_per_expert, e = idx[j];
+            const float wj = wts[j];
+            const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
+            v = (e >= 0 && e < moe.n_expert) ? v * wj : zero;
+        }
+        return v;
     };
 
     /* the wave's first super-block of x; later ones are fetched where they are used */
-    auto load_x = [&](int kc) { return *reinterpret_cast<const v4f *>(x + (size_t)(16 * kc + wv) * 256 + 4 * lane); };
+    auto load_x = [&](int kc) {
+        if (MOE == 1) { /* bf16 activations */
+            const uint2 b = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(x) + (size_t)(16 * kc + wv) * 256 + 4 * lane);
+            const v4f v = {__uint_as_float(b.x << 16), __uint_as_float(b.x & 0xFFFF0000u), __uint_as_float(b.y << 16),
+                           __uint_as_float(b.y & 0xFFFF0000u)};
+            return v;
+        }
+        return *reinterpret_cast<const v4f *>(x + (size_t)(16 * kc + wv) * 256 + 4 * lane);
+    };
     v4f xq = {0.0f, 0.0f, 0.0f, 0.0f};
     if (n_kc > 0) xq = load_x(0);
 
@@ -1025,8 +1082,7 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
 #pragma unroll
         for (int q = 0; q < NF; q++) {
             if (long_rows ? q >= 2 : q >= D) break;
-            const uint8_t *blk = long_rows ? row_pointer(0) + (size_t)(q < n_kc ? q : 0) * (16 * F::kBlock)
-                                           : row_pointer(q < n_rg ? q : 0);
+            const uint8_t *blk = long_rows ? row_pointer(0) + sb_off(q < n_kc ? q : 0) : row_pointer(q < n_rg ? q : 0) + sb_off(0);
             first[q] = F::load(blk, g);
             first_sh[q] = shift_of(blk);
         }
@@ -1049,12 +1105,12 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
 #pragma unroll
         for (int kc = 0; kc < NKC; kc++) {
             if (kc < n_kc) {
-                prepare(xq, xo);
+                prepare(moe_x(xq, kc), xo);
                 if (kc + 1 < n_kc) xq = load_x(kc + 1); /* on its way while this super-block is multiplied */
                 acc += F::item(xo, first[kc & 1], first_sh[kc & 1], tab, g);
             }
             if (kc + 2 < n_kc) { /* into the registers just used */
-                const uint8_t *blk = blk0 + (size_t)(kc + 2) * (16 * F::kBlock);
+                const uint8_t *blk = blk0 + sb_off(kc + 2);
                 first[kc & 1] = F::load(blk, g);
                 first_sh[kc & 1] = shift_of(blk);
             }
@@ -1065,12 +1121,12 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
         for (int kc = 0; kc < n_kc; kc++) {
             v4f v = xq;
             if (kc > 0) v = load_x(kc);
-            prepare(v, xo);
+            prepare(moe_x(v, kc), xo);
             /* D row groups in flight: a group's registers are refilled as soon as it has been multiplied */
             if (kc > 0) {
 #pragma unroll
                 for (int q = 0; q < D; q++) {
-                    const uint8_t *blk = row_pointer(q < n_rg ? q : 0) + (size_t)kc * (16 * F::kBlock);
+                    const uint8_t *blk = row_pointer(q < n_rg ? q : 0) + sb_off(kc);
                     first[q] = F::load(blk, g);
                     first_sh[q] = shift_of(blk);
                 }
@@ -1080,7 +1136,7 @@ gemv_grid_kernel(const JobView job, const float *__restrict__ x, int n_sb, int r
                 for (int q = 0; q < D; q++) {
                     if (rg + q < n_rg) store_partial(rg + q, F::item(xo, first[q], first_sh[q], tab, g), kc > 0);
                     if (rg + q + D < n_rg) {
-                        const uint8_t *blk = row_pointer(rg + q + D) + (size_t)kc * (16 * F::kBlock);
+                        const uint8_t *blk = row_pointer(rg + q + D) + sb_off(kc);
                         first[q] = F::load(blk, g);
                         first_sh[q] = shift_of(blk);
                     }
@@ -1170,15 +1226,103 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
     const size_t lds_bytes = (size_t)rows_per_wg * n_mats_here * kWaves * 4; /* the partial sums; the rest is static */
     const JobView view = job_view(job);
     const size_t pitch = row_stride ? row_stride : (size_t)n_sb * GridFmt<T>::kBlock;
+    const MoeArgs none = {nullptr, nullptr, 0, 0, 0, 0, 0};
     if (short_rows)
-        hipLaunchKernelGGL((gemv_grid_kernel<T, 1>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch);
+        hipLaunchKernelGGL((gemv_grid_kernel<T, 1>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none);
     else
-        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch);
+        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none);
     *err = hipGetLastError();
     return true;
 }
 
 }  // namespace
+
+namespace {
+
+template <uint32_t T>
+bool moe1_up_typed(const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h, int n_tok, int top_k,
+                   int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry, hipError_t *err) {
+    using F = GridFmt<T>;
+    const int n_sb = n_embd / 256;
+    const size_t row_bytes = (size_t)n_sb * F::kBlock, expert_bytes = (size_t)n_ff * row_bytes;
+    if (n_embd % 256 != 0 || n_sb > 16 * kMaxKc || n_ff < 1 || top_k < 1 || n_tok < 1) return false;
+    if (((uintptr_t)gate | (uintptr_t)up | expert_bytes) % F::kAlign || ((uintptr_t)X & 7) || ((uintptr_t)h & 15)) return false;
+    if (dry) return true;
+    constexpr int max_rows = F::kGridBytes > 0 ? 128 : kMaxRowsPerWg;
+    const int n_pairs = n_tok * top_k;
+    const int tiles = n_cu / n_pairs > 0 ? n_cu / n_pairs : 1;
+    int rows_per_wg = (n_ff + tiles - 1) / tiles;
+    if (2 * rows_per_wg > max_rows) rows_per_wg = max_rows / 2;
+    GemvJob job = {};
+    job.W[0] = gate; job.W[1] = up; job.y[0] = h;
+    job.n_rows[0] = job.n_rows[1] = n_ff;
+    job.n_mat = 2;
+    job.mode = kSiluMul;
+    const MoeArgs moe = {idx, nullptr, top_k, n_expert, n_sb, n_embd, expert_bytes};
+    const dim3 grid((n_ff + rows_per_wg - 1) / rows_per_wg, n_pairs);
+    const size_t lds_bytes = (size_t)2 * rows_per_wg * kWaves * 4;
+    const float *x = reinterpret_cast<const float *>(X);
+    if (n_sb <= 16)
+        hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 1>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_sb, rows_per_wg, row_bytes, moe);
+    else
+        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 1>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_sb, rows_per_wg, row_bytes, moe);
+    *err = hipGetLastError();
+    return true;
+}
+
+template <uint32_t T>
+bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
+                     int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry, hipError_t *err) {
+    using F = GridFmt<T>;
+    const int sbpe = n_ff / 256, n_sb = top_k * sbpe; /* the row of a token: top_k experts' rows side by side */
+    const size_t row_bytes = (size_t)sbpe * F::kBlock, expert_bytes = (size_t)n_embd * row_bytes;
+    if (n_ff % 256 != 0 || n_sb > 16 * kMaxKc || n_embd < 1 || top_k < 1 || n_tok < 1) return false;
+    if (((uintptr_t)down | row_bytes) % F::kAlign || ((uintptr_t)h & 15)) return false;
+    if (dry) return true;
+    constexpr int max_rows = F::kGridBytes > 0 ? 128 : kMaxRowsPerWg;
+    const int tiles = n_cu / n_tok > 0 ? n_cu / n_tok : 1;
+    int rows_per_wg = (n_embd + tiles - 1) / tiles;
+    if (rows_per_wg > max_rows) rows_per_wg = max_rows;
+    GemvJob job = single_job(down, out, n_embd);
+    const MoeArgs moe = {idx, w, top_k, n_expert, sbpe, 0, expert_bytes};
+    const dim3 grid((n_embd + rows_per_wg - 1) / rows_per_wg, n_tok);
+    const size_t lds_bytes = (size_t)rows_per_wg * kWaves * 4;
+    if (n_sb <= 16)
+        hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), h, n_sb, rows_per_wg, row_bytes, moe);
+    else
+        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), h, n_sb, rows_per_wg, row_bytes, moe);
+    *err = hipGetLastError();
+    return true;
+}
+
+}  // namespace
+
+/* the expert formats of the K-quant and 4-bit mixes; the others keep the grouped kernels */
+#define QLIN_MOE1_TYPES(X) X(T_Q6_K) X(T_Q5_K) X(T_Q8_0) X(T_Q4_0) X(T_IQ4_NL) X(T_IQ4_XS) X(T_Q2_K) X(T_Q3_K) X(T_MXFP4)
+
+bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h,
+                         int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
+                         hipError_t *err) {
+    *err = hipSuccess;
+    switch (type) {
+#define QLIN_CASE(TT) case TT: return moe1_up_typed<TT>(gate, up, X, idx, h, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, dry, err);
+    QLIN_MOE1_TYPES(QLIN_CASE)
+#undef QLIN_CASE
+    default: return false;
+    }
+}
+
+bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, const int32_t *idx, const float *w, float *out,
+                           int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
+                           hipError_t *err) {
+    *err = hipSuccess;
+    switch (type) {
+#define QLIN_CASE(TT) case TT: return moe1_down_typed<TT>(down, h, idx, w, out, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, dry, err);
+    QLIN_MOE1_TYPES(QLIN_CASE)
+#undef QLIN_CASE
+    default: return false;
+    }
+}
 
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||

@@ -406,32 +406,40 @@ moe1_q4k_kernel(const uint8_t *__restrict__ Wa, const uint8_t *__restrict__ Wb, 
     }
 }
 
-/* false: not a shape for the two launches above (the caller takes its general path) */
-bool launch_moe1_q4k(const void *gate, const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
-                     float *out, float *h, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream,
-                     hipError_t *err) {
+/* The two launches above, one function each; false: not a shape for it (the caller takes its general path).
+ * dry: only say whether it would be taken. h: n_tok * top_k * n_ff floats of scratch. */
+bool launch_moe1_q4k_up(const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h, int n_tok,
+                        int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry, hipError_t *err) {
     *err = hipSuccess;
-    if (n_embd % 256 != 0 || n_ff % 256 != 0 || top_k < 1 || n_tok < 1 || n_cu < 1) return false;
-    if ((((uintptr_t)gate | (uintptr_t)up | (uintptr_t)down | (uintptr_t)h) & 15) || ((uintptr_t)X & 7)) return false;
-    auto lds_of = [](int waves, int local_rows) { return (size_t)waves * kXScratch + (size_t)local_rows * waves * 4; };
-    {   /* gate, up, SiLU: top_k experts x n_ff row pairs over the compute units */
-        const int n_pairs = n_tok * top_k;
-        const int tiles = n_cu / n_pairs > 0 ? n_cu / n_pairs : 1;
-        int rows_per_wg = (n_ff + tiles - 1) / tiles;
-        if (2 * rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / 2;
-        const int waves = n_embd / 256 <= 8 ? 8 : kWaves;
-        hipLaunchKernelGGL(moe1_q4k_kernel<false>, dim3((n_ff + rows_per_wg - 1) / rows_per_wg, n_pairs), dim3(waves * 64),
-                           lds_of(waves, 2 * rows_per_wg), stream, (const uint8_t *)gate, (const uint8_t *)up, (const void *)X, idx,
-                           w, h, top_k, n_expert, n_ff, n_embd / 256, rows_per_wg, n_embd);
-    }
-    {
-        const int tiles = n_cu / n_tok > 0 ? n_cu / n_tok : 1;
-        int rows_per_wg = (n_embd + tiles - 1) / tiles;
-        if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
-        hipLaunchKernelGGL(moe1_q4k_kernel<true>, dim3((n_embd + rows_per_wg - 1) / rows_per_wg, n_tok), dim3(kWaves * 64),
-                           lds_of(kWaves, rows_per_wg), stream, (const uint8_t *)down, (const uint8_t *)down, (const void *)h, idx, w,
-                           out, top_k, n_expert, n_embd, n_ff / 256, rows_per_wg, 0);
-    }
+    if (n_embd % 256 != 0 || n_ff < 1 || top_k < 1 || n_tok < 1 || n_cu < 1) return false;
+    if ((((uintptr_t)gate | (uintptr_t)up | (uintptr_t)h) & 15) || ((uintptr_t)X & 7)) return false;
+    if (dry) return true;
+    /* n_tok * top_k experts x n_ff row pairs over the compute units */
+    const int n_pairs = n_tok * top_k;
+    const int tiles = n_cu / n_pairs > 0 ? n_cu / n_pairs : 1;
+    int rows_per_wg = (n_ff + tiles - 1) / tiles;
+    if (2 * rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg / 2;
+    const int waves = n_embd / 256 <= 8 ? 8 : kWaves;
+    hipLaunchKernelGGL(moe1_q4k_kernel<false>, dim3((n_ff + rows_per_wg - 1) / rows_per_wg, n_pairs), dim3(waves * 64),
+                       (size_t)waves * kXScratch + (size_t)2 * rows_per_wg * waves * 4, stream, (const uint8_t *)gate,
+                       (const uint8_t *)up, (const void *)X, idx, (const float *)nullptr, h, top_k, n_expert, n_ff, n_embd / 256,
+                       rows_per_wg, n_embd);
+    *err = hipGetLastError();
+    return true;
+}
+
+bool launch_moe1_q4k_down(const void *down, const float *h, const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
+                          int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry, hipError_t *err) {
+    *err = hipSuccess;
+    if (n_ff % 256 != 0 || n_embd < 1 || top_k < 1 || n_tok < 1 || n_cu < 1) return false;
+    if (((uintptr_t)down | (uintptr_t)h) & 15) return false;
+    if (dry) return true;
+    const int tiles = n_cu / n_tok > 0 ? n_cu / n_tok : 1;
+    int rows_per_wg = (n_embd + tiles - 1) / tiles;
+    if (rows_per_wg > kMaxRowsPerWg) rows_per_wg = kMaxRowsPerWg;
+    hipLaunchKernelGGL(moe1_q4k_kernel<true>, dim3((n_embd + rows_per_wg - 1) / rows_per_wg, n_tok), dim3(kWaves * 64),
+                       (size_t)kWaves * kXScratch + (size_t)rows_per_wg * kWaves * 4, stream, (const uint8_t *)down,
+                       (const uint8_t *)down, (const void *)h, idx, w, out, top_k, n_expert, n_embd, n_ff / 256, rows_per_wg, 0);
     *err = hipGetLastError();
     return true;
 }

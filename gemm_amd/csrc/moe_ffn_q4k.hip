@@ -1645,17 +1645,34 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
     /* One token (the reference's own case), or up to eight that will mostly meet different experts (two pairs or
      * fewer per four experts): each token on its own through two launches of the Q4_K matvec, no grouping and no
      * combine. 128 experts of 768 x 2048, top-8, us: 1 token 19.9 -> 10.6, 2: 24.3 -> 13.5, 4: 33.5 -> 19.2,
-     * 8: 49.1 -> 37.6; at 12 tokens (76.9 against 61.0) the experts that tokens share are read once per token too often. */
-    if ((n_tok == 1 || (n_tok <= 8 && 2 * n_pairs <= n_expert)) && type_gate == T_Q4_K && type_up == T_Q4_K &&
-        type_down == T_Q4_K) {
+     * 8: 49.1 -> 37.6; at 12 tokens (76.9 against 61.0) the experts that tokens share are read once per token too often.
+     * Q4_K experts on the Q4_K matvec, the other common expert formats on the matrix-instruction matvec (gate and up of
+     * one type; 1 token: Q4_K/Q4_K/Q6_K 21.6 -> 13.5, Q6_K 25.9 -> 15.7, Q8_0 26.0 -> 13.2, IQ4_XS 62.7 -> 12.4). */
+    if (n_tok == 1 || (n_tok <= 8 && 2 * n_pairs <= n_expert)) {
         static int n_cu = 0;
         if (n_cu == 0) {
             int dev = 0, v = 0;
             if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n_cu = v;
             else n_cu = 256;
         }
-        hipError_t e1;
-        if (launch_moe1_q4k(gate, up, down, X, idx, w, out, ws.g32, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, &e1)) return e1;
+        hipError_t e1 = hipSuccess;
+        auto up_step = [&](bool dry) {
+            if (type_gate == T_Q4_K && type_up == T_Q4_K)
+                return launch_moe1_q4k_up(gate, up, X, idx, ws.g32, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, dry, &e1);
+            return type_gate == type_up &&
+                   launch_moe1_grid_up(type_gate, gate, up, X, idx, ws.g32, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, dry, &e1);
+        };
+        auto down_step = [&](bool dry) {
+            if (type_down == T_Q4_K)
+                return launch_moe1_q4k_down(down, ws.g32, idx, w, out, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, dry, &e1);
+            return launch_moe1_grid_down(type_down, down, ws.g32, idx, w, out, n_tok, top_k, n_embd, n_ff, n_expert, n_cu, stream, dry, &e1);
+        };
+        if (up_step(true) && down_step(true)) {
+            up_step(false);
+            if (e1 != hipSuccess) return e1;
+            down_step(false);
+            return e1;
+        }
     }
     /* few pairs per expert: the matrix kernels look their expert up in the list of those that have tokens, and
      * the launch covers no more experts than there are pairs */

@@ -83,11 +83,19 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
                       hipStream_t stream, hipError_t *err, size_t row_stride = 0);
 bool gemv_grid_covers(uint32_t type); /* the formats it has an item for */
 /* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
-/* a few tokens, each on its own, through their top_k Q4_K experts as two matvec launches (h: n_tok * top_k * n_ff
- * floats of scratch; X [n_tok, n_embd] bf16); false: not its shape */
-bool launch_moe1_q4k(const void *gate, const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
-                     float *out, float *h, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream,
-                     hipError_t *err);
+/* A few tokens, each on its own, through their top_k experts as two matvec launches: gate + up + SiLU into h
+ * (n_tok * top_k * n_ff floats, X [n_tok, n_embd] bf16), then down with the routing weights folded into h. Q4_K experts
+ * and the formats of the matrix-instruction matvec (gate and up of one type). false: not a shape for it; dry: only say so. */
+bool launch_moe1_q4k_up(const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h, int n_tok,
+                        int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry, hipError_t *err);
+bool launch_moe1_q4k_down(const void *down, const float *h, const int32_t *idx, const float *w, float *out, int n_tok, int top_k,
+                          int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry, hipError_t *err);
+bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h,
+                         int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
+                         hipError_t *err);
+bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, const int32_t *idx, const float *w, float *out,
+                           int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
+                           hipError_t *err);
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu,
                            size_t row_stride = 0);
 

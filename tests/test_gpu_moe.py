@@ -76,7 +76,7 @@ def numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=(Q4K, Q4K,
         g, u = X[toks] @ G.T, X[toks] @ U.T
         with np.errstate(over="ignore"):  # exp(-g) -> inf gives h -> 0, as in fp32
             h = g / (1.0 + np.exp(-g)) * u
-        out[toks] += w[toks, ks].astype(np.float64)[:, None] * (h @ D.T)
+        np.add.at(out, toks, w[toks, ks].astype(np.float64)[:, None] * (h @ D.T))  # a token may name an expert twice
     return out
 
 
@@ -121,6 +121,37 @@ def test_few_tokens_many_experts(oracle, n_tok):
     want2 = oracle_ffn(oracle, gate, up, down, Xb, idx3, w3, n_embd, n_ff)
     for t in range(n_tok):
         assert rel_l2(got2[t], want2[t]) <= DESIGNED, t
+
+
+Q6K, Q5K = synth.GGML_Q6_K, synth.GGML_Q5_K
+FEW_TOKEN_TYPES = [(Q4K, Q4K, Q6K), (Q6K, Q6K, Q6K), (Q5K, Q5K, Q6K), (synth.GGML_Q8_0,) * 3, (synth.GGML_IQ4_XS,) * 3,
+                   (synth.GGML_MXFP4,) * 3, (synth.GGML_Q3_K, synth.GGML_Q3_K, Q4K), (synth.GGML_Q2_K,) * 3,
+                   (synth.GGML_IQ4_NL, synth.GGML_IQ4_NL, synth.GGML_Q4_0), (Q4K, Q6K, Q4K)]
+
+
+@pytest.mark.parametrize("n_tok", [1, 3, 8])
+@pytest.mark.parametrize("types", FEW_TOKEN_TYPES, ids=lambda t: "-".join(ALL_NAMES[x] for x in t))
+def test_few_tokens_other_expert_formats(oracle, types, n_tok):
+    """the same route with the experts in the formats of the matrix-instruction matvec, gate/up and down of different
+    types (the last case, gate and up of different types, keeps the grouped kernels); a repeated expert and an index
+    out of range as above"""
+    n_expert, n_embd, n_ff, k = 64, 512, 768, 4
+    gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=950, types=types)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=960 + n_tok, tokens=n_tok))
+    idx, w = route(oracle, synth.make_router_logits(n_tok, n_expert, seed=970 + n_tok), k)
+    idx[0, 1] = idx[0, 0]
+    got = run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types)
+    want = numpy_ffn(oracle, gate, up, down, Xb, idx, w, n_embd, n_ff, types=types)
+    for t in range(n_tok):
+        assert rel_l2(got[t], want[t]) <= DESIGNED, t
+    idx2 = idx.copy()
+    idx2[-1, 2] = -3
+    w0 = w.copy()
+    w0[-1, 2] = 0.0
+    dropped = run_ffn(gate, up, down, Xb, idx2, w, n_embd, n_ff, n_expert, types=types)
+    zeroed = run_ffn(gate, up, down, Xb, idx, w0, n_embd, n_ff, n_expert, types=types)
+    assert rel_l2(dropped, zeroed) <= 1e-7
+    assert np.array_equal(run_ffn(gate, up, down, Xb, idx, w, n_embd, n_ff, n_expert, types=types), got)
 
 
 def test_grouped_ffn_all_tokens_one_expert(oracle):
