@@ -488,8 +488,8 @@ def probe(args):
     elif args.probe == "decode_step":
         print(json.dumps({"probe": args.probe, **time_decode_step_linear()}))
     elif args.probe == "moe":
-        m, b, fl, routed = time_moe(max(10, args.steps // 20), 3)
-        print(json.dumps({"probe": "moe", "ms_per_step": m, "bytes": b, "routed": routed}))
+        m, b, fl, routed = time_moe(max(10, args.steps // 20), 3, n_tok=args.ptok)  # --ptok N: that many tokens
+        print(json.dumps({"probe": "moe", "tokens": args.ptok, "ms_per_step": m, "bytes": b, "routed": routed}))
     elif args.probe == "gemm":
         ms = time_gemm(512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
@@ -585,6 +585,7 @@ def main():
     ap.add_argument("--ptype", default="iq2_xxs", help="--probe gemv_any: format name")
     ap.add_argument("--prows", type=int, default=4096)
     ap.add_argument("--pcols", type=int, default=14336)
+    ap.add_argument("--ptok", type=int, default=64, help="--probe moe: tokens in the batch")
     ap.add_argument("--probe", choices=["gemv_any", "copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
