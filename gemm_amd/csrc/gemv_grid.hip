@@ -1,7 +1,7 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
@@ -9,7 +9,7 @@
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
  * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
- * :2832-2848 (NVFP4), :3161-3176 (TQ2_0).
+ * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -263,6 +263,93 @@ template <> struct GridFmt<T_IQ3_S> {
             acc = fmaf(join_digits(c) * xo.meta[2 * g + h], (float)(1u + 2u * nib), acc);
         }
         return d * acc;
+    }
+};
+
+/* IQ2_XS [d][32 x (9-bit grid index | 7 sign bits << 9)][8 scale bytes] (common/ggml_dequant.h:2975-2994), 74 bytes:
+ * d * (0.5 + nibble) * 0.25 * grid byte * sign, an eight-byte grid entry per 16-bit code, one scale nibble per 16
+ * elements. Lane group g takes groups 2g, 2g + 1: eight codes; an instruction is the two codes of one nibble. */
+template <> struct GridFmt<T_IQ2_XS> {
+    static constexpr int kBlock = 74, kGridBytes = 4096;
+    static constexpr int kAlign = 2, kPiece = 2;
+    static constexpr int kStep = 16;
+    static constexpr bool kAInRegs = true, kSums = false;
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    __device__ static const uint32_t *grid_src() { return reinterpret_cast<const uint32_t *>(qlin_iq2xs_grid); }
+    struct Raw {
+        Raw16 qs;
+        uint32_t sc, d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load16(blk + 2 + 16 * g);
+        r.sc = *reinterpret_cast<const uint16_t *>(blk + 66 + 2 * g);
+        r.d = *reinterpret_cast<const uint16_t *>(blk);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t, int g) {
+        uint32_t w[4];
+        bytes16(r.qs, sh, w);
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const uint32_t u0 = w[st] & 0xFFFFu, u1 = w[st] >> 16;
+            const uint2 m0 = grid[u0 & 511u], m1 = grid[u1 & 511u];
+            const uint2 s0 = t.sign128[u0 >> 9], s1 = t.sign128[u1 >> 9];
+            const v4i b = {apply_signs(m0.x, s0.x), apply_signs(m0.y, s0.y), apply_signs(m1.x, s1.x), apply_signs(m1.y, s1.y)};
+            const v4i zero = {0, 0, 0, 0};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[st], b, zero, 0, 0, 0);
+            const uint32_t nib = (r.sc >> (8 * (st >> 1) + 4 * (st & 1))) & 15u;
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + (st >> 1)], 0.5f + (float)nib, acc);
+        }
+        return half_bits_fast(r.d) * 0.25f * acc;
+    }
+};
+
+/* IQ2_S [d][32 index bytes][32 sign bytes][qh 8][8 scale bytes] (:2996-3020), 82 bytes: as IQ2_XS with a 10-bit
+ * index (two high bits per code in qh) into a 1024-entry grid and explicit sign bytes. */
+template <> struct GridFmt<T_IQ2_S> {
+    static constexpr int kBlock = 82, kGridBytes = 8192;
+    static constexpr int kAlign = 2, kPiece = 2;
+    static constexpr int kStep = 16;
+    static constexpr bool kAInRegs = true, kSums = false;
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    __device__ static const uint32_t *grid_src() { return reinterpret_cast<const uint32_t *>(qlin_iq2s_grid); }
+    struct Raw {
+        Raw8 qs, sg;
+        uint32_t qh, sc, d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load8(blk + 2 + 8 * g);
+        r.sg = load8(blk + 34 + 8 * g);
+        r.qh = *reinterpret_cast<const uint16_t *>(blk + 66 + 2 * g);
+        r.sc = *reinterpret_cast<const uint16_t *>(blk + 74 + 2 * g);
+        r.d = *reinterpret_cast<const uint16_t *>(blk);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t, int g) {
+        uint32_t q[2], sg[2];
+        bytes8(r.qs, sh, q);
+        bytes8(r.sg, sh, sg);
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const int h = st >> 1, l0 = 2 * (st & 1);
+            const uint32_t qhb = (r.qh >> (8 * h)) & 0xFFu;
+            const uint32_t i0 = ((q[h] >> (8 * l0)) & 0xFFu) | ((qhb << (8 - 2 * l0)) & 0x300u);
+            const uint32_t i1 = ((q[h] >> (8 * l0 + 8)) & 0xFFu) | ((qhb << (6 - 2 * l0)) & 0x300u);
+            const uint2 m0 = grid[i0], m1 = grid[i1];
+            const uint2 s0 = t.sign256[(sg[h] >> (8 * l0)) & 0xFFu], s1 = t.sign256[(sg[h] >> (8 * l0 + 8)) & 0xFFu];
+            const v4i b = {apply_signs(m0.x, s0.x), apply_signs(m0.y, s0.y), apply_signs(m1.x, s1.x), apply_signs(m1.y, s1.y)};
+            const v4i zero = {0, 0, 0, 0};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[st], b, zero, 0, 0, 0);
+            const uint32_t nib = (r.sc >> (8 * h + 4 * (st & 1))) & 15u;
+            acc = fmaf(join_digits(c) * xo.meta[2 * g + h], 0.5f + (float)nib, acc);
+        }
+        return half_bits_fast(r.d) * 0.25f * acc;
     }
 };
 
@@ -1187,6 +1274,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     if (n_sb < 8) return false;
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
+    case T_IQ2_XS: return true; /* 14336: 12.0 -> 10.3, 151936: 90 -> 64; IQ2_S (12.7 against 13.0, 95 against 101) stays */
     case T_MXFP4: case T_NVFP4: case T_TQ2_0: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5, 11.7 -> 7.4; 151936: 98 -> 74, 162 -> 88, 93 -> 43 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
@@ -1327,7 +1415,7 @@ bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, cons
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1351,6 +1439,8 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_MXFP4: return grid_typed<T_MXFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_NVFP4: return grid_typed<T_NVFP4>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_TQ2_0: return grid_typed<T_TQ2_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ2_XS: return grid_typed<T_IQ2_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ2_S: return grid_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
