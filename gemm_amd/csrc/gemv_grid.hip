@@ -976,8 +976,10 @@ template <> struct GridFmt<T_IQ4_XS> {
 struct MoeArgs {
     const int32_t *idx;
     const float *wts;
-    int top_k, n_expert, sb_per_expert, ldx; /* ldx: elements between two tokens' activations (MOE = 1) */
+    int top_k, n_expert, sb_per_expert;
+    int ldx; /* elements between two tokens' activations (MOE = 1) or rows of h (MOE = 2) */
     size_t expert_bytes;
+    int sb0; /* MOE = 2: the launch covers super-blocks sb0, sb0 + 1, ... of the token's row (x points at sb0's) */
 };
 
 template <uint32_t T, int NKC, int MOE = 0>
@@ -997,7 +999,7 @@ gemv_grid_kernel(const JobView job_in, const float *__restrict__ x, int n_sb, in
     } else if (MOE == 2) {
         idx += (size_t)blockIdx.y * moe.top_k;
         wts += (size_t)blockIdx.y * moe.top_k;
-        x += (size_t)blockIdx.y * n_sb * 256;
+        x += (size_t)blockIdx.y * moe.ldx;
         job.y0 += (size_t)blockIdx.y * job.n0;
     }
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -1057,15 +1059,15 @@ gemv_grid_kernel(const JobView job_in, const float *__restrict__ x, int n_sb, in
     auto sb_off = [&](int kc) {
         const int s = wv + 16 * kc;
         if (MOE == 2) {
-            const int j = s / moe.sb_per_expert, e = idx[j];
+            const int v = moe.sb0 + s, j = v / moe.sb_per_expert, e = idx[j];
             const bool valid = e >= 0 && e < moe.n_expert;
-            return (size_t)(valid ? e : 0) * moe.expert_bytes + (size_t)(s - j * moe.sb_per_expert) * F::kBlock;
+            return (size_t)(valid ? e : 0) * moe.expert_bytes + (size_t)(v - j * moe.sb_per_expert) * F::kBlock;
         }
         return (size_t)s * F::kBlock;
     };
     auto moe_x = [&](v4f v, int kc) { /* MOE = 2: the routing weight of the super-block's expert goes onto x */
         if (MOE == 2) {
-            const int j = (wv + 16 * kc) / moe.sb_per_expert, e = idx[j];
+            const int j = (moe.sb0 + wv + 16 * kc) / moe.sb_per_expert, e = idx[j];
             const float wj = wts[j];
             const v4f zero = {0.0f, 0.0f, 0.0f, 0.0f};
             v = (e >= 0 && e < moe.n_expert) ? v * wj : zero;
@@ -1314,7 +1316,7 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
     const size_t lds_bytes = (size_t)rows_per_wg * n_mats_here * kWaves * 4; /* the partial sums; the rest is static */
     const JobView view = job_view(job);
     const size_t pitch = row_stride ? row_stride : (size_t)n_sb * GridFmt<T>::kBlock;
-    const MoeArgs none = {nullptr, nullptr, 0, 0, 0, 0, 0};
+    const MoeArgs none = {nullptr, nullptr, 0, 0, 0, 0, 0, 0};
     if (short_rows)
         hipLaunchKernelGGL((gemv_grid_kernel<T, 1>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none);
     else
@@ -1346,7 +1348,7 @@ bool moe1_up_typed(const void *gate, const void *up, const uint16_t *X, const in
     job.n_rows[0] = job.n_rows[1] = n_ff;
     job.n_mat = 2;
     job.mode = kSiluMul;
-    const MoeArgs moe = {idx, nullptr, top_k, n_expert, n_sb, n_embd, expert_bytes};
+    const MoeArgs moe = {idx, nullptr, top_k, n_expert, n_sb, n_embd, expert_bytes, 0};
     const dim3 grid((n_ff + rows_per_wg - 1) / rows_per_wg, n_pairs);
     const size_t lds_bytes = (size_t)2 * rows_per_wg * kWaves * 4;
     const float *x = reinterpret_cast<const float *>(X);
@@ -1364,21 +1366,26 @@ bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const
     using F = GridFmt<T>;
     const int sbpe = n_ff / 256, n_sb = top_k * sbpe; /* the row of a token: top_k experts' rows side by side */
     const size_t row_bytes = (size_t)sbpe * F::kBlock, expert_bytes = (size_t)n_embd * row_bytes;
-    if (n_ff % 256 != 0 || n_sb > 16 * kMaxKc || n_embd < 1 || top_k < 1 || n_tok < 1) return false;
+    if (n_ff % 256 != 0 || n_embd < 1 || top_k < 1 || n_tok < 1) return false;
     if (((uintptr_t)down | row_bytes) % F::kAlign || ((uintptr_t)h & 15)) return false;
     if (dry) return true;
     constexpr int max_rows = F::kGridBytes > 0 ? 128 : kMaxRowsPerWg;
     const int tiles = n_cu / n_tok > 0 ? n_cu / n_tok : 1;
     int rows_per_wg = (n_embd + tiles - 1) / tiles;
     if (rows_per_wg > max_rows) rows_per_wg = max_rows;
-    GemvJob job = single_job(down, out, n_embd);
-    const MoeArgs moe = {idx, w, top_k, n_expert, sbpe, 0, expert_bytes};
     const dim3 grid((n_embd + rows_per_wg - 1) / rows_per_wg, n_tok);
     const size_t lds_bytes = (size_t)rows_per_wg * kWaves * 4;
-    if (n_sb <= 16)
-        hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), h, n_sb, rows_per_wg, row_bytes, moe);
-    else
-        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), h, n_sb, rows_per_wg, row_bytes, moe);
+    /* a launch takes 64 super-blocks of the row; a longer row (wide experts) goes in ranges, the later ones adding */
+    for (int sb0 = 0; sb0 < n_sb; sb0 += 16 * kMaxKc) {
+        const int n_here = n_sb - sb0 < 16 * kMaxKc ? n_sb - sb0 : 16 * kMaxKc;
+        GemvJob job = single_job(down, out, n_embd, sb0 == 0 ? kStore : kAdd);
+        const MoeArgs moe = {idx, w, top_k, n_expert, sbpe, n_sb * 256, expert_bytes, sb0};
+        const float *x = h + (size_t)sb0 * 256;
+        if (n_here <= 16)
+            hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_here, rows_per_wg, row_bytes, moe);
+        else
+            hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_here, rows_per_wg, row_bytes, moe);
+    }
     *err = hipGetLastError();
     return true;
 }

@@ -157,8 +157,8 @@ def test_few_tokens_other_expert_formats(oracle, types, n_tok):
 @pytest.mark.parametrize("types", [(Q4K, Q4K, Q4K), (Q4K, Q4K, Q6K), (Q6K, Q6K, Q4K)], ids=["q4k", "q4k_q4k_q6k", "q6k_q6k_q4k"])
 def test_one_token_wide_experts(oracle, types):
     """one token, top-2 of 8 experts with 8704-column down projections (a Mixtral-like shape, scaled): the down step
-    is a row of 68 super-blocks - more than the matrix-instruction kernel takes per launch, so a Q6_K down keeps the
-    grouped kernels while a Q4_K down takes the matvec route"""
+    is a row of 68 super-blocks - more than the matrix-instruction kernel takes per launch, so a Q6_K down runs as
+    two ranges of that row, the second adding; a Q4_K down walks the row in one launch"""
     n_expert, n_embd, n_ff, k, n_tok = 8, 1024, 8704, 2, 1
     gate, up, down = make_experts(n_expert, n_embd, n_ff, seed=980, types=types)
     Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=981, tokens=n_tok) * np.float32(0.05))
