@@ -1,7 +1,7 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
@@ -9,7 +9,7 @@
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
  * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
- * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S).
+ * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S), :1491-1503 (Q1_0).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -597,6 +597,49 @@ template <> struct GridFmt<T_TQ2_0> {
             const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
             const int e0 = elem0(g, l);
             acc += fmaf(join_digits(c), xo.meta[e0 >> 5], -xo.meta[8 + (e0 >> 4)]);
+        }
+        return half_bits_fast(r.d) * acc;
+    }
+};
+
+/* Q1_0 [d][128 bits] per 128 elements (common/ggml_dequant.h:1491-1503), 18 bytes: bit set -> +d, clear -> -d; 36
+ * bytes per 256 elements. Lane group g takes 64 bits of block g / 2, which start 2 (mod 4) bytes into the 36 for the
+ * first block: aligned dwords and a funnel shift there. The codes are the bits; 2 * (bits . x) - sum of x. */
+template <> struct GridFmt<T_Q1_0> {
+    static constexpr int kBlock = 36, kGridBytes = 0;
+    static constexpr int kPiece = 0, kAlign = 4;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        u32x2_a4 q;
+        uint32_t tail, d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        const int off = 18 * (g >> 1) + 2 + 8 * (g & 1); /* 2, 10, 20, 28 */
+        const uint8_t *p = blk + (off & ~3);
+        r.q = *reinterpret_cast<const u32x2_a4 *>(p);
+        r.tail = 0;
+        if (g < 2) r.tail = *reinterpret_cast<const uint32_t *>(p + 8); /* the second block's bits start on a dword */
+        r.d = *reinterpret_cast<const uint16_t *>(blk + 18 * (g >> 1));
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &, int g) {
+        const uint32_t sh = g < 2 ? 16u : 0u;
+        const uint32_t bits[2] = {__builtin_amdgcn_alignbit(r.q.y, r.q.x, sh), __builtin_amdgcn_alignbit(r.tail, r.q.y, sh)};
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const uint32_t b16 = bits[st >> 1] >> (16 * (st & 1));
+            const v4i b = {(int)spread4(b16), (int)spread4(b16 >> 4), (int)spread4(b16 >> 8), (int)spread4(b16 >> 12)};
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * st);
+            const v4i a = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, zero, 0, 0, 0);
+            const int e0 = elem0(g, st);
+            acc += fmaf(2.0f * join_digits(c), xo.meta[e0 >> 5], -xo.meta[8 + (e0 >> 4)]);
         }
         return half_bits_fast(r.d) * acc;
     }
@@ -1277,6 +1320,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
     case T_IQ2_XS: return true; /* 14336: 12.0 -> 10.3, 151936: 90 -> 64; IQ2_S (12.7 against 13.0, 95 against 101) stays */
+    case T_Q1_0: return true; /* 14336: 10.9 -> 7.5, 151936: 89 -> 44 */
     case T_MXFP4: case T_NVFP4: case T_TQ2_0: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5, 11.7 -> 7.4; 151936: 98 -> 74, 162 -> 88, 93 -> 43 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
@@ -1422,7 +1466,7 @@ bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, cons
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1448,6 +1492,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_TQ2_0: return grid_typed<T_TQ2_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ2_XS: return grid_typed<T_IQ2_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ2_S: return grid_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_Q1_0: return grid_typed<T_Q1_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
