@@ -1046,6 +1046,16 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
+    /* up to four tokens of any other block format: each through the matvec (exact weights; 14336 x 4096 IQ4_XS, four
+     * tokens: 44 us against 95 us for decode + dense product), x widened to fp32 at the start of the workspace */
+    if (n_tok <= kMatvecTokens && type != T_F32 && type != T_F16 && type != T_BF16) {
+        float *xf = (float *)workspace;
+        HIP_TRY(launch_dequant(T_BF16, X, nullptr, 0, xf, 1, (n_tok - 1) * ldx + n_cols, 0, (hipStream_t)stream));
+        for (int t = 0; t < n_tok; t++)
+            HIP_TRY(dispatch_gemv_job(type, single_job(W, Y + (size_t)t * ldy, n_rows), xf + (size_t)t * ldx, n_cols,
+                                      (hipStream_t)stream));
+        return QLIN_OK;
+    }
     const uint16_t *Wd = (const uint16_t *)W; /* bf16 weights are used where they are */
     if (type != T_BF16) {
         HIP_TRY(launch_dequant_bf16(type, W, (uint16_t *)workspace, n_rows, n_cols, row_size(type, n_cols), (hipStream_t)stream));

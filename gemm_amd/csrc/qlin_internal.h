@@ -77,12 +77,11 @@ bool launch_gemv_int(uint32_t type, const GemvJob &job, const float *x, int n_co
                      hipStream_t stream, hipError_t *err, size_t row_stride = 0);
 /* the formats whose rows launch_gemv_int reads from any even address (the others want 16-byte boundaries) */
 bool gemv_int_takes_any_even_address(uint32_t type);
-/* matrix-instruction matvec for the codebook formats IQ2_XXS, IQ3_XXS and IQ3_S (gemv_grid.hip): n_cols % 256 == 0,
- * n_cols <= 16384; same contract as launch_gemv_stream */
+/* matrix-instruction matvec for the formats of gemv_grid_covers (gemv_grid.hip): n_cols % 256 == 0, n_cols <= 16384,
+ * rows of up to 4096 elements only where it measured faster; same contract as launch_gemv_stream */
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu,
                       hipStream_t stream, hipError_t *err, size_t row_stride = 0);
 bool gemv_grid_covers(uint32_t type); /* the formats it has an item for */
-/* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 /* A few tokens, each on its own, through their top_k experts as two matvec launches: gate + up + SiLU into h
  * (n_tok * top_k * n_ff floats, X [n_tok, n_embd] bf16), then down with the routing weights folded into h. Q4_K experts
  * and the formats of the matrix-instruction matvec (gate and up of one type). false: not a shape for it; dry: only say so. */
@@ -96,6 +95,7 @@ bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const 
 bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, const int32_t *idx, const float *w, float *out,
                            int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
                            hipError_t *err);
+/* tuned Q4_K matvec: n_cols % 256 == 0, n_cols <= 16384, W and x 16-byte aligned */
 hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipStream_t stream, int n_cu,
                            size_t row_stride = 0);
 
@@ -124,6 +124,7 @@ constexpr int kKqFewTokens = 24; /* up to this many tokens Q6_K, Q5_K, Q3_K, Q2_
 /* false: not a shape for this kernel (the caller takes another route); true: launched, *err says how it went */
 bool launch_gemm_kq_fewtok(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                            int ldx, int ldy, hipStream_t stream, hipError_t *err);
+constexpr int kMatvecTokens = 4; /* qlin_gemm_bf16_any_dev: up to this many tokens of a format without a few-token kernel go through the matvec */
 constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
 hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                   int ldx, int ldy, hipStream_t stream);

@@ -45,8 +45,11 @@ KQ = {synth.GGML_Q6_K, synth.GGML_Q5_K, synth.GGML_Q3_K, synth.GGML_Q2_K, synth.
 
 
 def streams_exact_weights(tid, n_tok, n_rows, n_cols):
-    """few tokens of these formats go through a kernel that multiplies the unrounded weights"""
-    return tid in KQ and n_tok <= 24 and n_cols % 256 == 0 and n_rows * synth.row_bytes(tid, n_cols) % 16 == 0
+    """few tokens of these formats go through a kernel that multiplies the unrounded weights; up to four tokens of any
+    other block format (Q4_K has its own route) go through the matvec"""
+    if tid in KQ and n_tok <= 24 and n_cols % 256 == 0 and n_rows * synth.row_bytes(tid, n_cols) % 16 == 0:
+        return True
+    return n_tok <= 4 and tid not in synth.DENSE_TYPES and tid != synth.GGML_Q4_K
 
 
 def references(oracle, tid, W, Xb, n_cols):
@@ -82,6 +85,24 @@ def test_shapes(oracle, tid, n_tok, n_rows, n_cols, dense_kernel):
     exact, designed = references(oracle, tid, W, Xb, n_cols)
     assert rel_l2(Y, exact if streams_exact_weights(tid, n_tok, n_rows, n_cols) else designed) <= 2e-5, (ALL[tid], n_tok, n_rows, n_cols)
     assert rel_l2(Y, exact) <= 3e-3
+
+
+BLOCK_NOT_KQ = sorted(t for t in ALL if t not in KQ and t not in synth.DENSE_TYPES and t != Q4K)
+
+
+@pytest.mark.parametrize("n_tok", [1, 4, 5])
+@pytest.mark.parametrize("tid", BLOCK_NOT_KQ, ids=lambda t: ALL[t])
+def test_up_to_four_tokens_take_the_matvec(oracle, tid, n_tok):
+    """formats without a few-token kernel: up to four tokens go one by one through the matvec (exact weights, padded
+    X and Y rows left alone), five through decode + dense product"""
+    n_rows, n_cols = 203, 4608
+    W = synth.make_weights(tid, n_rows, n_cols, seed=70 + tid)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=71 + n_tok, tokens=n_tok))
+    ldx, ldy = n_cols + 24, n_rows + 5
+    Y = run(tid, W, Xb, n_rows, n_cols, n_tok, ldx=ldx, ldy=ldy)
+    exact, designed = references(oracle, tid, W, Xb, n_cols)
+    assert rel_l2(Y[:, :n_rows], exact if n_tok <= 4 else designed) <= 2e-5, (ALL[tid], n_tok)
+    assert np.all(Y[:, n_rows:] == -3.0)
 
 
 @pytest.mark.parametrize("n_tok", [1, 8, 9, 24, 25])
