@@ -1436,8 +1436,10 @@ bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const
 
 }  // namespace
 
-/* the expert formats of the K-quant and 4-bit mixes; the others keep the grouped kernels */
-#define QLIN_MOE1_TYPES(X) X(T_Q6_K) X(T_Q5_K) X(T_Q8_0) X(T_Q4_0) X(T_IQ4_NL) X(T_IQ4_XS) X(T_Q2_K) X(T_Q3_K) X(T_MXFP4)
+/* every format of this kernel (Q4_K experts take moe1_q4k_kernel, gemv_q4k.hip) */
+#define QLIN_MOE1_TYPES(X)                                                                                           \
+    X(T_Q6_K) X(T_Q5_K) X(T_Q8_0) X(T_Q4_0) X(T_Q4_1) X(T_Q5_0) X(T_Q5_1) X(T_IQ4_NL) X(T_IQ4_XS) X(T_Q2_K) X(T_Q3_K)  \
+    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S)
 
 bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h,
                          int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
