@@ -1,7 +1,7 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ1_S, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
@@ -9,7 +9,8 @@
  * the codes of common/ggml_dequant.h:2793-2816, :2916-2940, :3022-3058 (grid formats), :1653-1687 (Q6_K),
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
  * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
- * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S), :1491-1503 (Q1_0).
+ * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S), :1491-1503 (Q1_0),
+ * :3062-3083 (IQ1_S).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -350,6 +351,56 @@ template <> struct GridFmt<T_IQ2_S> {
             acc = fmaf(join_digits(c) * xo.meta[2 * g + h], 0.5f + (float)nib, acc);
         }
         return half_bits_fast(r.d) * 0.25f * acc;
+    }
+};
+
+/* IQ1_S [d][32 index bytes][8 x u16: 4 x 3 high index bits, 3-bit scale, shift sign] (common/ggml_dequant.h:3062-3083),
+ * 50 bytes: d * (2 s + 1) * (t + delta), t in {-1, 0, 1} from an eight-byte entry of a 2048-entry grid, delta = +-1/8
+ * per 32 elements. The grid bytes are the signed codes; delta goes onto the sum of x. */
+template <> struct GridFmt<T_IQ1_S> {
+    static constexpr int kBlock = 50, kGridBytes = 16384;
+    static constexpr int kAlign = 2, kPiece = 2;
+    static constexpr int kStep = 16;
+    static constexpr bool kAInRegs = true, kSums = true;
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    __device__ static const uint32_t *grid_src() { return reinterpret_cast<const uint32_t *>(qlin_iq1s_grid); }
+    struct Raw {
+        Raw8 qs;
+        uint32_t qh_q, qh_tail, d; /* the two u16 of groups 2g, 2g + 1: aligned dword and, off the grid, the tail */
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = load8(blk + 2 + 8 * g);
+        const uint8_t *p = blk + 34 + 4 * g;
+        const uint32_t odd = (uint32_t)(uintptr_t)p & 2u;
+        r.qh_q = *reinterpret_cast<const uint32_t *>(p - odd);
+        r.qh_tail = 0;
+        if (odd) r.qh_tail = *reinterpret_cast<const uint16_t *>(p + 2);
+        r.d = *reinterpret_cast<const uint16_t *>(blk);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &t, int g) {
+        uint32_t q[2];
+        bytes8(r.qs, sh, q);
+        const uint32_t qh2 = __builtin_amdgcn_alignbit(r.qh_tail, r.qh_q, sh);
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const int h = st >> 1, l0 = 2 * (st & 1);
+            const uint32_t qh = (qh2 >> (16 * h)) & 0xFFFFu;
+            const uint32_t i0 = ((q[h] >> (8 * l0)) & 0xFFu) | (((qh >> (3 * l0)) & 7u) << 8);
+            const uint32_t i1 = ((q[h] >> (8 * l0 + 8)) & 0xFFu) | (((qh >> (3 * l0 + 3)) & 7u) << 8);
+            const uint2 m0 = grid[i0], m1 = grid[i1];
+            const v4i b = {(int)m0.x, (int)m0.y, (int)m1.x, (int)m1.y};
+            const v4i zero = {0, 0, 0, 0};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[st], b, zero, 0, 0, 0);
+            const float dl = (float)(2u * ((qh >> 12) & 7u) + 1u);
+            const float delta = (qh & 0x8000u) ? -0.125f : 0.125f;
+            const int e0 = elem0(g, st);
+            acc = fmaf(dl, fmaf(join_digits(c), xo.meta[e0 >> 5], delta * xo.meta[8 + (e0 >> 4)]), acc);
+        }
+        return half_bits_fast(r.d) * acc;
     }
 };
 
@@ -1320,7 +1371,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
     case T_IQ2_XS: return true; /* 14336: 12.0 -> 10.3, 151936: 90 -> 64; IQ2_S (12.7 against 13.0, 95 against 101) stays */
-    case T_Q1_0: return true; /* 14336: 10.9 -> 7.5, 151936: 89 -> 44 */
+    case T_Q1_0: case T_IQ1_S: return true; /* 14336: 10.9 -> 7.5, 13.9 -> 10.5; 151936: 89 -> 44, 111 -> 75 */
     case T_MXFP4: case T_NVFP4: case T_TQ2_0: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5, 11.7 -> 7.4; 151936: 98 -> 74, 162 -> 88, 93 -> 43 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
@@ -1439,7 +1490,7 @@ bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const
 /* every format of this kernel (Q4_K experts take moe1_q4k_kernel, gemv_q4k.hip) */
 #define QLIN_MOE1_TYPES(X)                                                                                           \
     X(T_Q6_K) X(T_Q5_K) X(T_Q8_0) X(T_Q4_0) X(T_Q4_1) X(T_Q5_0) X(T_Q5_1) X(T_IQ4_NL) X(T_IQ4_XS) X(T_Q2_K) X(T_Q3_K)  \
-    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S)
+    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S) X(T_IQ1_S)
 
 bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h,
                          int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
@@ -1468,7 +1519,7 @@ bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, cons
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0 || type == T_IQ1_S;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1495,6 +1546,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_IQ2_XS: return grid_typed<T_IQ2_XS>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ2_S: return grid_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q1_0: return grid_typed<T_Q1_0>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ1_S: return grid_typed<T_IQ1_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }
