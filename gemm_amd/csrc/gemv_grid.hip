@@ -1,7 +1,7 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ1_S, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
@@ -10,7 +10,7 @@
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
  * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
  * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S), :1491-1503 (Q1_0),
- * :3062-3083 (IQ1_S).
+ * :3062-3126 (IQ1_S, IQ1_M).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -401,6 +401,55 @@ template <> struct GridFmt<T_IQ1_S> {
             acc = fmaf(dl, fmaf(join_digits(c), xo.meta[e0 >> 5], delta * xo.meta[8 + (e0 >> 4)]), acc);
         }
         return half_bits_fast(r.d) * acc;
+    }
+};
+
+/* IQ1_M [32 index bytes][qh 16][8 scale bytes] (common/ggml_dequant.h:3084-3126), 56 bytes and no d field (its
+ * four nibbles sit on top of the four scale words): d * (2 s + 1) * (t + delta) with the IQ1_S grid, a 3-bit scale
+ * per 16 elements and delta = +-1/8 per 8. The codes are 8 t + (+-1), signed bytes picked from a four-byte table by
+ * the grid byte's two low bits (t = -1, 0, 1 are 0xFF, 0, 1), and the scale carries the 1/8. */
+template <> struct GridFmt<T_IQ1_M> {
+    static constexpr int kBlock = 56, kGridBytes = 16384;
+    static constexpr int kAlign = 4, kPiece = 0;
+    static constexpr int kStep = 16;
+    static constexpr bool kAInRegs = true, kSums = false;
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    __device__ static const uint32_t *grid_src() { return reinterpret_cast<const uint32_t *>(qlin_iq1s_grid); }
+    struct Raw {
+        u32x2_a4 qs, sc;
+        uint32_t qh;
+    };
+    __device__ static Raw load(const uint8_t *blk, int g) {
+        Raw r;
+        r.qs = *reinterpret_cast<const u32x2_a4 *>(blk + 8 * g);
+        r.qh = *reinterpret_cast<const uint32_t *>(blk + 32 + 4 * g);
+        r.sc = *reinterpret_cast<const u32x2_a4 *>(blk + 48);
+        return r;
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t, const Tables &t, int g) {
+        const uint32_t q[2] = {r.qs.x, r.qs.y};
+        const uint2 *grid = reinterpret_cast<const uint2 *>(t.grid);
+        const uint32_t dbits = ((r.sc.x >> 12) & 0x000Fu) | ((r.sc.x >> 24) & 0x00F0u) | ((r.sc.y >> 4) & 0x0F00u) | ((r.sc.y >> 16) & 0xF000u);
+        const uint32_t scg = ((g & 2) ? r.sc.y : r.sc.x) >> (16 * (g & 1)); /* scale word g: groups 2g and 2g + 1 */
+        /* codes of t = 0, 1, (unused), -1 for delta = +1/8 and -1/8, as 8 t + (+-1) */
+        constexpr uint32_t kPlus = 0xF9000901u, kMinus = 0xF70007FFu;
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const int h = st >> 1, l0 = 2 * (st & 1);
+            const uint32_t qb = (r.qh >> (8 * (2 * h + (st & 1)))) & 0xFFu;
+            const uint32_t i0 = ((q[h] >> (8 * l0)) & 0xFFu) | ((qb << 8) & 0x700u);
+            const uint32_t i1 = ((q[h] >> (8 * l0 + 8)) & 0xFFu) | ((qb << 4) & 0x700u);
+            const uint2 m0 = grid[i0], m1 = grid[i1];
+            const uint32_t t0 = (qb & 0x08u) ? kMinus : kPlus, t1 = (qb & 0x80u) ? kMinus : kPlus;
+            const v4i b = {(int)__builtin_amdgcn_perm(0u, t0, m0.x & 0x03030303u), (int)__builtin_amdgcn_perm(0u, t0, m0.y & 0x03030303u),
+                           (int)__builtin_amdgcn_perm(0u, t1, m1.x & 0x03030303u), (int)__builtin_amdgcn_perm(0u, t1, m1.y & 0x03030303u)};
+            const v4i zero = {0, 0, 0, 0};
+            const v4i c = __builtin_amdgcn_mfma_i32_16x16x64_i8(xo.A[st], b, zero, 0, 0, 0);
+            const uint32_t s3 = (scg >> (6 * h + 3 * (st & 1))) & 7u;
+            acc = fmaf((float)(2u * s3 + 1u), join_digits(c) * xo.meta[2 * g + h], acc);
+        }
+        return half_bits_fast(dbits) * 0.125f * acc;
     }
 };
 
@@ -1371,7 +1420,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
     case T_IQ2_XS: return true; /* 14336: 12.0 -> 10.3, 151936: 90 -> 64; IQ2_S (12.7 against 13.0, 95 against 101) stays */
-    case T_Q1_0: case T_IQ1_S: return true; /* 14336: 10.9 -> 7.5, 13.9 -> 10.5; 151936: 89 -> 44, 111 -> 75 */
+    case T_Q1_0: case T_IQ1_S: case T_IQ1_M: return true; /* 14336: 10.9 -> 7.5, 13.9 -> 10.5, 16.0 -> 10.7; 151936: 89 -> 44, 111 -> 75, 135 -> 67 */
     case T_MXFP4: case T_NVFP4: case T_TQ2_0: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5, 11.7 -> 7.4; 151936: 98 -> 74, 162 -> 88, 93 -> 43 */
     case T_Q3_K: return n_rows >= 4096;
     case T_Q5_K: return n_rows <= 16384;
@@ -1490,7 +1539,7 @@ bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const
 /* every format of this kernel (Q4_K experts take moe1_q4k_kernel, gemv_q4k.hip) */
 #define QLIN_MOE1_TYPES(X)                                                                                           \
     X(T_Q6_K) X(T_Q5_K) X(T_Q8_0) X(T_Q4_0) X(T_Q4_1) X(T_Q5_0) X(T_Q5_1) X(T_IQ4_NL) X(T_IQ4_XS) X(T_Q2_K) X(T_Q3_K)  \
-    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S) X(T_IQ1_S)
+    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S) X(T_IQ1_S) X(T_IQ1_M)
 
 bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h,
                          int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
@@ -1519,7 +1568,7 @@ bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, cons
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0 || type == T_IQ1_S;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0 || type == T_IQ1_S || type == T_IQ1_M;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1547,6 +1596,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_IQ2_S: return grid_typed<T_IQ2_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_Q1_0: return grid_typed<T_Q1_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ1_S: return grid_typed<T_IQ1_S>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_IQ1_M: return grid_typed<T_IQ1_M>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }

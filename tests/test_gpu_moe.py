@@ -129,7 +129,7 @@ FEW_TOKEN_TYPES = [(Q4K, Q4K, Q6K), (Q6K, Q6K, Q6K), (Q5K, Q5K, Q6K), (synth.GGM
                    (synth.GGML_IQ4_NL, synth.GGML_IQ4_NL, synth.GGML_Q4_0), (synth.GGML_IQ2_XXS,) * 3,
                    (synth.GGML_IQ2_XS, synth.GGML_IQ2_XS, synth.GGML_IQ3_S), (synth.GGML_IQ3_XXS, synth.GGML_IQ3_XXS, synth.GGML_IQ2_S),
                    (synth.GGML_TQ2_0, synth.GGML_TQ2_0, synth.GGML_Q1_0), (synth.GGML_Q5_0, synth.GGML_Q5_0, synth.GGML_Q5_1),
-                   (synth.GGML_NVFP4, synth.GGML_NVFP4, synth.GGML_Q4_1), (synth.GGML_IQ1_S,) * 3, (Q4K, Q6K, Q4K)]
+                   (synth.GGML_NVFP4, synth.GGML_NVFP4, synth.GGML_Q4_1), (synth.GGML_IQ1_S, synth.GGML_IQ1_S, synth.GGML_IQ1_M), (Q4K, Q6K, Q4K)]
 
 
 @pytest.mark.parametrize("n_tok", [1, 3, 8])
