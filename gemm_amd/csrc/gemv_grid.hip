@@ -1,7 +1,7 @@
 /*
  * gemv_grid.hip - batch-1 matvec for rows of more than 4096 elements (and, where it measured faster, of 2048 to
  * 4096) on gfx950, for the codebook ("grid") formats
- * IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
+ * IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS and IQ3_S and for Q6_K, Q5_K, Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ1_0, TQ2_0, Q1_0, Q2_K and Q3_K: the inner products run on the 8-bit
  * integer matrix instruction; the grid formats look their codebook and sign masks up in LDS, the others build their
  * codes in registers and read the x operand from LDS for every item.
  *
@@ -10,7 +10,7 @@
  * :1620-1651 (Q5_K), :1479-1489 (Q8_0), :2850-2862 (Q4_0), :2942-2954 (IQ4_NL), :2956-2973 (IQ4_XS),
  * :1505-1534 (Q2_K), :1536-1580 (Q3_K), :2864-2915 (Q4_1, Q5_0, Q5_1), :2818-2830 (MXFP4) and
  * :2832-2848 (NVFP4), :3161-3176 (TQ2_0), :2975-3020 (IQ2_XS, IQ2_S), :1491-1503 (Q1_0),
- * :3062-3126 (IQ1_S, IQ1_M).
+ * :3062-3126 (IQ1_S, IQ1_M), :3127-3160 (TQ1_0).
  *
  *  1. x -> fixed point per 32-element group, three signed base-256 digits (the Q4_K matvec, gemv_q4k.hip,
  *     keeps four): X = rint(x * 2^(22-e)), e the exponent of the group's largest |x|; the error is at most
@@ -758,6 +758,69 @@ __device__ __forceinline__ Raw4 load4(const uint8_t *p) {
     return r;
 }
 
+/* TQ1_0 [qs 48][qh 4][d] (common/ggml_dequant.h:3127-3160), 54 bytes: base-3 digits, five to a byte of qs and four to
+ * a byte of qh; digit n of byte b is ((uint8)(b * 3^n) * 3) >> 8, the value (digit - 1) * d. Elements in runs of 16:
+ * runs 0..9 are digit n = run / 2 of qs[16 (run % 2) ..], runs 10..14 digit run - 10 of qs[32..48), run 15 the digits
+ * 0..3 of qh[0..4) (element 4 n + j = digit n of qh[j]). Lane group g takes runs 4g..4g + 3; every lane reads the
+ * three 16-byte pieces of qs and qh and picks. The codes stay unsigned (0..2); the -1 goes onto the sum of x. */
+template <> struct GridFmt<T_TQ1_0> {
+    static constexpr int kBlock = 54, kGridBytes = 0;
+    static constexpr int kPiece = 0, kAlign = 2;
+    static constexpr int kStep = 16;
+    static constexpr bool kSums = true, kAInRegs = false;
+    __device__ static const uint32_t *grid_src() { return nullptr; }
+    __device__ static int elem0(int g, int st) { return 64 * g + 16 * st; }
+    struct Raw {
+        Raw16 a, b, c;
+        Raw4 qh;
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *blk, int) {
+        Raw r;
+        r.a = load16(blk);
+        r.b = load16(blk + 16);
+        r.c = load16(blk + 32);
+        r.qh = load4(blk + 48);
+        r.d = *reinterpret_cast<const uint16_t *>(blk + 52);
+        return r;
+    }
+    /* digit of four bytes: ((b * pw) mod 256) * 3 >> 8, two bytes at a time in the halves of a dword */
+    __device__ static uint32_t digits4(uint32_t w, uint32_t pw) {
+        const uint32_t lo = (((w & 0x00FF00FFu) * pw) & 0x00FF00FFu) * 3u, hi = ((((w >> 8) & 0x00FF00FFu) * pw) & 0x00FF00FFu) * 3u;
+        return ((lo >> 8) & 0x00030003u) | (hi & 0x03000300u);
+    }
+    __device__ static float item(const XOperand &xo, const Raw &r, uint32_t sh, const Tables &, int g) {
+        uint32_t a[4], b[4], c[4];
+        bytes16(r.a, sh, a);
+        bytes16(r.b, sh, b);
+        bytes16(r.c, sh, c);
+        const uint32_t qh = __builtin_amdgcn_alignbit(r.qh.tail, r.qh.q, sh);
+        /* power of 3 of run 4g + st: runs 0..9 -> run / 2, runs 10..14 -> run - 10 */
+        float acc = 0.0f;
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const int run = 4 * g + st;
+            const bool from_c = run >= 10, special = run == 15;
+            const int n = from_c ? run - 10 : run >> 1;
+            const uint32_t pw = n == 0 ? 1u : n == 1 ? 3u : n == 2 ? 9u : n == 3 ? 27u : 81u;
+            v4i code;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t src = special ? qh : from_c ? c[i] : (run & 1) ? b[i] : a[i];
+                const uint32_t p = special ? (i == 0 ? 1u : i == 1 ? 3u : i == 2 ? 9u : 27u) : pw;
+                code[i] = (int)digits4(src, p);
+            }
+            const v4i zero = {0, 0, 0, 0};
+            const uint4 av = *reinterpret_cast<const uint4 *>(xo.arows + kStep * st);
+            const v4i av4 = {(int)av.x, (int)av.y, (int)av.z, (int)av.w};
+            const v4i cc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av4, code, zero, 0, 0, 0);
+            const int e0 = elem0(g, st);
+            acc += fmaf(join_digits(cc), xo.meta[e0 >> 5], -xo.meta[8 + (e0 >> 4)]);
+        }
+        return half_bits_fast(r.d) * acc;
+    }
+};
+
 /* Q3_K [hmask 32][qs 64][12 packed scale bytes][d] (:1536-1580), 110 bytes: element 128 h + 32 j + l (l < 32) is
  * bits 2j, 2j+1 of qs[32 h + l], minus 4 unless bit 4 h + j of hmask[l] is set, times d * (6-bit scale - 32) of
  * index 8 h + 2 j + l / 16: low nibbles in bytes 0..7 (index & 7, the high nibble for indices 8..15), the two high
@@ -1420,6 +1483,7 @@ bool short_rows_pay(uint32_t type, int n_sb, int n_rows) {
     switch (type) {
     case T_IQ4_NL: case T_IQ4_XS: case T_Q4_0: case T_Q2_K: case T_IQ2_XXS: case T_IQ3_XXS: case T_IQ3_S: return true;
     case T_IQ2_XS: return true; /* 14336: 12.0 -> 10.3, 151936: 90 -> 64; IQ2_S (12.7 against 13.0, 95 against 101) stays */
+    case T_TQ1_0: return true; /* 14336: 31.7 -> 15.7, 151936: 306 -> 107 */
     case T_Q1_0: case T_IQ1_S: case T_IQ1_M: return true; /* 14336: 10.9 -> 7.5, 13.9 -> 10.5, 16.0 -> 10.7; 151936: 89 -> 44, 111 -> 75, 135 -> 67 */
     case T_MXFP4: case T_NVFP4: case T_TQ2_0: return true; /* 14336: 13.4 -> 11.2, 17.9 -> 12.5, 11.7 -> 7.4; 151936: 98 -> 74, 162 -> 88, 93 -> 43 */
     case T_Q3_K: return n_rows >= 4096;
@@ -1539,7 +1603,7 @@ bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const
 /* every format of this kernel (Q4_K experts take moe1_q4k_kernel, gemv_q4k.hip) */
 #define QLIN_MOE1_TYPES(X)                                                                                           \
     X(T_Q6_K) X(T_Q5_K) X(T_Q8_0) X(T_Q4_0) X(T_Q4_1) X(T_Q5_0) X(T_Q5_1) X(T_IQ4_NL) X(T_IQ4_XS) X(T_Q2_K) X(T_Q3_K)  \
-    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S) X(T_IQ1_S) X(T_IQ1_M)
+    X(T_MXFP4) X(T_NVFP4) X(T_TQ2_0) X(T_Q1_0) X(T_IQ2_XXS) X(T_IQ2_XS) X(T_IQ2_S) X(T_IQ3_XXS) X(T_IQ3_S) X(T_IQ1_S) X(T_IQ1_M) X(T_TQ1_0)
 
 bool launch_moe1_grid_up(uint32_t type, const void *gate, const void *up, const uint16_t *X, const int32_t *idx, float *h,
                          int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int n_cu, hipStream_t stream, bool dry,
@@ -1568,7 +1632,7 @@ bool launch_moe1_grid_down(uint32_t type, const void *down, const float *h, cons
 bool gemv_grid_covers(uint32_t type) {
     return type == T_IQ2_XXS || type == T_IQ3_XXS || type == T_IQ3_S || type == T_Q6_K || type == T_Q5_K || type == T_Q8_0 ||
            type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K ||
-           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0 || type == T_IQ1_S || type == T_IQ1_M;
+           type == T_Q4_1 || type == T_Q5_0 || type == T_Q5_1 || type == T_MXFP4 || type == T_NVFP4 || type == T_TQ2_0 || type == T_IQ2_XS || type == T_IQ2_S || type == T_Q1_0 || type == T_IQ1_S || type == T_IQ1_M || type == T_TQ1_0;
 }
 
 bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_cols, int n_cu, hipStream_t stream,
@@ -1597,6 +1661,7 @@ bool launch_gemv_grid(uint32_t type, const GemvJob &job, const float *x, int n_c
     case T_Q1_0: return grid_typed<T_Q1_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ1_S: return grid_typed<T_IQ1_S>(job, x, n_cols, n_cu, stream, err, row_stride);
     case T_IQ1_M: return grid_typed<T_IQ1_M>(job, x, n_cols, n_cu, stream, err, row_stride);
+    case T_TQ1_0: return grid_typed<T_TQ1_0>(job, x, n_cols, n_cu, stream, err, row_stride);
     default: return false;
     }
 }

@@ -1,5 +1,5 @@
 """GPU parity of the matrix-instruction matvec for the codebook formats IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS, IQ3_S and for Q6_K, Q5_K,
-Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ2_0, Q1_0, Q2_K, Q3_K (rows longer than 4096 elements take it, and most of these formats' rows from 2048 elements) against the CPU oracle, through the C ABI: plain, ragged row counts, several
+Q8_0, Q4_0, Q4_1, Q5_0, Q5_1, IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ1_0, TQ2_0, Q1_0, Q2_K, Q3_K (rows longer than 4096 elements take it, and most of these formats' rows from 2048 elements) against the CPU oracle, through the C ABI: plain, ragged row counts, several
 matrices in one launch, gate+up+SiLU, projection+residual, non-finite x. Relative L2 <= 1e-5."""
 import numpy as np
 import pytest
@@ -14,7 +14,7 @@ GRID = {synth.GGML_IQ2_XXS: "iq2_xxs", synth.GGML_IQ3_XXS: "iq3_xxs", synth.GGML
         synth.GGML_Q6_K: "q6_K", synth.GGML_Q5_K: "q5_K", synth.GGML_Q8_0: "q8_0", synth.GGML_IQ4_NL: "iq4_nl",
         synth.GGML_IQ4_XS: "iq4_xs", synth.GGML_Q4_0: "q4_0", synth.GGML_Q2_K: "q2_K", synth.GGML_Q3_K: "q3_K",
         synth.GGML_Q4_1: "q4_1", synth.GGML_Q5_0: "q5_0", synth.GGML_Q5_1: "q5_1", synth.GGML_MXFP4: "mxfp4", synth.GGML_NVFP4: "nvfp4", synth.GGML_TQ2_0: "tq2_0",
-        synth.GGML_IQ2_XS: "iq2_xs", synth.GGML_IQ2_S: "iq2_s", synth.GGML_Q1_0: "q1_0", synth.GGML_IQ1_S: "iq1_s", synth.GGML_IQ1_M: "iq1_m"}
+        synth.GGML_IQ2_XS: "iq2_xs", synth.GGML_IQ2_S: "iq2_s", synth.GGML_Q1_0: "q1_0", synth.GGML_IQ1_S: "iq1_s", synth.GGML_IQ1_M: "iq1_m", synth.GGML_TQ1_0: "tq1_0"}
 
 
 # 17 super-blocks (one wave with two), 43 (ragged over the 16 waves), 56 and 64 (the most a wave takes);

@@ -16,7 +16,8 @@ TOL = 1e-5
 # formats whose matvec runs on integer dot products with x in per-32-element fixed point
 FIXED_POINT = {synth.GGML_Q4_K, synth.GGML_Q8_0, synth.GGML_Q4_0, synth.GGML_Q4_1, synth.GGML_Q5_0, synth.GGML_Q5_1,
                synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q2_K, synth.GGML_Q3_K, synth.GGML_IQ4_NL, synth.GGML_IQ4_XS,
-               synth.GGML_MXFP4, synth.GGML_IQ2_XXS, synth.GGML_IQ3_XXS, synth.GGML_IQ3_S, synth.GGML_IQ2_XS, synth.GGML_IQ2_S}
+               synth.GGML_MXFP4, synth.GGML_IQ2_XXS, synth.GGML_IQ3_XXS, synth.GGML_IQ3_S, synth.GGML_IQ2_XS, synth.GGML_IQ2_S,
+               synth.GGML_NVFP4, synth.GGML_TQ1_0, synth.GGML_TQ2_0, synth.GGML_Q1_0, synth.GGML_IQ1_S, synth.GGML_IQ1_M}
 
 
 def x_step(tid):
