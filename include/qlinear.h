@@ -269,7 +269,10 @@ int qlin_gemm_f32_any_dev(uint32_t ggml_type, const void *W, const float *X, flo
  *   out fp32 [n_tok, n_embd] (overwritten). workspace: qlin_moe_workspace_bytes() bytes.
  * Q4_K, Q5_K, Q6_K, Q3_K, Q2_K and Q8_0 matrices run on the matrix cores with unrounded codes; every other format
  * (block-quantized or dense) runs through the bit-exact decoder in fp32, several times slower. qlin_moe_ffn_types_dev takes one format
- * per tensor: K-quant mixes store part of the down projections as Q6_K beside Q4_K gate and up. */
+ * per tensor: K-quant mixes store part of the down projections as Q6_K beside Q4_K gate and up.
+ * One token - the reference's own call - and up to eight tokens when there are at most two (token, choice) pairs per
+ * four experts go token by token through two launches of the matvec kernels instead, for every block format (gate and
+ * up of one format): no rounding of activations or weights, the sum over a token's experts in a fixed order. */
 size_t qlin_moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
 int qlin_moe_route_dev(const float *router_logits, int n_tok, int n_expert, int top_k,
                        int32_t *expert_idx, float *expert_w, void *stream);
