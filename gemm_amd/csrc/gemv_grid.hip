@@ -1190,7 +1190,8 @@ struct MoeArgs {
 
 template <uint32_t T, int NKC, int MOE = 0>
 __global__ void __launch_bounds__(kWaves * 64)
-gemv_grid_kernel(const JobView job_in, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes, const MoeArgs moe) {
+gemv_grid_kernel(const JobView job_in, const float *__restrict__ x, int n_sb, int rows_per_wg, size_t row_bytes, const MoeArgs moe,
+                 int lone_ahead) {
     using F = GridFmt<T>;
     JobView job = job_in;
     const int32_t *idx = moe.idx;
@@ -1366,7 +1367,7 @@ gemv_grid_kernel(const JobView job_in, const float *__restrict__ x, int n_sb, in
 
     /* the first blocks are requested before the tables are built and x is prepared: the wave's first two
      * super-blocks of a lone row group (long rows), else its first super-block of the first row groups */
-    const bool long_rows = NKC > 1 && n_rg < 2;
+    const bool long_rows = NKC > 1 && n_rg < 2 && lone_ahead;
     /* row groups of a super-block column in flight per wave: with sixteen waves per compute unit one is enough, and
      * two or four measured slower for every format (IQ2_XXS 8192 x 28672: 38.8 us with four, 29.6 with one) */
     constexpr int D = 1;
@@ -1526,9 +1527,16 @@ bool grid_typed(const GemvJob &job, const float *x, int n_cols, int n_cu, hipStr
     const size_t pitch = row_stride ? row_stride : (size_t)n_sb * GridFmt<T>::kBlock;
     const MoeArgs none = {nullptr, nullptr, 0, 0, 0, 0, 0, 0};
     if (short_rows)
-        hipLaunchKernelGGL((gemv_grid_kernel<T, 1>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none);
+        hipLaunchKernelGGL((gemv_grid_kernel<T, 1>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none, 1);
     else
-        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none);
+        {
+        /* a lone row group per workgroup: two super-blocks requested ahead, except for the two formats with the most
+         * loads per item where every compute unit has a workgroup - there one super-block at a time measured faster
+         * (Q6_K 4096 x 8192: 11.3 -> 9.9 us, 4096 x 14336: 14.9 -> 14.6; IQ3_S 10.7 -> 9.9, 13.5 -> 13.0) */
+        const bool one_at_a_time = (T == T_Q6_K || T == T_IQ3_S) && grid >= n_cu;
+        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc>), dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, pitch, none,
+                           one_at_a_time ? 0 : 1);
+    }
     *err = hipGetLastError();
     return true;
 }
@@ -1561,9 +1569,9 @@ bool moe1_up_typed(const void *gate, const void *up, const uint16_t *X, const in
     const size_t lds_bytes = (size_t)2 * rows_per_wg * kWaves * 4;
     const float *x = reinterpret_cast<const float *>(X);
     if (n_sb <= 16)
-        hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 1>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_sb, rows_per_wg, row_bytes, moe);
+        hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 1>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_sb, rows_per_wg, row_bytes, moe, 1);
     else
-        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 1>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_sb, rows_per_wg, row_bytes, moe);
+        hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 1>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_sb, rows_per_wg, row_bytes, moe, 1);
     *err = hipGetLastError();
     return true;
 }
@@ -1590,9 +1598,9 @@ bool moe1_down_typed(const void *down, const float *h, const int32_t *idx, const
         const MoeArgs moe = {idx, w, top_k, n_expert, sbpe, n_sb * 256, expert_bytes, sb0};
         const float *x = h + (size_t)sb0 * 256;
         if (n_here <= 16)
-            hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_here, rows_per_wg, row_bytes, moe);
+            hipLaunchKernelGGL((gemv_grid_kernel<T, 1, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_here, rows_per_wg, row_bytes, moe, 1);
         else
-            hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_here, rows_per_wg, row_bytes, moe);
+            hipLaunchKernelGGL((gemv_grid_kernel<T, kMaxKc, 2>), grid, dim3(kWaves * 64), lds_bytes, stream, job_view(job), x, n_here, rows_per_wg, row_bytes, moe, 1);
     }
     *err = hipGetLastError();
     return true;
