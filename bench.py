@@ -42,7 +42,7 @@ Q4K = synth.GGML_Q4_K
 # same counter reads for a device-to-device copy of known size, as recorded with its commands in
 # PROFILED_TRAFFIC_SOURCE. It changes only when the kernel's loads change and the profile is taken again;
 # tests/test_profiles.py fails when the two files disagree.
-PROFILED_TRAFFIC_BYTES = 33270573
+PROFILED_TRAFFIC_BYTES = 33277536
 PROFILED_TRAFFIC_SOURCE = "profiles/gemv_q4k_14336x4096.md"
 
 
