@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <climits>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -1048,9 +1049,11 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     }
     /* up to four tokens of any other block format: each through the matvec (exact weights; 14336 x 4096 IQ4_XS, four
      * tokens: 44 us against 95 us for decode + dense product), x widened to fp32 at the start of the workspace */
-    if (n_tok <= kMatvecTokens && type != T_F32 && type != T_F16 && type != T_BF16) {
+    const size_t x_span = (size_t)(n_tok - 1) * ldx + n_cols; /* elements of X from the first token's to the last's */
+    if (n_tok <= kMatvecTokens && type != T_F32 && type != T_F16 && type != T_BF16 && x_span <= (size_t)INT_MAX &&
+        x_span * sizeof(float) <= workspace_bytes) { /* a very wide ldx: the dense route below */
         float *xf = (float *)workspace;
-        HIP_TRY(launch_dequant(T_BF16, X, nullptr, 0, xf, 1, (n_tok - 1) * ldx + n_cols, 0, (hipStream_t)stream));
+        HIP_TRY(launch_dequant(T_BF16, X, nullptr, 0, xf, 1, (int)x_span, 0, (hipStream_t)stream));
         for (int t = 0; t < n_tok; t++)
             HIP_TRY(dispatch_gemv_job(type, single_job(W, Y + (size_t)t * ldy, n_rows), xf + (size_t)t * ldx, n_cols,
                                       (hipStream_t)stream));

@@ -105,6 +105,31 @@ def test_up_to_four_tokens_take_the_matvec(oracle, tid, n_tok):
     assert np.all(Y[:, n_rows:] == -3.0)
 
 
+def test_few_tokens_whose_rows_lie_far_apart(oracle):
+    """three tokens of X with a leading dimension so wide that their fp32 copy would not fit the workspace: the call
+    must not write past it (it takes the decode + dense route instead)"""
+    tid = synth.GGML_IQ4_XS
+    n_rows, n_cols, n_tok = 16, 256, 3
+    ws_bytes = qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols)
+    ldx = (ws_bytes // 4 // (n_tok - 1) + 8) // 8 * 8  # (n_tok - 1) * ldx * 4 bytes > the workspace
+    W = synth.make_weights(tid, n_rows, n_cols, seed=91)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=92, tokens=n_tok))
+    Xpad = np.zeros((n_tok - 1) * ldx + n_cols, np.uint16)
+    for t in range(n_tok):
+        Xpad[t * ldx:t * ldx + n_cols] = Xb[t]
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xpad)
+    dY = qlinear.DevBuf.from_numpy(np.full((n_tok, n_rows), -3.0, np.float32))
+    guard = 1 << 20
+    ws = qlinear.DevBuf.from_numpy(np.full(ws_bytes + guard, 0x5A, np.uint8))
+    # the workspace is declared without its guard megabyte, which has to come back untouched
+    qlinear.check(qlinear.load().qlin_gemm_bf16_any_dev(tid, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, n_rows,
+                                                        ws.ptr, ws_bytes, None))
+    qlinear.sync()
+    exact, designed = references(oracle, tid, W, Xb, n_cols)
+    assert rel_l2(dY.to_numpy(np.float32, (n_tok, n_rows)), designed) <= 2e-5
+    assert np.all(ws.to_numpy(np.uint8, (ws_bytes + guard,))[ws_bytes:] == 0x5A)
+
+
 @pytest.mark.parametrize("n_tok", [1, 8, 9, 24, 25])
 @pytest.mark.parametrize("tid", sorted(KQ), ids=lambda t: ALL[t])
 def test_few_tokens_of_a_k_quant_or_q8_0_tensor(oracle, tid, n_tok):
