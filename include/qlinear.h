@@ -234,7 +234,8 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
  * Q8_0 tensor (n_cols % 256 == 0, the tensor's bytes a multiple of 16) also run in one fused kernel with
  * unrounded weights (~1e-6) and leave the workspace alone (it may be NULL then). Up to 4 tokens of any other
  * block format go one by one through the matvec kernels (exact weights, ~1e-6; the workspace holds their
- * activations as fp32). workspace: device memory, 256-byte aligned, at least
+ * activations as fp32, and when ldx is so wide that (n_tok - 1) * ldx + n_cols floats do not fit it they take the
+ * decode + dense route). workspace: device memory, 256-byte aligned, at least
  * qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes (2 bytes per weight + 32 MiB for the library);
  * calls that share a workspace must be ordered on one stream. Relative L2 of Y against exact weights
  * <= 2e-3.
