@@ -380,6 +380,8 @@ hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int 
      * half-empty 256-token tiles (128 tokens at 14336 x 4096: 51.7 -> 39.5 us, 64 tokens: 50.7 -> 34.4) */
     if (n_tok <= 128) return launch_tiled<2, 1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     if (m_tiles * n_tiles_128 < 200) return launch_tiled<4, 1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    /* a chip's worth of 256-token x 128-row tiles or more: the four-wave kernel (its 32-bit offsets hold 256 rows of X) */
+    if (ldx < (1 << 22)) return launch_gemm_q4k_bf16_wave4(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     return launch_tiled<4, 2>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
 }
 
