@@ -19,10 +19,12 @@
  * So nothing is stored to LDS by a wave:
  *   - activations go from global memory to LDS by the load-to-LDS path, 256 tokens x 64 k per tile, whole 128-byte
  *     row segments per 8 lanes, four stages deep;
- *   - weights never touch LDS: wave w owns rows 32 w .. 32 w + 31 of the workgroup's 128 and all 256 tokens, its lane
- *     (row i, half kg) loads 16 of the 32 code bytes of a quarter super-block of its row and decodes them straight into
- *     the matrix instruction's first-operand layout (8 consecutive k of one row per lane): no decode is done twice
- *     in the workgroup, and there is nothing to exchange;
+ *   - decoded weights never touch LDS: wave w owns rows 32 w .. 32 w + 31 of the workgroup's 128 and all 256 tokens,
+ *     its lane (row i, half kg) takes 16 of the 32 code bytes of a quarter super-block of its row and decodes them
+ *     straight into the matrix instruction's first-operand layout (8 consecutive k of one row per lane): no decode
+ *     is done twice in the workgroup, and there is nothing to exchange. The raw blocks of a wave's rows come the same
+ *     way as the activations (whole 144-byte blocks, consecutive lanes consecutive bytes; a lane reading its own
+ *     row from global memory costs the memory pipe four times as much) and are read back by the wave itself;
  *   - per matrix instruction one ds_read_b128 (a 32-token x 16-k activation fragment) and about three vector
  *     instructions of decode.
  *
@@ -33,8 +35,8 @@
  * LDS: four stages of [256 tokens][64 k] bf16 = 32 KB; 16-byte chunk c of token row r sits at chunk position
  * c ^ f(r), f = bits 1 and 2 of (r >> 1) & 7 swapped, so that the 16 rows of a fragment fetch hit 16 different
  * 16-byte bank groups. One tile = 32 slots of [matrix instruction, fragment fetch for the next k-step, side work],
- * nothing moves between slots; side work = the load-to-LDS requests of the tile three ahead, the raw codes of the
- * next super-block, and the decode of the next tile in 44 pieces of at most two vector instructions. Before the last
+ * nothing moves between slots; side work = the load-to-LDS requests of the tile three ahead and of the raw blocks
+ * two super-blocks ahead, and the decode of the next tile in 44 pieces of at most two vector instructions. Before the last
  * k-step: wait for this wave's requests of the next tile, barrier (the next tile is complete; nobody reads the
  * stage that is requested next, its last fragments were fetched a k-step earlier).
  */
@@ -62,6 +64,9 @@ __shared__ __attribute__((aligned(1024))) uint8_t w4_stage0[kXStage];
 __shared__ __attribute__((aligned(1024))) uint8_t w4_stage1[kXStage];
 __shared__ __attribute__((aligned(1024))) uint8_t w4_stage2[kXStage];
 __shared__ __attribute__((aligned(1024))) uint8_t w4_stage3[kXStage];
+/* raw blocks of one super-block of a wave's 32 weight rows (32 x 144 bytes, rounded up to five requests of 1 KB) */
+constexpr int kWRaw = 5 * 1024;
+__shared__ __attribute__((aligned(1024))) uint8_t w4_wraw[4 * kWRaw];
 
 #define QLIN_INL __device__ __forceinline__ __attribute__((always_inline))
 
@@ -123,8 +128,8 @@ struct Ctx {
     float w0, w1, w2, w3;
     uint32_t xrd;            /* byte offset of this lane's fragment fetches in a stage: k-step 0, token block 0 */
     __amdgpu_buffer_rsrc_t w_rsrc, x_rsrc;
-    uint32_t w_off, w_offq, x_off[8];
-    int wv;                  /* wave of the workgroup */
+    uint32_t w_off[5], w_rd, x_off[8];
+    int wv, kg;              /* wave of the workgroup; lane half */
     int sb, n_sb;            /* super-block of the tile in use */
     float unit;
 };
@@ -164,10 +169,16 @@ template <int CQ, int WB, int PP> QLIN_INL void decode_piece(Ctx &c, const u32x4
     }
 }
 
-template <int WHICH> QLIN_INL void load_sb(Ctx &c, SbRegs &r, int sb) {
-    const int so = min(sb, c.n_sb - 1) * 144; /* past the end: a harmless re-read */
-    if constexpr (WHICH == 0) r.hdr = __builtin_amdgcn_raw_buffer_load_b128(c.w_rsrc, c.w_off, so, 0);
-    else r.q[WHICH - 1] = __builtin_amdgcn_raw_buffer_load_b128(c.w_rsrc, c.w_offq + 32 * (WHICH - 1), so, 0);
+/* request Q (0..4) of this wave for the raw blocks of super-block `sb` of its 32 rows: 64 consecutive 16-byte
+ * pieces of the 32 x 9 (past the end of K: a harmless re-read) */
+template <int Q> QLIN_INL void request_w(Ctx &c, int sb) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(c.w_rsrc, (lds_void *)(w4_wraw + c.wv * kWRaw + Q * 1024), 16, c.w_off[Q],
+                                             min(sb, c.n_sb - 1) * 144, 0, 0);
+}
+/* this lane's part WHICH (0: header, 1..4: its 16 code bytes of quarter WHICH - 1) of the raw blocks in LDS */
+template <int WHICH> QLIN_INL void load_sb(Ctx &c, SbRegs &r) {
+    if constexpr (WHICH == 0) r.hdr = *reinterpret_cast<const u32x4 *>(w4_wraw + c.w_rd);
+    else r.q[WHICH - 1] = *reinterpret_cast<const u32x4 *>(w4_wraw + c.w_rd + 16 + 32 * (WHICH - 1) + 16 * c.kg);
 }
 
 /* request I (0..7) of this wave for 64-k tile `tile` into stage ST: token rows 64 wv + 8 I .. + 7, 128 bytes each */
@@ -186,14 +197,17 @@ template <int U, int T> QLIN_INL void slot(Ctx &c) {
     constexpr int s = T / 8, bj = T % 8;
     if constexpr (T == 24) {
         /* this wave's requests of the next tile have landed: younger are the 8 of the tile after it, 6 of the one
-         * after that, and the code loads of the tiles with U = 0 */
-        wait_vmcnt<14 + (U == 0 || U == 1 ? 5 : 0)>();
+         * after that, and the five weight requests of the tiles with U = 1 */
+        wait_vmcnt<14 + (U == 1 || U == 2 ? 5 : 0)>();
         __builtin_amdgcn_s_barrier();
     }
     c.acc[bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, c.wa[U & 1][s]), c.xf[s & 1][bj], c.acc[bj], 0, 0, 0);
     c.xf[(s + 1) & 1][bj] = load_frag<(s == 3 ? (U + 1) & 3 : U), (s + 1) & 3, bj>(c);
     if constexpr (T % 4 == 2) request_x<(U + 3) & 3, T / 4>(c, 4 * c.sb + U + 3);
-    if constexpr (U == 0 && T % 4 == 1 && T / 4 < 5) load_sb<T / 4>(c, c.nxt, c.sb + 1);
+    /* U = 0: the raw blocks of the next super-block (requested three tiles ago) into registers; U = 1: request the
+     * ones after it into the same place */
+    if constexpr (U == 0 && T % 4 == 1 && T / 4 < 5) load_sb<T / 4>(c, c.nxt);
+    if constexpr (U == 1 && T % 4 == 1 && T / 4 < 5) request_w<T / 4>(c, c.sb + 2);
     if constexpr (U == 3 && T % 8 == 4 && T / 8 < 3) c.cur.q[T / 8 + 1] = c.nxt.q[T / 8 + 1];
     /* decode of the next tile: quarter (U + 1) & 3, for U = 3 of the next super-block, whose header is unpacked first */
     constexpr int n_pieces = U == 3 ? 48 : 44;
@@ -249,8 +263,13 @@ gemm_q4k_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__rest
     const int w_rows = min(kBN, n_rows - tile_n * kBN);
     c.w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(W) + (size_t)tile_n * kBN * row_bytes, 0,
                                                  w_rows * row_bytes, 0x00020000);
-    c.w_off = (uint32_t)min(32 * c.wv + li, w_rows - 1) * row_bytes;
-    c.w_offq = c.w_off + 16 + 16 * kg;
+    c.kg = kg;
+#pragma unroll
+    for (int q = 0; q < 5; q++) {
+        const int id = min(64 * q + lane, 32 * 9 - 1); /* piece id % 9 of row id / 9; the fifth request is half padding */
+        c.w_off[q] = (uint32_t)min(32 * c.wv + id / 9, w_rows - 1) * row_bytes + 16 * (id % 9);
+    }
+    c.w_rd = (uint32_t)(c.wv * kWRaw + li * 144);
     /* Activation requests: request I of this wave fills 1 KB of a stage, lane l the 16 bytes at chunk position l % 8 of
      * token row 64 wv + 8 I + l / 8, i.e. chunk (l % 8) ^ f(row) of that token's 128 bytes; tokens past the end
      * re-read the last one (never stored) */
@@ -272,13 +291,17 @@ gemm_q4k_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__rest
 
     /* ---- prologue: codes of super-block 0, tiles 0..2 requested; tile 0 decoded; fragments of its k-step 0 fetched */
     c.sb = 0;
-    load_sb<0>(c, c.cur, 0); load_sb<1>(c, c.cur, 0); load_sb<2>(c, c.cur, 0); load_sb<3>(c, c.cur, 0); load_sb<4>(c, c.cur, 0);
+    request_w<0>(c, 0); request_w<1>(c, 0); request_w<2>(c, 0); request_w<3>(c, 0); request_w<4>(c, 0);
     request_tile<0>(c, 0, std::make_integer_sequence<int, 8>{});
+    wait_vmcnt<8>();
+    load_sb<0>(c, c.cur); load_sb<1>(c, c.cur); load_sb<2>(c, c.cur); load_sb<3>(c, c.cur); load_sb<4>(c, c.cur);
+    __builtin_amdgcn_s_waitcnt(0xC07F); /* lgkmcnt(0): the registers hold super-block 0 before its place is requested again */
+    request_w<0>(c, 1); request_w<1>(c, 1); request_w<2>(c, 1); request_w<3>(c, 1); request_w<4>(c, 1);
     request_tile<1>(c, 1, std::make_integer_sequence<int, 8>{});
     request_tile<2>(c, 2, std::make_integer_sequence<int, 8>{});
     unpack0(c, c.cur.hdr); unpack1(c, c.cur.hdr); unpack2(c, c.cur.hdr); unpack3(c, c.cur.hdr);
     decode_first(c, std::make_integer_sequence<int, 44>{});
-    wait_vmcnt<16>(); /* tile 0 is in LDS as far as this wave's requests go */
+    wait_vmcnt<21>(); /* tile 0 is in LDS as far as this wave's requests go */
     __builtin_amdgcn_s_barrier();
     c.xf[0][0] = load_frag<0, 0, 0>(c); c.xf[0][1] = load_frag<0, 0, 1>(c); c.xf[0][2] = load_frag<0, 0, 2>(c);
     c.xf[0][3] = load_frag<0, 0, 3>(c); c.xf[0][4] = load_frag<0, 0, 4>(c); c.xf[0][5] = load_frag<0, 0, 5>(c);
