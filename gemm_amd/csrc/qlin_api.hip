@@ -724,7 +724,7 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
         const uint16_t *Xb = (const uint16_t *)g.tmp[2].p;
         float *Yd = (float *)g.tmp[1].p;
         const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-        if (type == T_Q4_K && (n_tok <= kFewTokens || (n_tok <= 512 && tiles >= 200))) {
+        if (type == T_Q4_K && (n_tok <= kFewTokens || tiles >= 200)) {
             HIP_TRY(launch_gemm_q4k_bf16(dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
         } else {
             const uint16_t *Wd = (const uint16_t *)dW;
@@ -1024,12 +1024,12 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
     if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
         return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
-    /* Q4_K: the fused kernels (no workspace) for a few tokens, and up to 512 tokens where their 256-token x
-     * 128-row tiles fill the chip; with fewer than 200 tiles (4096 rows: 64) the decode + library route is
-     * faster (4096 x 14336 at 512 tokens: 105 vs 162 us; 14336 x 4096: 96 vs 77 us) */
+    /* Q4_K: the fused kernels (no workspace) for a few tokens, and wherever their 256-token x 128-row tiles fill
+     * the chip (14336 x 4096: 60 us at 512 tokens, 231 at 2048; decode + library product 96 and 231); with fewer
+     * than 200 tiles (4096 rows at 512 tokens: 64) the decode + library route is faster (4096 x 14336: 105 vs 162 us) */
     if (type == T_Q4_K) {
         const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-        if (n_tok <= kFewTokens || (n_tok <= 512 && tiles >= 200))
+        if (n_tok <= kFewTokens || tiles >= 200)
             return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     }
     /* a few tokens of a Q6_K, Q5_K, Q3_K, Q2_K or Q8_0 tensor: streamed once per eight tokens with exact codes
