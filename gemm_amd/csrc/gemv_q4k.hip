@@ -45,6 +45,7 @@
  */
 #include "qlin_device.h"
 #include "qlin_internal.h"
+#include <stdlib.h>
 
 namespace qlin {
 
@@ -308,6 +309,109 @@ gemv_q4k_kernel(const JobView job, const float *__restrict__ x, int n_sb, int ro
     }
 }
 
+/* The same matvec for one matrix of rows of at most 4096 elements and at most kDmaRows rows per workgroup, with the
+ * blocks fetched by the load-to-LDS path: wave w copies super-block w of all the workgroup's rows (runs of 144
+ * contiguous bytes, consecutive lanes consecutive 16-byte pieces) into its own LDS image with eight requests
+ * issued at once, and takes the matrix operands of a row group from there as soon as the requests that cover it
+ * have landed (requests complete in order: three cover the first 16 rows, five the first 32, seven the first 48).
+ * What the memory pipe sees is then 64 contiguous bytes per four lanes instead of four rows per four lanes.
+ * All vector-memory instructions of the loop are written out with their own waits: the compiler's counters
+ * would make the first wait cover every request. */
+/* s_waitcnt vmcnt(N) that the compiler moves no memory access across (and, with an argument, no use of it) */
+template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
+template <int N> __device__ __forceinline__ void wait_vm(v4f &v) { asm volatile("s_waitcnt vmcnt(%1)" : "+v"(v) : "n"(N) : "memory"); }
+constexpr int kDmaRows = 56;
+constexpr int kDmaImage = 8192; /* 56 x 144 B = 8064 */
+
+/* NQ: requests per wave = ceil(rows per workgroup x 9 / 64) */
+template <int NQ>
+__global__ void __launch_bounds__(kWaves * 64)
+gemv_q4k_dma_kernel(const uint8_t *__restrict__ W, float *__restrict__ y, const float *__restrict__ x, int n_rows,
+                    int n_sb, int add, int rows_per_wg, size_t row_bytes) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * rows_per_wg;
+    int rows_here = n_rows - row0;
+    if (rows_here > rows_per_wg) rows_here = rows_per_wg;
+    const int n_rg = (rows_here + 15) >> 4;
+    /* LDS map: images [kWaves][kDmaImage] | x scratch [kWaves][kXScratch] | partial sums [rows][kWaves] */
+    uint8_t *img = lds + wv * kDmaImage;
+    uint8_t *xs = lds + kWaves * kDmaImage + wv * kXScratch;
+    float *partial = reinterpret_cast<float *>(lds + kWaves * (kDmaImage + kXScratch));
+
+    auto store_partial = [&](int rg, float v) { /* the four lane groups hold four sub-blocks' shares of the same row */
+        v = sum_lane_groups(v);
+        const int lr = 16 * rg + n;
+        if (lane < 16 && lr < rows_here) partial[lr * kWaves + wv] = v;
+    };
+    if (wv >= n_sb) { /* a wave without a super-block (K < 4096) contributes zeros */
+        for (int rg = 0; rg < n_rg; rg++) store_partial(rg, 0.0f);
+    } else {
+        /* x first, then the eight requests: piece id = 64 q + lane is part id % 9 of row id / 9 */
+        v4f xv;
+        const uint32_t x_off = (uint32_t)(wv * 256 + 4 * lane) * 4u;
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(xv) : "v"(x_off), "s"(x) : "memory");
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint8_t *>(W) + (size_t)row0 * row_bytes + (size_t)wv * 144, 0,
+            (int)((size_t)(rows_here - 1) * row_bytes + 144), 0x00020000);
+        const uint32_t img_base = (uint32_t)(uintptr_t)img; /* LDS addresses are the low 32 bits of the flat ones */
+        /* 64 = 7 x 9 + 1: from one request to the next a lane moves on seven rows and one part (eight rows when the
+         * part wraps). Pieces past the last row lie outside the descriptor and arrive as zeros. */
+        uint32_t part = (uint32_t)lane % 9u, voff = ((uint32_t)lane / 9u) * (uint32_t)row_bytes + 16u * part;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                         :
+                         : "s"(img_base + 1024u * q), "v"(voff), "s"(rsrc)
+                         : "memory");
+            const bool wrap = part == 8u;
+            part = wrap ? 0u : part + 1u;
+            voff += 7u * (uint32_t)row_bytes + (wrap ? (uint32_t)row_bytes - 128u : 16u);
+        }
+        wait_vm<NQ>(xv);
+        XOperand xo;
+        q4k_prepare(xv, xo, xs, lane);
+        auto run = [&](int rg) {
+            int lr = 16 * rg + n;
+            if (lr >= rows_here) lr = rows_here - 1; /* rows past the end: the last one, never stored */
+            const uint8_t *blk = img + lr * 144;
+            const uint4 h = *reinterpret_cast<const uint4 *>(blk);
+            const uint4 q0 = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+            const uint4 q1 = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
+            store_partial(rg, q4k_item(xo, h, q0, q1, g));
+        };
+        /* row group rg is covered by requests 0 .. (144 (rg + 1) - 1) / 64 */
+        wait_vm<(NQ - 3 > 0 ? NQ - 3 : 0)>();
+        run(0);
+        if (n_rg > 1) {
+            wait_vm<(NQ - 5 > 0 ? NQ - 5 : 0)>();
+            run(1);
+        }
+        if (n_rg > 2) {
+            wait_vm<(NQ - 7 > 0 ? NQ - 7 : 0)>();
+            run(2);
+        }
+        if (n_rg > 3) {
+            wait_vm<0>();
+            run(3);
+        }
+        wait_vm<0>(); /* nothing on its way into LDS when the wave ends */
+    }
+    __syncthreads();
+    for (int lr = threadIdx.x; lr < rows_here; lr += kWaves * 64) {
+        const float4 *p = reinterpret_cast<const float4 *>(partial + lr * kWaves);
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kWaves / 4; k++) {
+            const float4 v = p[k];
+            s += (v.x + v.y) + (v.z + v.w);
+        }
+        y[row0 + lr] = add ? y[row0 + lr] + s : s;
+    }
+}
+
 /* A token (or a few, each on its own) through its top_k routed experts, Q4_K expert tensors (the reference's MoE block for a token,
  * common/transformer.h:4045-4131: sum_j w_j * down_e(silu(gate_e x) * up_e x), e = idx[j]), as two launches of the
  * matvec above:
@@ -467,6 +571,31 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, row_stride,
                            grid < n_cu ? 1 : 0);
     };
+    static const bool no_dma = getenv("QLIN_GEMV_NODMA") != nullptr; /* DEV */
+    if (!no_dma && one && n_sb <= 16 && rows_per_wg <= kDmaRows && (size_t)kDmaRows * row_stride < ((size_t)1 << 31)) {
+        auto launch_dma = [&](auto kernel, OnceFlag &lds_raised) {
+            if (!lds_raised.is_set()) {
+                hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                lds_raised.set();
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64),
+                               (size_t)kWaves * (kDmaImage + kXScratch) + (size_t)rows_per_wg * kWaves * 4, stream,
+                               (const uint8_t *)job.W[0], job.y[0], x, n_rows, n_sb, job.mode == kAdd ? 1 : 0, rows_per_wg, row_stride);
+            return hipGetLastError();
+        };
+        static OnceFlag raised[8];
+        switch ((rows_per_wg * 9 + 63) / 64) {
+        case 1: return launch_dma(gemv_q4k_dma_kernel<1>, raised[0]);
+        case 2: return launch_dma(gemv_q4k_dma_kernel<2>, raised[1]);
+        case 3: return launch_dma(gemv_q4k_dma_kernel<3>, raised[2]);
+        case 4: return launch_dma(gemv_q4k_dma_kernel<4>, raised[3]);
+        case 5: return launch_dma(gemv_q4k_dma_kernel<5>, raised[4]);
+        case 6: return launch_dma(gemv_q4k_dma_kernel<6>, raised[5]);
+        case 7: return launch_dma(gemv_q4k_dma_kernel<7>, raised[6]);
+        default: return launch_dma(gemv_q4k_dma_kernel<8>, raised[7]);
+        }
+    }
     if (n_sb <= 16) {
         if (one) launch(gemv_q4k_kernel<1, true>);
         else launch(gemv_q4k_kernel<1, false>);
