@@ -45,7 +45,6 @@
  */
 #include "qlin_device.h"
 #include "qlin_internal.h"
-#include <stdlib.h>
 
 namespace qlin {
 
@@ -571,8 +570,8 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds_bytes, stream, view, x, n_sb, rows_per_wg, row_stride,
                            grid < n_cu ? 1 : 0);
     };
-    static const bool no_dma = getenv("QLIN_GEMV_NODMA") != nullptr; /* DEV */
-    if (!no_dma && one && n_sb <= 16 && rows_per_wg <= kDmaRows && (size_t)kDmaRows * row_stride < ((size_t)1 << 31)) {
+    /* one matrix, rows of up to 4096 elements, at most 56 rows per workgroup: the load-to-LDS kernel */
+    if (one && n_sb <= 16 && rows_per_wg <= kDmaRows && (size_t)kDmaRows * row_stride < ((size_t)1 << 31)) {
         auto launch_dma = [&](auto kernel, OnceFlag &lds_raised) {
             if (!lds_raised.is_set()) {
                 hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
