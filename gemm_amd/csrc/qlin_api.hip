@@ -726,6 +726,8 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
         const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
         if (type == T_Q4_K && (n_tok <= kFewTokens || tiles >= 200)) {
             HIP_TRY(launch_gemm_q4k_bf16(dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
+        } else if (gemm_kq_wave4_covers(type) && tiles >= 200 && n_cols % 256 == 0 && n_cols < (1 << 22)) {
+            HIP_TRY(launch_gemm_kq_bf16_wave4(type, dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
         } else {
             const uint16_t *Wd = (const uint16_t *)dW;
             if (type != T_BF16) {
@@ -1041,12 +1043,19 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
             return QLIN_OK;
         }
     }
-    if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols))
-        return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes");
     {
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
+    /* Q5_K and Q6_K where the fused kernel's tiles fill the chip: decoded into the matrix operand like Q4_K, no
+     * workspace (14336 x 4096 at 512 tokens: decode + library product 92 and 84 us) */
+    if (gemm_kq_wave4_covers(type) && n_cols % 256 == 0 && ldx < (1 << 22) &&
+        (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256) >= 200) {
+        HIP_TRY(launch_gemm_kq_bf16_wave4(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        return QLIN_OK;
+    }
+    if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+        return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes");
     /* up to four tokens of any other block format: each through the matvec (exact weights; 14336 x 4096 IQ4_XS, four
      * tokens: 44 us against 95 us for decode + dense product), x widened to fp32 at the start of the workspace */
     const size_t x_span = (size_t)(n_tok - 1) * ldx + n_cols; /* elements of X from the first token's to the last's */

@@ -128,7 +128,11 @@ constexpr int kMatvecTokens = 4; /* qlin_gemm_bf16_any_dev: up to this many toke
 constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
 hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                   int ldx, int ldy, hipStream_t stream);
-/* 256-token x 128-row tiles on four waves, one per SIMD (gemm_q4k_wave4.hip): n_cols % 256 == 0, ldx < 2^22 */
+/* 256-token x 128-row tiles on four waves, one per SIMD, weights decoded from their blocks into the matrix operand
+ * (gemm_kq_wave4.hip): the formats of gemm_kq_wave4_covers, n_cols % 256 == 0, ldx < 2^22 */
+bool gemm_kq_wave4_covers(uint32_t type);
+hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                                     int n_tok, int ldx, int ldy, hipStream_t stream);
 hipError_t launch_gemm_q4k_bf16_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                       int ldx, int ldy, hipStream_t stream);
 hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,

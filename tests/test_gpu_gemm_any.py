@@ -87,6 +87,54 @@ def test_shapes(oracle, tid, n_tok, n_rows, n_cols, dense_kernel):
     assert rel_l2(Y, exact) <= 3e-3
 
 
+FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K]
+
+
+@pytest.mark.parametrize("tid", FUSED, ids=lambda t: ALL[t])
+@pytest.mark.parametrize("n_tok,n_rows,n_cols", [
+    (260, 12805, 256),   # 101 x 2 tiles: one super-block, ragged rows and tokens
+    (1030, 5130, 768),   # 41 x 5 tiles, an odd super-block count
+    (513, 8500, 1024),
+])
+def test_fused_tile_kernel_shapes(oracle, tid, n_tok, n_rows, n_cols):
+    """200 or more 256-token x 128-row tiles: Q4_K, Q5_K and Q6_K are decoded inside the product (no workspace is
+    read: none is passed); weights rounded once to bf16, as the decode + dense route rounds them"""
+    W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + tid)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=n_tok + tid, tokens=n_tok))
+    ldx, ldy = n_cols + 8, n_rows + 3
+    Xpad = np.zeros((n_tok, ldx), np.uint16)
+    Xpad[:, :n_cols] = Xb
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xpad)
+    dY = qlinear.DevBuf.from_numpy(np.full((n_tok, ldy), -3.0, np.float32))
+    qlinear.check(qlinear.load().qlin_gemm_bf16_any_dev(tid, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy,
+                                                        None, 0, None))
+    qlinear.sync()
+    Y = dY.to_numpy(np.float32, (n_tok, ldy))
+    for buf in (dW, dX, dY):
+        buf.free()
+    assert np.all(Y[:, n_rows:] == -3.0)
+    rows = np.unique(np.concatenate([np.random.default_rng(n_tok).choice(n_rows, 300, replace=False),
+                                     np.arange(n_rows - 140, n_rows)]))  # a sample, and the ragged last tiles whole
+    exact, designed = references(oracle, tid, W[rows], Xb, n_cols)
+    assert rel_l2(Y[:, rows], designed) <= 2e-5, (ALL[tid], n_tok, n_rows, n_cols)
+    assert rel_l2(Y[:, rows], exact) <= 3e-3
+
+
+@pytest.mark.parametrize("tid", [synth.GGML_Q5_K, synth.GGML_Q6_K], ids=lambda t: ALL[t])
+def test_fused_tile_kernel_full_size_config(oracle, tid):
+    """14336 x 4096 at 512 tokens; the oracle on a sample of rows, and scaling X by two scales Y exactly"""
+    n_rows, n_cols, n_tok = 14336, 4096, 512
+    W = synth.make_weights(tid, n_rows, n_cols, seed=43)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=44, tokens=n_tok))
+    Y = run(tid, W, Xb, n_rows, n_cols, n_tok)
+    rows = np.random.default_rng(2).choice(n_rows, 160, replace=False)
+    exact, designed = references(oracle, tid, W[rows], Xb, n_cols)
+    assert rel_l2(Y[:, rows], designed) <= 2e-5
+    assert rel_l2(Y[:, rows], exact) <= 3e-3
+    Y2 = run(tid, W, synth.to_bf16_bits(2.0 * synth.bf16_bits_to_f32(Xb)), n_rows, n_cols, n_tok)
+    assert np.array_equal(Y2, 2.0 * Y)
+
+
 BLOCK_NOT_KQ = sorted(t for t in ALL if t not in KQ and t not in synth.DENSE_TYPES and t != Q4K)
 
 
