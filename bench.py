@@ -5,8 +5,8 @@
 
 A step is one Q4_K matvec y = W.x with W 14336 x 4096 (the decode-shape weight the headline
 metric is quoted on), x fp32, all inputs resident in HBM before the clock starts. Successive
-steps walk through enough distinct copies of W (> 256 MB in total) that no step finds its
-weights in the 256 MB last-level cache, so the figure is an HBM figure. The timed region is
+steps walk through enough distinct copies of W (1 GiB in total, four times the 256 MB last-level
+cache) that no step finds a useful part of its weights there, so the figure is an HBM figure. The timed region is
 bracketed by stream synchronisation and timed with HIP events recorded on the stream the
 kernels are launched on.
 
@@ -54,7 +54,7 @@ SPIN_UP_MS = 40.0  # untimed launches of the measured kernel before the warm-up 
 # memory clocks of an idle device take tens of milliseconds of work to settle (a step is 8-9 us)
 
 
-def time_gemv(type_id, n_rows, n_cols, steps, warmup, min_total_bytes=320 << 20, max_copies=24, spin_up_ms=0.0):
+def time_gemv(type_id, n_rows, n_cols, steps, warmup, min_total_bytes=1 << 30, max_copies=40, spin_up_ms=0.0):
     """-> (ms per step, number of weight copies)"""
     W = synth.make_weights(type_id, n_rows, n_cols, seed=20260 + type_id)
     x = synth.make_activation(n_cols, seed=7)
@@ -455,7 +455,7 @@ def probe(args):
         print(json.dumps({"probe": "gemv", "ms_per_step": ms, "copies": copies}))
     elif args.probe in ("gemv_q8_0", "gemv_q6_K"):
         tid, r, c = (synth.GGML_Q8_0, 4096, 4096) if args.probe == "gemv_q8_0" else (synth.GGML_Q6_K, 151936, 4096)
-        ms, copies = time_gemv(tid, r, c, max(10, args.steps // 8), 3, max_copies=24 if r < 100000 else 2)
+        ms, copies = time_gemv(tid, r, c, max(10, args.steps // 8), 3)
         print(json.dumps({"probe": args.probe, "ms_per_step": ms, "copies": copies}))
     elif args.probe == "gemv_any":  # --ptype NAME --prows R --pcols C: that matvec only
         tid = {v: k for k, v in list(synth.TYPE_NAMES.items()) + list(synth.DENSE_TYPES.items())}[args.ptype]
@@ -493,9 +493,12 @@ def probe(args):
     elif args.probe == "gemm":
         ms = time_gemm(512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm", "ms_per_step": ms}))
-    elif args.probe == "gemm_any_q6_K":  # decode to bf16 + dense library GEMM, Q6_K, 512 tokens
+    elif args.probe == "gemm_any_q6_K":  # Q6_K, 512 tokens: decoded inside the tile kernel
         ms = time_gemm_any(synth.GGML_Q6_K, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_any_q6_K", "ms_per_step": ms}))
+    elif args.probe == "gemm_any_q8_0":  # Q8_0, 512 tokens: decode to bf16 + dense library GEMM
+        ms = time_gemm_any(synth.GGML_Q8_0, 512, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_any_q8_0", "ms_per_step": ms}))
     elif args.probe == "gemm_f32_any_q4_K":  # decode to fp32 + dense fp32 library GEMM, Q4_K, 512 tokens
         ms = time_gemm_f32_any(Q4K, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_f32_any_q4_K", "ms_per_step": ms}))
@@ -505,7 +508,8 @@ def probe(args):
 
 
 def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
-    """Prefill GEMM for any format: decode to bf16 in a workspace + dense library GEMM. -> ms per step"""
+    """Prefill GEMM for any format (qlin_gemm_bf16_any_dev: decoded inside the tile kernel for the formats that has,
+    else decode to bf16 in a workspace + dense library GEMM). -> ms per step"""
     W = synth.make_weights(type_id, n_rows, n_cols, seed=70 + type_id)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=71, tokens=n_tok))
     dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xb)
@@ -519,6 +523,35 @@ def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
         qlinear.gemm_bf16_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
     ms = qlinear.timer_end() / steps
     for b in (dW, dX, dY, ws):
+        b.free()
+    return ms
+
+
+FUSED_GEMM_TYPES = (Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K)  # decoded inside the tile kernel where its tiles fill the chip
+
+
+def time_gemm_two_kernels(type_id, n_tok, n_rows, n_cols, steps, warmup):
+    """The route the fused kernel replaces, for comparison: decode the weights to bf16 in a workspace, then the
+    dense bf16 product on them. -> ms per step"""
+    W = synth.make_weights(type_id, n_rows, n_cols, seed=70 + type_id)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=71, tokens=n_tok))
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xb)
+    dY = qlinear.DevBuf(n_tok * n_rows * 4)
+    ws = qlinear.DevBuf(qlinear.gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+    dB = qlinear.DevBuf(n_rows * n_cols * 2)
+
+    def step():
+        qlinear.dequant_bf16_dev(type_id, dW, dB, n_rows, n_cols)
+        qlinear.gemm_bf16_any_dev(synth.GGML_BF16, dB, dX, dY, n_rows, n_cols, n_tok, n_cols, n_rows, ws)
+
+    for _ in range(warmup):
+        step()
+    qlinear.sync()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        step()
+    ms = qlinear.timer_end() / steps
+    for b in (dW, dX, dY, ws, dB):
         b.free()
     return ms
 
@@ -543,6 +576,24 @@ def time_gemm_f32_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
     return ms
 
 
+def time_hbm_read_rotating(nbytes=33030144, reps=200, total=1 << 30):
+    """A read-only streaming kernel over buffers of the headline's weight size, one launch per buffer, rotating
+    through 1 GiB of them like the headline: what one launch of that size can reach on this part, launch and
+    drain included. -> GB/s"""
+    copies = max(2, -(-total // nbytes))
+    bufs = [qlinear.DevBuf(nbytes) for _ in range(copies)]
+    for b in bufs:
+        qlinear.probe_hbm_read(b)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for i in range(reps):
+        qlinear.probe_hbm_read(bufs[i % copies])
+    ms = qlinear.timer_end() / reps
+    for b in bufs:
+        b.free()
+    return nbytes / (ms * 1e-3) / 1e9
+
+
 def time_achievable():
     """What the part sustains on the two priced resources: a register-only loop of the GEMM's matrix
     instruction (with the shader clock it ran at) and a streaming read of 512 MiB / of the headline's
@@ -557,19 +608,14 @@ def time_achievable():
         best = max(best, fl / (ms * 1e-3) / 1e12)
     out["mfma_bf16_32x32x16_register_loop_TFLOP/s"] = round(best, 1)
     out["shader_clock_MHz_in_that_loop"] = round(qlinear.probe_clocks(), 0)
-    for label, nbytes, reps in (("hbm_read_512MiB_GB/s", 512 << 20, 10), ("hbm_read_33MB_rotating_GB/s", 33030144, 40)):
-        copies = 1 if nbytes > (256 << 20) else 11
-        bufs = [qlinear.DevBuf(nbytes) for _ in range(copies)]
-        for b in bufs:
-            qlinear.probe_hbm_read(b)
-        qlinear.sync()
-        qlinear.timer_begin()
-        for i in range(reps):
-            qlinear.probe_hbm_read(bufs[i % copies])
-        ms = qlinear.timer_end() / reps
-        out[label] = round(nbytes / (ms * 1e-3) / 1e9, 1)
-        for b in bufs:
-            b.free()
+    big = qlinear.DevBuf(512 << 20)
+    qlinear.probe_hbm_read(big)
+    qlinear.sync()
+    qlinear.timer_begin()
+    for i in range(10):
+        qlinear.probe_hbm_read(big)
+    out["hbm_read_512MiB_GB/s"] = round((512 << 20) / (qlinear.timer_end() / 10 * 1e-3) / 1e9, 1)
+    big.free()
     return out
 
 
@@ -586,7 +632,7 @@ def main():
     ap.add_argument("--prows", type=int, default=4096)
     ap.add_argument("--pcols", type=int, default=14336)
     ap.add_argument("--ptok", type=int, default=64, help="--probe moe: tokens in the batch")
-    ap.add_argument("--probe", choices=["gemv_any", "copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["gemv_any", "copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
@@ -602,6 +648,7 @@ def main():
     t0 = time.time()
     ms, copies = time_gemv(Q4K, n_rows, n_cols, args.steps, args.warmup, spin_up_ms=args.spin_up_ms)
     gbps = nbytes / (ms * 1e-3) / 1e9
+    floor_gbps = time_hbm_read_rotating()
 
     extra = {}
     if not args.no_extra:
@@ -615,7 +662,7 @@ def main():
         gemv = {}
         for tname, tid, r, c in shapes:
             st = max(20, args.steps // 8)
-            m, _ = time_gemv(tid, r, c, st, 4, max_copies=24 if r < 100000 else 2)
+            m, _ = time_gemv(tid, r, c, st, 4)
             b = gemv_bytes(tid, r, c)
             gemv["%s_%dx%d" % (tname, r, c)] = {"us": round(m * 1e3, 2), "GB/s": round(b / (m * 1e-3) / 1e9, 1)}
         extra["gemv_other_shapes"] = gemv
@@ -627,16 +674,24 @@ def main():
         extra["q4k_prefill_gemm_14336x4096_bf16"] = gemm
         tf = gemm["M=512"]["TFLOP/s"]
         anyfmt = {}
-        for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("q8_0", synth.GGML_Q8_0, 512), ("q5_K", synth.GGML_Q5_K, 512),
+        for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q8_0", synth.GGML_Q8_0, 512),
                               ("iq4_nl", synth.GGML_IQ4_NL, 512), ("bf16", synth.GGML_BF16, 512), ("q4_K", Q4K, 2048),
-                              ("q6_K", synth.GGML_Q6_K, 2048)):
+                              ("q5_K", synth.GGML_Q5_K, 2048), ("q6_K", synth.GGML_Q6_K, 2048)):
             m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
-            anyfmt["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
-        extra["prefill_gemm_any_format_14336x4096_decode_to_bf16_plus_library_gemm"] = anyfmt
+            anyfmt["%s_M=%d" % (tname, M)] = {
+                "us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1),
+                "route": "decoded inside the product, no workspace" if tid in FUSED_GEMM_TYPES else
+                         "dense library product" if tid == synth.GGML_BF16 else "decode to bf16 + dense library product"}
+        extra["prefill_gemm_any_format_14336x4096"] = anyfmt
+        two = {}
+        for tname, tid, M in (("q4_K", Q4K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q6_K", synth.GGML_Q6_K, 512)):
+            m = time_gemm_two_kernels(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
+            two["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
+        extra["prefill_gemm_14336x4096_decode_to_bf16_plus_library_gemm_for_comparison"] = two
         own = {}
         qlinear.check(qlinear.load().qlin_set_dense_gemm_own(1))
         try:
-            for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("bf16", synth.GGML_BF16, 512), ("q6_K", synth.GGML_Q6_K, 2048)):
+            for tname, tid, M in (("q8_0", synth.GGML_Q8_0, 512), ("bf16", synth.GGML_BF16, 512), ("q8_0", synth.GGML_Q8_0, 2048)):
                 m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
                 own["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
         finally:
@@ -705,7 +760,12 @@ def main():
                    "device_spin_up": "untimed launches of the same kernel ahead of the warm-up steps until the clocks "
                                      "of the idle device have settled; the timed region is the given steps only"},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": PROFILED_TRAFFIC_BYTES,
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "launch_floor_frac": round(floor_gbps / HBM_PEAK_GBPS, 4),
+                     "launch_floor": "a read-only streaming kernel over the same 33 MB per launch, same rotation: %.1f GB/s; "
+                                     "what is left of the peak once a launch of this size has filled and drained the "
+                                     "chip" % floor_gbps,
+                     "traffic": PROFILED_TRAFFIC_BYTES,
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, scaled by a copy of "
                                        "known size; not re-measured by this run (" + PROFILED_TRAFFIC_SOURCE + ")"},
     }

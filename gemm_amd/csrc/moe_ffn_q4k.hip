@@ -504,20 +504,13 @@ __device__ __forceinline__ TileElem tile_elem(int idx) {
 __device__ __forceinline__ int live_slots(int cnt, int t0) { return cnt - t0 < 16 ? cnt - t0 : 16; }
 
 /* ---- 2. gate and up for RT * 16 rows of one expert, all of its tokens ---- */
-#ifndef MOE_GU_WAVES
-#define MOE_GU_WAVES 2
-#endif
-#ifndef MOE_DN_WAVES
-#define MOE_DN_WAVES 2
-#endif
-#ifndef MOE_GU_WG_WAVES
-#define MOE_GU_WG_WAVES 4
-#endif
-#ifndef MOE_GU_RT
-#define MOE_GU_RT 1
-#endif
+/* launch shape of the grouped kernels, as measured best at 128 experts of 768 x 2048, 64 tokens, top-8 */
+constexpr int kGuWavesPerSimd = 2; /* gate+up kernel: waves per SIMD the registers are budgeted for */
+constexpr int kDnWavesPerSimd = 2; /* down kernels: the same */
+constexpr int kGuWgWaves = 4;      /* gate+up kernel: waves of a workgroup (each takes a share of K) */
+constexpr int kGuRowTiles = 1;     /* gate+up kernel: 16-row tiles per workgroup */
 template <int RT>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_GU_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(kGuWavesPerSimd)))
 moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__ up,
                    const uint16_t *__restrict__ X, const int32_t *__restrict__ head,
                    const int32_t *__restrict__ order, uint16_t *__restrict__ h_hi, uint16_t *__restrict__ h_lo,
@@ -613,11 +606,9 @@ moe_gate_up_kernel(const uint8_t *__restrict__ gate, const uint8_t *__restrict__
 }
 
 /* ---- 3. down for RT * 16 rows of one expert ---- */
-#ifndef MOE_DN_RT
-#define MOE_DN_RT 2
-#endif
+constexpr int kDnRowTiles = 2; /* down kernels: 16-row tiles per workgroup */
 template <int RT>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(kDnWavesPerSimd)))
 moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                 const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets, float *__restrict__ part,
                 int n_embd, int n_ff, const int32_t *__restrict__ routed) {
@@ -663,11 +654,9 @@ moe_down_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h
  * expert's activations and routing weights are fetched once for all NT groups. A (expert, 32 rows)
  * workgroup lives for four or five memory round trips and moves 14 KB of weights; with a handful of them
  * on a compute unit that bounded the kernel at a quarter of HBM speed. */
-#ifndef MOE_DN_NT
-#define MOE_DN_NT 4
-#endif
+constexpr int kDnColTiles = 4; /* wide down kernel: row-tile groups that share one workgroup's activations */
 template <int RT, int NT>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(MOE_DN_WAVES)))
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(kDnWavesPerSimd)))
 moe_down_walk_kernel(const uint8_t *__restrict__ down, const uint16_t *__restrict__ h_hi,
                      const uint16_t *__restrict__ h_lo, const int32_t *__restrict__ offsets,
                      float *__restrict__ part, int n_embd, int n_ff, const int32_t *__restrict__ routed) {
@@ -1639,7 +1628,7 @@ size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_exp
 
 hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
                           const void *down, const uint16_t *X, const int32_t *idx, const float *w, float *out, int n_tok,
-                          int top_k, int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream) {
+                          int top_k, int n_embd, int n_ff, int n_expert, int n_cu, void *workspace, hipStream_t stream) {
     const Workspace ws = carve(workspace, n_tok, top_k, n_embd, n_ff, n_expert);
     const int n_pairs = n_tok * top_k;
     /* One token (the reference's own case), or up to eight that will mostly meet different experts (two pairs or
@@ -1649,12 +1638,6 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
      * Q4_K experts on the Q4_K matvec, the other common expert formats on the matrix-instruction matvec (gate and up of
      * one type; 1 token: Q4_K/Q4_K/Q6_K 21.6 -> 13.5, Q6_K 25.9 -> 15.7, Q8_0 26.0 -> 13.2, IQ4_XS 62.7 -> 12.4). */
     if (n_tok == 1 || (n_tok <= 8 && 2 * n_pairs <= n_expert)) {
-        static int n_cu = 0;
-        if (n_cu == 0) {
-            int dev = 0, v = 0;
-            if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n_cu = v;
-            else n_cu = 256;
-        }
         hipError_t e1 = hipSuccess;
         auto up_step = [&](bool dry) {
             if (type_gate == T_Q4_K && type_up == T_Q4_K)
@@ -1685,22 +1668,22 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                        n_pairs, n_expert, ws.offsets, ws.order, ws.slot_of, ws.head, top_k);
     static OnceFlag lds_raised;
     if (!lds_raised.is_set()) {
-        hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<MOE_GU_RT>,
+        hipError_t e1 = hipFuncSetAttribute((const void *)moe_gate_up_kernel<kGuRowTiles>,
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e1 != hipSuccess) return e1;
         lds_raised.set();
     }
     /* Q4_K matrices take the matrix-core kernels; any other format (or a shape their tiles do not divide)
      * the any-format kernel, matrix by matrix: gate and up -> fp32 by slot -> silu(g)*u as head + tail */
-    const bool fast_gu = type_gate == T_Q4_K && type_up == T_Q4_K && n_embd % 256 == 0 && n_ff % (16 * MOE_GU_RT) == 0;
-    const bool fast_dn = type_down == T_Q4_K && n_ff % 256 == 0 && n_embd % (16 * MOE_DN_RT) == 0;
+    const bool fast_gu = type_gate == T_Q4_K && type_up == T_Q4_K && n_embd % 256 == 0 && n_ff % (16 * kGuRowTiles) == 0;
+    const bool fast_dn = type_down == T_Q4_K && n_ff % 256 == 0 && n_embd % (16 * kDnRowTiles) == 0;
     /* waves per workgroup = super-blocks of K, at most 4 for gate/up (a wave then walks several
      * super-blocks one after the other) and 8 for down. The gate/up kernel needs 138 registers, so a
      * compute unit holds 12 of its waves: three 4-wave workgroups in different phases instead of one
      * 8-wave workgroup that loads, computes and reduces with nothing beside it (75 -> 65 us). */
-    const int gu_waves = n_embd / 256 < MOE_GU_WG_WAVES ? n_embd / 256 : MOE_GU_WG_WAVES, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
+    const int gu_waves = n_embd / 256 < kGuWgWaves ? n_embd / 256 : kGuWgWaves, dn_waves = n_ff / 256 < 8 ? n_ff / 256 : 8;
     if (fast_gu) {
-        constexpr int RT = MOE_GU_RT;
+        constexpr int RT = kGuRowTiles;
         hipLaunchKernelGGL(moe_gate_up_kernel<RT>, dim3(n_ff / (16 * RT), grid_y), dim3(64 * gu_waves),
                            (size_t)gu_waves * 2 * RT * (1024 + 16 * kQ4KBlock + 256), stream,
                            (const uint8_t *)gate, (const uint8_t *)up, X, ws.head, ws.order, ws.h_hi, ws.h_lo, n_embd,
@@ -1731,9 +1714,9 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
                            ws.h_hi, ws.h_lo, n);
     }
     /* a handful of routed experts: the walk's 128-row workgroups would leave most compute units idle */
-    const bool few_tiles = routed && (long long)grid_y * (n_embd / (16 * MOE_DN_RT * MOE_DN_NT)) < 512;
-    if (fast_dn && n_ff / 256 <= dn_waves && n_embd % (16 * MOE_DN_RT * MOE_DN_NT) == 0 && !few_tiles) {
-        constexpr int DRT = MOE_DN_RT, DNT = MOE_DN_NT;
+    const bool few_tiles = routed && (long long)grid_y * (n_embd / (16 * kDnRowTiles * kDnColTiles)) < 512;
+    if (fast_dn && n_ff / 256 <= dn_waves && n_embd % (16 * kDnRowTiles * kDnColTiles) == 0 && !few_tiles) {
+        constexpr int DRT = kDnRowTiles, DNT = kDnColTiles;
         static OnceFlag walk_lds_raised;
         if (!walk_lds_raised.is_set()) { /* 8 waves: 90 KB */
             hipError_t e1 = hipFuncSetAttribute((const void *)moe_down_walk_kernel<DRT, DNT>,
@@ -1776,7 +1759,7 @@ hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_do
         default: go(KqQ8_0()); break;
         }
     } else if (fast_dn) {
-        constexpr int DRT = MOE_DN_RT;
+        constexpr int DRT = kDnRowTiles;
         hipLaunchKernelGGL(moe_down_kernel<DRT>, dim3(n_embd / (16 * DRT), grid_y), dim3(64 * dn_waves),
                            (size_t)dn_waves * DRT * (1024 + 16 * kQ4KBlock), stream,
                            (const uint8_t *)down, ws.h_hi, ws.h_lo, ws.offsets, ws.part, n_embd, n_ff, routed);
@@ -1811,13 +1794,13 @@ hipError_t moe_static_scratch_setup(int device) {
 hipError_t launch_moe_ffn_static(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate,
                                  const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
                                  float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int device,
-                                 hipStream_t stream) {
+                                 int n_cu, hipStream_t stream) {
     if (device < 0 || device >= kMaxScratchDevices || !g_scratch_ptr[device]) return hipErrorNotInitialized;
     if (moe_workspace_bytes(n_tok, top_k, n_embd, n_ff, n_expert) > kMoeStaticScratchBytes) return hipErrorInvalidValue;
     /* nothing in the workspace has to start at zero: the grouping kernel writes every offset, slot and weight
      * it later reads, and the expert kernels write every slot row the combine step reads */
     return launch_moe_ffn(type_gate, type_up, type_down, gate, up, down, X, idx, w, out, n_tok, top_k, n_embd, n_ff,
-                          n_expert, g_scratch_ptr[device], stream);
+                          n_expert, n_cu, g_scratch_ptr[device], stream);
 }
 
 }  // namespace qlin

@@ -17,6 +17,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <map>
 #include <vector>
 #include <mutex>
@@ -30,6 +31,21 @@ namespace {
 using namespace qlin;
 
 thread_local std::string t_error;
+
+/* qlin_timer_begin / _end: the event pair belongs to the calling thread, so that threads timing their own streams do
+ * not overwrite each other's start event; it goes when the thread ends or calls qlin_shutdown */
+struct ThreadTimer {
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool begun = false;
+    void reset() {
+        if (ev0) (void)hipEventDestroy(ev0);
+        if (ev1) (void)hipEventDestroy(ev1);
+        ev0 = ev1 = nullptr;
+        begun = false;
+    }
+    ~ThreadTimer() { reset(); }
+};
+thread_local ThreadTimer t_timer;
 
 int fail(int code, const char *fmt, ...) {
     char buf[512];
@@ -107,13 +123,17 @@ struct State {
     size_t up_used = 0, down_used = 0;
     struct Pending { void *host; const void *staged; size_t bytes; };
     std::vector<Pending> pending;
-    bool dense_gemm_library = true; /* bf16 products by the vendor library (faster); QLIN_DENSE_GEMM=own or
-                                       qlin_set_dense_gemm_own(1): by this library's tile kernel */
+    /* 0: the vendor library, 1: this library's tile kernel, 2: neither (the vector-ALU kernel); read by device-pointer
+     * calls outside the lock */
+    std::atomic<int> dense_gemm_mode{0}; /* bf16 products by the vendor library (faster) unless QLIN_DENSE_GEMM=own or
+                                            qlin_set_dense_gemm_own say otherwise */
     bool prefill_bf16 = false; /* qlin_gemm_tokenmajor on the matrix cores (opt-in: costs accuracy) */
 } g;
 
 int ensure_init_locked(int device) {
     if (!g.pending.empty() || g.up_used || g.down_used) { /* left by a call that failed before it finished */
+        /* its kernels may still be reading or writing the staging regions that the offsets are about to hand out again */
+        if (g.stream) (void)hipStreamSynchronize(g.stream);
         g.pending.clear();
         g.up_used = g.down_used = 0;
     }
@@ -129,7 +149,7 @@ int ensure_init_locked(int device) {
     HIP_TRY(hipStreamCreate(&g.stream));
     g.device = device;
     if (const char *e = getenv("QLIN_PREFILL_MATRIX_CORES")) g.prefill_bf16 = e[0] == '1';
-    if (const char *e = getenv("QLIN_DENSE_GEMM")) g.dense_gemm_library = e[0] != 'o';
+    if (const char *e = getenv("QLIN_DENSE_GEMM")) g.dense_gemm_mode = e[0] == 'o' ? 1 : 0;
     if (hipHostMalloc((void **)&g.pinned, 2 * kPinnedHalf, hipHostMallocMapped) != hipSuccess) {
         g.pinned = nullptr; /* transfers then go straight from and to the caller's memory */
         (void)hipGetLastError();
@@ -137,7 +157,15 @@ int ensure_init_locked(int device) {
         g.pinned_dev = nullptr;
         (void)hipGetLastError();
     }
-    HIP_TRY(moe_static_scratch_setup(device)); /* address of the no-allocation entry point's scratch on this device */
+    /* address of the no-allocation entry point's scratch on this device */
+    if (hipError_t e = moe_static_scratch_setup(device); e != hipSuccess) {
+        /* a retry starts from nothing: no second stream, no second staging buffer */
+        if (g.pinned) (void)hipHostFree(g.pinned);
+        g.pinned = g.pinned_dev = nullptr;
+        (void)hipStreamDestroy(g.stream);
+        g.stream = nullptr;
+        return fail(QLIN_ERR_DEVICE, "looking up the built-in scratch failed: %s", hipGetErrorString(e));
+    }
     g.ready = true;
     return QLIN_OK;
 }
@@ -452,6 +480,7 @@ void qlin_shutdown(void) {
     (void)hipStreamDestroy(g.stream);
     g.stream = nullptr;
     g.ready = false;
+    t_timer.reset();
 }
 
 const char *qlin_last_error(void) { return t_error.c_str(); }
@@ -774,7 +803,8 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
 int qlin_set_dense_gemm_own(int enable) {
     std::lock_guard<std::mutex> lk(g.mu);
     if (int rc = ensure_init_locked(0)) return rc;
-    g.dense_gemm_library = enable == 0;
+    if (enable < 0 || enable > 2) return fail(QLIN_ERR_ARG, "0: vendor library, 1: own tile kernel, 2: vector-ALU kernel");
+    g.dense_gemm_mode = enable;
     return QLIN_OK;
 }
 
@@ -1077,18 +1107,28 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
      * when asked for (QLIN_DENSE_GEMM=own, qlin_set_dense_gemm_own) - this library's own tile kernel
      * (gemm_dense_mfma.hip; K a multiple of 256) */
     const bool own_ok = n_cols % 256 == 0 && aligned(Wd, 16);
-    if (own_ok && !g.dense_gemm_library) {
+    const int mode = g.dense_gemm_mode;
+    if (own_ok && mode == 1) {
         HIP_TRY(launch_gemm_dense_own(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
         return QLIN_OK;
     }
     void *lib_ws = (char *)workspace + dense_gemm_weight_bytes(n_rows, n_cols);
-    if (const char *err = launch_gemm_dense_bf16(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, lib_ws, kDenseLibWorkspace,
-                                                 (hipStream_t)stream)) {
-        if (own_ok) { /* a shape the library has no kernel for */
-            HIP_TRY(launch_gemm_dense_own(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
-            return QLIN_OK;
-        }
-        return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+    const char *err = mode == 2 ? "switched off" : launch_gemm_dense_bf16(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, lib_ws,
+                                                                          kDenseLibWorkspace, (hipStream_t)stream);
+    if (!err) return QLIN_OK;
+    if (own_ok && mode != 2) { /* a shape the library has no kernel for */
+        HIP_TRY(launch_gemm_dense_own(Wd, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        return QLIN_OK;
+    }
+    /* neither takes the shape: the vector-ALU kernel on the weights as they came, the activations widened to fp32 a
+     * band of tokens at a time in the library's part of the workspace */
+    const size_t band = kDenseLibWorkspace / ((size_t)n_cols * sizeof(float));
+    if (band == 0) return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
+    float *xf = (float *)lib_ws;
+    for (size_t t0 = 0; t0 < (size_t)n_tok; t0 += band) {
+        const int nt = (int)std::min<size_t>(band, (size_t)n_tok - t0);
+        HIP_TRY(launch_dequant(T_BF16, X + t0 * ldx, nullptr, 0, xf, nt, n_cols, (size_t)ldx * 2, (hipStream_t)stream));
+        HIP_TRY(launch_gemm_f32(type, W, xf, Y + t0 * ldy, n_rows, n_cols, nt, n_cols, ldy, (hipStream_t)stream));
     }
     return QLIN_OK;
 }
@@ -1181,7 +1221,7 @@ int qlin_moe_ffn_types_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_d
         if (int rc = ensure_init_locked(0)) return rc;
     }
     HIP_TRY(launch_moe_ffn(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
-                           n_tok, top_k, n_embd, n_ff, n_expert, workspace, (hipStream_t)stream));
+                           n_tok, top_k, n_embd, n_ff, n_expert, g.n_cu, workspace, (hipStream_t)stream));
     return QLIN_OK;
 }
 
@@ -1197,15 +1237,16 @@ int qlin_moe_ffn_static_dev(uint32_t type_gate, uint32_t type_up, uint32_t type_
     if (need > (size_t)QLIN_MOE_STATIC_SCRATCH_BYTES)
         return fail(QLIN_ERR_ARG, "this shape needs %zu bytes of scratch, the built-in scratch holds %zu: use qlin_moe_ffn_types_dev "
                                   "with a workspace", need, (size_t)QLIN_MOE_STATIC_SCRATCH_BYTES);
-    int device;
+    int device, n_cu;
     {
         std::lock_guard<std::mutex> lk(g.mu);
         if (!g.ready) /* initialising would allocate (stream, events): that is qlin_init's job, not this call's */
             return fail(QLIN_ERR_DEVICE, "qlin_init() must have run before qlin_moe_ffn_static_dev");
         device = g.device;
+        n_cu = g.n_cu;
     }
     HIP_TRY(launch_moe_ffn_static(type_gate, type_up, type_down, gate_exps, up_exps, down_exps, X, expert_idx, expert_w, out,
-                                  n_tok, top_k, n_embd, n_ff, n_expert, device, (hipStream_t)stream));
+                                  n_tok, top_k, n_embd, n_ff, n_expert, device, n_cu, (hipStream_t)stream));
     return QLIN_OK;
 }
 
@@ -1241,16 +1282,6 @@ int qlin_probe_hbm_read(const void *buf, size_t n_bytes, void *stream) {
     HIP_TRY(launch_probe_read(buf, n_bytes, (hipStream_t)stream));
     return QLIN_OK;
 }
-
-/* the event pair belongs to the calling thread, so that threads timing their own streams do not overwrite
- * each other's start event */
-namespace {
-struct ThreadTimer {
-    hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    bool begun = false;
-};
-thread_local ThreadTimer t_timer;
-}  // namespace
 
 int qlin_timer_begin(void *stream) {
     {

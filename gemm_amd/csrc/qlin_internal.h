@@ -143,7 +143,7 @@ hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int 
 size_t moe_workspace_bytes(int n_tok, int top_k, int n_embd, int n_ff, int n_expert);
 hipError_t launch_moe_ffn(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
                           const void *down, const uint16_t *X, const int32_t *idx, const float *w, float *out, int n_tok,
-                          int top_k, int n_embd, int n_ff, int n_expert, void *workspace, hipStream_t stream);
+                          int top_k, int n_embd, int n_ff, int n_expert, int n_cu, void *workspace, hipStream_t stream);
 
 /* the same with the workspace in a device array of the library (at most kMoeStaticScratchBytes); setup once per
  * device with that device current, before the first launch there */
@@ -153,7 +153,7 @@ hipError_t moe_static_scratch_setup(int device);
 hipError_t launch_moe_ffn_static(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate,
                                  const void *up, const void *down, const uint16_t *X, const int32_t *idx, const float *w,
                                  float *out, int n_tok, int top_k, int n_embd, int n_ff, int n_expert, int device,
-                                 hipStream_t stream);
+                                 int n_cu, hipStream_t stream);
 
 /* MoE pieces */
 hipError_t launch_moe_route(const float *logits, int n_tok, int n_expert, int top_k, int32_t *idx,

@@ -195,9 +195,10 @@ int qlin_dequant_bf16_dev(uint32_t ggml_type, const void *W, uint16_t *out, int 
  * An id outside [0, n_table_rows) gives a row of zeros (the reference refuses such a token, :3501). */
 int qlin_embed_rows_dev(uint32_t ggml_type, const void *table, int n_table_rows, const int32_t *row_ids,
                         int n_ids, float *out, int n_cols, void *stream);
-/* y[n_rows] = W . x, x fp32. Besides the block formats W may be dense F16, BF16 or F32 rows
- * (n_cols a multiple of 8, W 16-byte aligned): the fp32 dot of the widened row with x, as
- * tf_qmatvec does for these types (common/transformer.h:1051-1075). Rows of any length in whole blocks: rows
+/* y[n_rows] = W . x, x fp32 (16-byte aligned), W 2-byte aligned (F32: 4-byte). Besides the block formats W may be
+ * dense F16, BF16 or F32 rows of any length: the fp32 dot of the widened row with x, as tf_qmatvec does for these
+ * types (common/transformer.h:1051-1075); dense rows whose length is not a multiple of 8, or that do not start on
+ * 16-byte addresses, take a one-element-per-lane kernel. Rows of any length in whole blocks: rows
  * of more than 16384 elements run as several launches over column ranges, the later ones adding to y (still one
  * call, ordered on `stream`). */
 int qlin_gemv_dev(uint32_t ggml_type, const void *W, const float *x, float *y, int n_rows,
@@ -229,8 +230,10 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
  * tf_gemm_f16_mt_tokenmajor for the formats it re-decodes once per token (common/transformer.h:4535-4572):
  * W is decoded once to bf16 (nearest even) into `workspace` and multiplied by the dense matrix-core GEMM of
  * the vendor library. Q4_K takes the fused kernels of qlin_gemm_bf16_dev instead, and leaves the
- * workspace alone, for up to 48 tokens and for up to 512 tokens when the tensor has enough rows to fill
- * the chip with their tiles (about 12800 rows at 512 tokens). Up to 24 tokens of a Q6_K, Q5_K, Q3_K, Q2_K or
+ * workspace alone, for up to 48 tokens and wherever the tensor has enough rows to fill the chip with
+ * 256-token x 128-row tiles (200 of them: 12800 rows at 257..512 tokens, 6400 at 513..1024, ...); Q5_K and Q6_K
+ * tensors (n_cols % 256 == 0) take the same tile kernel under the same condition, decoded inside the product
+ * with the same single rounding to bf16, workspace untouched (it may be NULL then). Up to 24 tokens of a Q6_K, Q5_K, Q3_K, Q2_K or
  * Q8_0 tensor (n_cols % 256 == 0, the tensor's bytes a multiple of 16) also run in one fused kernel with
  * unrounded weights (~1e-6) and leave the workspace alone (it may be NULL then). Up to 4 tokens of any other
  * block format go one by one through the matvec kernels (exact weights, ~1e-6; the workspace holds their
@@ -242,7 +245,9 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
  * qlin_set_dense_gemm_own(1), or QLIN_DENSE_GEMM=own in the environment when the library initialises,
  * replaces the vendor library's dense GEMM by this library's own bf16 tile kernel (rows of a multiple of
  * 256 elements; about 0.8x the vendor kernel's speed at 512 tokens, 0.6x at 2048); the own kernel also
- * takes over whenever the vendor library offers no kernel for a shape. */
+ * takes over whenever the vendor library offers no kernel for a shape, and where neither takes it the
+ * vector-ALU kernel of qlin_gemm_f32_dev does (exact weights, activations widened to fp32 a band of tokens at a
+ * time in the workspace) - qlin_set_dense_gemm_own(2) sends every dense product there (a test switch: slow). */
 int qlin_set_dense_gemm_own(int enable);
 size_t qlin_gemm_bf16_any_workspace_bytes(int n_rows, int n_cols);
 int qlin_gemm_bf16_any_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,

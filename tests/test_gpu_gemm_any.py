@@ -135,6 +135,25 @@ def test_fused_tile_kernel_full_size_config(oracle, tid):
     assert np.array_equal(Y2, 2.0 * Y)
 
 
+@pytest.mark.parametrize("tid,n_tok,n_rows,n_cols", [
+    (synth.GGML_IQ4_NL, 70, 130, 512), (synth.GGML_Q8_0, 33, 257, 96), (synth.GGML_BF16, 40, 64, 1024),
+    (synth.GGML_Q4_0, 9000, 16, 1024),  # more tokens than one band of the workspace holds as fp32
+])
+def test_neither_dense_kernel_takes_the_shape(oracle, tid, n_tok, n_rows, n_cols):
+    """with both dense products switched off the call still answers: the vector-ALU kernel on the exact weights"""
+    W = synth.make_weights(tid, n_rows, n_cols, seed=5 + tid)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=6 + tid, tokens=n_tok))
+    qlinear.check(qlinear.load().qlin_set_dense_gemm_own(2))
+    try:
+        Y = run(tid, W, Xb, n_rows, n_cols, n_tok, ldx=n_cols + 16, ldy=n_rows + 5)
+    finally:
+        qlinear.check(qlinear.load().qlin_set_dense_gemm_own(0))
+    assert np.all(Y[:, n_rows:] == -3.0)
+    exact, _ = references(oracle, tid, W, Xb, n_cols)
+    assert rel_l2(Y[:, :n_rows], exact) <= 2e-5
+    assert qlinear.load().qlin_set_dense_gemm_own(3) == qlinear.ERR_ARG
+
+
 BLOCK_NOT_KQ = sorted(t for t in ALL if t not in KQ and t not in synth.DENSE_TYPES and t != Q4K)
 
 

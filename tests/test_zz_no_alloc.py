@@ -71,3 +71,73 @@ def test_static_scratch_rejects_what_does_not_fit():
     # the benchmark's shape fits
     assert qlinear.moe_workspace_bytes(64, 8, 2048, 768, 128) <= 16 << 20
     d.free()
+
+
+def test_static_entry_records_into_a_graph_and_replays_bit_identically(oracle):
+    """Stream capture refuses a call that allocates or synchronises, so recording qlin_moe_ffn_static_dev (after one
+    eager call has done its once-only kernel set-up) shows that it does neither. The graph is replayed three times
+    with eager work of the same entry point on another shape between the replays; every replay reproduces the eager
+    result bit for bit."""
+    import ctypes as C
+    lib = qlinear.load()
+    assert lib.qlin_init(0) == 0
+    hip = C.CDLL("libamdhip64.so")
+    vp = C.c_void_p
+    hip.hipStreamCreate.argtypes = [C.POINTER(vp)]
+    hip.hipStreamBeginCapture.argtypes = [vp, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [vp, C.POINTER(vp)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(vp), vp, vp, vp, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [vp, vp]
+    hip.hipStreamSynchronize.argtypes = [vp]
+    hip.hipGraphExecDestroy.argtypes = [vp]
+    hip.hipGraphDestroy.argtypes = [vp]
+    hip.hipStreamDestroy.argtypes = [vp]
+
+    types = (Q4K, Q4K, Q6K)
+    n_expert, n_embd, n_ff, n_tok, top_k = 16, 1024, 512, 40, 4
+    gate = synth.make_weights(types[0], n_expert * n_ff, n_embd, seed=171)
+    up = synth.make_weights(types[1], n_expert * n_ff, n_embd, seed=172)
+    down = synth.make_weights(types[2], n_expert * n_embd, n_ff, seed=173)
+
+    def inputs(n, k, seed):
+        Xb = synth.to_bf16_bits(synth.make_activation(n_embd, seed=seed, tokens=n))
+        logits = synth.make_router_logits(n, n_expert, seed=seed + 1)
+        idx, w = np.zeros((n, k), np.int32), np.zeros((n, k), np.float32)
+        for t in range(n):
+            idx[t], w[t] = oracle.moe_route(logits[t], k)
+        return [qlinear.DevBuf.from_numpy(a) for a in (Xb, idx, w)]
+
+    wbufs = [qlinear.DevBuf.from_numpy(a) for a in (gate, up, down)]
+    main_in, other_in = inputs(n_tok, top_k, 300), inputs(9, 2, 310)
+    dout = qlinear.DevBuf.from_numpy(np.full((n_tok, n_embd), -7.0, np.float32))
+    dother = qlinear.DevBuf(9 * n_embd * 4)
+
+    stream = vp()
+    assert hip.hipStreamCreate(C.byref(stream)) == 0
+    qlinear.moe_ffn_static_dev(types, *wbufs, *main_in, dout, n_tok, top_k, n_embd, n_ff, n_expert, stream)
+    qlinear.sync(stream)
+    eager = dout.to_numpy(np.float32, (n_tok, n_embd))
+
+    graph, gexec = vp(), vp()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0  # hipStreamCaptureModeGlobal
+    rc = lib.qlin_moe_ffn_static_dev(types[0], types[1], types[2], *[b.ptr for b in wbufs], *[b.ptr for b in main_in],
+                                     dout.ptr, n_tok, top_k, n_embd, n_ff, n_expert, stream)
+    end = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0, lib.qlin_last_error()
+    assert end == 0 and graph.value
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+    for replay in range(3):
+        fill = np.full((n_tok, n_embd), -7.0, np.float32)  # the output starts from a known value each time
+        assert lib.qlin_dev_upload(dout.ptr, fill.ctypes.data_as(vp), fill.nbytes) == 0
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        assert hip.hipStreamSynchronize(stream) == 0
+        got = dout.to_numpy(np.float32, (n_tok, n_embd))
+        assert np.array_equal(got.view(np.uint32), eager.view(np.uint32)), replay
+        # eager work of the same entry point on another shape overwrites the shared scratch between replays
+        qlinear.moe_ffn_static_dev(types, *wbufs, *other_in, dother, 9, 2, n_embd, n_ff, n_expert, stream)
+        qlinear.sync(stream)
+    assert hip.hipGraphExecDestroy(gexec) == 0
+    assert hip.hipGraphDestroy(graph) == 0
+    assert hip.hipStreamDestroy(stream) == 0
+    for b in wbufs + main_in + other_in + [dout, dother]:
+        b.free()
