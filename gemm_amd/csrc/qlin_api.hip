@@ -1122,13 +1122,14 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     }
     /* neither takes the shape: the vector-ALU kernel on the weights as they came, the activations widened to fp32 a
      * band of tokens at a time in the library's part of the workspace */
-    const size_t band = kDenseLibWorkspace / ((size_t)n_cols * sizeof(float));
+    const size_t band = kDenseLibWorkspace / ((size_t)ldx * sizeof(float)); /* tokens widened at a time, gaps and all */
     if (band == 0) return fail(QLIN_ERR_DEVICE, "dense bf16 GEMM: %s", err);
     float *xf = (float *)lib_ws;
     for (size_t t0 = 0; t0 < (size_t)n_tok; t0 += band) {
         const int nt = (int)std::min<size_t>(band, (size_t)n_tok - t0);
-        HIP_TRY(launch_dequant(T_BF16, X + t0 * ldx, nullptr, 0, xf, nt, n_cols, (size_t)ldx * 2, (hipStream_t)stream));
-        HIP_TRY(launch_gemm_f32(type, W, xf, Y + t0 * ldy, n_rows, n_cols, nt, n_cols, ldy, (hipStream_t)stream));
+        const size_t span = (size_t)(nt - 1) * ldx + n_cols;
+        HIP_TRY(launch_dequant(T_BF16, X + t0 * ldx, nullptr, 0, xf, 1, (int)span, 0, (hipStream_t)stream));
+        HIP_TRY(launch_gemm_f32(type, W, xf, Y + t0 * ldy, n_rows, n_cols, nt, ldx, ldy, (hipStream_t)stream));
     }
     return QLIN_OK;
 }

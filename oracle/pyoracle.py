@@ -68,6 +68,8 @@ class Oracle:
         L.qo_moe_route.argtypes = [_fp, C.c_int, C.c_int, _ip, _fp]
         for f in (L.qo_moe_ffn_token_f64, L.qo_moe_ffn_token_f32):
             f.argtypes = [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _fp, _ip, _fp, C.c_int, _fp]
+        L.qo_moe_ffn_token_types.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, _fp, _ip,
+                                             _fp, C.c_int, _fp, C.c_int]
 
     # ---- codec
     def fp16_table(self):
@@ -180,6 +182,20 @@ class Oracle:
         assert rc == 0, rc
         return out
 
+    def moe_ffn_token_types(self, types, gate, up, down, n_embd, n_ff, x, idx, w, f64=True):
+        """the three expert tensors in a format each (gate, up, down)"""
+        gate, pg = _u8(gate)
+        up, pu = _u8(up)
+        down, pd = _u8(down)
+        x, px = _f32(x)
+        idx = np.ascontiguousarray(idx, np.int32)
+        w, pw = _f32(w)
+        out = np.zeros(n_embd, np.float32)
+        rc = self.lib.qo_moe_ffn_token_types(types[0], types[1], types[2], pg, pu, pd, n_embd, n_ff, px,
+                                             idx.ctypes.data_as(_ip), pw, len(idx), out.ctypes.data_as(_fp), 1 if f64 else 0)
+        assert rc == 0, rc
+        return out
+
 
 class Reference:
     """The reference's own functions, compiled from its sources (oracle/_ref/libref.so).
@@ -256,6 +272,20 @@ class Reference:
         self.lib.ref_tf_gemm_tokenmajor(Y.ctypes.data_as(_fp), pw, type_id, px, n_rows, n_cols, n_tok, n_rows,
                                         X.shape[1], n_threads)
         return Y
+
+    def softmax(self, x):
+        """tf_softmax (common/transformer.h:1537-1586), on a copy"""
+        x = np.array(x, np.float32, copy=True)
+        self.lib.ref_tf_softmax(x.ctypes.data_as(_fp), x.shape[0])
+        return x
+
+    def silu_mul(self, gate, up):
+        """tf_silu_mul_avx2 (common/transformer.h:4679-4694): silu(gate) * up"""
+        gate, pg = _f32(gate)
+        up, pu = _f32(up)
+        out = np.zeros(gate.shape[0], np.float32)
+        self.lib.ref_tf_silu_mul(out.ctypes.data_as(_fp), pg, pu, gate.shape[0])
+        return out
 
     def qmatvec_pool_time(self, type_id, W, x, n_cols, n_threads, iters):
         W, pw = _u8(W)

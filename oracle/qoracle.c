@@ -17,11 +17,14 @@
  *                          and the compiled reference's tf_qmatvec on the same inputs.
  *   qo_gemm_tokmajor_*     pinned: equals per-token gemv (brute force) and numpy matmul.
  *   qo_moe_route           pinned: weights sum to 1, index set == argsort top-k, weights ==
- *                          softmax over the selected logits. The ORDER in which the k survivors
- *                          come out (heap order) is restated from the source only: the routing
- *                          code is inline in the reference's forward pass and cannot be called
- *                          on its own. The order affects nothing but fp32 summation order.
- *   qo_moe_ffn_token_*     pinned: numpy float64 restatement on decoded expert slices.
+ *                          softmax over the selected logits; and ids (in order) and weights against the
+ *                          fixture of the MoE block below, whose selection ran on the compiled reference's
+ *                          tf_softmax (the heap itself is inline in the reference's forward pass and is
+ *                          restated beside that fixture's generator, independently of this file).
+ *   qo_moe_ffn_token_*     pinned: numpy float64 restatement on decoded expert slices, and the fixture
+ *                          of one token's whole block composed from the compiled reference's tf_softmax,
+ *                          tf_qmatvec_expert (x3) and tf_silu_mul_avx2 (tests/golden/make_golden.py), to
+ *                          5e-6: that SiLU uses a polynomial exp, this file expf.
  */
 #include "qoracle.h"
 #include "qoracle_tables.h"
@@ -561,12 +564,13 @@ void qo_moe_route(const float *logits, int n_expert, int top_k, int *idx, float 
     free(p);
 }
 
-static int moe_token(uint32_t type, const void *gate, const void *up, const void *down, int n_embd,
-                     int n_ff, const float *x, const int *idx, const float *w, int top_k,
+static int moe_token(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
+                     const void *down, int n_embd, int n_ff, const float *x, const int *idx, const float *w, int top_k,
                      float *out, int use_f64) {
-    const size_t rb_in = qo_row_size(type, n_embd);  /* gate/up rows have n_embd columns */
-    const size_t rb_dn = qo_row_size(type, n_ff);    /* down rows have n_ff columns */
-    if (!rb_in || !rb_dn) return -1;
+    const size_t rb_g = qo_row_size(type_gate, n_embd); /* gate/up rows have n_embd columns */
+    const size_t rb_u = qo_row_size(type_up, n_embd);
+    const size_t rb_dn = qo_row_size(type_down, n_ff);  /* down rows have n_ff columns */
+    if (!rb_g || !rb_u || !rb_dn) return -1;
     const int mx = n_embd > n_ff ? n_embd : n_ff;
     float *tmp = (float *)calloc((size_t)mx, sizeof(float));
     float *g = (float *)calloc((size_t)n_ff, sizeof(float));
@@ -576,13 +580,13 @@ static int moe_token(uint32_t type, const void *gate, const void *up, const void
     for (int i = 0; i < n_embd; i++) out[i] = 0.0f;
     for (int k = 0; k < top_k; k++) {
         /* expert slice = base + expert * rows_per_expert * row_bytes (common/transformer.h:525) */
-        const uint8_t *ge = (const uint8_t *)gate + (size_t)idx[k] * n_ff * rb_in;
-        const uint8_t *ue = (const uint8_t *)up + (size_t)idx[k] * n_ff * rb_in;
+        const uint8_t *ge = (const uint8_t *)gate + (size_t)idx[k] * n_ff * rb_g;
+        const uint8_t *ue = (const uint8_t *)up + (size_t)idx[k] * n_ff * rb_u;
         const uint8_t *de = (const uint8_t *)down + (size_t)idx[k] * n_embd * rb_dn;
         for (int r = 0; r < n_ff; r++) {
-            qo_dequant_row(type, ue + (size_t)r * rb_in, tmp, n_embd);
+            qo_dequant_row(type_up, ue + (size_t)r * rb_u, tmp, n_embd);
             u[r] = use_f64 ? (float)dot_f64(tmp, x, n_embd) : dot_f32(tmp, x, n_embd);
-            qo_dequant_row(type, ge + (size_t)r * rb_in, tmp, n_embd);
+            qo_dequant_row(type_gate, ge + (size_t)r * rb_g, tmp, n_embd);
             g[r] = use_f64 ? (float)dot_f64(tmp, x, n_embd) : dot_f32(tmp, x, n_embd);
         }
         /* h = silu(gate) * up, written over gate (common/transformer.h:4108, scalar form :4690) */
@@ -591,7 +595,7 @@ static int moe_token(uint32_t type, const void *gate, const void *up, const void
             else g[r] = g[r] / (1.0f + expf(-g[r])) * u[r];
         }
         for (int r = 0; r < n_embd; r++) {
-            qo_dequant_row(type, de + (size_t)r * rb_dn, tmp, n_ff);
+            qo_dequant_row(type_down, de + (size_t)r * rb_dn, tmp, n_ff);
             q[r] = use_f64 ? (float)dot_f64(tmp, g, n_ff) : dot_f32(tmp, g, n_ff);
         }
         if (use_f64) for (int i = 0; i < n_embd; i++) acc[i] += (double)w[k] * (double)q[i];
@@ -605,10 +609,15 @@ static int moe_token(uint32_t type, const void *gate, const void *up, const void
 int qo_moe_ffn_token_f64(uint32_t type, const void *gate, const void *up, const void *down,
                          int n_embd, int n_ff, const float *x, const int *idx, const float *w,
                          int top_k, float *out) {
-    return moe_token(type, gate, up, down, n_embd, n_ff, x, idx, w, top_k, out, 1);
+    return moe_token(type, type, type, gate, up, down, n_embd, n_ff, x, idx, w, top_k, out, 1);
 }
 int qo_moe_ffn_token_f32(uint32_t type, const void *gate, const void *up, const void *down,
                          int n_embd, int n_ff, const float *x, const int *idx, const float *w,
                          int top_k, float *out) {
-    return moe_token(type, gate, up, down, n_embd, n_ff, x, idx, w, top_k, out, 0);
+    return moe_token(type, type, type, gate, up, down, n_embd, n_ff, x, idx, w, top_k, out, 0);
+}
+int qo_moe_ffn_token_types(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
+                           const void *down, int n_embd, int n_ff, const float *x, const int *idx, const float *w,
+                           int top_k, float *out, int use_f64) {
+    return moe_token(type_gate, type_up, type_down, gate, up, down, n_embd, n_ff, x, idx, w, top_k, out, use_f64);
 }

@@ -124,6 +124,10 @@ int qo_moe_ffn_token_f64(uint32_t type, const void *gate, const void *up, const 
 int qo_moe_ffn_token_f32(uint32_t type, const void *gate, const void *up, const void *down,
                          int n_embd, int n_ff, const float *x, const int *idx, const float *w,
                          int top_k, float *out);
+/* the three matrices in a format each; use_f64 as the two above */
+int qo_moe_ffn_token_types(uint32_t type_gate, uint32_t type_up, uint32_t type_down, const void *gate, const void *up,
+                           const void *down, int n_embd, int n_ff, const float *x, const int *idx, const float *w,
+                           int top_k, float *out, int use_f64);
 
 #ifdef __cplusplus
 }

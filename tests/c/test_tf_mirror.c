@@ -6,6 +6,7 @@
  * Exit code 0 = all checks passed.
  */
 #define QLINEAR_TF_REFERENCE_NAMES
+#define QLINEAR_GGML_REFERENCE_NAMES
 #include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -13,6 +14,7 @@
 
 #include "qlinear.h"
 #include "qlinear_tf.h"
+#include "qlinear_ggml.h"
 
 static uint64_t rng_state = 0x9E3779B97F4A7C15ull;
 static uint32_t rnd(void) {
@@ -59,6 +61,75 @@ static void check_rows(const char *what, const qtensor *t, int row0, int n_rows,
     const double rel = sqrt(num / (den > 0 ? den : 1));
     printf("%-28s rel-L2 %.3e %s\n", what, rel, rel <= 1e-5 ? "ok" : "FAIL");
     if (!(rel <= 1e-5)) failures++;
+}
+
+/* the codec under the names of common/ggml_dequant.h: every per-type decoder once against dequant_row of its type
+ * (bit for bit), the row sizes, the half conversion over all 65536 patterns, and the Q8_0 products */
+typedef void (*row_decoder)(const void *, float *, int);
+static void check_ggml_names(void) {
+    static const struct { const char *name; uint32_t type; int block_elems, block_bytes; row_decoder fn; } dec[] = {
+        {"q2_K", 10, 256, 84, dequantize_row_q2_K},       {"q3_K", 11, 256, 110, dequantize_row_q3_K},
+        {"q8_0", 8, 32, 34, dequantize_row_q8_0},         {"q1_0", 41, 128, 18, dequantize_row_q1_0},
+        {"mxfp4", 39, 32, 17, dequantize_row_mxfp4},      {"nvfp4", 40, 64, 36, dequantize_row_nvfp4},
+        {"q4_K", 12, 256, 144, dequantize_row_q4_K},      {"q5_K", 13, 256, 176, dequantize_row_q5_K},
+        {"q6_K", 14, 256, 210, dequantize_row_q6_K},      {"iq2_xxs", 16, 256, 66, dequantize_row_iq2_xxs},
+        {"q4_0", 2, 32, 18, dequantize_row_q4_0},         {"q4_1", 3, 32, 20, dequantize_row_q4_1},
+        {"q5_0", 6, 32, 22, dequantize_row_q5_0},         {"q5_1", 7, 32, 24, dequantize_row_q5_1},
+        {"iq2_xs", 17, 256, 74, dequantize_row_iq2_xs},   {"iq2_s", 22, 256, 82, dequantize_row_iq2_s},
+        {"iq3_xxs", 18, 256, 98, dequantize_row_iq3_xxs}, {"iq3_s", 21, 256, 110, dequantize_row_iq3_s},
+        {"iq4_nl", 20, 32, 18, dequantize_row_iq4_nl},    {"iq4_xs", 23, 256, 136, dequantize_row_iq4_xs},
+        {"iq1_s", 19, 256, 50, dequantize_row_iq1_s},     {"iq1_m", 29, 256, 56, dequantize_row_iq1_m},
+        {"tq1_0", 34, 256, 54, dequantize_row_tq1_0},     {"tq2_0", 35, 256, 66, dequantize_row_tq2_0},
+        {"bf16", 30, 1, 2, dequantize_row_bf16},
+    };
+    const int n = 512;
+    uint8_t *src = (uint8_t *)malloc(2 * n + 4096);
+    float *a = (float *)malloc(sizeof(float) * n), *b = (float *)malloc(sizeof(float) * n);
+    int bad = 0;
+    for (size_t i = 0; i < sizeof dec / sizeof dec[0]; i++) {
+        const size_t bytes = (size_t)(n / dec[i].block_elems) * dec[i].block_bytes;
+        if (dequant_row_size(dec[i].type, n) != bytes) { printf("dequant_row_size %s FAIL\n", dec[i].name); bad++; }
+        for (size_t j = 0; j < bytes; j++) src[j] = (uint8_t)rnd();
+        memset(a, 0xAA, sizeof(float) * n);
+        memset(b, 0x55, sizeof(float) * n);
+        dec[i].fn(src, a, n);
+        if (dequant_row(dec[i].type, src, b, n) != 0 || memcmp(a, b, sizeof(float) * n) != 0) {
+            printf("dequantize_row_%s vs dequant_row FAIL\n", dec[i].name);
+            bad++;
+        }
+    }
+    if (dequant_row(9, src, a, n) != -1 || dequant_row_size(9, n) != 0) { printf("unsupported type FAIL\n"); bad++; }
+    printf("%-28s %s\n", "ggml decoder names (25)", bad ? "FAIL" : "ok");
+    failures += bad;
+
+    /* ggml_fp16_to_fp32 against the library's F16 decoder, all patterns, bit for bit */
+    uint16_t *h = (uint16_t *)malloc(2 * 65536);
+    float *f = (float *)malloc(4 * 65536);
+    for (int i = 0; i < 65536; i++) h[i] = (uint16_t)i;
+    bad = dequant_row(1, h, f, 65536) != 0;
+    for (int i = 0; i < 65536 && !bad; i++) {
+        const float g = ggml_fp16_to_fp32((uint16_t)i);
+        if (memcmp(&g, &f[i], 4) != 0 && !(g != g && f[i] != f[i])) { printf("fp16 0x%04x FAIL\n", i); bad = 1; }
+    }
+    printf("%-28s %s\n", "ggml_fp16_to_fp32 (65536)", bad ? "FAIL" : "ok");
+    failures += bad;
+    free(h); free(f); free(src); free(a); free(b);
+
+    /* Q8_0 row dot, one-row matvec, token-major GEMM */
+    const int K = 1024, R = 40, N = 3;
+    qtensor w = make_tensor(8, R, K);
+    float *x = (float *)malloc(sizeof(float) * K * N), *Y = (float *)malloc(sizeof(float) * N * 64);
+    for (int i = 0; i < K * N; i++) x[i] = rndf();
+    float one[1], two[1];
+    one[0] = vec_dot_q8_0_f32((const uint8_t *)w.data + 5 * dequant_row_size(8, K), x, K);
+    check_rows("vec_dot_q8_0_f32", &w, 5, 1, x, one);
+    matvec_q8_0_f32(two, (const uint8_t *)w.data + 7 * dequant_row_size(8, K), x, K);
+    check_rows("matvec_q8_0_f32", &w, 7, 1, x, two);
+    for (int i = 0; i < N * 64; i++) Y[i] = -5.0f;
+    gemm_q8_0_f32_tokmajor(Y, w.data, x, R, K, N, 64, K);
+    for (int t = 0; t < N; t++) check_rows("gemm_q8_0_f32_tokmajor", &w, 0, R, x + (size_t)t * K, Y + (size_t)t * 64);
+    if (Y[R] != -5.0f || Y[63] != -5.0f) { printf("gemm_q8_0 wrote outside its rows FAIL\n"); failures++; }
+    free(x); free(Y); free(w.data);
 }
 
 int main(void) {
@@ -145,6 +216,8 @@ int main(void) {
     for (int i = 0; i < 256; i++) zeros &= (y[i] == 0.0f);
     printf("%-28s %s\n", "unsupported type zero-fill", zeros ? "ok" : "FAIL");
     if (!zeros) failures++;
+
+    check_ggml_names();
 
     qtf_unregister_tensor(&a);
     qlin_shutdown();

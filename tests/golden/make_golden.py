@@ -128,6 +128,63 @@ def gguf_fixture(ref):
     return out
 
 
+MOE_EXPERTS, MOE_TOP, MOE_EMBD, MOE_FF = 16, 4, 512, 256
+
+
+def heap_top_k(probs, k):
+    """The selection of the reference's MoE block (common/transformer.h:4056-4090): one pass over the experts that
+    keeps the k largest probabilities in a min-heap (ties keep the earlier expert), then the weights divided by their
+    sum, added up in heap order in fp32. -> (expert ids, weights) in the heap's final order."""
+    ids, val = [], []
+
+    def swap(a, b):
+        ids[a], ids[b] = ids[b], ids[a]
+        val[a], val[b] = val[b], val[a]
+
+    for e, p in enumerate(probs):
+        if len(ids) < k:
+            ids.append(e)
+            val.append(p)
+            child = len(ids) - 1
+            while child > 0 and val[child] < val[(child - 1) // 2]:
+                swap(child, (child - 1) // 2)
+                child = (child - 1) // 2
+        elif p > val[0]:
+            ids[0], val[0] = e, p
+            node = 0
+            while True:
+                least = node
+                for c in (2 * node + 1, 2 * node + 2):
+                    if c < k and val[c] < val[least]:
+                        least = c
+                if least == node:
+                    break
+                swap(node, least)
+                node = least
+    total = np.float32(0.0)
+    for v in val:
+        total = np.float32(total + v)
+    w = np.array(val, np.float32)
+    if total > 0:
+        w = (w / total).astype(np.float32)
+    return np.array(ids, np.int32), w
+
+
+def moe_block(ref, types, gate, up, down, logits, x):
+    """One token through the reference's MoE FFN block (common/transformer.h:4045-4131), composed from its own
+    compiled functions: tf_softmax, the selection above, tf_qmatvec_expert for up, gate and down, tf_silu_mul_avx2,
+    and the weighted sum (one rounding per element and expert, as its fused multiply-add gives)."""
+    idx, w = heap_top_k(ref.softmax(logits), MOE_TOP)
+    out = np.zeros(MOE_EMBD, np.float32)
+    for e, ew in zip(idx, w):
+        u = ref.qmatvec_expert(types[1], up, int(e), x, MOE_FF, MOE_EMBD)
+        g = ref.qmatvec_expert(types[0], gate, int(e), x, MOE_FF, MOE_EMBD)
+        h = ref.silu_mul(g, u)
+        q = ref.qmatvec_expert(types[2], down, int(e), h, MOE_EMBD, MOE_FF)
+        out = (np.float64(ew) * q.astype(np.float64) + out.astype(np.float64)).astype(np.float32)
+    return idx, w, out
+
+
 def main():
     ref = Reference()
     manifest = {"generator": "tests/golden/make_golden.py", "source": "reference C compiled via oracle/ref_shim.c"}
@@ -187,6 +244,25 @@ def main():
         lin[name + "_Y_tokmajor"] = ref.gemm_tokenmajor(tid, W, X, LIN_COLS)
         # expert slice: the 24 rows seen as 3 experts of 8 rows
         lin[name + "_y_expert1"] = ref.qmatvec_expert(tid, W, 1, x, 8, LIN_COLS)
+    # the MoE FFN block, one token at a time; the expert matrices are drawn from fixed seeds (their hashes are in the
+    # manifest), two tokens per format mix
+    Q4K, Q6K = synth.GGML_Q4_K, synth.GGML_Q6_K
+    moe_manifest = {"n_expert": MOE_EXPERTS, "top_k": MOE_TOP, "n_embd": MOE_EMBD, "n_ff": MOE_FF, "cases": {}}
+    for label, types in (("q4k", (Q4K, Q4K, Q4K)), ("q4k_down_q6k", (Q4K, Q4K, Q6K))):
+        seeds = (5100 + types[2], 5200 + types[2], 5300 + types[2])
+        gate = synth.make_weights(types[0], MOE_EXPERTS * MOE_FF, MOE_EMBD, seed=seeds[0])
+        up = synth.make_weights(types[1], MOE_EXPERTS * MOE_FF, MOE_EMBD, seed=seeds[1])
+        down = synth.make_weights(types[2], MOE_EXPERTS * MOE_EMBD, MOE_FF, seed=seeds[2])
+        logits = synth.make_router_logits(2, MOE_EXPERTS, seed=5400 + types[2])
+        xs = synth.make_activation(MOE_EMBD, seed=5500 + types[2], tokens=2)
+        res = [moe_block(ref, types, gate, up, down, logits[t], xs[t]) for t in range(2)]
+        lin["moe_%s_logits" % label], lin["moe_%s_x" % label] = logits, xs
+        lin["moe_%s_idx" % label] = np.stack([r[0] for r in res])
+        lin["moe_%s_w" % label] = np.stack([r[1] for r in res])
+        lin["moe_%s_out" % label] = np.stack([r[2] for r in res])
+        moe_manifest["cases"][label] = {"types": list(types), "weight_seeds": list(seeds),
+                                        "weights_sha256": [sha(gate), sha(up), sha(down)]}
+    manifest["moe_block"] = moe_manifest
     np.savez_compressed(os.path.join(OUT, "linear_golden.npz"), **lin)
 
     manifest["gguf_fixture"] = gguf_fixture(ref)

@@ -165,6 +165,34 @@ def test_weight_registry(oracle):
     assert np.all(qlinear.matvec(tid, W, x, n_cols) == 0)
 
 
+@pytest.mark.parametrize("label", ["q4k", "q4k_down_q6k"])
+def test_moe_token_ffn_against_the_compiled_reference(manifest, linear_golden, label):
+    """qlin_moe_ffn_token_types from router logits to output against the fixture of the reference's own block
+    (tf_softmax, heap selection, tf_qmatvec_expert x3, tf_silu_mul_avx2, weighted sum). Bar 2e-4: the reference's
+    softmax and SiLU use a polynomial exp that moves the expert weights by up to 5e-5."""
+    from tests.conftest import moe_block_case
+    c = moe_block_case(manifest, linear_golden, label)
+    lib = qlinear.load()
+    for t in range(c["logits"].shape[0]):
+        out = np.zeros(c["n_embd"], np.float32)
+        logits, x = np.ascontiguousarray(c["logits"][t]), np.ascontiguousarray(c["x"][t])
+        assert lib.qlin_moe_ffn_token_types(out.ctypes.data, c["gate"].ctypes.data, c["up"].ctypes.data, c["down"].ctypes.data,
+                                            c["types"][0], c["types"][1], c["types"][2], c["n_embd"], c["n_ff"],
+                                            c["n_expert"], c["top_k"], logits.ctypes.data, x.ctypes.data) == 0
+        assert rel_l2(out, c["out"][t]) <= 2e-4, (label, t)
+        # the device routing picks the reference's experts with the reference's weights (the order of the k is the
+        # device's own: it only decides the order of an fp32 sum)
+        dl = qlinear.DevBuf.from_numpy(logits)
+        di, dw = qlinear.DevBuf(c["top_k"] * 4), qlinear.DevBuf(c["top_k"] * 4)
+        assert lib.qlin_moe_route_dev(dl.ptr, 1, c["n_expert"], c["top_k"], di.ptr, dw.ptr, None) == 0
+        qlinear.sync()
+        gi, gw = di.to_numpy(np.int32, (c["top_k"],)), dw.to_numpy(np.float32, (c["top_k"],))
+        assert np.array_equal(np.sort(gi), np.sort(c["idx"][t]))
+        assert np.allclose(gw[np.argsort(gi)], c["w"][t][np.argsort(c["idx"][t])], rtol=5e-5, atol=0)
+        for b in (dl, di, dw):
+            b.free()
+
+
 def test_moe_route_and_token_ffn(oracle):
     lib = qlinear.load()
     tid, n_expert, n_embd, n_ff, k = synth.GGML_Q4_K, 16, 512, 256, 4

@@ -115,3 +115,22 @@ def test_moe_ffn_token_against_numpy(oracle):
     got32 = oracle.moe_ffn_token(tid, gate, up, down, n_embd, n_ff, x, idx, w, f64=False)
     assert rel_l2(got64, want) < 1e-6
     assert rel_l2(got32, want) < 1e-5
+
+
+@pytest.mark.parametrize("label", ["q4k", "q4k_down_q6k"])
+def test_moe_block_against_the_compiled_reference(oracle, manifest, linear_golden, label):
+    """One token's MoE FFN block as the reference's own compiled pieces compute it (tf_softmax, the heap selection,
+    tf_qmatvec_expert three times per expert, tf_silu_mul_avx2, the weighted sum): the oracle's routing gives the same
+    experts in the same order, the same weights up to the polynomial exp of the reference's softmax (5e-5; the oracle
+    calls expf), and its fp32 and double-precision blocks the same output to 5e-6 (measured 2e-7 .. 8e-7: the exp
+    inside the reference's SiLU is a polynomial too)."""
+    from tests.conftest import moe_block_case
+    c = moe_block_case(manifest, linear_golden, label)
+    for t in range(c["logits"].shape[0]):
+        idx, w = oracle.moe_route(c["logits"][t], c["top_k"])
+        assert np.array_equal(idx, c["idx"][t])
+        assert np.allclose(w, c["w"][t], rtol=5e-5, atol=0)
+        for f64 in (False, True):
+            got = oracle.moe_ffn_token_types(c["types"], c["gate"], c["up"], c["down"], c["n_embd"], c["n_ff"], c["x"][t],
+                                             c["idx"][t], c["w"][t], f64=f64)
+            assert rel_l2(got, c["out"][t]) <= 5e-6, (label, t, f64)
