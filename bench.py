@@ -42,7 +42,7 @@ Q4K = synth.GGML_Q4_K
 # same counter reads for a device-to-device copy of known size, as recorded with its commands in
 # PROFILED_TRAFFIC_SOURCE. It changes only when the kernel's loads change and the profile is taken again;
 # tests/test_profiles.py fails when the two files disagree.
-PROFILED_TRAFFIC_BYTES = 33277536
+PROFILED_TRAFFIC_BYTES = 33297298
 PROFILED_TRAFFIC_SOURCE = "profiles/gemv_q4k_14336x4096.md"
 
 
@@ -450,9 +450,18 @@ def probe(args):
             assert hip.hipMemcpy(b.ptr, a.ptr, n, 3) == 0  # hipMemcpyDeviceToDevice
         qlinear.sync()
         print(json.dumps({"probe": "copy", "bytes_each": n, "copies": 4}))
+    elif args.probe == "tiny":  # a launch that does next to nothing (reads 4 KB): what a launch costs, with and without a profiler
+        buf = qlinear.DevBuf(4096)
+        for _ in range(200):
+            qlinear.probe_hbm_read(buf)
+        qlinear.sync()
+        qlinear.timer_begin()
+        for _ in range(args.steps):
+            qlinear.probe_hbm_read(buf)
+        print(json.dumps({"probe": "tiny", "ms_per_step": qlinear.timer_end() / args.steps, "steps": args.steps}))
     elif args.probe == "gemv":
         ms, copies = time_gemv(Q4K, 14336, 4096, args.steps, args.warmup, spin_up_ms=args.spin_up_ms)
-        print(json.dumps({"probe": "gemv", "ms_per_step": ms, "copies": copies}))
+        print(json.dumps({"probe": "gemv", "ms_per_step": ms, "copies": copies, "steps": args.steps, "warmup": args.warmup}))
     elif args.probe in ("gemv_q8_0", "gemv_q6_K"):
         tid, r, c = (synth.GGML_Q8_0, 4096, 4096) if args.probe == "gemv_q8_0" else (synth.GGML_Q6_K, 151936, 4096)
         ms, copies = time_gemv(tid, r, c, max(10, args.steps // 8), 3)
@@ -632,7 +641,7 @@ def main():
     ap.add_argument("--prows", type=int, default=4096)
     ap.add_argument("--pcols", type=int, default=14336)
     ap.add_argument("--ptok", type=int, default=64, help="--probe moe: tokens in the batch")
-    ap.add_argument("--probe", choices=["gemv_any", "copy", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["gemv_any", "copy", "tiny", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
