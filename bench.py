@@ -505,7 +505,7 @@ def probe(args):
     elif args.probe == "gemm_any_q6_K":  # Q6_K, 512 tokens: decoded inside the tile kernel
         ms = time_gemm_any(synth.GGML_Q6_K, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_any_q6_K", "ms_per_step": ms}))
-    elif args.probe == "gemm_any_q8_0":  # Q8_0, 512 tokens: decode to bf16 + dense library GEMM
+    elif args.probe == "gemm_any_q8_0":  # Q8_0, 512 tokens: decoded inside the tile kernel
         ms = time_gemm_any(synth.GGML_Q8_0, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_any_q8_0", "ms_per_step": ms}))
     elif args.probe == "gemm_f32_any_q4_K":  # decode to fp32 + dense fp32 library GEMM, Q4_K, 512 tokens
@@ -536,7 +536,8 @@ def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
     return ms
 
 
-FUSED_GEMM_TYPES = (Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K)  # decoded inside the tile kernel where its tiles fill the chip
+# decoded inside the tile kernel where its tiles fill the chip, up to this many tokens when a workspace is passed
+FUSED_GEMM_MAX_TOKENS = {Q4K: 1536, synth.GGML_Q5_K: 1536, synth.GGML_Q6_K: 512, synth.GGML_Q8_0: 512}
 
 
 def time_gemm_two_kernels(type_id, n_tok, n_rows, n_cols, steps, warmup):
@@ -684,23 +685,24 @@ def main():
         tf = gemm["M=512"]["TFLOP/s"]
         anyfmt = {}
         for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q8_0", synth.GGML_Q8_0, 512),
-                              ("iq4_nl", synth.GGML_IQ4_NL, 512), ("bf16", synth.GGML_BF16, 512), ("q4_K", Q4K, 2048),
-                              ("q5_K", synth.GGML_Q5_K, 2048), ("q6_K", synth.GGML_Q6_K, 2048)):
+                              ("iq4_nl", synth.GGML_IQ4_NL, 512), ("bf16", synth.GGML_BF16, 512), ("q4_K", Q4K, 1024),
+                              ("q5_K", synth.GGML_Q5_K, 1024), ("q4_K", Q4K, 2048), ("q6_K", synth.GGML_Q6_K, 2048)):
             m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
             anyfmt["%s_M=%d" % (tname, M)] = {
                 "us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1),
-                "route": "decoded inside the product, no workspace" if tid in FUSED_GEMM_TYPES else
+                "route": "decoded inside the product, no workspace" if M <= FUSED_GEMM_MAX_TOKENS.get(tid, 0) else
                          "dense library product" if tid == synth.GGML_BF16 else "decode to bf16 + dense library product"}
         extra["prefill_gemm_any_format_14336x4096"] = anyfmt
         two = {}
-        for tname, tid, M in (("q4_K", Q4K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q6_K", synth.GGML_Q6_K, 512)):
+        for tname, tid, M in (("q4_K", Q4K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q6_K", synth.GGML_Q6_K, 512),
+                              ("q8_0", synth.GGML_Q8_0, 512)):
             m = time_gemm_two_kernels(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
             two["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
         extra["prefill_gemm_14336x4096_decode_to_bf16_plus_library_gemm_for_comparison"] = two
         own = {}
         qlinear.check(qlinear.load().qlin_set_dense_gemm_own(1))
         try:
-            for tname, tid, M in (("q8_0", synth.GGML_Q8_0, 512), ("bf16", synth.GGML_BF16, 512), ("q8_0", synth.GGML_Q8_0, 2048)):
+            for tname, tid, M in (("iq4_nl", synth.GGML_IQ4_NL, 512), ("bf16", synth.GGML_BF16, 512), ("iq4_nl", synth.GGML_IQ4_NL, 2048)):
                 m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
                 own["%s_M=%d" % (tname, M)] = {"us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1)}
         finally:

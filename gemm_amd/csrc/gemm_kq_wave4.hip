@@ -1,12 +1,13 @@
 /*
- * gemm_kq_wave4.hip - Q4_K, Q5_K and Q6_K x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup, one
- * per SIMD.
+ * gemm_kq_wave4.hip - Q4_K, Q5_K, Q6_K and Q8_0 x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup,
+ * one per SIMD.
  *
  *   Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k]      X bf16, Y fp32, fp32 accumulate
  *
  * The contraction of tf_gemm_f16_mt_tokenmajor (common/transformer.h:4487, generic branch :4535-4572) with the
- * weights decoded as dequantize_row_q4_K / _q5_K / _q6_K do (common/ggml_dequant.h:1592-1618, :1620-1660, :1662-1700;
- * y = (d*sc)*q - dmin*m, resp. d*sc*(q - 32), in fp32) and rounded once to bf16, nearest even. What the reference's
+ * weights decoded as dequantize_row_q4_K / _q5_K / _q6_K / _q8_0 do (common/ggml_dequant.h:1592-1618, :1620-1660,
+ * :1662-1700, :1479-1489; y = (d*sc)*q - dmin*m, resp. d*sc*(q - 32), resp. d*q, in fp32) and rounded once to bf16,
+ * nearest even. What the reference's
  * fused kernel does per tile for every type (rdna4/dequant/bench_dequant.c:359-459), on this part's terms.
  *
  * What the shape follows from, measured on MI355X with one wave per SIMD (cycles that the matrix pipe waits for
@@ -30,9 +31,10 @@
  *   - per matrix instruction one ds_read_b128 (a 32-token x 16-k activation fragment) and about three vector
  *     instructions of decode.
  *
- * The three formats differ in what a lane takes from its row's block (Q4_K: 16 code bytes per quarter; Q5_K: those
+ * The formats differ in what a lane takes from its row's block (Q4_K: 16 code bytes per quarter; Q5_K: those
  * and 16 bytes of fifth bits per super-block; Q6_K: two runs of 16 nibble bytes and 16 bytes of bit pairs per half
- * super-block) and in the arithmetic of a piece; the tile loop is one template over a format description.
+ * super-block; Q8_0: the 32 codes of one block per tile, scales straight from memory) and in the arithmetic of a
+ * piece; the tile loop is one template over a format description.
  *
  * k inside a tile is permuted so that a lane's 16 code bytes serve its four k-steps (Q4_K; the others alike): k-step s of lane half kg covers
  * the low (s < 2) or high nibbles of code bytes 16 kg + 8 (s & 1) .. + 7, i.e. tile k 32 (s >> 1) + 16 kg + 8 (s & 1) ..;
@@ -46,6 +48,7 @@
  * k-step: wait for this wave's requests of the next tile, barrier (the next tile is complete; nobody reads the
  * stage that is requested next, its last fragments were fetched a k-step earlier).
  */
+#include <climits>
 #include <utility>
 
 #include "qlin_device.h"
@@ -114,8 +117,8 @@ template <int N> QLIN_INL void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-/* where a lane finds vector J of its raw data in its row's image: byte offset, and whether the lane half adds 16 */
-struct VecAt { int off; bool by_half; };
+/* where a lane finds vector J of its raw data in its row's image: byte offset, and what the upper lane half adds */
+struct VecAt { int off; int by_half; };
 
 /* scratch of the decode that all formats share */
 struct Temps {
@@ -130,12 +133,14 @@ template <class F> struct Ctx {
     floatx16 acc[8];         /* [token block]: 32 rows x 32 tokens each */
     bf16x8 xf[2][8];         /* activation fragments of the k-step in use and of the next: [k-step & 1][token block] */
     u32x4 wa[2][4];          /* decoded weights of the tile in use and of the next: [tile & 1][k-step] */
-    u32x4 cur[F::kLaneVec], nxt[F::kLaneVec]; /* raw data of the super-block of the tile being decoded, and of the next */
+    u32x4 cur[F::kLaneVec + F::kExtraVec], nxt[F::kLaneVec + F::kExtraVec]; /* raw data of the super-block of the tile being
+                                decoded, and of the next: kLaneVec vectors out of the LDS image, kExtraVec straight from memory */
     typename F::Scales sc;   /* of the super-block being decoded */
     Temps t;
     uint32_t xrd;            /* byte offset of this lane's fragment fetches in a stage: k-step 0, token block 0 */
     __amdgpu_buffer_rsrc_t w_rsrc, x_rsrc;
-    uint32_t w_off[F::kReq], w_rd, x_off[8];
+    uint32_t w_off[F::kReq], w_rd, w_swz, w_own, x_off[8]; /* w_swz: see kSwizzle; w_own: byte offset of the lane's own
+                                                               row in the weight tile */
     uint8_t *raw;            /* the workgroup's raw-block area in LDS */
     int wv, kg;              /* wave of the workgroup; lane half */
     int sb, n_sb;            /* super-block of the tile in use */
@@ -184,11 +189,15 @@ template <int TC, int P, class C> QLIN_INL void k4_tile_scales(C &c) {
  * the lane's bytes 8 (s & 1) .. + 7. */
 struct FQ4K {
     static constexpr int kBlockBytes = 144, kPieces = 9, kReq = 5, kLaneVec = 5, kPrepPieces = 4, kTilePieces = 44;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
     typedef K4Scales Scales;
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
-    static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, false} : VecAt{16 + 32 * (j - 1), true}; }
-    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec]) { k4_unpack<P>(c, raw[0], c.unit); }
-    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec]) {
+    static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, 0} : VecAt{16 + 32 * (j - 1), 16}; }
+    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) { k4_unpack<P>(c, raw[0], c.unit); }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
         Temps &t = c.t;
         if constexpr (P < 4) k4_tile_scales<TC, P>(c);
         else {
@@ -210,11 +219,15 @@ struct FQ4K {
  * code goes through the byte-to-float conversion (the fp8 reading is linear up to 15 only). */
 struct FQ5K {
     static constexpr int kBlockBytes = 176, kPieces = 11, kReq = 6, kLaneVec = 6, kPrepPieces = 4, kTilePieces = 60;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
     typedef K4Scales Scales;
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
-    static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, false} : j == 1 ? VecAt{16, true} : VecAt{48 + 32 * (j - 2), true}; }
-    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec]) { k4_unpack<P>(c, raw[0], 1.0f); }
-    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec]) {
+    static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, 0} : j == 1 ? VecAt{16, 16} : VecAt{48 + 32 * (j - 2), 16}; }
+    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) { k4_unpack<P>(c, raw[0], 1.0f); }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
         Temps &t = c.t;
         if constexpr (P < 4) k4_tile_scales<TC, P>(c);
         else {
@@ -235,13 +248,17 @@ struct FQ5K {
 struct Q6Scales { float d; };
 struct FQ6K {
     static constexpr int kBlockBytes = 210, kPieces = 15, kReq = 8, kLaneVec = 8, kPrepPieces = 1, kTilePieces = 60;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
     typedef Q6Scales Scales;
     static QLIN_INL uint32_t piece_src(int part) { return part < 13 ? 16u * part : part == 13 ? 194u : 0u; }
     static constexpr VecAt vec_at(int j) {
-        return j < 4 ? VecAt{64 * (j >> 1) + 32 * (j & 1), true} : j < 6 ? VecAt{128 + 32 * (j - 4), true} : j == 6 ? VecAt{192, false} : VecAt{208, false};
+        return j < 4 ? VecAt{64 * (j >> 1) + 32 * (j & 1), 16} : j < 6 ? VecAt{128 + 32 * (j - 4), 16} : j == 6 ? VecAt{192, 0} : VecAt{208, 0};
     }
-    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec]) { c.sc.d = half_bits_fast(raw[7].w >> 16); }
-    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec]) {
+    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) { c.sc.d = half_bits_fast(raw[7].w >> 16); }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
         Temps &t = c.t;
         constexpr int half = TC >> 1, p = TC & 1;
         if constexpr (P < 4) {
@@ -262,6 +279,40 @@ struct FQ6K {
     }
 };
 
+/* ---- Q8_0: 34-byte blocks = d | 32 int8 codes; eight of them are the unit of the pipeline. Only the codes go through
+ * LDS (two 16-byte pieces per block, fetched from 34 b + 2 and 34 b + 18: the load-to-LDS path takes any source
+ * alignment, and the image's vectors come out aligned), 512 bytes per row: with the four activation stages that is all
+ * of the 160 KB. The scales come straight from memory into registers, four two-byte loads per lane and unit. So that
+ * four suffice, the k order inside a tile differs from the K-quants': lane half kg takes ALL codes of block 2 c + kg of
+ * tile c, k-step s its codes 8 s .. 8 s + 7, and the activation fragment of that lane half is chunk 4 kg + s. */
+struct FQ8_0 {
+    static constexpr int kBlockBytes = 272, kPieces = 16, kReq = 8, kLaneVec = 8, kPrepPieces = 0, kTilePieces = 49;
+    static constexpr int kExtraVec = 1, kExtraLoads = 4, kKgChunk = 4;
+    /* a row's image is 256 bytes, a whole turn of the LDS banks: piece p of row r sits at position p ^ (r % 16) of the
+     * row, so that 16 rows reading the same piece hit 16 different bank groups */
+    static constexpr bool kSwizzle = true;
+    struct Scales {};
+    static constexpr int frag_xor(int s) { return s << 4; }
+    static QLIN_INL uint32_t piece_src(int part) { return 34u * (part >> 1) + 2u + 16u * (part & 1); }
+    /* vector j: half j & 1 of the codes of block 2 (j >> 1) + kg */
+    static constexpr VecAt vec_at(int j) { return VecAt{64 * (j >> 1) + 16 * (j & 1), 32}; }
+    /* scale J (0..3) of super-block `sb`: d of block 2 J + kg of the lane's own row, kept as the 16 bits that came */
+    template <int J, class C> static QLIN_INL void extra_load(C &c, u32x4 (&raw)[kLaneVec + kExtraVec], int sb) {
+        raw[kLaneVec][J] = __builtin_amdgcn_raw_buffer_load_b16(c.w_rsrc, c.w_own + 34u * c.kg + 68u * J, sb * kBlockBytes, 0);
+    }
+    template <int P, class C> static QLIN_INL void prep(C &, const u32x4 (&)[kLaneVec + kExtraVec]) {}
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        Temps &t = c.t;
+        if constexpr (P == 0) { t.dl_a = half_bits_fast(raw[kLaneVec][TC] & 0xFFFFu); t.nml_a = -128.0f * t.dl_a; }
+        else {
+            /* the int8 code with its sign bit flipped is code + 128 as an unsigned byte */
+            constexpr int dw = (P - 1) / 6, ph = (P - 1) % 6;
+            if constexpr (ph == 0) t.cm = raw[2 * TC + (dw >> 2)][dw & 3] ^ 0x80808080u;
+            else bytes4_piece<ph + 1, dw & 1>(c, t.dl_a, t.nml_a, c.wa[WB][dw >> 1]);
+        }
+    }
+};
+
 /* one load-to-LDS request: lane l's 16 bytes from voff + soff of the buffer land at lds + 16 l */
 QLIN_INL void dma16(__amdgpu_buffer_rsrc_t rsrc, uint8_t *lds, uint32_t voff, uint32_t soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void *)lds, 16, voff, soff, 0, 0);
@@ -275,7 +326,7 @@ template <class F, int Q> QLIN_INL void request_w(Ctx<F> &c, int sb) {
 /* vector J of this lane's raw data out of its row's image */
 template <class F, int J> QLIN_INL u32x4 load_raw(Ctx<F> &c) {
     constexpr VecAt at = F::vec_at(J);
-    return *reinterpret_cast<const u32x4 *>(c.raw + c.w_rd + at.off + (at.by_half ? 16 * c.kg : 0));
+    return *reinterpret_cast<const u32x4 *>(c.raw + c.w_rd + ((uint32_t)(at.off + at.by_half * c.kg) ^ c.w_swz));
 }
 
 /* request I (0..7) of this wave for 64-k tile `tile` into stage ST: token rows 64 wv + 8 I .. + 7, 128 bytes each */
@@ -285,7 +336,7 @@ template <class F, int ST, int I> QLIN_INL void request_x(Ctx<F> &c, int tile) {
 
 /* activation fragment of token block BJ, k-step S of stage ST */
 template <class F, int ST, int S, int BJ> QLIN_INL bf16x8 load_frag(Ctx<F> &c) {
-    return *reinterpret_cast<const bf16x8 *>(stage_ptr<ST>() + (c.xrd ^ (uint32_t)(((S & 1) << 4) | ((S >> 1) << 6))) + BJ * 4096);
+    return *reinterpret_cast<const bf16x8 *>(stage_ptr<ST>() + (c.xrd ^ (uint32_t)F::frag_xor(S)) + BJ * 4096);
 }
 
 /* slot T (0..31) of tile 4 sb + U */
@@ -293,9 +344,10 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     constexpr int s = T / 8, bj = T % 8;
     if constexpr (T == 24) {
         /* this wave's requests of the next tile have landed: younger are the 8 of the tile after it, 6 of the one
-         * after that, and the weight requests of a tile with U = 1 (all of them if that was the tile before, those of
-         * its first 24 slots if it is this one) */
-        wait_vmcnt<14 + (U == 1 ? (F::kReq < 6 ? F::kReq : 6) : 0) + (U == 2 ? F::kReq : 0)>();
+         * after that, the weight requests of a tile with U = 1 and the scale loads of one with U = 0 (all of them if
+         * that was the tile before, those of its first 24 slots if it is this one) */
+        constexpr int w_now = F::kReq < 6 ? F::kReq : 6, x_now = F::kExtraLoads < 6 ? F::kExtraLoads : 6;
+        wait_vmcnt<14 + (U == 0 ? x_now : 0) + (U == 1 ? w_now + F::kExtraLoads : 0) + (U == 2 ? F::kReq : 0)>();
         __builtin_amdgcn_s_barrier();
     }
     c.acc[bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, c.wa[U & 1][s]), c.xf[s & 1][bj], c.acc[bj], 0, 0, 0);
@@ -305,8 +357,9 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
      * one after it into the same place; U = 3: the tile being decoded is the first of the next super-block, which
      * then becomes the one in work */
     if constexpr (U == 0 && T % 4 == 1 && T / 4 < F::kLaneVec) c.nxt[T / 4] = load_raw<F, T / 4>(c);
+    if constexpr (U == 0 && T % 4 == 1 && T / 4 < F::kExtraLoads) F::template extra_load<T / 4>(c, c.nxt, min(c.sb + 1, c.n_sb - 1));
     if constexpr (U == 1 && T % 4 == 1 && T / 4 < F::kReq) request_w<F, T / 4>(c, c.sb + 2);
-    if constexpr (U == 3 && T % 4 == 3 && T / 4 < F::kLaneVec) c.cur[T / 4] = c.nxt[T / 4];
+    if constexpr (U == 3 && T % 3 == 2 && T / 3 < F::kLaneVec + F::kExtraVec) c.cur[T / 3] = c.nxt[T / 3];
     constexpr int n_pieces = F::kTilePieces + (U == 3 ? F::kPrepPieces : 0);
     constexpr int p0 = (T * n_pieces + 31) / 32, p1 = ((T + 1) * n_pieces + 31) / 32; /* pieces p with p * 32 / n_pieces == T */
     auto piece = [&](auto pc) {
@@ -332,6 +385,7 @@ template <class F, int... P> QLIN_INL void decode_first(Ctx<F> &c, std::integer_
 template <class F, int ST, int... I> QLIN_INL void request_tile(Ctx<F> &c, int tile, std::integer_sequence<int, I...>) { (request_x<F, ST, I>(c, tile), ...); }
 template <class F, int... Q> QLIN_INL void request_raw(Ctx<F> &c, int sb, std::integer_sequence<int, Q...>) { (request_w<F, Q>(c, sb), ...); }
 template <class F, int... J> QLIN_INL void load_cur(Ctx<F> &c, std::integer_sequence<int, J...>) { ((c.cur[J] = load_raw<F, J>(c)), ...); }
+template <class F, int... J> QLIN_INL void load_cur_extra(Ctx<F> &c, std::integer_sequence<int, J...>) { (F::template extra_load<J>(c, c.cur, 0), ...); }
 
 }  // namespace
 
@@ -368,9 +422,12 @@ gemm_kq_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__restr
 #pragma unroll
     for (int q = 0; q < F::kReq; q++) {
         const int id = min(64 * q + lane, 32 * F::kPieces - 1); /* past the last piece: padding */
-        c.w_off[q] = (uint32_t)min(32 * c.wv + id / F::kPieces, w_rows - 1) * row_bytes + F::piece_src(id % F::kPieces);
+        const int part = F::kSwizzle ? (id % F::kPieces) ^ ((id / F::kPieces) & 15) : id % F::kPieces;
+        c.w_off[q] = (uint32_t)min(32 * c.wv + id / F::kPieces, w_rows - 1) * row_bytes + F::piece_src(part);
     }
     c.w_rd = (uint32_t)(c.wv * F::kReq * 1024 + li * F::kPieces * 16);
+    c.w_swz = F::kSwizzle ? (uint32_t)(li & 15) << 4 : 0u;
+    c.w_own = (uint32_t)min(32 * c.wv + li, w_rows - 1) * row_bytes;
     /* Activation requests: request I of this wave fills 1 KB of a stage, lane l the 16 bytes at chunk position l % 8 of
      * token row 64 wv + 8 I + l / 8, i.e. chunk (l % 8) ^ f(row) of that token's 128 bytes; tokens past the end
      * re-read the last one (never stored) */
@@ -382,8 +439,8 @@ gemm_kq_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__restr
         const int row = 64 * c.wv + 8 * i + (lane >> 3);
         c.x_off[i] = (uint32_t)min(row, x_rows - 1) * (uint32_t)(2 * ldx) + (uint32_t)((((lane & 7) ^ fsw(row))) << 4);
     }
-    /* fragment fetches: token li of each block of 32, chunk 4 (s >> 1) + 2 kg + (s & 1) */
-    c.xrd = (uint32_t)(li * 128 + (((2 * kg) ^ fsw(li)) << 4));
+    /* fragment fetches: token li of each block of 32; chunk 4 (s >> 1) + 2 kg + (s & 1) for the K-quants */
+    c.xrd = (uint32_t)(li * 128 + (((F::kKgChunk * kg) ^ fsw(li)) << 4));
 
 #pragma unroll
     for (int i = 0; i < 8; i++)
@@ -393,6 +450,7 @@ gemm_kq_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__restr
     /* ---- prologue: raw blocks of super-block 0 fetched and read back, those of super-block 1 and tiles 0..2
      * requested; tile 0 decoded; fragments of its k-step 0 fetched */
     c.sb = 0;
+    load_cur_extra<F>(c, std::make_integer_sequence<int, F::kExtraLoads>{});
     request_raw<F>(c, 0, std::make_integer_sequence<int, F::kReq>{});
     request_tile<F, 0>(c, 0, std::make_integer_sequence<int, 8>{});
     wait_vmcnt<8>();
@@ -457,7 +515,21 @@ hipError_t launch_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, 
 }
 }  // namespace
 
-bool gemm_kq_wave4_covers(uint32_t type) { return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K; }
+bool gemm_kq_wave4_covers(uint32_t type) { return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K || type == T_Q8_0; }
+
+/* Every 256 tokens decode the weights again, which costs more the more there is to decode, while decoding once into
+ * a workspace costs 27 - 38 us whatever the token count. 14336 x 4096, this kernel against decode + the vendor library's
+ * product, us: at 512 tokens Q4_K 61 / 86, Q5_K 62 / 92, Q6_K 66 / 84, Q8_0 71 / 83; at 1024 118 / 125, 121 / 135,
+ * 131 / 126, 139 / 121; at 1536 181 / 190, 185 / 195, 206 / 184, 216 / 177; at 2048 267 / 244, 262 / 260, 273 / 240,
+ * 311 / 224 (Q8_0's extra is mostly its scale loads). Above these token counts the decode + dense route is taken
+ * where a workspace is at hand. */
+int gemm_kq_wave4_max_tokens(uint32_t type) {
+    switch (type) {
+    case T_Q4_K: case T_Q5_K: return 1536;
+    case T_Q6_K: case T_Q8_0: return 512;
+    default: return INT_MAX;
+    }
+}
 
 hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
                                      int n_tok, int ldx, int ldy, hipStream_t stream) {
@@ -465,6 +537,7 @@ hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_
     case T_Q4_K: return launch_wave4<FQ4K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q5_K: return launch_wave4<FQ5K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q6_K: return launch_wave4<FQ6K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q8_0: return launch_wave4<FQ8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }

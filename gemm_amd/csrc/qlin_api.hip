@@ -753,9 +753,10 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
         const uint16_t *Xb = (const uint16_t *)g.tmp[2].p;
         float *Yd = (float *)g.tmp[1].p;
         const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-        if (type == T_Q4_K && (n_tok <= kFewTokens || tiles >= 200)) {
+        if (type == T_Q4_K && (n_tok <= kFewTokens || (tiles >= 200 && n_tok <= gemm_kq_wave4_max_tokens(type)))) {
             HIP_TRY(launch_gemm_q4k_bf16(dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
-        } else if (gemm_kq_wave4_covers(type) && tiles >= 200 && n_cols % 256 == 0 && n_cols < (1 << 22)) {
+        } else if (gemm_kq_wave4_covers(type) && tiles >= 200 && n_cols % 256 == 0 && n_cols < (1 << 22) &&
+                   n_tok <= gemm_kq_wave4_max_tokens(type)) {
             HIP_TRY(launch_gemm_kq_bf16_wave4(type, dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
         } else {
             const uint16_t *Wd = (const uint16_t *)dW;
@@ -1057,11 +1058,13 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
         return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
     /* Q4_K: the fused kernels (no workspace) for a few tokens, and wherever their 256-token x 128-row tiles fill
-     * the chip (14336 x 4096: 60 us at 512 tokens, 231 at 2048; decode + library product 96 and 231); with fewer
-     * than 200 tiles (4096 rows at 512 tokens: 64) the decode + library route is faster (4096 x 14336: 105 vs 162 us) */
+     * the chip (14336 x 4096: 60 us at 512 tokens, 181 at 1536; decode + library product 86 and 190); with fewer
+     * than 200 tiles (4096 rows at 512 tokens: 64) the decode + library route is faster (4096 x 14336: 105 vs 162 us),
+     * and so it is from 2048 tokens on (267 vs 244 us) */
+    const bool ws_ok = workspace && aligned(workspace, 256) && workspace_bytes >= qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols);
     if (type == T_Q4_K) {
         const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-        if (n_tok <= kFewTokens || tiles >= 200)
+        if (n_tok <= kFewTokens || (tiles >= 200 && (n_tok <= gemm_kq_wave4_max_tokens(type) || !ws_ok)))
             return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     }
     /* a few tokens of a Q6_K, Q5_K, Q3_K, Q2_K or Q8_0 tensor: streamed once per eight tokens with exact codes
@@ -1077,14 +1080,16 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
-    /* Q5_K and Q6_K where the fused kernel's tiles fill the chip: decoded into the matrix operand like Q4_K, no
-     * workspace (14336 x 4096 at 512 tokens: decode + library product 92 and 84 us) */
+    /* Q5_K, Q6_K and Q8_0 where the fused kernel's tiles fill the chip: decoded into the matrix operand like Q4_K, no
+     * workspace (14336 x 4096 at 512 tokens: 62, 66 and 71 us; decode + library product 92, 84 and 83) - up to the
+     * token count from which decoding once pays, if the caller brought the workspace for that */
     if (gemm_kq_wave4_covers(type) && n_cols % 256 == 0 && ldx < (1 << 22) &&
-        (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256) >= 200) {
+        (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256) >= 200 &&
+        (n_tok <= gemm_kq_wave4_max_tokens(type) || !ws_ok)) {
         HIP_TRY(launch_gemm_kq_bf16_wave4(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
         return QLIN_OK;
     }
-    if (!workspace || !aligned(workspace, 256) || workspace_bytes < qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols))
+    if (!ws_ok)
         return fail(QLIN_ERR_ARG, "workspace must be 256-byte aligned and hold qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols) bytes");
     /* up to four tokens of any other block format: each through the matvec (exact weights; 14336 x 4096 IQ4_XS, four
      * tokens: 44 us against 95 us for decode + dense product), x widened to fp32 at the start of the workspace */

@@ -131,6 +131,7 @@ hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, in
 /* 256-token x 128-row tiles on four waves, one per SIMD, weights decoded from their blocks into the matrix operand
  * (gemm_kq_wave4.hip): the formats of gemm_kq_wave4_covers, n_cols % 256 == 0, ldx < 2^22 */
 bool gemm_kq_wave4_covers(uint32_t type);
+int gemm_kq_wave4_max_tokens(uint32_t type); /* above this many tokens decode + dense product is faster, given a workspace */
 hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
                                      int n_tok, int ldx, int ldy, hipStream_t stream);
 hipError_t launch_gemm_q4k_bf16_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,

@@ -231,9 +231,10 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
  * W is decoded once to bf16 (nearest even) into `workspace` and multiplied by the dense matrix-core GEMM of
  * the vendor library. Q4_K takes the fused kernels of qlin_gemm_bf16_dev instead, and leaves the
  * workspace alone, for up to 48 tokens and wherever the tensor has enough rows to fill the chip with
- * 256-token x 128-row tiles (200 of them: 12800 rows at 257..512 tokens, 6400 at 513..1024, ...); Q5_K and Q6_K
- * tensors (n_cols % 256 == 0) take the same tile kernel under the same condition, decoded inside the product
- * with the same single rounding to bf16, workspace untouched (it may be NULL then). Up to 24 tokens of a Q6_K, Q5_K, Q3_K, Q2_K or
+ * 256-token x 128-row tiles (200 of them: 12800 rows at 257..512 tokens, 6400 at 513..1024, ...); Q5_K, Q6_K and
+ * Q8_0 tensors (n_cols % 256 == 0) take the same tile kernel under the same condition, decoded inside the product
+ * with the same single rounding to bf16, workspace untouched (it may be NULL then) - with a workspace, up to 1536
+ * tokens (Q4_K, Q5_K) or 512 (Q6_K, Q8_0): beyond, decoding once into it is faster. Up to 24 tokens of a Q6_K, Q5_K, Q3_K, Q2_K or
  * Q8_0 tensor (n_cols % 256 == 0, the tensor's bytes a multiple of 16) also run in one fused kernel with
  * unrounded weights (~1e-6) and leave the workspace alone (it may be NULL then). Up to 4 tokens of any other
  * block format go one by one through the matvec kernels (exact weights, ~1e-6; the workspace holds their

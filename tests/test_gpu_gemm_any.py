@@ -75,6 +75,8 @@ def test_every_format(oracle, tid, dense_kernel):
 @pytest.mark.parametrize("tid,n_tok,n_rows,n_cols", [
     (synth.GGML_Q6_K, 1, 16, 256), (synth.GGML_Q6_K, 515, 1000, 1024), (synth.GGML_Q8_0, 130, 257, 96),
     (synth.GGML_Q5_K, 64, 2048, 768), (synth.GGML_IQ4_NL, 200, 130, 4096), (Q4K, 513, 384, 512),
+    # enough tiles for the fused kernel, but more tokens than it keeps when there is a workspace to decode into
+    (synth.GGML_Q6_K, 1030, 5130, 512), (synth.GGML_Q8_0, 770, 8200, 256),
     (Q4K, 1100, 300, 256), (Q4K, 300, 25700, 256), (synth.GGML_BF16, 33, 100, 264), (synth.GGML_F16, 300, 64, 1000),
     (synth.GGML_BF16, 700, 3000, 1024), (synth.GGML_Q6_K, 257, 129, 2048), (synth.GGML_Q8_0, 100, 4100, 512),
 ])
@@ -87,7 +89,7 @@ def test_shapes(oracle, tid, n_tok, n_rows, n_cols, dense_kernel):
     assert rel_l2(Y, exact) <= 3e-3
 
 
-FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K]
+FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0]
 
 
 @pytest.mark.parametrize("tid", FUSED, ids=lambda t: ALL[t])
@@ -97,7 +99,7 @@ FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K]
     (513, 8500, 1024),
 ])
 def test_fused_tile_kernel_shapes(oracle, tid, n_tok, n_rows, n_cols):
-    """200 or more 256-token x 128-row tiles: Q4_K, Q5_K and Q6_K are decoded inside the product (no workspace is
+    """200 or more 256-token x 128-row tiles: Q4_K, Q5_K, Q6_K and Q8_0 are decoded inside the product (no workspace is
     read: none is passed); weights rounded once to bf16, as the decode + dense route rounds them"""
     W = synth.make_weights(tid, n_rows, n_cols, seed=n_rows + tid)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=n_tok + tid, tokens=n_tok))
@@ -120,7 +122,7 @@ def test_fused_tile_kernel_shapes(oracle, tid, n_tok, n_rows, n_cols):
     assert rel_l2(Y[:, rows], exact) <= 3e-3
 
 
-@pytest.mark.parametrize("tid", [synth.GGML_Q5_K, synth.GGML_Q6_K], ids=lambda t: ALL[t])
+@pytest.mark.parametrize("tid", [synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0], ids=lambda t: ALL[t])
 def test_fused_tile_kernel_full_size_config(oracle, tid):
     """14336 x 4096 at 512 tokens; the oracle on a sample of rows, and scaling X by two scales Y exactly"""
     n_rows, n_cols, n_tok = 14336, 4096, 512
