@@ -536,8 +536,12 @@ def time_gemm_any(type_id, n_tok, n_rows, n_cols, steps, warmup):
     return ms
 
 
-# decoded inside the tile kernel where its tiles fill the chip, up to this many tokens when a workspace is passed
-FUSED_GEMM_MAX_TOKENS = {Q4K: 1536, synth.GGML_Q5_K: 1536, synth.GGML_Q6_K: 512, synth.GGML_Q8_0: 512}
+def gemm_route(type_id, n_tok, n_rows, n_cols):
+    """what qlin_gemm_bf16_any_dev does with this shape when it is handed a workspace"""
+    r = qlinear.load().qlin_probe_gemm_route(type_id, n_rows, n_cols, n_tok, n_cols, 1)
+    if r:
+        return "decoded inside the product (%s tiles), no workspace" % ("256-token x 128-row" if r == 1 else "128-token x 64-row")
+    return "dense library product" if type_id == synth.GGML_BF16 else "decode to bf16 + dense library product"
 
 
 def time_gemm_two_kernels(type_id, n_tok, n_rows, n_cols, steps, warmup):
@@ -690,9 +694,16 @@ def main():
             m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
             anyfmt["%s_M=%d" % (tname, M)] = {
                 "us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * 14336 * 4096 / (m * 1e-3) / 1e12, 1),
-                "route": "decoded inside the product, no workspace" if M <= FUSED_GEMM_MAX_TOKENS.get(tid, 0) else
-                         "dense library product" if tid == synth.GGML_BF16 else "decode to bf16 + dense library product"}
+                "route": gemm_route(tid, M, 14336, 4096)}
         extra["prefill_gemm_any_format_14336x4096"] = anyfmt
+        small = {}
+        for tname, tid, M, r, c in (("q4_K", Q4K, 512, 4096, 4096), ("q4_K", Q4K, 512, 6144, 4096), ("q4_K", Q4K, 512, 4096, 14336),
+                                    ("q4_K", Q4K, 256, 14336, 4096), ("q6_K", synth.GGML_Q6_K, 128, 14336, 4096),
+                                    ("q6_K", synth.GGML_Q6_K, 512, 4096, 14336), ("q8_0", synth.GGML_Q8_0, 512, 4096, 4096)):
+            m = time_gemm_any(tid, M, r, c, max(5, args.steps // 40), 2)
+            small["%s_M=%d_%dx%d" % (tname, M, r, c)] = {
+                "us": round(m * 1e3, 1), "TFLOP/s": round(2.0 * M * r * c / (m * 1e-3) / 1e12, 1), "route": gemm_route(tid, M, r, c)}
+        extra["prefill_gemm_other_shapes"] = small
         two = {}
         for tname, tid, M in (("q4_K", Q4K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q6_K", synth.GGML_Q6_K, 512),
                               ("q8_0", synth.GGML_Q8_0, 512)):

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libqlinear.so")
 TF_LIB = os.path.join(HERE, "libqlinear_tf.so")
-SOURCES = ["qlin_api.hip", "dequant.hip", "gemv_generic.hip", "gemv_q4k.hip", "gemv_stream.hip", "gemv_int.hip", "gemv_grid.hip", "gemm_q4k_mfma.hip", "gemm_kq_wave4.hip", "gemm_dense_mfma.hip", "moe.hip", "moe_ffn_q4k.hip", "argmax.hip", "gguf_upload.hip", "probe.hip", "gemm_dense_lt.hip"]
+SOURCES = ["qlin_api.hip", "dequant.hip", "gemv_generic.hip", "gemv_q4k.hip", "gemv_stream.hip", "gemv_int.hip", "gemv_grid.hip", "gemm_q4k_mfma.hip", "gemm_kq_wave4.hip", "gemm_kq_wave4s.hip", "gemm_dense_mfma.hip", "moe.hip", "moe_ffn_q4k.hip", "argmax.hip", "gguf_upload.hip", "probe.hip", "gemm_dense_lt.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 

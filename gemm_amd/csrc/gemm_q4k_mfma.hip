@@ -374,14 +374,14 @@ hipError_t launch_gemm_q4k_bf16(const void *W, const uint16_t *X, float *Y, int 
     /* up to 48 tokens the weights are better streamed once per 16 tokens with exact codes (13-39 us at
      * 14336 x 4096) than pushed through a 256-token tile (54 us whatever the count) */
     if (n_tok <= kFewTokens) return launch_gemm_q4k_fewtok(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    /* 128-row tiles unless they would leave compute units without a workgroup */
+    /* the four-wave kernels, large or small tiles by how many there are (their 32-bit offsets hold 256 rows of X) */
+    const FusedTile tile = choose_fused_tile(T_Q4_K, n_rows, n_cols, n_tok, ldx, false);
+    if (tile != kFusedNone) return launch_fused_tile(tile, T_Q4_K, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    /* a row pitch of 4 M elements or more: the eight-wave kernel of this file, which addresses with 64 bits.
+     * 128-row tiles unless they would leave compute units without a workgroup */
     const int m_tiles = (n_tok + 255) / 256, n_tiles_128 = (n_rows + 127) / 128;
-    /* up to 128 tokens: 128-token x 64-row tiles of four waves, two workgroups per compute unit, instead of
-     * half-empty 256-token tiles (128 tokens at 14336 x 4096: 51.7 -> 39.5 us, 64 tokens: 50.7 -> 34.4) */
     if (n_tok <= 128) return launch_tiled<2, 1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     if (m_tiles * n_tiles_128 < 200) return launch_tiled<4, 1>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    /* a chip's worth of 256-token x 128-row tiles or more: the four-wave kernel (its 32-bit offsets hold 256 rows of X) */
-    if (ldx < (1 << 22)) return launch_gemm_q4k_bf16_wave4(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     return launch_tiled<4, 2>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
 }
 

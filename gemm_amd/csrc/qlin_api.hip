@@ -752,12 +752,11 @@ int qlin_gemm_tokenmajor(float *Y, const void *W, uint32_t type, int n_cols, con
         HIP_TRY(launch_dequant_bf16(T_F32, g.tmp[0].p, (uint16_t *)g.tmp[2].p, n_tok, n_cols, (size_t)n_cols * 4, g.stream));
         const uint16_t *Xb = (const uint16_t *)g.tmp[2].p;
         float *Yd = (float *)g.tmp[1].p;
-        const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-        if (type == T_Q4_K && (n_tok <= kFewTokens || (tiles >= 200 && n_tok <= gemm_kq_wave4_max_tokens(type)))) {
+        const FusedTile tile = choose_fused_tile(type, n_rows, n_cols, n_tok, n_cols, true);
+        if (type == T_Q4_K && n_tok <= kFewTokens) {
             HIP_TRY(launch_gemm_q4k_bf16(dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
-        } else if (gemm_kq_wave4_covers(type) && tiles >= 200 && n_cols % 256 == 0 && n_cols < (1 << 22) &&
-                   n_tok <= gemm_kq_wave4_max_tokens(type)) {
-            HIP_TRY(launch_gemm_kq_bf16_wave4(type, dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
+        } else if (tile != kFusedNone) {
+            HIP_TRY(launch_fused_tile(tile, type, dW, Xb, Yd, n_rows, n_cols, n_tok, n_cols, n_rows, g.stream));
         } else {
             const uint16_t *Wd = (const uint16_t *)dW;
             if (type != T_BF16) {
@@ -1057,16 +1056,10 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
     if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
         return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
-    /* Q4_K: the fused kernels (no workspace) for a few tokens, and wherever their 256-token x 128-row tiles fill
-     * the chip (14336 x 4096: 60 us at 512 tokens, 181 at 1536; decode + library product 86 and 190); with fewer
-     * than 200 tiles (4096 rows at 512 tokens: 64) the decode + library route is faster (4096 x 14336: 105 vs 162 us),
-     * and so it is from 2048 tokens on (267 vs 244 us) */
+    /* Q4_K, a few tokens: its few-token kernel (exact codes, no workspace) */
     const bool ws_ok = workspace && aligned(workspace, 256) && workspace_bytes >= qlin_gemm_bf16_any_workspace_bytes(n_rows, n_cols);
-    if (type == T_Q4_K) {
-        const long long tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-        if (n_tok <= kFewTokens || (tiles >= 200 && (n_tok <= gemm_kq_wave4_max_tokens(type) || !ws_ok)))
-            return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    }
+    if (type == T_Q4_K && n_tok <= kFewTokens)
+        return qlin_gemm_bf16_dev(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     /* a few tokens of a Q6_K, Q5_K, Q3_K, Q2_K or Q8_0 tensor: streamed once per eight tokens with exact codes
      * (14336 x 4096 Q6_K, 8 tokens: decode + library GEMM about 75 us) */
     {
@@ -1080,13 +1073,10 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
-    /* Q5_K, Q6_K and Q8_0 where the fused kernel's tiles fill the chip: decoded into the matrix operand like Q4_K, no
-     * workspace (14336 x 4096 at 512 tokens: 62, 66 and 71 us; decode + library product 92, 84 and 83) - up to the
-     * token count from which decoding once pays, if the caller brought the workspace for that */
-    if (gemm_kq_wave4_covers(type) && n_cols % 256 == 0 && ldx < (1 << 22) &&
-        (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256) >= 200 &&
-        (n_tok <= gemm_kq_wave4_max_tokens(type) || !ws_ok)) {
-        HIP_TRY(launch_gemm_kq_bf16_wave4(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+    /* Q4_K, Q5_K, Q6_K and Q8_0: decoded into the matrix operand inside the product, no workspace, in large or small
+     * tiles by the shape - except where decoding once into the caller's workspace measured faster */
+    if (const FusedTile tile = choose_fused_tile(type, n_rows, n_cols, n_tok, ldx, ws_ok); tile != kFusedNone) {
+        HIP_TRY(launch_fused_tile(tile, type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
         return QLIN_OK;
     }
     if (!ws_ok)
@@ -1278,6 +1268,27 @@ int qlin_probe_clocks(void *stream, double *shader_mhz) {
     HIP_TRY(read_probe_clocks(c));
     if (c[1] == 0) return fail(QLIN_ERR_ARG, "qlin_probe_mfma_bf16 has not run");
     *shader_mhz = (double)c[0] * 100.0 / (double)c[1];
+    return QLIN_OK;
+}
+
+int qlin_probe_gemm_route(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, int have_workspace) {
+    return (int)choose_fused_tile(type, n_rows, n_cols, n_tok, ldx, have_workspace != 0);
+}
+
+int qlin_probe_gemm_tile(int tile, uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                         int n_tok, int ldx, int ldy, void *stream) {
+    if (tile < 0 || tile > 1) return fail(QLIN_ERR_ARG, "tile: 0 (256 x 128) or 1 (128 x 64)");
+    if (!gemm_kq_wave4_covers(type)) return fail(QLIN_ERR_TYPE, "no fused tile kernel for type %u", type);
+    if (int rc = check_linear_shape(type, n_rows, n_cols)) return rc;
+    if (n_tok < 0 || ldx < n_cols || ldy < n_rows || n_cols % 256 || ldx >= (1 << 22))
+        return fail(QLIN_ERR_ARG, "bad token count, leading dimension or row length");
+    if (n_rows == 0 || n_tok == 0) return QLIN_OK;
+    if (!W || !X || !Y) return fail(QLIN_ERR_ARG, "null pointer");
+    if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
+        return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
+    if (int rc = init_once()) return rc;
+    HIP_TRY((tile ? launch_gemm_kq_bf16_wave4s : launch_gemm_kq_bf16_wave4)(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy,
+                                                                            (hipStream_t)stream));
     return QLIN_OK;
 }
 

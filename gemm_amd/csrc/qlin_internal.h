@@ -125,13 +125,21 @@ constexpr int kKqFewTokens = 24; /* up to this many tokens Q6_K, Q5_K, Q3_K, Q2_
 bool launch_gemm_kq_fewtok(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                            int ldx, int ldy, hipStream_t stream, hipError_t *err);
 constexpr int kMatvecTokens = 4; /* qlin_gemm_bf16_any_dev: up to this many tokens of a format without a few-token kernel go through the matvec */
-constexpr int kFewTokens = 48; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel */
+constexpr int kFewTokens = 32; /* launch_gemm_q4k_bf16 hands token counts up to this to the few-token kernel (14336 x 4096:
+                                  24 us at 32 tokens, 34 at 48; the small-tile kernel 26 for up to 128) */
 hipError_t launch_gemm_q4k_fewtok(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,
                                   int ldx, int ldy, hipStream_t stream);
 /* 256-token x 128-row tiles on four waves, one per SIMD, weights decoded from their blocks into the matrix operand
  * (gemm_kq_wave4.hip): the formats of gemm_kq_wave4_covers, n_cols % 256 == 0, ldx < 2^22 */
 bool gemm_kq_wave4_covers(uint32_t type);
-int gemm_kq_wave4_max_tokens(uint32_t type); /* above this many tokens decode + dense product is faster, given a workspace */
+/* the same in 128-token x 64-row tiles, two workgroups per compute unit (gemm_kq_wave4s.hip) */
+hipError_t launch_gemm_kq_bf16_wave4s(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                                      int n_tok, int ldx, int ldy, hipStream_t stream);
+/* the fused kernel for a shape (kFusedNone: decode + dense product, or the format has none) and its launch */
+enum FusedTile { kFusedNone = 0, kFusedLarge, kFusedSmall };
+FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, bool have_workspace);
+hipError_t launch_fused_tile(FusedTile tile, uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows,
+                             int n_cols, int n_tok, int ldx, int ldy, hipStream_t stream);
 hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
                                      int n_tok, int ldx, int ldy, hipStream_t stream);
 hipError_t launch_gemm_q4k_bf16_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,

@@ -118,6 +118,8 @@ SIGNATURES = {
     "qlin_probe_mfma_bf16": (C.c_int, [C.c_int, _vp, C.POINTER(C.c_double)]),
     "qlin_probe_clocks": (C.c_int, [_vp, C.POINTER(C.c_double)]),
     "qlin_probe_hbm_read": (C.c_int, [_vp, C.c_size_t, _vp]),
+    "qlin_probe_gemm_route": (C.c_int, [C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "qlin_probe_gemm_tile": (C.c_int, [C.c_int, C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp]),
     "qlin_timer_begin": (C.c_int, [_vp]),
     "qlin_timer_end": (C.c_int, [_vp, _fp]),
 }
@@ -370,6 +372,10 @@ def probe_clocks(stream=None):
     mhz = C.c_double(0)
     check(load().qlin_probe_clocks(stream, C.byref(mhz)))
     return mhz.value
+
+
+def probe_gemm_tile(tile, type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, stream=None):
+    check(load().qlin_probe_gemm_tile(tile, type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy, stream))
 
 
 def probe_hbm_read(buf, n_bytes=None, stream=None):

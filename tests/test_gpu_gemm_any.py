@@ -41,6 +41,7 @@ def dense_kernel(request):
     qlinear.check(qlinear.load().qlin_set_dense_gemm_own(0))
 
 
+FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0]  # decoded inside the tile kernels
 KQ = {synth.GGML_Q6_K, synth.GGML_Q5_K, synth.GGML_Q3_K, synth.GGML_Q2_K, synth.GGML_Q8_0}
 
 
@@ -89,9 +90,6 @@ def test_shapes(oracle, tid, n_tok, n_rows, n_cols, dense_kernel):
     assert rel_l2(Y, exact) <= 3e-3
 
 
-FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0]
-
-
 @pytest.mark.parametrize("tid", FUSED, ids=lambda t: ALL[t])
 @pytest.mark.parametrize("n_tok,n_rows,n_cols", [
     (260, 12805, 256),   # 101 x 2 tiles: one super-block, ragged rows and tokens
@@ -120,6 +118,33 @@ def test_fused_tile_kernel_shapes(oracle, tid, n_tok, n_rows, n_cols):
     exact, designed = references(oracle, tid, W[rows], Xb, n_cols)
     assert rel_l2(Y[:, rows], designed) <= 2e-5, (ALL[tid], n_tok, n_rows, n_cols)
     assert rel_l2(Y[:, rows], exact) <= 3e-3
+
+
+@pytest.mark.parametrize("tile", [0, 1], ids=["256x128", "128x64"])
+@pytest.mark.parametrize("tid", FUSED, ids=lambda t: ALL[t])
+@pytest.mark.parametrize("n_tok,n_rows,n_cols", [
+    (5, 7, 256), (130, 70, 512), (300, 200, 1280), (64, 129, 2048), (513, 65, 256),
+])
+def test_each_tile_kernel_on_small_and_ragged_shapes(oracle, tile, tid, n_tok, n_rows, n_cols):
+    """both tile kernels called by name, on shapes the shape-based choice would give to other kernels: one super-block,
+    an odd count of them, single rows and tokens, ragged last tiles, padded leading dimensions"""
+    W = synth.make_weights(tid, n_rows, n_cols, seed=3 * n_rows + tid + tile)
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=n_tok + tid, tokens=n_tok))
+    ldx, ldy = n_cols + 16, n_rows + 1
+    Xpad = np.zeros((n_tok, ldx), np.uint16)
+    Xpad[:, :n_cols] = Xb
+    dW, dX = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xpad)
+    dY = qlinear.DevBuf.from_numpy(np.full((n_tok, ldy), -3.0, np.float32))
+    qlinear.probe_gemm_tile(tile, tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy)
+    qlinear.sync()
+    Y = dY.to_numpy(np.float32, (n_tok, ldy))
+    for buf in (dW, dX, dY):
+        buf.free()
+    assert np.all(Y[:, n_rows:] == -3.0)
+    exact, designed = references(oracle, tid, W, Xb, n_cols)
+    assert rel_l2(Y[:, :n_rows], designed) <= 2e-5, (ALL[tid], tile, n_tok, n_rows, n_cols)
+    if n_tok * n_rows >= 1000:  # the bar on the bf16 rounding of the weights is a statistical one
+        assert rel_l2(Y[:, :n_rows], exact) <= 3e-3
 
 
 @pytest.mark.parametrize("tid", [synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0], ids=lambda t: ALL[t])
@@ -202,8 +227,9 @@ def test_few_tokens_whose_rows_lie_far_apart(oracle):
 @pytest.mark.parametrize("n_tok", [1, 8, 9, 24, 25])
 @pytest.mark.parametrize("tid", sorted(KQ), ids=lambda t: ALL[t])
 def test_few_tokens_of_a_k_quant_or_q8_0_tensor(oracle, tid, n_tok):
-    """up to 24 tokens: one kernel, unrounded weights, no workspace, rows and padding of any count; 25 tokens: the
-    decode + dense route, which needs the workspace"""
+    """up to 24 tokens: one kernel, unrounded weights, no workspace, rows and padding of any count; 25 tokens: weights
+    rounded to bf16 - inside the tile kernel for the formats that has (no workspace either), else by the decode + dense
+    route, which needs the workspace"""
     # 5 super-blocks over 4 waves, a last row tile of 8 rows; the kernel wants the tensor to end on a 16-byte
     # boundary (210-, 110- and 84-byte blocks: a row count that is a multiple of 8)
     n_rows, n_cols = 296, 1280
@@ -218,6 +244,9 @@ def test_few_tokens_of_a_k_quant_or_q8_0_tensor(oracle, tid, n_tok):
     if n_tok <= 24:
         qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, None)
         want = exact
+    elif tid in FUSED:
+        qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, None)
+        want = designed
     else:
         with pytest.raises(qlinear.QlinError):
             qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, None)
@@ -231,7 +260,7 @@ def test_few_tokens_of_a_k_quant_or_q8_0_tensor(oracle, tid, n_tok):
 
 
 def test_q4k_few_tokens_is_the_fused_path_and_needs_no_workspace(oracle):
-    n_tok, n_rows, n_cols = 40, 96, 512
+    n_tok, n_rows, n_cols = 30, 96, 512
     W = synth.make_weights(Q4K, n_rows, n_cols, seed=1)
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=2, tokens=n_tok))
     dW, dX, dY = qlinear.DevBuf.from_numpy(W), qlinear.DevBuf.from_numpy(Xb), qlinear.DevBuf(n_tok * n_rows * 4)
@@ -281,10 +310,12 @@ def test_argument_checks():
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 300, 4, 304, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ragged K
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 260, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ldx % 8
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 100, ws.ptr, need, None) == qlinear.ERR_ARG      # ldy < rows
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
-    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, None, 0, None) == 0  # few tokens: no workspace needed
+    NL = synth.GGML_IQ4_NL  # a format that always takes the decode + dense route above four tokens
+    assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
+    assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
+    assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 128, None, 0, None) == 0   # few tokens: no workspace needed
+    assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, None, 0, None) == 0  # nor by the tile kernels
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 0, 256, 4, 256, 128, None, 0, None) == 0
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 0, 256, 128, None, 0, None) == 0
     assert lib.qlin_gemm_bf16_any_workspace_bytes(0, 256) == 0
@@ -304,8 +335,10 @@ def test_decode_to_bf16_is_the_codec_rounded_once(oracle, tid):
     n_tok = 70
     Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=7, tokens=n_tok))
     Y_cached = run(synth.GGML_BF16, got.view(np.uint8).reshape(n_rows, -1), Xb, n_rows, n_cols, n_tok)
-    Y_direct = run(tid, W, Xb, n_rows, n_cols, n_tok) if not (tid == Q4K) else None
-    if Y_direct is not None:
+    Y_direct = run(tid, W, Xb, n_rows, n_cols, n_tok)
+    if tid in FUSED:  # the same rounded weights inside the tile kernel, summed in another order
+        assert rel_l2(Y_direct, Y_cached) <= 2e-6
+    else:
         assert np.array_equal(Y_cached, Y_direct)
     dW.free()
     dout.free()
