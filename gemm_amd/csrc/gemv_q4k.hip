@@ -369,6 +369,8 @@ gemv_q4k_dma_kernel(const uint8_t *__restrict__ W, float *__restrict__ y, const 
             part = wrap ? 0u : part + 1u;
             voff += 7u * (uint32_t)row_bytes + (wrap ? (uint32_t)row_bytes - 128u : 16u);
         }
+        /* xv is written by the load above without the compiler knowing when: this wait is its first use, in the
+         * registers the load wrote (the compiled code is checked for a copy ahead of it whenever this kernel changes) */
         wait_vm<NQ>(xv);
         XOperand xo;
         q4k_prepare(xv, xo, xs, lane);
@@ -397,6 +399,117 @@ gemv_q4k_dma_kernel(const uint8_t *__restrict__ W, float *__restrict__ y, const 
             run(3);
         }
         wait_vm<0>(); /* nothing on its way into LDS when the wave ends */
+    }
+    __syncthreads();
+    for (int lr = threadIdx.x; lr < rows_here; lr += kWaves * 64) {
+        const float4 *p = reinterpret_cast<const float4 *>(partial + lr * kWaves);
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < kWaves / 4; k++) {
+            const float4 v = p[k];
+            s += (v.x + v.y) + (v.z + v.w);
+        }
+        y[row0 + lr] = add ? y[row0 + lr] + s : s;
+    }
+}
+
+/* The load-to-LDS matvec for one matrix of longer rows (17 to 64 super-blocks) and at most kDmaLongRows rows per
+ * workgroup - the down projection, 4096 x 14336: 16 rows per compute unit. Wave w takes super-blocks w, w + 16, ... of
+ * the workgroup's rows, one pass each; the image of a pass is rows x 144 bytes (NQ requests), two image slots per wave:
+ * the pass after next is requested as soon as a pass has been multiplied, so a wave has two passes in flight or in
+ * work instead of one round trip after the other. A pass's 256 activations come by the same path into the last KB of
+ * its slot (a register load would have to be waited for by a counter the compiler cannot see). A row's shares of
+ * all passes are added in registers. */
+constexpr int kDmaLongRows = 21;   /* 21 x 144 B = 3024: a 4 KB slot holds the image (3 requests) and 1 KB of activations */
+constexpr int kDmaLongPasses = 4;
+
+template <int NQ>
+__global__ void __launch_bounds__(kWaves * 64)
+gemv_q4k_dma_long_kernel(const uint8_t *__restrict__ W, float *__restrict__ y, const float *__restrict__ x, int n_rows,
+                         int n_sb, int add, int rows_per_wg, size_t row_bytes) {
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+    const int lane = threadIdx.x & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * rows_per_wg;
+    int rows_here = n_rows - row0;
+    if (rows_here > rows_per_wg) rows_here = rows_per_wg;
+    const int n_rg = (rows_here + 15) >> 4; /* 1 or 2 */
+    const int n_kc = (n_sb - wv + 15) >> 4; /* this wave's passes: 1 .. 4 (n_sb > 16) */
+    /* LDS map: image slots [kWaves][2][4 KB] | x scratch [kWaves][kXScratch] | partial sums [rows][kWaves] */
+    uint8_t *img = lds + wv * kDmaImage;
+    uint8_t *xs = lds + kWaves * kDmaImage + wv * kXScratch;
+    float *partial = reinterpret_cast<float *>(lds + kWaves * (kDmaImage + kXScratch));
+
+    static_assert(NQ <= 3, "a slot is three requests of weights and one of activations");
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(x), 0, n_sb * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t *>(W) + (size_t)row0 * row_bytes, 0, (int)((size_t)(rows_here - 1) * row_bytes + (size_t)n_sb * 144),
+        0x00020000);
+    const uint32_t img_base = (uint32_t)(uintptr_t)img;
+    /* piece id = 64 q + lane is part id % 9 of row id / 9; pieces past the last row arrive as zeros */
+    uint32_t voff0[NQ];
+    {
+        uint32_t part = (uint32_t)lane % 9u, row = (uint32_t)lane / 9u;
+#pragma unroll
+        for (int q = 0; q < NQ; q++) {
+            voff0[q] = row < (uint32_t)rows_here ? row * (uint32_t)row_bytes + 16u * part : 0xFFFFFFF0u;
+            const bool wrap = part == 8u;
+            part = wrap ? 0u : part + 1u;
+            row += wrap ? 8u : 7u;
+        }
+    }
+    const uint32_t x_voff = 16u * (uint32_t)lane;
+    auto request = [&](int kc) { /* pass kc into slot kc & 1: its activations, then its blocks */
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :
+                     : "s"(img_base + 4096u * (kc & 1) + 3072u), "v"(x_voff), "s"(x_rsrc), "s"((uint32_t)(16 * kc + wv) * 1024u)
+                     : "memory");
+        const uint32_t soff = (uint32_t)(16 * kc + wv) * 144u;
+#pragma unroll
+        for (int q = 0; q < NQ; q++)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :
+                         : "s"(img_base + 4096u * (kc & 1) + 1024u * q), "v"(voff0[q]), "s"(rsrc), "s"(soff)
+                         : "memory");
+    };
+    request(0);
+    if (n_kc > 1) request(1);
+    float acc[2] = {0.0f, 0.0f};
+    XOperand xo;
+#pragma unroll
+    for (int kc = 0; kc < kDmaLongPasses; kc++) {
+        if (kc < n_kc) {
+            /* the requests of this pass are in when at most those of the next one are outstanding */
+            if (kc + 1 < n_kc) wait_vm<NQ + 1>();
+            else wait_vm<0>();
+            const uint8_t *slot = img + 4096 * (kc & 1);
+            q4k_prepare(*reinterpret_cast<const v4f *>(slot + 3072 + 16 * lane), xo, xs, lane);
+#pragma unroll
+            for (int rg = 0; rg < 2; rg++) {
+                if (rg < n_rg) {
+                    int lr = 16 * rg + n;
+                    if (lr >= rows_here) lr = rows_here - 1; /* rows past the end: the last one, never stored */
+                    const uint8_t *blk = slot + lr * 144;
+                    const uint4 h = *reinterpret_cast<const uint4 *>(blk);
+                    const uint4 q0 = *reinterpret_cast<const uint4 *>(blk + 16 + 16 * g);
+                    const uint4 q1 = *reinterpret_cast<const uint4 *>(blk + 80 + 16 * g);
+                    acc[rg] += q4k_item(xo, h, q0, q1, g);
+                }
+            }
+            if (kc + 2 < n_kc) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); /* the slot has been read before it is refilled */
+                request(kc + 2);
+            }
+        }
+    }
+#pragma unroll
+    for (int rg = 0; rg < 2; rg++) {
+        if (rg < n_rg) {
+            const float v = sum_lane_groups(acc[rg]);
+            const int lr = 16 * rg + n;
+            if (lane < 16 && lr < rows_here) partial[lr * kWaves + wv] = v;
+        }
     }
     __syncthreads();
     for (int lr = threadIdx.x; lr < rows_here; lr += kWaves * 64) {
@@ -593,6 +706,30 @@ hipError_t launch_gemv_q4k(const GemvJob &job, const float *x, int n_cols, hipSt
         case 6: return launch_dma(gemv_q4k_dma_kernel<6>, raised[5]);
         case 7: return launch_dma(gemv_q4k_dma_kernel<7>, raised[6]);
         default: return launch_dma(gemv_q4k_dma_kernel<8>, raised[7]);
+        }
+    }
+    /* one matrix, rows of 17 to 64 super-blocks, at most 21 rows per workgroup: the load-to-LDS kernel for long rows */
+    /* (1 GiB rotation, this kernel / the register-load kernel below, us: 4096 x 14336 9.1 / 9.8, 2048 x 16384 8.2 / 9.5,
+     * 4096 x 8192 6.3 / 7.1, 1024 x 14336 6.6 / 7.7, 4096 x 5120 5.0 / 5.2; with three passes for most waves and two for
+     * the rest, 4096 x 11008, it measured 8.3 / 7.7, so rows of 33 to 48 super-blocks stay with the other kernel) */
+    if (one && n_sb > 16 && n_sb <= 16 * kDmaLongPasses && (n_sb <= 32 || n_sb > 48) && rows_per_wg <= kDmaLongRows &&
+        (size_t)kDmaLongRows * row_stride < ((size_t)1 << 31)) {
+        auto launch_long = [&](auto kernel, OnceFlag &lds_raised) {
+            if (!lds_raised.is_set()) {
+                hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                if (e != hipSuccess) return e;
+                lds_raised.set();
+            }
+            hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64),
+                               (size_t)kWaves * (kDmaImage + kXScratch) + (size_t)rows_per_wg * kWaves * 4, stream,
+                               (const uint8_t *)job.W[0], job.y[0], x, n_rows, n_sb, job.mode == kAdd ? 1 : 0, rows_per_wg, row_stride);
+            return hipGetLastError();
+        };
+        static OnceFlag raised_long[3];
+        switch ((rows_per_wg * 9 + 63) / 64) {
+        case 1: return launch_long(gemv_q4k_dma_long_kernel<1>, raised_long[0]);
+        case 2: return launch_long(gemv_q4k_dma_long_kernel<2>, raised_long[1]);
+        default: return launch_long(gemv_q4k_dma_long_kernel<3>, raised_long[2]);
         }
     }
     if (n_sb <= 16) {
