@@ -61,7 +61,7 @@ struct VecAt { int off; int by_half; };
 
 /* scratch of the decode that all formats share */
 struct Temps {
-    uint32_t cm, hb;
+    uint32_t cm, hb, lo, hi;
     float2v cp0, cp1;
     float f0, f1, f2, f3, w0, w1, w2, w3;
     float s_a, s_b, m_a, m_b, dl_a, dl_b, nml_a, nml_b; /* of the two sub-blocks (scale groups) of the tile in work */
@@ -229,6 +229,60 @@ struct FQ8_0 {
             constexpr int dw = (P - 1) / 6, ph = (P - 1) % 6;
             if constexpr (ph == 0) t.cm = raw[2 * TC + (dw >> 2)][dw & 3] ^ 0x80808080u;
             else bytes4_piece<ph + 1, dw & 1>(c, t.dl_a, t.nml_a, c.wa[WB][dw >> 1]);
+        }
+    }
+};
+
+/* ---- IQ4_NL: 18-byte blocks = d | 16 bytes whose low nibbles are elements 0..15 and high nibbles 16..31, each nibble an
+ * index into a table of 16 int8 values (common/ggml_dequant.h:2942-2954); eight blocks (144 bytes, like a Q4_K
+ * super-block) are the unit. Both lane halves take the same bytes - half kg their nibble kg - so a lane keeps the whole
+ * 144-byte image of its row in nine vectors and cuts a block's four code dwords out of them at offsets known at
+ * compile time (blocks with an even index start two bytes into a dword: one v_alignbyte per dword). The table lookup
+ * is two byte permutes (entries 0..7, 8..15, stored with 128 added so that they are unsigned bytes) and a select on
+ * bit 3 of the index: about 5 vector instructions per weight, more than one wave per SIMD can issue beside the matrix
+ * instructions, but far fewer than the decode to bf16 in memory costs. */
+struct FIQ4NL {
+    static constexpr int kBlockBytes = 144, kPieces = 9, kReq = 5, kLaneVec = 9, kPrepPieces = 0, kTilePieces = 82;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    struct Scales {};
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
+    static constexpr VecAt vec_at(int j) { return VecAt{16 * j, 0}; }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
+    template <int P, class C> static QLIN_INL void prep(C &, const u32x4 (&)[kLaneVec + kExtraVec]) {}
+    /* dword I of the row image */
+    template <int I> static QLIN_INL uint32_t image_dword(const u32x4 (&raw)[kLaneVec + kExtraVec]) { return raw[I >> 2][I & 3]; }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        Temps &t = c.t;
+        if constexpr (P < 2) {
+            /* d of block 2 TC + P: bytes 18 b, 18 b + 1 of the image */
+            constexpr int b = 2 * TC + P, at = 18 * b;
+            const float d = half_bits_fast((image_dword<(at >> 2)>(raw) >> (8 * (at & 3))) & 0xFFFFu);
+            if constexpr (P == 0) { t.dl_a = d; t.nml_a = -128.0f * d; }
+            else { t.dl_b = d; t.nml_b = -128.0f * d; }
+        } else {
+            constexpr int dw = (P - 2) / 10, ph = (P - 2) % 10, b = 2 * TC + (dw >> 2), at = 18 * b + 2 + 4 * (dw & 3);
+            const float dl = (dw >> 2) ? t.dl_b : t.dl_a, off = (dw >> 2) ? t.nml_b : t.nml_a;
+            if constexpr (ph == 0) {
+                uint32_t src;
+                if constexpr ((at & 3) == 0) src = image_dword<(at >> 2)>(raw);
+                else src = __builtin_amdgcn_alignbyte(image_dword<(at >> 2) + 1>(raw), image_dword<(at >> 2)>(raw), at & 3);
+                t.hb = src >> (4u * (uint32_t)c.kg); /* the lane half's nibble of every byte */
+            } else if constexpr (ph == 1) {
+                t.cm = t.hb & 0x0F0F0F0Fu;
+                t.hb = t.cm & 0x07070707u;
+            } else if constexpr (ph == 2) {
+                t.lo = __builtin_amdgcn_perm(0x766A5D4Fu, 0x3F2D1801u, t.hb); /* table entries 0..7, + 128 */
+                t.hi = __builtin_amdgcn_perm(0xF1D9C5B5u, 0xA6998D81u, t.hb); /* entries 8..15 */
+            } else if constexpr (ph == 3) {
+                t.hb = (t.cm >> 3) & 0x01010101u;
+            } else if constexpr (ph == 4) {
+                t.hb *= 255u; /* 0xFF in the bytes whose index is 8 or more */
+                t.cm = (t.hb & t.hi) | (~t.hb & t.lo);
+            } else {
+                bytes4_piece<ph - 3, dw & 1>(c, dl, off, c.wa[WB][dw >> 1]);
+            }
         }
     }
 };

@@ -1,5 +1,5 @@
 /*
- * gemm_kq_wave4.hip - Q4_K, Q5_K, Q6_K and Q8_0 x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup,
+ * gemm_kq_wave4.hip - Q4_K, Q5_K, Q6_K, Q8_0 and IQ4_NL x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup,
  * one per SIMD.
  *
  *   Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k]      X bf16, Y fp32, fp32 accumulate
@@ -135,7 +135,7 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     /* U = 0: the raw data of the next super-block (requested three tiles ago) into registers; U = 1: request the
      * one after it into the same place; U = 3: the tile being decoded is the first of the next super-block, which
      * then becomes the one in work */
-    if constexpr (U == 0 && T % 4 == 1 && T / 4 < F::kLaneVec) c.nxt[T / 4] = load_raw<F, T / 4>(c);
+    if constexpr (U == 0 && T % 3 == 1 && T / 3 < F::kLaneVec) c.nxt[T / 3] = load_raw<F, T / 3>(c);
     if constexpr (U == 0 && T % 4 == 1 && T / 4 < F::kExtraLoads) F::template extra_load<T / 4>(c, c.nxt, min(c.sb + 1, c.n_sb - 1));
     if constexpr (U == 1 && T % 4 == 1 && T / 4 < F::kReq) request_w<F, T / 4>(c, c.sb + 2);
     if constexpr (U == 3 && T % 3 == 2 && T / 3 < F::kLaneVec + F::kExtraVec) c.cur[T / 3] = c.nxt[T / 3];
@@ -154,7 +154,8 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     };
     piece(std::integral_constant<int, p0>{});
     piece(std::integral_constant<int, p0 + 1>{});
-    static_assert(p1 - p0 <= 2, "at most two pieces per slot");
+    piece(std::integral_constant<int, p0 + 2>{});
+    static_assert(p1 - p0 <= 3, "at most three pieces per slot");
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -294,7 +295,9 @@ hipError_t launch_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, 
 }
 }  // namespace
 
-bool gemm_kq_wave4_covers(uint32_t type) { return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K || type == T_Q8_0; }
+bool gemm_kq_wave4_covers(uint32_t type) {
+    return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K || type == T_Q8_0 || type == T_IQ4_NL;
+}
 
 /* Which kernel takes a prefill GEMM of a format with a fused kernel, beyond the token counts of the few-token kernels.
  * 200 or more 256-token x 128-row tiles fill the chip: the large-tile kernel - up to a token count, because it decodes
@@ -304,13 +307,16 @@ bool gemm_kq_wave4_covers(uint32_t type) { return type == T_Q4_K || type == T_Q5
  * 139 / 121; at 1536 181 / 190, 185 / 195, 206 / 184, 216 / 177; at 2048 267 / 244, 262 / 260, 273 / 240, 311 / 224).
  * Fewer large tiles: the small-tile kernel (4096 x 4096 at 512 tokens, small tiles / decode + library: Q4_K 29 / 45,
  * Q6_K 34 / 40, Q8_0 36 / 39; 4096 x 14336: 89 / 100, 104 / 100, 110 / 101; 14336 x 4096 at 128 tokens: 28 / 74,
- * 33 / 73, 36 / 72; at 256: 46 / 77, 55 / 84, 63 / 81), for Q6_K and Q8_0 up to 256 tokens.
+ * 33 / 73, 36 / 72; at 256: 46 / 77, 55 / 84, 63 / 81), for Q6_K, Q8_0 and IQ4_NL up to 256 tokens. IQ4_NL (a table
+ * lookup per weight): large tiles 62 / 95 at 512 tokens, 123 / 132 at 1024, 279 / 254 at 2048; small tiles 4096 x 4096
+ * 38 / 45, 4096 x 14336 120 / 108, 14336 x 4096 at 128 tokens 37 / 80.
  * Without a workspace there is no decode + dense route to prefer. */
 FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, bool have_workspace) {
     if (!gemm_kq_wave4_covers(type) || n_cols % 256 != 0 || ldx >= (1 << 22)) return kFusedNone;
     const long long large_tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
     const bool light = type == T_Q4_K || type == T_Q5_K; /* less to decode per weight */
-    if (large_tiles >= 200) return (n_tok <= (light ? 1536 : 512) || !have_workspace) ? kFusedLarge : kFusedNone;
+    if (large_tiles >= 200)
+        return (n_tok <= (light || type == T_IQ4_NL ? 1536 : 512) || !have_workspace) ? kFusedLarge : kFusedNone;
     return (light || n_tok <= 256 || !have_workspace) ? kFusedSmall : kFusedNone;
 }
 
@@ -328,6 +334,7 @@ hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_
     case T_Q5_K: return launch_wave4<FQ5K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q6_K: return launch_wave4<FQ6K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q8_0: return launch_wave4<FQ8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_IQ4_NL: return launch_wave4<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }

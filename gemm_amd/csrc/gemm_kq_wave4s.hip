@@ -1,5 +1,5 @@
 /*
- * gemm_kq_wave4s.hip - the fused Q4_K / Q5_K / Q6_K / Q8_0 x bf16 prefill GEMM in 128-token x 64-row tiles, for the
+ * gemm_kq_wave4s.hip - the fused Q4_K / Q5_K / Q6_K / Q8_0 / IQ4_NL x bf16 prefill GEMM in 128-token x 64-row tiles, for the
  * shapes whose 256-token x 128-row tiles (gemm_kq_wave4.hip) would leave most of the chip idle: 4096-row projections
  * at 512 tokens (64 large tiles, 256 small ones), 14336 rows at 129..256 tokens.
  *
@@ -99,7 +99,7 @@ template <class F, int U, int P0, int P1, int... I> QLIN_INL void pieces(Ctx<F> 
 /* slot T (0..7) of tile 4 sb + U: k-step T / 2, token block T % 2 */
 template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     constexpr int s = T / 2, bj = T % 2, nW = Ctx<F>::kMyReq, nE = F::kExtraLoads, nV = F::kLaneVec + F::kExtraVec;
-    static_assert(nE <= 4 && nW <= 4 && F::kLaneVec <= 8 && nV <= 10, "side work is laid out over the first slots of a tile");
+    static_assert(nE <= 4 && nW <= 4 && F::kLaneVec <= 10 && nV <= 10, "side work is laid out over the first slots of a tile");
     if constexpr (T == 6) {
         /* this wave's requests of the next tile have landed: younger are the 4 of the tile after it, 3 of the one
          * after that, the weight requests of a tile with U = 1 and the scale loads of one with U = 0 */
@@ -111,7 +111,7 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     c.acc[bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, c.wa[U & 1][s]), c.xf[s & 1][bj], c.acc[bj], 0, 0, 0);
     c.xf[(s + 1) & 1][bj] = load_frag<F, (s == 3 ? (U + 1) & 3 : U), (s + 1) & 3, bj>(c);
     if constexpr (T % 2 == 1) request_x<F, (U + 3) & 3, T / 2>(c, 4 * c.sb + U + 3);
-    if constexpr (U == 0 && T < 4) {
+    if constexpr (U == 0 && T < 5) { /* all before the barrier of this tile */
         if constexpr (2 * T < F::kLaneVec) c.nxt[2 * T] = load_raw<F, 2 * T>(c);
         if constexpr (2 * T + 1 < F::kLaneVec) c.nxt[2 * T + 1] = load_raw<F, 2 * T + 1>(c);
         if constexpr (T < nE) F::template extra_load<T>(c, c.nxt, min(c.sb + 1, c.n_sb - 1));
@@ -123,8 +123,8 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     }
     constexpr int n_pieces = F::kTilePieces + (U == 3 ? F::kPrepPieces : 0);
     constexpr int p0 = (T * n_pieces + 7) / 8, p1 = ((T + 1) * n_pieces + 7) / 8; /* pieces p with p * 8 / n_pieces == T */
-    static_assert(p1 - p0 <= 8, "at most eight pieces per slot");
-    pieces<F, U, p0, p1>(c, std::make_integer_sequence<int, 8>{});
+    static_assert(p1 - p0 <= 11, "at most eleven pieces per slot");
+    pieces<F, U, p0, p1>(c, std::make_integer_sequence<int, 11>{});
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -274,6 +274,7 @@ hipError_t launch_gemm_kq_bf16_wave4s(uint32_t type, const void *W, const uint16
     case T_Q5_K: return launch_wave4s<FQ5K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q6_K: return launch_wave4s<FQ6K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q8_0: return launch_wave4s<FQ8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_IQ4_NL: return launch_wave4s<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }
