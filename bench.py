@@ -508,6 +508,12 @@ def probe(args):
     elif args.probe == "gemm_any_q8_0":  # Q8_0, 512 tokens: decoded inside the tile kernel
         ms = time_gemm_any(synth.GGML_Q8_0, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_any_q8_0", "ms_per_step": ms}))
+    elif args.probe == "gemm_small_q4_K":  # Q4_K 4096 x 4096 at 512 tokens: the 128-token x 64-row tile kernel
+        ms = time_gemm_any(Q4K, 512, 4096, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_small_q4_K", "ms_per_step": ms}))
+    elif args.probe == "gemm_any_iq4_nl":  # IQ4_NL, 512 tokens: decoded inside the large-tile kernel
+        ms = time_gemm_any(synth.GGML_IQ4_NL, 512, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_any_iq4_nl", "ms_per_step": ms}))
     elif args.probe == "gemm_f32_any_q4_K":  # decode to fp32 + dense fp32 library GEMM, Q4_K, 512 tokens
         ms = time_gemm_f32_any(Q4K, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_f32_any_q4_K", "ms_per_step": ms}))
@@ -646,7 +652,7 @@ def main():
     ap.add_argument("--prows", type=int, default=4096)
     ap.add_argument("--pcols", type=int, default=14336)
     ap.add_argument("--ptok", type=int, default=64, help="--probe moe: tokens in the batch")
-    ap.add_argument("--probe", choices=["gemv_any", "copy", "tiny", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["gemv_any", "copy", "tiny", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_small_q4_K", "gemm_any_iq4_nl", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "
