@@ -287,6 +287,94 @@ struct FIQ4NL {
     }
 };
 
+/* ---- Q4_0: 18-byte blocks = d | 16 bytes, elements 0..15 in the low nibbles, 16..31 in the high ones, value d (q - 8)
+ * (common/ggml_dequant.h:2850-2862). The layout and the lane roles of IQ4_NL with the arithmetic of Q4_K: the nibbles
+ * go through the fp8 reading. */
+struct FQ4_0 {
+    static constexpr int kBlockBytes = 144, kPieces = 9, kReq = 5, kLaneVec = 9, kPrepPieces = 0, kTilePieces = 50;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    struct Scales {};
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
+    static constexpr VecAt vec_at(int j) { return VecAt{16 * j, 0}; }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
+    template <int P, class C> static QLIN_INL void prep(C &, const u32x4 (&)[kLaneVec + kExtraVec]) {}
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        Temps &t = c.t;
+        if constexpr (P < 2) {
+            constexpr int b = 2 * TC + P, at = 18 * b;
+            const float d = half_bits_fast((FIQ4NL::image_dword<(at >> 2)>(raw) >> (8 * (at & 3))) & 0xFFFFu);
+            if constexpr (P == 0) { t.dl_a = d * c.unit; t.nml_a = -8.0f * d; }
+            else { t.dl_b = d * c.unit; t.nml_b = -8.0f * d; }
+        } else {
+            constexpr int dw = (P - 2) / 6, ph = (P - 2) % 6, b = 2 * TC + (dw >> 2), at = 18 * b + 2 + 4 * (dw & 3);
+            const float dl = (dw >> 2) ? t.dl_b : t.dl_a, off = (dw >> 2) ? t.nml_b : t.nml_a;
+            if constexpr (ph == 0) {
+                uint32_t src;
+                if constexpr ((at & 3) == 0) src = FIQ4NL::image_dword<(at >> 2)>(raw);
+                else src = __builtin_amdgcn_alignbyte(FIQ4NL::image_dword<(at >> 2) + 1>(raw), FIQ4NL::image_dword<(at >> 2)>(raw), at & 3);
+                t.hb = src >> (4u * (uint32_t)c.kg);
+            } else if constexpr (ph == 1) t.cm = t.hb & 0x0F0F0F0Fu;
+            else if constexpr (ph == 2) { t.cp0 = fp8_pair_lo(t.cm); t.cp1 = fp8_pair_hi(t.cm); }
+            else if constexpr (ph == 3) { t.w0 = fmaf(t.cp0.x, dl, off); t.w1 = fmaf(t.cp0.y, dl, off); }
+            else if constexpr (ph == 4) { t.w2 = fmaf(t.cp1.x, dl, off); t.w3 = fmaf(t.cp1.y, dl, off); }
+            else if constexpr ((dw & 1) == 0) { c.wa[WB][dw >> 1].x = pack_bf16(t.w0, t.w1); c.wa[WB][dw >> 1].y = pack_bf16(t.w2, t.w3); }
+            else { c.wa[WB][dw >> 1].z = pack_bf16(t.w0, t.w1); c.wa[WB][dw >> 1].w = pack_bf16(t.w2, t.w3); }
+        }
+    }
+};
+
+/* ---- IQ4_XS: 136-byte super-blocks = d | 8 x 2 high scale bits | 8 x 4 low scale bits | 8 x 16 code bytes; sub-block g
+ * (32 elements) = the nibbles of bytes 8 + 16 g .. + 15 as in IQ4_NL, through the same table, times d (ls_g - 32)
+ * (common/ggml_dequant.h:2956-2973). A row's image is nine 16-byte pieces (the last one half belongs to the next
+ * super-block); the code dwords are aligned. */
+struct XsScales { float d; };
+struct FIQ4XS {
+    static constexpr int kBlockBytes = 136, kPieces = 9, kReq = 5, kLaneVec = 9, kPrepPieces = 1, kTilePieces = 88;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    typedef XsScales Scales;
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
+    static constexpr VecAt vec_at(int j) { return VecAt{16 * j, 0}; }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
+    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        c.sc.d = half_bits_fast(raw[0].x & 0xFFFFu);
+    }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        Temps &t = c.t;
+        if constexpr (P < 8) {
+            /* four pieces per sub-block g = 2 TC + P / 4: the 6-bit scale, then d (ls - 32) and -128 times that */
+            constexpr int g = 2 * TC + (P >> 2), q = P & 3;
+            float &dl = (P >> 2) ? t.dl_b : t.dl_a, &nml = (P >> 2) ? t.nml_b : t.nml_a;
+            if constexpr (q == 0) { t.lo = (raw[0].y >> (8 * (g >> 1) + 4 * (g & 1))) & 15u; t.hi = (raw[0].x >> (16 + 2 * g)) & 3u; }
+            else if constexpr (q == 1) t.lo = (t.lo | (t.hi << 4)) - 32u;
+            else if constexpr (q == 2) dl = c.sc.d * (float)(int)t.lo;
+            else nml = -128.0f * dl;
+        } else {
+            constexpr int dw = (P - 8) / 10, ph = (P - 8) % 10, g = 2 * TC + (dw >> 2);
+            const float dl = (dw >> 2) ? t.dl_b : t.dl_a, off = (dw >> 2) ? t.nml_b : t.nml_a;
+            if constexpr (ph == 0) {
+                t.hb = FIQ4NL::image_dword<2 + 4 * g + (dw & 3)>(raw) >> (4u * (uint32_t)c.kg);
+            } else if constexpr (ph == 1) {
+                t.cm = t.hb & 0x0F0F0F0Fu;
+                t.hb = t.cm & 0x07070707u;
+            } else if constexpr (ph == 2) {
+                t.lo = __builtin_amdgcn_perm(0x766A5D4Fu, 0x3F2D1801u, t.hb);
+                t.hi = __builtin_amdgcn_perm(0xF1D9C5B5u, 0xA6998D81u, t.hb);
+            } else if constexpr (ph == 3) {
+                t.hb = (t.cm >> 3) & 0x01010101u;
+            } else if constexpr (ph == 4) {
+                t.hb *= 255u;
+                t.cm = (t.hb & t.hi) | (~t.hb & t.lo);
+            } else {
+                bytes4_piece<ph - 3, dw & 1>(c, dl, off, c.wa[WB][dw >> 1]);
+            }
+        }
+    }
+};
+
 /* one load-to-LDS request: lane l's 16 bytes from voff + soff of the buffer land at lds + 16 l */
 QLIN_INL void dma16(__amdgpu_buffer_rsrc_t rsrc, uint8_t *lds, uint32_t voff, uint32_t soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void *)lds, 16, voff, soff, 0, 0);

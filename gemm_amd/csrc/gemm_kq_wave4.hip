@@ -1,5 +1,5 @@
 /*
- * gemm_kq_wave4.hip - Q4_K, Q5_K, Q6_K, Q8_0 and IQ4_NL x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup,
+ * gemm_kq_wave4.hip - Q4_K, Q5_K, Q6_K, Q8_0, IQ4_NL, IQ4_XS and Q4_0 x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup,
  * one per SIMD.
  *
  *   Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k]      X bf16, Y fp32, fp32 accumulate
@@ -296,7 +296,8 @@ hipError_t launch_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, 
 }  // namespace
 
 bool gemm_kq_wave4_covers(uint32_t type) {
-    return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K || type == T_Q8_0 || type == T_IQ4_NL;
+    return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K || type == T_Q8_0 || type == T_IQ4_NL || type == T_IQ4_XS ||
+           type == T_Q4_0;
 }
 
 /* Which kernel takes a prefill GEMM of a format with a fused kernel, beyond the token counts of the few-token kernels.
@@ -309,15 +310,23 @@ bool gemm_kq_wave4_covers(uint32_t type) {
  * Q6_K 34 / 40, Q8_0 36 / 39; 4096 x 14336: 89 / 100, 104 / 100, 110 / 101; 14336 x 4096 at 128 tokens: 28 / 74,
  * 33 / 73, 36 / 72; at 256: 46 / 77, 55 / 84, 63 / 81), for Q6_K, Q8_0 and IQ4_NL up to 256 tokens. IQ4_NL (a table
  * lookup per weight): large tiles 62 / 95 at 512 tokens, 123 / 132 at 1024, 279 / 254 at 2048; small tiles 4096 x 4096
- * 38 / 45, 4096 x 14336 120 / 108, 14336 x 4096 at 128 tokens 37 / 80.
+ * 38 / 45, 4096 x 14336 120 / 108, 14336 x 4096 at 128 tokens 37 / 80. IQ4_XS: large 68 / 99, 133 / 139, 305 / 270; small
+ * 39 / 45, 123 / 111, 38 / 79. Q4_0: large 62 / 81, 122 / 120, 272 / 241; small 30 / 41, 93 / 93, 30 / 67.
  * Without a workspace there is no decode + dense route to prefer. */
 FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, bool have_workspace) {
     if (!gemm_kq_wave4_covers(type) || n_cols % 256 != 0 || ldx >= (1 << 22)) return kFusedNone;
     const long long large_tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
-    const bool light = type == T_Q4_K || type == T_Q5_K; /* less to decode per weight */
-    if (large_tiles >= 200)
-        return (n_tok <= (light || type == T_IQ4_NL ? 1536 : 512) || !have_workspace) ? kFusedLarge : kFusedNone;
-    return (light || n_tok <= 256 || !have_workspace) ? kFusedSmall : kFusedNone;
+    /* token counts up to which the large-tile and the small-tile kernel measured faster than decode + dense */
+    int large_max = 512, small_max = 256;
+    switch (type) {
+    case T_Q4_K: case T_Q5_K: large_max = 1536; small_max = INT_MAX; break;
+    case T_Q4_0: large_max = 1024; small_max = INT_MAX; break;
+    case T_IQ4_NL: large_max = 1536; break;
+    case T_IQ4_XS: large_max = 1024; break;
+    default: break; /* Q6_K, Q8_0 */
+    }
+    if (large_tiles >= 200) return (n_tok <= large_max || !have_workspace) ? kFusedLarge : kFusedNone;
+    return (n_tok <= small_max || !have_workspace) ? kFusedSmall : kFusedNone;
 }
 
 hipError_t launch_fused_tile(FusedTile tile, uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows,
@@ -335,6 +344,8 @@ hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_
     case T_Q6_K: return launch_wave4<FQ6K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q8_0: return launch_wave4<FQ8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_IQ4_NL: return launch_wave4<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_IQ4_XS: return launch_wave4<FIQ4XS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q4_0: return launch_wave4<FQ4_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }

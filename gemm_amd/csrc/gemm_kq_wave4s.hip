@@ -1,5 +1,5 @@
 /*
- * gemm_kq_wave4s.hip - the fused Q4_K / Q5_K / Q6_K / Q8_0 / IQ4_NL x bf16 prefill GEMM in 128-token x 64-row tiles, for the
+ * gemm_kq_wave4s.hip - the fused Q4_K / Q5_K / Q6_K / Q8_0 / IQ4_NL / IQ4_XS / Q4_0 x bf16 prefill GEMM in 128-token x 64-row tiles, for the
  * shapes whose 256-token x 128-row tiles (gemm_kq_wave4.hip) would leave most of the chip idle: 4096-row projections
  * at 512 tokens (64 large tiles, 256 small ones), 14336 rows at 129..256 tokens.
  *
@@ -123,8 +123,8 @@ template <class F, int U, int T> QLIN_INL void slot(Ctx<F> &c) {
     }
     constexpr int n_pieces = F::kTilePieces + (U == 3 ? F::kPrepPieces : 0);
     constexpr int p0 = (T * n_pieces + 7) / 8, p1 = ((T + 1) * n_pieces + 7) / 8; /* pieces p with p * 8 / n_pieces == T */
-    static_assert(p1 - p0 <= 11, "at most eleven pieces per slot");
-    pieces<F, U, p0, p1>(c, std::make_integer_sequence<int, 11>{});
+    static_assert(p1 - p0 <= 12, "at most twelve pieces per slot");
+    pieces<F, U, p0, p1>(c, std::make_integer_sequence<int, 12>{});
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -275,6 +275,8 @@ hipError_t launch_gemm_kq_bf16_wave4s(uint32_t type, const void *W, const uint16
     case T_Q6_K: return launch_wave4s<FQ6K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q8_0: return launch_wave4s<FQ8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_IQ4_NL: return launch_wave4s<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_IQ4_XS: return launch_wave4s<FIQ4XS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q4_0: return launch_wave4s<FQ4_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }

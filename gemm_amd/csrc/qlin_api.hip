@@ -1075,8 +1075,8 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     }
     /* Q4_K, Q5_K, Q6_K, Q8_0 and IQ4_NL: decoded into the matrix operand inside the product, no workspace, in large or small
      * tiles by the shape - except where decoding once into the caller's workspace measured faster */
-    /* (up to four tokens of IQ4_NL, which has no few-token kernel, are faster one by one through the matvec below) */
-    const bool matvec_first = type == T_IQ4_NL && n_tok <= kMatvecTokens && ws_ok;
+    /* (up to four tokens of the formats without a few-token kernel are faster one by one through the matvec below) */
+    const bool matvec_first = (type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0) && n_tok <= kMatvecTokens && ws_ok;
     if (const FusedTile tile = matvec_first ? kFusedNone : choose_fused_tile(type, n_rows, n_cols, n_tok, ldx, ws_ok);
         tile != kFusedNone) {
         HIP_TRY(launch_fused_tile(tile, type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));

@@ -26,7 +26,7 @@ int qlin_probe_hbm_read(const void *buf, size_t n_bytes, void *stream);
 
 /* One tile kernel of the fused prefill GEMM by name, whatever the shape-based choice of qlin_gemm_bf16_any_dev would be:
  * tile 0 = 256 tokens x 128 rows, 1 = 128 tokens x 64 rows. Arguments and result as qlin_gemm_bf16_any_dev without a
- * workspace; Q4_K, Q5_K, Q6_K, Q8_0, IQ4_NL; n_cols % 256 == 0. For timing one against the other and for the parity tests of
+ * workspace; Q4_K, Q5_K, Q6_K, Q8_0, IQ4_NL, IQ4_XS, Q4_0; n_cols % 256 == 0. For timing one against the other and for the parity tests of
  * each on small shapes. */
 /* which of them qlin_gemm_bf16_any_dev picks for a shape above the few-token kernels' token counts: 1 = the 256 x 128
  * tile kernel, 2 = the 128 x 64 one, 0 = neither (decode to bf16 + dense product) */

@@ -41,7 +41,8 @@ def dense_kernel(request):
     qlinear.check(qlinear.load().qlin_set_dense_gemm_own(0))
 
 
-FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ4_NL]  # decoded inside the tile kernels
+FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ4_NL, synth.GGML_IQ4_XS,
+         synth.GGML_Q4_0]  # decoded inside the tile kernels
 KQ = {synth.GGML_Q6_K, synth.GGML_Q5_K, synth.GGML_Q3_K, synth.GGML_Q2_K, synth.GGML_Q8_0}
 
 
@@ -163,8 +164,8 @@ def test_fused_tile_kernel_full_size_config(oracle, tid):
 
 
 @pytest.mark.parametrize("tid,n_tok,n_rows,n_cols", [
-    (synth.GGML_IQ4_XS, 70, 130, 512), (synth.GGML_Q8_0, 33, 257, 96), (synth.GGML_BF16, 40, 64, 1024),
-    (synth.GGML_Q4_0, 9000, 16, 1024),  # more tokens than one band of the workspace holds as fp32
+    (synth.GGML_IQ3_S, 70, 130, 512), (synth.GGML_Q8_0, 33, 257, 96), (synth.GGML_BF16, 40, 64, 1024),
+    (synth.GGML_Q4_1, 9000, 16, 1024),  # more tokens than one band of the workspace holds as fp32
 ])
 def test_neither_dense_kernel_takes_the_shape(oracle, tid, n_tok, n_rows, n_cols):
     """with both dense products switched off the call still answers: the vector-ALU kernel on the exact weights"""
@@ -310,7 +311,7 @@ def test_argument_checks():
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 300, 4, 304, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ragged K
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 260, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ldx % 8
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 100, ws.ptr, need, None) == qlinear.ERR_ARG      # ldy < rows
-    NL = synth.GGML_IQ4_XS  # a format that always takes the decode + dense route above four tokens
+    NL = synth.GGML_Q3_K  # a format that always takes the decode + dense route above 24 tokens
     assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
     assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
     assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
