@@ -74,3 +74,59 @@ def test_decode_style_sequence_in_a_graph(oracle):
         qlinear.sync()
     assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
     assert hip.hipStreamDestroy(stream) == 0
+
+
+def test_prefill_sequence_in_a_graph(oracle):
+    """The fused prefill GEMMs take no workspace and only enqueue: a chunk's projections (large tiles, small tiles and
+    the few-token kernel, three formats) are captured with a NULL workspace and replayed bit-identically."""
+    hip = C.CDLL("libamdhip64.so")
+    Q5K, NL = synth.GGML_Q5_K, synth.GGML_IQ4_NL
+    K, n_tok = 512, 300
+    shapes = [(Q4K, 12900, n_tok), (Q5K, 640, n_tok), (NL, 300, n_tok), (Q6K, 200, 20)]  # large tiles, small, small, few tokens
+    host = [synth.make_weights(t, r, K, seed=20 + i) for i, (t, r, _) in enumerate(shapes)]
+    W = [qlinear.DevBuf.from_numpy(a) for a in host]
+    Xb = synth.to_bf16_bits(synth.make_activation(K, seed=30, tokens=n_tok))
+    dX = qlinear.DevBuf.from_numpy(Xb)
+    Y = [qlinear.DevBuf(m * r * 4) for (_, r, m) in shapes]
+    lib = qlinear.load()
+
+    def enqueue(stream):
+        for (t, r, m), w, y in zip(shapes, W, Y):
+            assert lib.qlin_gemm_bf16_any_dev(t, w.ptr, dX.ptr, y.ptr, r, K, m, K, r, None, 0, stream) == 0, lib.qlin_last_error()
+
+    def clear():
+        for (_, r, m), y in zip(shapes, Y):
+            z = np.full(m * r, -3.0, np.float32)
+            assert lib.qlin_dev_upload(y.ptr, z.ctypes.data, z.nbytes) == 0
+
+    enqueue(None)  # eager run: the reference for the replays, itself checked against the oracle
+    qlinear.sync()
+    want = [y.to_numpy(np.float32, (m, r)) for (_, r, m), y in zip(shapes, Y)]
+    Xf = synth.bf16_bits_to_f32(Xb).astype(np.float64)
+    for (t, r, m), h, got in zip(shapes, host, want):
+        dec = oracle.dequant_matrix(t, h, K)
+        if m > 24:
+            dec = synth.bf16_bits_to_f32(synth.to_bf16_bits(dec))
+        assert rel_l2(got, Xf[:m] @ dec.astype(np.float64).T) <= 2e-5, (t, r, m)
+
+    stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(stream)) == 0
+    assert hip.hipStreamBeginCapture(stream, 0) == 0  # hipStreamCaptureModeGlobal
+    enqueue(stream)
+    assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+    n_nodes = C.c_size_t(0)
+    assert hip.hipGraphGetNodes(graph, None, C.byref(n_nodes)) == 0
+    assert n_nodes.value == len(shapes)  # one kernel per product, nothing else
+    for replay in range(3):
+        clear()
+        assert hip.hipGraphLaunch(gexec, stream) == 0
+        assert hip.hipStreamSynchronize(stream) == 0
+        for (_, r, m), y, w_ in zip(shapes, Y, want):
+            assert np.array_equal(y.to_numpy(np.float32, (m, r)), w_), replay
+        qlinear.gemm_bf16_any_dev(Q5K, W[1], dX, Y[1], 640, K, 100, K, 640, None)  # eager work between replays
+        qlinear.sync()
+    assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
+    assert hip.hipStreamDestroy(stream) == 0
+    for b in W + Y + [dX]:
+        b.free()
