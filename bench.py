@@ -695,7 +695,9 @@ def main():
         tf = gemm["M=512"]["TFLOP/s"]
         anyfmt = {}
         for tname, tid, M in (("q6_K", synth.GGML_Q6_K, 512), ("q5_K", synth.GGML_Q5_K, 512), ("q8_0", synth.GGML_Q8_0, 512),
-                              ("iq4_nl", synth.GGML_IQ4_NL, 512), ("bf16", synth.GGML_BF16, 512), ("q4_K", Q4K, 1024),
+                              ("iq4_nl", synth.GGML_IQ4_NL, 512), ("iq4_xs", synth.GGML_IQ4_XS, 512), ("q4_0", synth.GGML_Q4_0, 512),
+                              ("q3_K", synth.GGML_Q3_K, 512), ("q2_K", synth.GGML_Q2_K, 512),
+                              ("bf16", synth.GGML_BF16, 512), ("q4_K", Q4K, 1024),
                               ("q5_K", synth.GGML_Q5_K, 1024), ("q4_K", Q4K, 2048), ("q6_K", synth.GGML_Q6_K, 2048)):
             m = time_gemm_any(tid, M, 14336, 4096, max(5, args.steps // 40), 2)
             anyfmt["%s_M=%d" % (tname, M)] = {

@@ -375,6 +375,108 @@ struct FIQ4XS {
     }
 };
 
+/* ---- Q2_K and Q3_K share their element order: half h (128 elements) of a super-block, shift j (0..3), 16-element group
+ * sub, element l: bits 2 j of code byte 32 h + 16 sub + l, scale 8 h + 2 j + sub (common/ggml_dequant.h:1505-1580). Tile c
+ * is half c >> 1, shifts 2 (c & 1) and 2 (c & 1) + 1; lane half kg takes sub = kg, so its 16 code bytes per half serve
+ * both tiles of the half, and its two scales of a tile are bytes kg and kg + 2 of dword 2 h + (c & 1) of the sixteen.
+ * k-step s: shift 2 (c & 1) + (s >> 1), the lane's bytes 8 (s & 1) .. + 7. The codes (0..3, with Q3_K's third bit 0..7) go
+ * through the fp8 reading. */
+template <int TC, int DW> struct K23 { static constexpr int half = TC >> 1, j = 2 * (TC & 1) + (DW >> 2), sdw = 2 * half + (TC & 1); };
+
+/* Q2_K: 84-byte blocks = 16 scale bytes (low nibble scale, high nibble min) | 64 code bytes | d | dmin; (d sc) q - dmin m.
+ * A row's image is the first five 16-byte pieces and bytes 68..83 as the sixth (d and dmin in its last dword; a fetch of
+ * bytes 80..95 would leave the row, and the buffer at its last row). */
+struct Q2Scales { float d, dmin; };
+struct FQ2K {
+    static constexpr int kBlockBytes = 84, kPieces = 6, kReq = 3, kLaneVec = 4, kPrepPieces = 1, kTilePieces = 44;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    typedef Q2Scales Scales;
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    static QLIN_INL uint32_t piece_src(int part) { return part < 5 ? 16u * part : 68u; }
+    /* vector 0: the scales; 1, 2: the lane's code bytes of half 0, 1; 3: the piece with d and dmin */
+    static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, 0} : j < 3 ? VecAt{16 + 32 * (j - 1), 16} : VecAt{80, 0}; }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
+    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        c.sc.d = half_bits_fast(raw[3].w & 0xFFFFu) * c.unit;
+        c.sc.dmin = half_bits_fast(raw[3].w >> 16);
+    }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        Temps &t = c.t;
+        if constexpr (P < 4) {
+            const uint32_t word = raw[0][K23<TC, 0>::sdw], at = 8u * (uint32_t)c.kg;
+            if constexpr (P == 0) { t.s_a = (float)__builtin_amdgcn_ubfe(word, at, 4); t.s_b = (float)__builtin_amdgcn_ubfe(word, at + 16, 4); }
+            else if constexpr (P == 1) { t.m_a = (float)__builtin_amdgcn_ubfe(word, at + 4, 4); t.m_b = (float)__builtin_amdgcn_ubfe(word, at + 20, 4); }
+            else if constexpr (P == 2) { t.dl_a = c.sc.d * t.s_a; t.dl_b = c.sc.d * t.s_b; }
+            else { t.nml_a = -(c.sc.dmin * t.m_a); t.nml_b = -(c.sc.dmin * t.m_b); }
+        } else {
+            constexpr int dw = (P - 4) / 5, ph = (P - 4) % 5;
+            typedef K23<TC, dw> G;
+            const float dl = dw < 4 ? t.dl_a : t.dl_b, nml = dw < 4 ? t.nml_a : t.nml_b;
+            if constexpr (ph == 0) t.cm = (raw[1 + G::half][dw & 3] >> (2 * G::j)) & 0x03030303u;
+            else if constexpr (ph == 1) { t.cp0 = fp8_pair_lo(t.cm); t.cp1 = fp8_pair_hi(t.cm); }
+            else if constexpr (ph == 2) { t.w0 = fmaf(t.cp0.x, dl, nml); t.w1 = fmaf(t.cp0.y, dl, nml); }
+            else if constexpr (ph == 3) { t.w2 = fmaf(t.cp1.x, dl, nml); t.w3 = fmaf(t.cp1.y, dl, nml); }
+            else if constexpr ((dw & 1) == 0) { c.wa[WB][dw >> 1].x = pack_bf16(t.w0, t.w1); c.wa[WB][dw >> 1].y = pack_bf16(t.w2, t.w3); }
+            else { c.wa[WB][dw >> 1].z = pack_bf16(t.w0, t.w1); c.wa[WB][dw >> 1].w = pack_bf16(t.w2, t.w3); }
+        }
+    }
+};
+
+/* Q3_K: 110-byte blocks = 32 bytes of third bits (bit 4 h + j of byte 16 sub + l) | 64 code bytes | 12 bytes of sixteen
+ * 6-bit scales | d; (d (sc - 32)) (q - 4) with q the three bits. A row's image is the first six pieces and bytes 94..109
+ * as the seventh (ending with the block, as Q2_K's last), 112 bytes: a stride that spreads 16 rows over all banks. The
+ * packed scales start two bytes into that piece; once per super-block they are cut out and spread to sixteen bytes. */
+struct Q3Scales { float d, dm4; uint32_t a0, a1, hi, sc[4]; }; /* d with the fp8 reading's factor, dm4 = -4 d without */
+struct FQ3K {
+    static constexpr int kBlockBytes = 110, kPieces = 7, kReq = 4, kLaneVec = 4, kPrepPieces = 4, kTilePieces = 52;
+    static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
+    static constexpr bool kSwizzle = false;
+    typedef Q3Scales Scales;
+    static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
+    static QLIN_INL uint32_t piece_src(int part) { return part < 6 ? 16u * part : 94u; }
+    /* vector 0: the lane's third-bit bytes; 1, 2: its code bytes of half 0, 1; 3: the piece with scales and d */
+    static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, 16} : j < 3 ? VecAt{32 + 32 * (j - 1), 16} : VecAt{96, 0}; }
+    template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
+    template <int P, class C> static QLIN_INL void prep(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        const u32x4 &v = raw[3]; /* block bytes 94..109: scale bytes 0..11 at 2..13, d at 14 */
+        if constexpr (P == 0) { c.sc.a0 = __builtin_amdgcn_alignbyte(v.y, v.x, 2); c.sc.a1 = __builtin_amdgcn_alignbyte(v.z, v.y, 2); }
+        else if constexpr (P == 1) {
+            c.sc.hi = __builtin_amdgcn_alignbyte(v.w, v.z, 2);
+            c.sc.dm4 = -4.0f * half_bits_fast(v.w >> 16);
+            c.sc.d = c.sc.dm4 * (-0.25f * c.unit);
+        }
+        else if constexpr (P == 2) {
+            c.sc.sc[0] = (c.sc.a0 & 0x0F0F0F0Fu) | ((c.sc.hi & 0x03030303u) << 4);
+            c.sc.sc[1] = (c.sc.a1 & 0x0F0F0F0Fu) | (((c.sc.hi >> 2) & 0x03030303u) << 4);
+        } else {
+            c.sc.sc[2] = ((c.sc.a0 >> 4) & 0x0F0F0F0Fu) | (((c.sc.hi >> 4) & 0x03030303u) << 4);
+            c.sc.sc[3] = ((c.sc.a1 >> 4) & 0x0F0F0F0Fu) | (((c.sc.hi >> 6) & 0x03030303u) << 4);
+        }
+    }
+    template <int TC, int WB, int P, class C> static QLIN_INL void tile_piece(C &c, const u32x4 (&raw)[kLaneVec + kExtraVec]) {
+        Temps &t = c.t;
+        if constexpr (P < 4) {
+            const uint32_t word = c.sc.sc[K23<TC, 0>::sdw], at = 8u * (uint32_t)c.kg;
+            if constexpr (P == 0) t.s_a = (float)((int)__builtin_amdgcn_ubfe(word, at, 8) - 32);
+            else if constexpr (P == 1) t.s_b = (float)((int)__builtin_amdgcn_ubfe(word, at + 16, 8) - 32);
+            else if constexpr (P == 2) { t.dl_a = c.sc.d * t.s_a; t.dl_b = c.sc.d * t.s_b; }
+            else { t.nml_a = c.sc.dm4 * t.s_a; t.nml_b = c.sc.dm4 * t.s_b; }
+        } else {
+            constexpr int dw = (P - 4) / 6, ph = (P - 4) % 6;
+            typedef K23<TC, dw> G;
+            const float dl = dw < 4 ? t.dl_a : t.dl_b, nml = dw < 4 ? t.nml_a : t.nml_b;
+            if constexpr (ph == 0) t.cm = (raw[1 + G::half][dw & 3] >> (2 * G::j)) & 0x03030303u;
+            else if constexpr (ph == 1) { t.hb = (raw[0][dw & 3] >> (4 * G::half + G::j)) & 0x01010101u; t.cm |= t.hb << 2; }
+            else if constexpr (ph == 2) { t.cp0 = fp8_pair_lo(t.cm); t.cp1 = fp8_pair_hi(t.cm); }
+            else if constexpr (ph == 3) { t.w0 = fmaf(t.cp0.x, dl, nml); t.w1 = fmaf(t.cp0.y, dl, nml); }
+            else if constexpr (ph == 4) { t.w2 = fmaf(t.cp1.x, dl, nml); t.w3 = fmaf(t.cp1.y, dl, nml); }
+            else if constexpr ((dw & 1) == 0) { c.wa[WB][dw >> 1].x = pack_bf16(t.w0, t.w1); c.wa[WB][dw >> 1].y = pack_bf16(t.w2, t.w3); }
+            else { c.wa[WB][dw >> 1].z = pack_bf16(t.w0, t.w1); c.wa[WB][dw >> 1].w = pack_bf16(t.w2, t.w3); }
+        }
+    }
+};
+
 /* one load-to-LDS request: lane l's 16 bytes from voff + soff of the buffer land at lds + 16 l */
 QLIN_INL void dma16(__amdgpu_buffer_rsrc_t rsrc, uint8_t *lds, uint32_t voff, uint32_t soff) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void *)lds, 16, voff, soff, 0, 0);

@@ -297,7 +297,7 @@ hipError_t launch_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, 
 
 bool gemm_kq_wave4_covers(uint32_t type) {
     return type == T_Q4_K || type == T_Q5_K || type == T_Q6_K || type == T_Q8_0 || type == T_IQ4_NL || type == T_IQ4_XS ||
-           type == T_Q4_0;
+           type == T_Q4_0 || type == T_Q2_K || type == T_Q3_K;
 }
 
 /* Which kernel takes a prefill GEMM of a format with a fused kernel, beyond the token counts of the few-token kernels.
@@ -311,7 +311,9 @@ bool gemm_kq_wave4_covers(uint32_t type) {
  * 33 / 73, 36 / 72; at 256: 46 / 77, 55 / 84, 63 / 81), for Q6_K, Q8_0 and IQ4_NL up to 256 tokens. IQ4_NL (a table
  * lookup per weight): large tiles 62 / 95 at 512 tokens, 123 / 132 at 1024, 279 / 254 at 2048; small tiles 4096 x 4096
  * 38 / 45, 4096 x 14336 120 / 108, 14336 x 4096 at 128 tokens 37 / 80. IQ4_XS: large 68 / 99, 133 / 139, 305 / 270; small
- * 39 / 45, 123 / 111, 38 / 79. Q4_0: large 62 / 81, 122 / 120, 272 / 241; small 30 / 41, 93 / 93, 30 / 67.
+ * 39 / 45, 123 / 111, 38 / 79. Q4_0: large 62 / 81, 122 / 120, 272 / 241; small 30 / 41, 93 / 93, 30 / 67. Q2_K: large
+ * 59 / 82, 117 / 120, 251 / 222; small 29 / 42, 89 / 95, 28 / 71. Q3_K: large 62 / 91, 127 / 128, 261 / 253; small 32 / 44,
+ * 99 / 103, 31 / 76.
  * Without a workspace there is no decode + dense route to prefer. */
 FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, bool have_workspace) {
     if (!gemm_kq_wave4_covers(type) || n_cols % 256 != 0 || ldx >= (1 << 22)) return kFusedNone;
@@ -320,7 +322,7 @@ FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, in
     int large_max = 512, small_max = 256;
     switch (type) {
     case T_Q4_K: case T_Q5_K: large_max = 1536; small_max = INT_MAX; break;
-    case T_Q4_0: large_max = 1024; small_max = INT_MAX; break;
+    case T_Q4_0: case T_Q2_K: case T_Q3_K: large_max = 1024; small_max = INT_MAX; break;
     case T_IQ4_NL: large_max = 1536; break;
     case T_IQ4_XS: large_max = 1024; break;
     default: break; /* Q6_K, Q8_0 */
@@ -346,6 +348,8 @@ hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_
     case T_IQ4_NL: return launch_wave4<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_IQ4_XS: return launch_wave4<FIQ4XS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q4_0: return launch_wave4<FQ4_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q2_K: return launch_wave4<FQ2K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q3_K: return launch_wave4<FQ3K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }

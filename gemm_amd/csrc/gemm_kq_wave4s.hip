@@ -277,6 +277,8 @@ hipError_t launch_gemm_kq_bf16_wave4s(uint32_t type, const void *W, const uint16
     case T_IQ4_NL: return launch_wave4s<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_IQ4_XS: return launch_wave4s<FIQ4XS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     case T_Q4_0: return launch_wave4s<FQ4_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q2_K: return launch_wave4s<FQ2K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q3_K: return launch_wave4s<FQ3K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -229,12 +229,12 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
 /* The same contraction for EVERY weight format (block-quantized and dense F16/BF16/F32), the role of
  * tf_gemm_f16_mt_tokenmajor for the formats it re-decodes once per token (common/transformer.h:4535-4572):
  * W is decoded once to bf16 (nearest even) into `workspace` and multiplied by the dense matrix-core GEMM of
- * the vendor library. Q4_K, Q5_K, Q6_K, Q8_0, IQ4_NL, IQ4_XS and Q4_0 tensors (n_cols % 256 == 0) are instead decoded inside the product
- * by this library's tile kernels, with the same single rounding to bf16, and leave the workspace alone (it may be NULL
+ * the vendor library. Q2_K, Q3_K, Q4_K, Q5_K, Q6_K, Q8_0, IQ4_NL, IQ4_XS and Q4_0 tensors (n_cols % 256 == 0) are instead
+ * decoded inside the product by this library's tile kernels, with the same single rounding to bf16, and leave the workspace alone (it may be NULL
  * for them): 256-token x 128-row tiles where 200 or more of them fill the chip (12800 rows at 257..512 tokens, 6400 at
  * 513..1024, ...), 128-token x 64-row tiles for smaller shapes (4096-row projections at 512 tokens, any row count at
  * 33..256 tokens). Given a workspace, the decode + dense route still takes the shapes where decoding once measured
- * faster: large-tile shapes above 1536 tokens (Q4_K, Q5_K, IQ4_NL), 1024 (IQ4_XS, Q4_0) or 512 (Q6_K, Q8_0), small-tile
+ * faster: large-tile shapes above 1536 tokens (Q4_K, Q5_K, IQ4_NL), 1024 (Q2_K, Q3_K, IQ4_XS, Q4_0) or 512 (Q6_K, Q8_0), small-tile
  * shapes of Q6_K, Q8_0, IQ4_NL and IQ4_XS above 256 tokens. Q4_K up to 32 tokens: the few-token kernel of qlin_gemm_bf16_dev.
  * Up to 24 tokens of a Q6_K, Q5_K, Q3_K, Q2_K or
  * Q8_0 tensor (n_cols % 256 == 0, the tensor's bytes a multiple of 16) also run in one fused kernel with

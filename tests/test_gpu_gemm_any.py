@@ -42,7 +42,7 @@ def dense_kernel(request):
 
 
 FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ4_NL, synth.GGML_IQ4_XS,
-         synth.GGML_Q4_0]  # decoded inside the tile kernels
+         synth.GGML_Q4_0, synth.GGML_Q2_K, synth.GGML_Q3_K]  # decoded inside the tile kernels
 KQ = {synth.GGML_Q6_K, synth.GGML_Q5_K, synth.GGML_Q3_K, synth.GGML_Q2_K, synth.GGML_Q8_0}
 
 
@@ -311,7 +311,7 @@ def test_argument_checks():
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 300, 4, 304, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ragged K
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 260, 128, ws.ptr, need, None) == qlinear.ERR_ARG      # ldx % 8
     assert f(Q6K, d.ptr, d.ptr, d.ptr, 128, 256, 4, 256, 100, ws.ptr, need, None) == qlinear.ERR_ARG      # ldy < rows
-    NL = synth.GGML_Q3_K  # a format that always takes the decode + dense route above 24 tokens
+    NL = synth.GGML_Q5_1  # a format that always takes the decode + dense route above 24 tokens
     assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, ws.ptr, need - 1, None) == qlinear.ERR_ARG  # small workspace
     assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, None, 0, None) == qlinear.ERR_ARG           # no workspace
     assert f(NL, d.ptr, d.ptr, d.ptr, 128, 256, 32, 256, 128, C.c_void_p(ws.ptr + 16), need, None) == qlinear.ERR_ARG
