@@ -220,7 +220,7 @@ def time_decode_step_linear(n_layers=32, steps=5, mix=False):
 def time_prefill_chunk_linear(n_tok=512, n_layers=32, steps=3):
     """The block-quantized linear operators of one 512-token prefill chunk of the same Llama-3-8B-shaped
     model: seven Q4_K x bf16 GEMMs per layer (Q, K, V, attention output, gate, up, down) through
-    qlin_gemm_bf16_any_dev (fused tile kernel for gate and up, decode + library GEMM for the 4096- and
+    qlin_gemm_bf16_any_dev (large-tile kernel for gate and up, small-tile kernel for the 4096- and
     1024-row tensors), each layer with its own weights; inputs are bf16 buffers of the right shapes (attention, norms, the SiLU product and
     the fp32 -> bf16 conversions between the operators are not run). -> dict"""
     K, FF, KV = 4096, 14336, 1024
@@ -244,6 +244,26 @@ def time_prefill_chunk_linear(n_tok=512, n_layers=32, steps=3):
         step()
     ms = qlinear.timer_end() / steps
     flops = 2.0 * n_tok * n_layers * sum(r * c for r, c in shapes)
+    # Q, K and V of a layer in one launch (qlin_gemm_bf16_multi_dev), gate and up in another, the other two as before
+    outs = [qlinear.DevBuf(n_tok * r * 4) for r, _ in shapes[:3]]
+    gu = [out, qlinear.DevBuf(n_tok * FF * 4)]
+
+    def step_qkv():
+        for W in layers:
+            qlinear.gemm_bf16_multi_dev(Q4K, W[:3], xk, outs, [r for r, _ in shapes[:3]], K, n_tok, K,
+                                        [r for r, _ in shapes[:3]], ws)
+            qlinear.gemm_bf16_any_dev(Q4K, W[3], xk, out, K, K, n_tok, K, K, ws)
+            qlinear.gemm_bf16_multi_dev(Q4K, W[4:6], xk, gu, [FF, FF], K, n_tok, K, [FF, FF], ws)
+            qlinear.gemm_bf16_any_dev(Q4K, W[6], xff, out, K, FF, n_tok, FF, K, ws)
+
+    step_qkv()
+    qlinear.sync()
+    qlinear.timer_begin()
+    for _ in range(steps):
+        step_qkv()
+    ms_qkv = qlinear.timer_end() / steps
+    for d in outs + gu[1:]:
+        d.free()
     # the same chunk for an engine that spends HBM on bf16 copies of its weights (decoded once at load):
     # every GEMM is then the dense library GEMM on the cached copy
     BF16 = synth.GGML_BF16
@@ -275,6 +295,8 @@ def time_prefill_chunk_linear(n_tok=512, n_layers=32, steps=3):
     return {"ms_per_chunk": round(ms, 3), "tokens": n_tok, "tokens_per_s": round(n_tok / (ms * 1e-3)),
             "launches": 7 * n_layers, "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 1),
             "mfma_frac": round(flops / (ms * 1e-3) / 1e12 / BF16_PEAK_TFLOPS, 4),
+            "with_q_k_v_in_one_launch_and_gate_up_in_one": {"ms_per_chunk": round(ms_qkv, 3), "tokens_per_s": round(n_tok / (ms_qkv * 1e-3)),
+                                         "launches": 4 * n_layers, "TFLOP/s": round(flops / (ms_qkv * 1e-3) / 1e12, 1)},
             "with_cached_bf16_copies_of_the_weights": {
                 "ms_per_chunk": round(ms_cached, 3), "tokens_per_s": round(n_tok / (ms_cached * 1e-3)),
                 "TFLOP/s": round(flops / (ms_cached * 1e-3) / 1e12, 1),
@@ -511,6 +533,9 @@ def probe(args):
     elif args.probe == "gemm_small_q4_K":  # Q4_K 4096 x 4096 at 512 tokens: the 128-token x 64-row tile kernel
         ms = time_gemm_any(Q4K, 512, 4096, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_small_q4_K", "ms_per_step": ms}))
+    elif args.probe == "gemm_small_q4_K_m128":  # Q4_K 14336 x 4096 at 128 tokens: the same kernel, one workgroup per compute unit
+        ms = time_gemm_any(Q4K, 128, 14336, 4096, max(3, args.steps // 20), 2)
+        print(json.dumps({"probe": "gemm_small_q4_K_m128", "ms_per_step": ms}))
     elif args.probe == "gemm_any_iq4_nl":  # IQ4_NL, 512 tokens: decoded inside the large-tile kernel
         ms = time_gemm_any(synth.GGML_IQ4_NL, 512, 14336, 4096, max(3, args.steps // 20), 2)
         print(json.dumps({"probe": "gemm_any_iq4_nl", "ms_per_step": ms}))
@@ -652,7 +677,7 @@ def main():
     ap.add_argument("--prows", type=int, default=4096)
     ap.add_argument("--pcols", type=int, default=14336)
     ap.add_argument("--ptok", type=int, default=64, help="--probe moe: tokens in the batch")
-    ap.add_argument("--probe", choices=["gemv_any", "copy", "tiny", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_small_q4_K", "gemm_any_iq4_nl", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
+    ap.add_argument("--probe", choices=["gemv_any", "copy", "tiny", "gemv", "gemv_q8_0", "gemv_q6_K", "gemv_q4_0", "gemv_silu", "dequant", "gemm", "gemm_any_q6_K", "gemm_any_q8_0", "gemm_small_q4_K", "gemm_small_q4_K_m128", "gemm_any_iq4_nl", "gemm_f32_any_q4_K", "gemm_fewtok", "moe", "decode_step"], help="device work only, for rocprofv3 runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus %d is not supported (the path shards by "

@@ -171,8 +171,7 @@ template <class F, int... J> QLIN_INL void load_cur_extra(Ctx<F> &c, std::intege
 
 template <class F>
 __global__ void __launch_bounds__(256)
-gemm_kq_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__restrict__ X, float *__restrict__ Y,
-                          int n_rows, int n_sb, int n_tok, int ldx, int ldy, int m_tiles) {
+gemm_kq_bf16_wave4_kernel(TileSet set, const uint16_t *__restrict__ X, int n_sb, int n_tok, int ldx, int m_tiles) {
     /* raw blocks of one super-block of each wave's 32 weight rows (32 x kPieces pieces, rounded up to whole requests) */
     __shared__ __attribute__((aligned(1024))) uint8_t w4_raw[4 * F::kReq * 1024];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -181,8 +180,12 @@ gemm_kq_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__restr
      * that share one weight tile get ids 8 apart and meet in the same L2 */
     const int xcd = blockIdx.x & 7, slot_id = blockIdx.x >> 3;
     const int tile_m = slot_id % m_tiles;
-    const int tile_n = (slot_id / m_tiles) * 8 + xcd;
-    if (tile_n * kBN >= n_rows) return;
+    const int tile_all = (slot_id / m_tiles) * 8 + xcd;
+    if (tile_all >= set.end[2]) return;
+    const TileOf t = tile_of(set, tile_all);
+    const uint8_t *W = t.W;
+    float *Y = t.Y;
+    const int n_rows = t.n_rows, ldy = t.ldy, tile_n = t.tile;
 
     Ctx<F> c;
     c.raw = w4_raw;
@@ -282,16 +285,22 @@ gemm_kq_bf16_wave4_kernel(const uint8_t *__restrict__ W, const uint16_t *__restr
 
 namespace {
 template <class F>
-hipError_t launch_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok, int ldx, int ldy,
-                        hipStream_t stream) {
+hipError_t launch_wave4(int n_mat, const void *const *W, const uint16_t *X, float *const *Y, const int *n_rows, int n_cols,
+                        int n_tok, int ldx, const int *ldy, hipStream_t stream) {
     const int n_sb = n_cols / 256;
     const int m_tiles = (n_tok + kBM - 1) / kBM;
-    const int n_tiles = (n_rows + kBN - 1) / kBN;
+    TileSet set;
+    const int n_tiles = fill_tile_set(set, n_mat, W, Y, n_rows, ldy, kBN);
     /* ids are dealt to 8 XCDs; pad the n-tile count to a multiple of 8 (surplus groups exit) */
     const int n_tiles_pad = (n_tiles + 7) / 8 * 8;
-    hipLaunchKernelGGL(gemm_kq_bf16_wave4_kernel<F>, dim3(n_tiles_pad * m_tiles), dim3(256), 0, stream,
-                       (const uint8_t *)W, X, Y, n_rows, n_sb, n_tok, ldx, ldy, m_tiles);
+    hipLaunchKernelGGL(gemm_kq_bf16_wave4_kernel<F>, dim3(n_tiles_pad * m_tiles), dim3(256), 0, stream, set, X, n_sb,
+                       n_tok, ldx, m_tiles);
     return hipGetLastError();
+}
+template <class F>
+hipError_t launch_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok, int ldx, int ldy,
+                        hipStream_t stream) {
+    return launch_wave4<F>(1, &W, X, &Y, &n_rows, n_cols, n_tok, ldx, &ldy, stream);
 }
 }  // namespace
 
@@ -304,28 +313,30 @@ bool gemm_kq_wave4_covers(uint32_t type) {
  * 200 or more 256-token x 128-row tiles fill the chip: the large-tile kernel - up to a token count, because it decodes
  * the weights again every 256 tokens, which costs more the more there is to decode, while decoding once into a workspace
  * costs 27 - 38 us whatever the token count (14336 x 4096, large tiles against decode + the vendor library's product, us:
- * at 512 tokens Q4_K 61 / 86, Q5_K 62 / 92, Q6_K 66 / 84, Q8_0 71 / 83; at 1024 118 / 125, 121 / 135, 131 / 126,
- * 139 / 121; at 1536 181 / 190, 185 / 195, 206 / 184, 216 / 177; at 2048 267 / 244, 262 / 260, 273 / 240, 311 / 224).
- * Fewer large tiles: the small-tile kernel (4096 x 4096 at 512 tokens, small tiles / decode + library: Q4_K 29 / 45,
- * Q6_K 34 / 40, Q8_0 36 / 39; 4096 x 14336: 89 / 100, 104 / 100, 110 / 101; 14336 x 4096 at 128 tokens: 28 / 74,
- * 33 / 73, 36 / 72; at 256: 46 / 77, 55 / 84, 63 / 81), for Q6_K, Q8_0 and IQ4_NL up to 256 tokens. IQ4_NL (a table
- * lookup per weight): large tiles 62 / 95 at 512 tokens, 123 / 132 at 1024, 279 / 254 at 2048; small tiles 4096 x 4096
- * 38 / 45, 4096 x 14336 120 / 108, 14336 x 4096 at 128 tokens 37 / 80. IQ4_XS: large 68 / 99, 133 / 139, 305 / 270; small
- * 39 / 45, 123 / 111, 38 / 79. Q4_0: large 62 / 81, 122 / 120, 272 / 241; small 30 / 41, 93 / 93, 30 / 67. Q2_K: large
- * 59 / 82, 117 / 120, 251 / 222; small 29 / 42, 89 / 95, 28 / 71. Q3_K: large 62 / 91, 127 / 128, 261 / 253; small 32 / 44,
- * 99 / 103, 31 / 76.
+ * at 512 tokens Q4_K 61 / 86, Q5_K 62 / 92, Q6_K 66 / 84, Q8_0 71 / 83, IQ4_NL 62 / 95, IQ4_XS 68 / 99, Q4_0 62 / 81,
+ * Q2_K 59 / 82, Q3_K 62 / 91; at 1024 118 / 125, 121 / 135, 131 / 126, 139 / 121, 123 / 132, 133 / 139, 122 / 120,
+ * 117 / 120, 127 / 128; at 1536 Q4_K 181 / 190, Q5_K 185 / 195, Q6_K 206 / 184, Q8_0 216 / 177; at 2048 267 / 244,
+ * 262 / 260, 273 / 240, 311 / 224, 279 / 254, 305 / 270, 272 / 241, 251 / 222, 261 / 253).
+ * Fewer large tiles: the small-tile kernel, up to a token count per format (small tiles / decode + library, us, at
+ * 4096 x 4096 and 4096 x 14336 with 512 tokens, the same two with 1024, 6144 x 4096 with 768, 14336 x 4096 with 256:
+ * Q4_K 24 / 43, 72 / 97, 42 / 52, 133 / 153, 57 / 59, 39 / 75; Q5_K 25 / 44, 74 / 104, 43 / 54, 139 / 158, 59 / 61, 41 / 80;
+ * Q6_K 29 / 40, 85 / 96, 49 / 51, 163 / 154, 68 / 57, 47 / 71; Q8_0 35 / 38, 109 / 97, 64 / 49, 216 / 152, 91 / 55, 62 / 75;
+ * IQ4_NL 27 / 45, 80 / 108, 46 / 55, 148 / 161, 63 / 63, 44 / 88; IQ4_XS 27 / 45, 82 / 110, 47 / 55, 154 / 162, 64 / 63,
+ * 45 / 80; Q4_0 24 / 41, 72 / 91, 41 / 50, 133 / 144, 57 / 56, 39 / 72; Q2_K 24 / 42, 70 / 94, 41 / 52, 132 / 149, 55 / 58,
+ * 38 / 74; Q3_K 26 / 45, 75 / 102, 44 / 54, 144 / 160, 61 / 61, 42 / 82).
  * Without a workspace there is no decode + dense route to prefer. */
 FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, bool have_workspace) {
     if (!gemm_kq_wave4_covers(type) || n_cols % 256 != 0 || ldx >= (1 << 22)) return kFusedNone;
     const long long large_tiles = (long long)((n_rows + 127) / 128) * ((n_tok + 255) / 256);
     /* token counts up to which the large-tile and the small-tile kernel measured faster than decode + dense */
-    int large_max = 512, small_max = 256;
+    int large_max = 512, small_max = 256; /* Q8_0 */
     switch (type) {
     case T_Q4_K: case T_Q5_K: large_max = 1536; small_max = INT_MAX; break;
     case T_Q4_0: case T_Q2_K: case T_Q3_K: large_max = 1024; small_max = INT_MAX; break;
-    case T_IQ4_NL: large_max = 1536; break;
-    case T_IQ4_XS: large_max = 1024; break;
-    default: break; /* Q6_K, Q8_0 */
+    case T_IQ4_NL: large_max = 1536; small_max = 1024; break;
+    case T_IQ4_XS: large_max = 1024; small_max = 1024; break;
+    case T_Q6_K: small_max = 512; break;
+    default: break;
     }
     if (large_tiles >= 200) return (n_tok <= large_max || !have_workspace) ? kFusedLarge : kFusedNone;
     return (n_tok <= small_max || !have_workspace) ? kFusedSmall : kFusedNone;
@@ -338,20 +349,27 @@ hipError_t launch_fused_tile(FusedTile tile, uint32_t type, const void *W, const
     return hipErrorInvalidValue;
 }
 
-hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
-                                     int n_tok, int ldx, int ldy, hipStream_t stream) {
+hipError_t launch_gemm_kq_bf16_wave4_multi(uint32_t type, int n_mat, const void *const *W, const uint16_t *X,
+                                           float *const *Y, const int *n_rows, int n_cols, int n_tok, int ldx,
+                                           const int *ldy, hipStream_t stream) {
+    if (n_mat < 1 || n_mat > 3) return hipErrorInvalidValue;
     switch (type) {
-    case T_Q4_K: return launch_wave4<FQ4K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_Q5_K: return launch_wave4<FQ5K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_Q6_K: return launch_wave4<FQ6K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_Q8_0: return launch_wave4<FQ8_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_IQ4_NL: return launch_wave4<FIQ4NL>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_IQ4_XS: return launch_wave4<FIQ4XS>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_Q4_0: return launch_wave4<FQ4_0>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_Q2_K: return launch_wave4<FQ2K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
-    case T_Q3_K: return launch_wave4<FQ3K>(W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q4_K: return launch_wave4<FQ4K>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q5_K: return launch_wave4<FQ5K>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q6_K: return launch_wave4<FQ6K>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q8_0: return launch_wave4<FQ8_0>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_IQ4_NL: return launch_wave4<FIQ4NL>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_IQ4_XS: return launch_wave4<FIQ4XS>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q4_0: return launch_wave4<FQ4_0>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q2_K: return launch_wave4<FQ2K>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
+    case T_Q3_K: return launch_wave4<FQ3K>(n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, stream);
     default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_gemm_kq_bf16_wave4(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
+                                     int n_tok, int ldx, int ldy, hipStream_t stream) {
+    return launch_gemm_kq_bf16_wave4_multi(type, 1, &W, X, &Y, &n_rows, n_cols, n_tok, ldx, &ldy, stream);
 }
 
 hipError_t launch_gemm_q4k_bf16_wave4(const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols, int n_tok,

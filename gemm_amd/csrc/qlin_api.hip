@@ -1132,6 +1132,43 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
     return QLIN_OK;
 }
 
+int qlin_gemm_bf16_multi_dev(uint32_t type, int n_mat, const void *const *W, const uint16_t *X, float *const *Y,
+                             const int *n_rows, int n_cols, int n_tok, int ldx, const int *ldy, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+    if (n_mat < 1 || n_mat > 3) return fail(QLIN_ERR_ARG, "one to three tensors per call");
+    if (!W || !Y || !n_rows || !ldy) return fail(QLIN_ERR_ARG, "null pointer");
+    /* one launch where every tensor on its own would take the same tile kernel; the checks are those of the
+     * single-tensor call, which a tensor that fails them goes through below to report it */
+    bool together = n_mat > 1 && n_tok > 0 && X && aligned(X, 16) && ldx % 8 == 0 && ldx >= n_cols && n_tok > kFewTokens;
+    FusedTile tile = kFusedNone;
+    for (int i = 0; i < n_mat && together; i++) {
+        const bool ws_ok = workspace && aligned(workspace, 256) &&
+                           workspace_bytes >= qlin_gemm_bf16_any_workspace_bytes(n_rows[i], n_cols);
+        together = n_rows[i] > 0 && W[i] && Y[i] && aligned(W[i], 16) && aligned(Y[i], 4) && ldy[i] >= n_rows[i] &&
+                   n_cols > 0; /* the chooser checks format and row length */
+        if (!together) break;
+        const FusedTile mine = choose_fused_tile(type, n_rows[i], n_cols, n_tok, ldx, ws_ok);
+        together = mine != kFusedNone && (i == 0 || mine == tile);
+        tile = mine;
+    }
+    if (together) {
+        {
+            std::lock_guard<std::mutex> lk(g.mu);
+            if (int rc = ensure_init_locked(0)) return rc;
+        }
+        if (tile == kFusedSmall)
+            HIP_TRY(launch_gemm_kq_bf16_wave4s_multi(type, n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        else
+            HIP_TRY(launch_gemm_kq_bf16_wave4_multi(type, n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        return QLIN_OK;
+    }
+    for (int i = 0; i < n_mat; i++)
+        if (int rc = qlin_gemm_bf16_any_dev(type, W[i], X, Y[i], n_rows[i], n_cols, n_tok, ldx, ldy[i], workspace,
+                                            workspace_bytes, stream))
+            return rc;
+    return QLIN_OK;
+}
+
 size_t qlin_gemm_f32_any_workspace_bytes(int n_rows, int n_cols) {
     if (n_rows <= 0 || n_cols <= 0) return 0;
     return dense_gemm_weight_bytes_f32(n_rows, n_cols) + kDenseLibWorkspace;

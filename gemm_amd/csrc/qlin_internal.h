@@ -135,6 +135,13 @@ bool gemm_kq_wave4_covers(uint32_t type);
 /* the same in 128-token x 64-row tiles, two workgroups per compute unit (gemm_kq_wave4s.hip) */
 hipError_t launch_gemm_kq_bf16_wave4s(uint32_t type, const void *W, const uint16_t *X, float *Y, int n_rows, int n_cols,
                                       int n_tok, int ldx, int ldy, hipStream_t stream);
+/* the same kernel over up to three tensors of one format and K in one launch (row tiles numbered through the tensors) */
+hipError_t launch_gemm_kq_bf16_wave4_multi(uint32_t type, int n_mat, const void *const *W, const uint16_t *X,
+                                           float *const *Y, const int *n_rows, int n_cols, int n_tok, int ldx,
+                                           const int *ldy, hipStream_t stream);
+hipError_t launch_gemm_kq_bf16_wave4s_multi(uint32_t type, int n_mat, const void *const *W, const uint16_t *X,
+                                            float *const *Y, const int *n_rows, int n_cols, int n_tok, int ldx,
+                                            const int *ldy, hipStream_t stream);
 /* the fused kernel for a shape (kFusedNone: decode + dense product, or the format has none) and its launch */
 enum FusedTile { kFusedNone = 0, kFusedLarge, kFusedSmall };
 FusedTile choose_fused_tile(uint32_t type, int n_rows, int n_cols, int n_tok, int ldx, bool have_workspace);

@@ -113,6 +113,7 @@ SIGNATURES = {
     "qlin_dequant_bf16_dev": (C.c_int, [C.c_uint32, _vp, _vp, C.c_int, C.c_int, _vp]),
     "qlin_gemm_bf16_any_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "qlin_gemm_bf16_any_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, C.c_size_t, _vp]),
+    "qlin_gemm_bf16_multi_dev": (C.c_int, [C.c_uint32, C.c_int, _vp, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, _vp, _vp, C.c_size_t, _vp]),
     "qlin_gemm_f32_any_workspace_bytes": (C.c_size_t, [C.c_int, C.c_int]),
     "qlin_gemm_f32_any_dev": (C.c_int, [C.c_uint32, _vp, _vp, _vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _vp, C.c_size_t, _vp]),
     "qlin_probe_mfma_bf16": (C.c_int, [C.c_int, _vp, C.POINTER(C.c_double)]),
@@ -321,6 +322,17 @@ def gemm_bf16_any_workspace_bytes(n_rows, n_cols):
 def gemm_bf16_any_dev(type_id, dW, dX, dY, n_rows, n_cols, n_tok, ldx, ldy, dws, stream=None):
     check(load().qlin_gemm_bf16_any_dev(type_id, dW.ptr, dX.ptr, dY.ptr, n_rows, n_cols, n_tok, ldx, ldy,
                                         dws.ptr if dws is not None else None, dws.nbytes if dws is not None else 0, stream))
+
+
+def gemm_bf16_multi_dev(type_id, dWs, dX, dYs, n_rows, n_cols, n_tok, ldx, ldys, dws, stream=None):
+    """dWs, dYs: lists of DevBuf; n_rows, ldys: lists of int (one entry per tensor)"""
+    n = len(dWs)
+    Wp = (C.c_void_p * n)(*[b.ptr for b in dWs])
+    Yp = (C.c_void_p * n)(*[b.ptr for b in dYs])
+    rows = (C.c_int * n)(*n_rows)
+    ld = (C.c_int * n)(*ldys)
+    check(load().qlin_gemm_bf16_multi_dev(type_id, n, Wp, dX.ptr, Yp, rows, n_cols, n_tok, ldx, ld,
+                                          dws.ptr if dws is not None else None, dws.nbytes if dws is not None else 0, stream))
 
 
 def gemm_f32_any_workspace_bytes(n_rows, n_cols):

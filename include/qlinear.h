@@ -235,7 +235,7 @@ int qlin_gemm_bf16_dev(uint32_t ggml_type, const void *W, const uint16_t *X, flo
  * 513..1024, ...), 128-token x 64-row tiles for smaller shapes (4096-row projections at 512 tokens, any row count at
  * 33..256 tokens). Given a workspace, the decode + dense route still takes the shapes where decoding once measured
  * faster: large-tile shapes above 1536 tokens (Q4_K, Q5_K, IQ4_NL), 1024 (Q2_K, Q3_K, IQ4_XS, Q4_0) or 512 (Q6_K, Q8_0), small-tile
- * shapes of Q6_K, Q8_0, IQ4_NL and IQ4_XS above 256 tokens. Q4_K up to 32 tokens: the few-token kernel of qlin_gemm_bf16_dev.
+ * shapes of Q8_0 above 256 tokens, of Q6_K above 512, of IQ4_NL and IQ4_XS above 1024. Q4_K up to 32 tokens: the few-token kernel of qlin_gemm_bf16_dev.
  * Up to 24 tokens of a Q6_K, Q5_K, Q3_K, Q2_K or
  * Q8_0 tensor (n_cols % 256 == 0, the tensor's bytes a multiple of 16) also run in one fused kernel with
  * unrounded weights (~1e-6) and leave the workspace alone (it may be NULL then). Up to 4 tokens of any other
@@ -256,6 +256,17 @@ size_t qlin_gemm_bf16_any_workspace_bytes(int n_rows, int n_cols);
 int qlin_gemm_bf16_any_dev(uint32_t ggml_type, const void *W, const uint16_t *X, float *Y, int n_rows,
                            int n_cols, int n_tok, int ldx, int ldy, void *workspace, size_t workspace_bytes,
                            void *stream);
+/* qlin_gemm_bf16_any_dev for one to three weight tensors of ONE format and row length against the same activations:
+ * the Q, K and V projections of a prefill chunk, which the reference multiplies tensor by tensor
+ * (tf_gemm_f16_mt_tokenmajor per projection, common/transformer.h:5256-5258). Y[i][t * ldy[i] + r] is tensor i's
+ * product. Where every tensor on its own would take the 128-token x 64-row tile kernel they share one launch, their row
+ * tiles numbered through (a 1024-row K or V projection alone is 64 workgroups at 512 tokens on 256 compute units;
+ * Q4_K 4096 + 1024 + 1024 rows x 4096 at 512 tokens: 36 us in one launch against 24 + 22 + 22); every other case is
+ * one qlin_gemm_bf16_any_dev call per tensor, with its argument checks and its use of the workspace (sized for the
+ * largest tensor). The arrays W, Y, n_rows and ldy are host memory and are read before the call returns. */
+int qlin_gemm_bf16_multi_dev(uint32_t ggml_type, int n_mat, const void *const *W, const uint16_t *X, float *const *Y,
+                             const int *n_rows, int n_cols, int n_tok, int ldx, const int *ldy, void *workspace,
+                             size_t workspace_bytes, void *stream);
 /* Same contraction in fp32 (X fp32, no rounding of weights or activations); any supported type.
  * Vector-ALU kernel, no workspace: the choice for a few tokens. */
 int qlin_gemm_f32_dev(uint32_t ggml_type, const void *W, const float *X, float *Y, int n_rows,

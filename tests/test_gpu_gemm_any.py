@@ -43,6 +43,7 @@ def dense_kernel(request):
 
 FUSED = [Q4K, synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ4_NL, synth.GGML_IQ4_XS,
          synth.GGML_Q4_0, synth.GGML_Q2_K, synth.GGML_Q3_K]  # decoded inside the tile kernels
+FEW = 32  # tokens up to which Q4_K takes its few-token kernel
 KQ = {synth.GGML_Q6_K, synth.GGML_Q5_K, synth.GGML_Q3_K, synth.GGML_Q2_K, synth.GGML_Q8_0}
 
 
@@ -146,6 +147,85 @@ def test_each_tile_kernel_on_small_and_ragged_shapes(oracle, tile, tid, n_tok, n
     assert rel_l2(Y[:, :n_rows], designed) <= 2e-5, (ALL[tid], tile, n_tok, n_rows, n_cols)
     if n_tok * n_rows >= 1000:  # the bar on the bf16 rounding of the weights is a statistical one
         assert rel_l2(Y[:, :n_rows], exact) <= 3e-3
+
+
+def multi_case(tid, rows, n_cols, n_tok, seed):
+    Ws = [synth.make_weights(tid, r, n_cols, seed=seed + i) for i, r in enumerate(rows)]
+    Xb = synth.to_bf16_bits(synth.make_activation(n_cols, seed=seed + 9, tokens=n_tok))
+    ldx = n_cols + 8
+    Xpad = np.zeros((n_tok, ldx), np.uint16)
+    Xpad[:, :n_cols] = Xb
+    ldys = [r + 1 + i for i, r in enumerate(rows)]
+    return Ws, Xb, Xpad, ldx, ldys
+
+
+def run_multi(tid, Ws, Xpad, rows, n_cols, n_tok, ldx, ldys, together, ws_bytes=0):
+    dWs = [qlinear.DevBuf.from_numpy(W) for W in Ws]
+    dX = qlinear.DevBuf.from_numpy(Xpad)
+    dYs = [qlinear.DevBuf.from_numpy(np.full((n_tok, ld), -3.0, np.float32)) for ld in ldys]
+    dws = qlinear.DevBuf(ws_bytes) if ws_bytes else None
+    if together:
+        qlinear.gemm_bf16_multi_dev(tid, dWs, dX, dYs, rows, n_cols, n_tok, ldx, ldys, dws)
+    else:
+        for dW, dY, r, ld in zip(dWs, dYs, rows, ldys):
+            qlinear.gemm_bf16_any_dev(tid, dW, dX, dY, r, n_cols, n_tok, ldx, ld, dws)
+    qlinear.sync()
+    Ys = [dY.to_numpy(np.float32, (n_tok, ld)) for dY, ld in zip(dYs, ldys)]
+    for b in dWs + dYs + [dX] + ([dws] if dws else []):
+        b.free()
+    return Ys
+
+
+@pytest.mark.parametrize("tid", FUSED, ids=lambda t: ALL[t])
+@pytest.mark.parametrize("rows,n_cols,n_tok", [
+    ((256, 64, 70), 512, 130),   # ragged last tiles of the second and third tensor, two token tiles
+    ((130, 129), 1280, 64),      # two tensors, neither a whole number of tiles
+    ((64, 64, 64), 256, 33),     # one tile each, one super-block
+    ((6400, 6500), 256, 1024),   # 200 and more 256-token x 128-row tiles each: the large-tile kernel
+])
+def test_several_tensors_in_one_launch_equal_one_call_each(oracle, tid, rows, n_cols, n_tok):
+    """qlin_gemm_bf16_multi_dev on shapes where every tensor takes the same tile kernel: bit for bit what one call per
+    tensor gives (the same workgroups run, numbered through the tensors), right against the oracle, and nothing written
+    past a tensor's rows"""
+    rows = list(rows)
+    Ws, Xb, Xpad, ldx, ldys = multi_case(tid, rows, n_cols, n_tok, seed=500 + tid)
+    one_by_one = run_multi(tid, Ws, Xpad, rows, n_cols, n_tok, ldx, ldys, together=False)
+    together = run_multi(tid, Ws, Xpad, rows, n_cols, n_tok, ldx, ldys, together=True)
+    for W, r, a, b in zip(Ws, rows, one_by_one, together):
+        if tid == Q4K and n_tok <= FEW:  # the single call takes the few-token kernel (exact codes): compare by value
+            assert rel_l2(b[:, :r], a[:, :r]) <= 3e-3
+        else:
+            assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), (ALL[tid], r)
+        assert np.all(b[:, r:] == -3.0)
+        exact, designed = references(oracle, tid, W, Xb, n_cols)
+        assert rel_l2(b[:, :r], designed) <= 2e-5, (ALL[tid], r)
+
+
+def test_several_tensors_fall_back_to_one_call_each(oracle):
+    """a format without a tile kernel, a few tokens, and a single tensor: the per-tensor route, same results and same errors"""
+    lib = qlinear.load()
+    for tid, n_tok in ((synth.GGML_Q5_1, 40), (synth.GGML_Q6_K, 8), (Q4K, 16)):
+        rows, n_cols = [96, 33], 512
+        Ws, Xb, Xpad, ldx, ldys = multi_case(tid, rows, n_cols, n_tok, seed=700 + tid)
+        ws_bytes = qlinear.gemm_bf16_any_workspace_bytes(max(rows), n_cols)
+        a = run_multi(tid, Ws, Xpad, rows, n_cols, n_tok, ldx, ldys, together=False, ws_bytes=ws_bytes)
+        b = run_multi(tid, Ws, Xpad, rows, n_cols, n_tok, ldx, ldys, together=True, ws_bytes=ws_bytes)
+        for x, y in zip(a, b):
+            assert np.array_equal(x.view(np.uint32), y.view(np.uint32)), ALL[tid]
+    # the formats without a tile kernel need the workspace here as well
+    rows, n_cols, n_tok = [96, 33], 512, 40
+    Ws, Xb, Xpad, ldx, ldys = multi_case(synth.GGML_Q5_1, rows, n_cols, n_tok, seed=3)
+    with pytest.raises(qlinear.QlinError):
+        run_multi(synth.GGML_Q5_1, Ws, Xpad, rows, n_cols, n_tok, ldx, ldys, together=True)
+    d = qlinear.DevBuf(4096)
+    import ctypes as C
+    one = (C.c_void_p * 1)(d.ptr)
+    n1 = (C.c_int * 1)(16)
+    f = lib.qlin_gemm_bf16_multi_dev
+    assert f(Q4K, 0, one, d.ptr, one, n1, 256, 4, 256, n1, None, 0, None) == qlinear.ERR_ARG   # no tensor
+    assert f(Q4K, 4, one, d.ptr, one, n1, 256, 4, 256, n1, None, 0, None) == qlinear.ERR_ARG   # more than three
+    assert f(Q4K, 1, None, d.ptr, one, n1, 256, 4, 256, n1, None, 0, None) == qlinear.ERR_ARG  # no array
+    d.free()
 
 
 @pytest.mark.parametrize("tid", [synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ4_NL], ids=lambda t: ALL[t])
