@@ -112,8 +112,8 @@ struct FQ4K {
     static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
     static constexpr bool kSwizzle = false;
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 4 ? -1 : ((P - 4) / 5) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 4 ? -1 : ((P - 4) / 5) >> 1; }
     template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
     typedef K4Scales Scales;
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
@@ -144,8 +144,8 @@ struct FQ5K {
     static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
     static constexpr bool kSwizzle = false;
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 4 ? -1 : ((P - 4) / 7) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 4 ? -1 : ((P - 4) / 7) >> 1; }
     template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
     typedef K4Scales Scales;
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
@@ -175,8 +175,8 @@ struct FQ6K {
     static constexpr int kExtraVec = 0, kExtraLoads = 0, kKgChunk = 2;
     static constexpr bool kSwizzle = false;
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 4 ? P >> 1 : ((P - 4) / 7) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 4 ? 4 + (P >> 1) : ((P - 4) / 7) >> 1; }
     template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
     typedef Q6Scales Scales;
     static QLIN_INL uint32_t piece_src(int part) { return part < 13 ? 16u * part : part == 13 ? 194u : 0u; }
@@ -219,8 +219,8 @@ struct FQ8_0 {
     static constexpr bool kSwizzle = true;
     struct Scales {};
     static constexpr int frag_xor(int s) { return s << 4; }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 1 ? -1 : ((P - 1) / 6) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 1 ? -1 : ((P - 1) / 6) >> 1; }
     static QLIN_INL uint32_t piece_src(int part) { return 34u * (part >> 1) + 2u + 16u * (part & 1); }
     /* vector j: half j & 1 of the codes of block 2 (j >> 1) + kg */
     static constexpr VecAt vec_at(int j) { return VecAt{64 * (j >> 1) + 16 * (j & 1), 32}; }
@@ -255,8 +255,8 @@ struct FIQ4NL {
     static constexpr bool kSwizzle = false;
     struct Scales {};
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 2 ? P : ((P - 2) / 10) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 2 ? 4 + P : ((P - 2) / 10) >> 1; }
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
     static constexpr VecAt vec_at(int j) { return VecAt{16 * j, 0}; }
     template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
@@ -306,8 +306,8 @@ struct FQ4_0 {
     static constexpr bool kSwizzle = false;
     struct Scales {};
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 2 ? P : ((P - 2) / 6) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 2 ? 4 + P : ((P - 2) / 6) >> 1; }
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
     static constexpr VecAt vec_at(int j) { return VecAt{16 * j, 0}; }
     template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
@@ -348,8 +348,8 @@ struct FIQ4XS {
     static constexpr bool kSwizzle = false;
     typedef XsScales Scales;
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 8 ? P >> 2 : ((P - 8) / 10) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 8 ? 4 + (P >> 2) : ((P - 8) / 10) >> 1; }
     static QLIN_INL uint32_t piece_src(int part) { return 16u * part; }
     static constexpr VecAt vec_at(int j) { return VecAt{16 * j, 0}; }
     template <int J, class C> static QLIN_INL void extra_load(C &, u32x4 (&)[kLaneVec + kExtraVec], int) {}
@@ -407,8 +407,8 @@ struct FQ2K {
     static constexpr bool kSwizzle = false;
     typedef Q2Scales Scales;
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 4 ? -1 : ((P - 4) / 5) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 4 ? -1 : ((P - 4) / 5) >> 1; }
     static QLIN_INL uint32_t piece_src(int part) { return part < 5 ? 16u * part : 68u; }
     /* vector 0: the scales; 1, 2: the lane's code bytes of half 0, 1; 3: the piece with d and dmin */
     static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, 0} : j < 3 ? VecAt{16 + 32 * (j - 1), 16} : VecAt{80, 0}; }
@@ -450,8 +450,8 @@ struct FQ3K {
     static constexpr bool kSwizzle = false;
     typedef Q3Scales Scales;
     static constexpr int frag_xor(int s) { return ((s & 1) << 4) | ((s >> 1) << 6); }
-    /* which half of a tile's k-steps (0: steps 0, 1; 1: steps 2, 3) tile piece P serves; -1: both */
-    static constexpr int piece_half(int P) { return P < 4 ? -1 : ((P - 4) / 6) >> 2; }
+    /* which k-step of a tile (0..3) tile piece P serves; 4, 5: both k-steps of half 0, 1; -1: all four */
+    static constexpr int piece_step(int P) { return P < 4 ? -1 : ((P - 4) / 6) >> 1; }
     static QLIN_INL uint32_t piece_src(int part) { return part < 6 ? 16u * part : 94u; }
     /* vector 0: the lane's third-bit bytes; 1, 2: its code bytes of half 0, 1; 3: the piece with scales and d */
     static constexpr VecAt vec_at(int j) { return j == 0 ? VecAt{0, 16} : j < 3 ? VecAt{32 + 32 * (j - 1), 16} : VecAt{96, 0}; }
@@ -495,39 +495,63 @@ struct FQ3K {
     }
 };
 
+/* Does a wave that takes half WK of a tile's k-steps (2 WK and 2 WK + 1) run tile piece q of format F? */
+template <class F, int WK> constexpr bool owns_piece(int q) {
+    const int st = F::piece_step(q);
+    return st < 0 || (st < 4 ? st >> 1 : st - 4) == WK;
+}
+/* The decode pieces of a tile that such a wave runs: the NPREP pieces of the next super-block's scales (last tile of
+ * a super-block), then its tile pieces, in their order. */
+template <class F, int WK, int NPREP> struct Owned {
+    static constexpr int count() {
+        int n = NPREP;
+        for (int q = 0; q < F::kTilePieces; q++) n += owns_piece<F, WK>(q) ? 1 : 0;
+        return n;
+    }
+    /* the i-th of them: below NPREP a prep piece, else NPREP + the tile piece's number */
+    static constexpr int nth(int i) {
+        if (i < NPREP) return i;
+        int n = NPREP;
+        for (int q = 0; q < F::kTilePieces; q++)
+            if (owns_piece<F, WK>(q)) {
+                if (n == i) return NPREP + q;
+                n++;
+            }
+        return -1;
+    }
+};
+
 /* Up to three weight tensors of one format and one K against the same activations in one launch (the Q, K and V
  * projections of a prefill chunk: a 1024-row tensor alone is 64 small tiles at 512 tokens; gate and up). Row tiles are
  * numbered through the tensors: tensor i owns tiles end[i - 1] .. end[i] - 1. */
-struct TileSet {
-    const uint8_t *W[3];
-    float *Y[3];
-    int n_rows[3], ldy[3], end[3];
+struct TileSet { /* named members, not arrays: the kernels pick by comparisons on scalar registers, never by an index */
+    const uint8_t *W0, *W1, *W2;
+    float *Y0, *Y1, *Y2;
+    int n_rows0, n_rows1, n_rows2, ldy0, ldy1, ldy2, end0, end1, end2;
 };
 /* host: entries past n_mat repeat the last tensor and own no tile -> the number of row tiles */
 inline int fill_tile_set(TileSet &set, int n_mat, const void *const *W, float *const *Y, const int *n_rows, const int *ldy,
                          int rows_per_tile) {
-    int n_tiles = 0;
+    int n_tiles = 0, end[3];
     for (int i = 0; i < 3; i++) {
-        const int j = i < n_mat ? i : n_mat - 1;
-        set.W[i] = (const uint8_t *)W[j];
-        set.Y[i] = Y[j];
-        set.n_rows[i] = n_rows[j];
-        set.ldy[i] = ldy[j];
         if (i < n_mat) n_tiles += (n_rows[i] + rows_per_tile - 1) / rows_per_tile;
-        set.end[i] = n_tiles;
+        end[i] = n_tiles;
     }
+    const int j1 = n_mat > 1 ? 1 : 0, j2 = n_mat > 2 ? 2 : j1;
+    set.W0 = (const uint8_t *)W[0]; set.W1 = (const uint8_t *)W[j1]; set.W2 = (const uint8_t *)W[j2];
+    set.Y0 = Y[0]; set.Y1 = Y[j1]; set.Y2 = Y[j2];
+    set.n_rows0 = n_rows[0]; set.n_rows1 = n_rows[j1]; set.n_rows2 = n_rows[j2];
+    set.ldy0 = ldy[0]; set.ldy1 = ldy[j1]; set.ldy2 = ldy[j2];
+    set.end0 = end[0]; set.end1 = end[1]; set.end2 = end[2];
     return n_tiles;
 }
-/* device: the tensor of row tile `tile_all` (below end[2]) and the tile's number inside it */
+/* device: the tensor of row tile `tile_all` (below end2) and the tile's number inside it */
 struct TileOf { const uint8_t *W; float *Y; int n_rows, ldy, tile; };
 QLIN_INL TileOf tile_of(const TileSet &set, int tile_all) {
-    const int mi = (tile_all >= set.end[0] ? 1 : 0) + (tile_all >= set.end[1] ? 1 : 0);
     TileOf t;
-    t.W = mi == 0 ? set.W[0] : mi == 1 ? set.W[1] : set.W[2];
-    t.Y = mi == 0 ? set.Y[0] : mi == 1 ? set.Y[1] : set.Y[2];
-    t.n_rows = mi == 0 ? set.n_rows[0] : mi == 1 ? set.n_rows[1] : set.n_rows[2];
-    t.ldy = mi == 0 ? set.ldy[0] : mi == 1 ? set.ldy[1] : set.ldy[2];
-    t.tile = tile_all - (mi == 0 ? 0 : mi == 1 ? set.end[0] : set.end[1]);
+    if (tile_all < set.end0) { t.W = set.W0; t.Y = set.Y0; t.n_rows = set.n_rows0; t.ldy = set.ldy0; t.tile = tile_all; }
+    else if (tile_all < set.end1) { t.W = set.W1; t.Y = set.Y1; t.n_rows = set.n_rows1; t.ldy = set.ldy1; t.tile = tile_all - set.end0; }
+    else { t.W = set.W2; t.Y = set.Y2; t.n_rows = set.n_rows2; t.ldy = set.ldy2; t.tile = tile_all - set.end1; }
     return t;
 }
 

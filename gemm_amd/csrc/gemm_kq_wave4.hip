@@ -181,7 +181,7 @@ gemm_kq_bf16_wave4_kernel(TileSet set, const uint16_t *__restrict__ X, int n_sb,
     const int xcd = blockIdx.x & 7, slot_id = blockIdx.x >> 3;
     const int tile_m = slot_id % m_tiles;
     const int tile_all = (slot_id / m_tiles) * 8 + xcd;
-    if (tile_all >= set.end[2]) return;
+    if (tile_all >= set.end2) return;
     const TileOf t = tile_of(set, tile_all);
     const uint8_t *W = t.W;
     float *Y = t.Y;

@@ -84,28 +84,6 @@ template <class F, int ST, int S, int BJ> QLIN_INL bf16x8 load_frag(Ctx<F> &c) {
     return *reinterpret_cast<const bf16x8 *>(stage_ptr<ST>() + (c.xrd ^ (uint32_t)F::frag_xor(S)) + BJ * 4096);
 }
 
-/* The decode pieces of a tile that wave half WK runs: the NPREP pieces of the next super-block's scales (last tile of
- * a super-block), then the tile pieces that serve its k-steps or both halves, in their order. */
-template <class F, int WK, int NPREP> struct Owned {
-    static constexpr bool own(int q) { return F::piece_half(q) < 0 || F::piece_half(q) == WK; }
-    static constexpr int count() {
-        int n = NPREP;
-        for (int q = 0; q < F::kTilePieces; q++) n += own(q) ? 1 : 0;
-        return n;
-    }
-    /* the i-th of them: below NPREP a prep piece, else NPREP + the tile piece's number */
-    static constexpr int nth(int i) {
-        if (i < NPREP) return i;
-        int n = NPREP;
-        for (int q = 0; q < F::kTilePieces; q++)
-            if (own(q)) {
-                if (n == i) return NPREP + q;
-                n++;
-            }
-        return -1;
-    }
-};
-
 /* owned pieces I0 + I of a slot, as far as they are below I1 */
 template <class F, int WK, int U, int I0, int I1, int... I> QLIN_INL void pieces(Ctx<F> &c, std::integer_sequence<int, I...>) {
     constexpr int n_prep = U == 3 ? F::kPrepPieces : 0;
@@ -249,7 +227,7 @@ gemm_kq_bf16_wave4s_kernel(TileSet set, const uint16_t *__restrict__ X, int n_sb
     const int xcd = blockIdx.x & 7, slot_id = blockIdx.x >> 3;
     const int tile_m = slot_id % m_tiles;
     const int tile_all = (slot_id / m_tiles) * 8 + xcd;
-    if (tile_all >= set.end[2]) return;
+    if (tile_all >= set.end2) return;
     const TileOf t = tile_of(set, tile_all);
     const uint8_t *W = t.W;
     float *Y = t.Y;

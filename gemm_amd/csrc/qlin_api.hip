@@ -1156,10 +1156,10 @@ int qlin_gemm_bf16_multi_dev(uint32_t type, int n_mat, const void *const *W, con
             std::lock_guard<std::mutex> lk(g.mu);
             if (int rc = ensure_init_locked(0)) return rc;
         }
-        if (tile == kFusedSmall)
-            HIP_TRY(launch_gemm_kq_bf16_wave4s_multi(type, n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
-        else
+        if (tile == kFusedLarge)
             HIP_TRY(launch_gemm_kq_bf16_wave4_multi(type, n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
+        else
+            HIP_TRY(launch_gemm_kq_bf16_wave4s_multi(type, n_mat, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy, (hipStream_t)stream));
         return QLIN_OK;
     }
     for (int i = 0; i < n_mat; i++)
@@ -1327,8 +1327,8 @@ int qlin_probe_gemm_tile(int tile, uint32_t type, const void *W, const uint16_t 
     if (!aligned(W, 16) || !aligned(X, 16) || !aligned(Y, 4) || ldx % 8)
         return fail(QLIN_ERR_ARG, "W and X need 16-byte alignment, Y 4-byte, ldx %% 8 == 0");
     if (int rc = init_once()) return rc;
-    HIP_TRY((tile ? launch_gemm_kq_bf16_wave4s : launch_gemm_kq_bf16_wave4)(type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy,
-                                                                            (hipStream_t)stream));
+    HIP_TRY(launch_fused_tile(tile == 0 ? kFusedLarge : kFusedSmall, type, W, X, Y, n_rows, n_cols, n_tok, ldx, ldy,
+                              (hipStream_t)stream));
     return QLIN_OK;
 }
 
