@@ -1,6 +1,6 @@
 /*
- * gemm_kq_wave4.hip - Q4_K, Q5_K, Q6_K, Q8_0, IQ4_NL, IQ4_XS and Q4_0 x bf16 prefill GEMM for more than 128 tokens: four waves per workgroup,
- * one per SIMD.
+ * gemm_kq_wave4.hip - the fused block-format x bf16 prefill GEMM (Q2_K ... Q6_K, Q8_0, IQ4_NL, IQ4_XS, Q4_0: the formats of
+ * gemm_kq_formats.h) in 256-token x 128-row tiles: four waves per workgroup, one per SIMD.
  *
  *   Y[t*ldy + r] = sum_k X[t*ldx + k] * decode(W)[r][k]      X bf16, Y fp32, fp32 accumulate
  *

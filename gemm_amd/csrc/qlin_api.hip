@@ -1073,7 +1073,7 @@ int qlin_gemm_bf16_any_dev(uint32_t type, const void *W, const uint16_t *X, floa
         std::lock_guard<std::mutex> lk(g.mu);
         if (int rc = ensure_init_locked(0)) return rc;
     }
-    /* Q4_K, Q5_K, Q6_K, Q8_0 and IQ4_NL: decoded into the matrix operand inside the product, no workspace, in large or small
+    /* the formats with a tile kernel (gemm_kq_formats.h): decoded into the matrix operand inside the product, no workspace, in large or small
      * tiles by the shape - except where decoding once into the caller's workspace measured faster */
     /* (up to four tokens of the formats without a few-token kernel are faster one by one through the matvec below) */
     const bool matvec_first = (type == T_IQ4_NL || type == T_IQ4_XS || type == T_Q4_0) && n_tok <= kMatvecTokens && ws_ok;
