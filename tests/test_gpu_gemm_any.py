@@ -228,7 +228,7 @@ def test_several_tensors_fall_back_to_one_call_each(oracle):
     d.free()
 
 
-@pytest.mark.parametrize("tid", [synth.GGML_Q5_K, synth.GGML_Q6_K, synth.GGML_Q8_0, synth.GGML_IQ4_NL], ids=lambda t: ALL[t])
+@pytest.mark.parametrize("tid", [t for t in FUSED if t != Q4K], ids=lambda t: ALL[t])  # Q4_K: test_gpu_gemm_bf16.py
 def test_fused_tile_kernel_full_size_config(oracle, tid):
     """14336 x 4096 at 512 tokens; the oracle on a sample of rows, and scaling X by two scales Y exactly"""
     n_rows, n_cols, n_tok = 14336, 4096, 512
