@@ -259,10 +259,11 @@ int qlin_gemm_bf16_any_dev(uint32_t ggml_type, const void *W, const uint16_t *X,
 /* qlin_gemm_bf16_any_dev for one to three weight tensors of ONE format and row length against the same activations:
  * the Q, K and V projections of a prefill chunk, which the reference multiplies tensor by tensor
  * (tf_gemm_f16_mt_tokenmajor per projection, common/transformer.h:5256-5258). Y[i][t * ldy[i] + r] is tensor i's
- * product. Where every tensor on its own would take the 128-token x 64-row tile kernel they share one launch, their row
- * tiles numbered through (a 1024-row K or V projection alone is 64 workgroups at 512 tokens on 256 compute units;
- * Q4_K 4096 + 1024 + 1024 rows x 4096 at 512 tokens: 36 us in one launch against 24 + 22 + 22); every other case is
- * one qlin_gemm_bf16_any_dev call per tensor, with its argument checks and its use of the workspace (sized for the
+ * product. Where every tensor on its own would take the same tile kernel (more than 32 tokens of a format with one)
+ * they share one launch, their row tiles numbered through, with the results of one call per tensor bit for bit: a
+ * 1024-row K or V projection alone is 64 workgroups of 128 tokens x 64 rows at 512 tokens on 256 compute units (Q4_K
+ * 4096 + 1024 + 1024 rows x 4096 at 512 tokens: 36 us in one launch against 24 + 22 + 22). Every other case is one
+ * qlin_gemm_bf16_any_dev call per tensor, with its argument checks and its use of the workspace (sized for the
  * largest tensor). The arrays W, Y, n_rows and ldy are host memory and are read before the call returns. */
 int qlin_gemm_bf16_multi_dev(uint32_t ggml_type, int n_mat, const void *const *W, const uint16_t *X, float *const *Y,
                              const int *n_rows, int n_cols, int n_tok, int ldx, const int *ldy, void *workspace,
