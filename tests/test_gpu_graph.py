@@ -78,7 +78,8 @@ def test_decode_style_sequence_in_a_graph(oracle):
 
 def test_prefill_sequence_in_a_graph(oracle):
     """The fused prefill GEMMs take no workspace and only enqueue: a chunk's projections (large tiles, small tiles and
-    the few-token kernel, three formats) are captured with a NULL workspace and replayed bit-identically."""
+    the few-token kernel, three formats, and three tensors in one launch of qlin_gemm_bf16_multi_dev) are captured with a
+    NULL workspace and replayed bit-identically."""
     hip = C.CDLL("libamdhip64.so")
     Q5K, NL = synth.GGML_Q5_K, synth.GGML_IQ4_NL
     K, n_tok = 512, 300
@@ -89,13 +90,22 @@ def test_prefill_sequence_in_a_graph(oracle):
     dX = qlinear.DevBuf.from_numpy(Xb)
     Y = [qlinear.DevBuf(m * r * 4) for (_, r, m) in shapes]
     lib = qlinear.load()
+    # three Q5_K tensors that share one launch (the shape of a chunk's Q, K and V projections)
+    qkv_rows = [640, 130, 70]
+    qkv_host = [synth.make_weights(Q5K, r, K, seed=40 + i) for i, r in enumerate(qkv_rows)]
+    qkv_W = [qlinear.DevBuf.from_numpy(a) for a in qkv_host]
+    qkv_Y = [qlinear.DevBuf(n_tok * r * 4) for r in qkv_rows]
+    Wp = (C.c_void_p * 3)(*[b.ptr for b in qkv_W])
+    Yp = (C.c_void_p * 3)(*[b.ptr for b in qkv_Y])
+    rows3 = (C.c_int * 3)(*qkv_rows)
 
     def enqueue(stream):
         for (t, r, m), w, y in zip(shapes, W, Y):
             assert lib.qlin_gemm_bf16_any_dev(t, w.ptr, dX.ptr, y.ptr, r, K, m, K, r, None, 0, stream) == 0, lib.qlin_last_error()
+        assert lib.qlin_gemm_bf16_multi_dev(Q5K, 3, Wp, dX.ptr, Yp, rows3, K, n_tok, K, rows3, None, 0, stream) == 0, lib.qlin_last_error()
 
     def clear():
-        for (_, r, m), y in zip(shapes, Y):
+        for r, m, y in [(r, m, y) for (_, r, m), y in zip(shapes, Y)] + [(r, n_tok, y) for r, y in zip(qkv_rows, qkv_Y)]:
             z = np.full(m * r, -3.0, np.float32)
             assert lib.qlin_dev_upload(y.ptr, z.ctypes.data, z.nbytes) == 0
 
@@ -108,6 +118,10 @@ def test_prefill_sequence_in_a_graph(oracle):
         if m > 24:
             dec = synth.bf16_bits_to_f32(synth.to_bf16_bits(dec))
         assert rel_l2(got, Xf[:m] @ dec.astype(np.float64).T) <= 2e-5, (t, r, m)
+    qkv_want = [y.to_numpy(np.float32, (n_tok, r)) for r, y in zip(qkv_rows, qkv_Y)]
+    for r, h, got in zip(qkv_rows, qkv_host, qkv_want):
+        dec = synth.bf16_bits_to_f32(synth.to_bf16_bits(oracle.dequant_matrix(Q5K, h, K)))
+        assert rel_l2(got, Xf @ dec.astype(np.float64).T) <= 2e-5, r
 
     stream, graph, gexec = C.c_void_p(), C.c_void_p(), C.c_void_p()
     assert hip.hipStreamCreate(C.byref(stream)) == 0
@@ -117,16 +131,18 @@ def test_prefill_sequence_in_a_graph(oracle):
     assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
     n_nodes = C.c_size_t(0)
     assert hip.hipGraphGetNodes(graph, None, C.byref(n_nodes)) == 0
-    assert n_nodes.value == len(shapes)  # one kernel per product, nothing else
+    assert n_nodes.value == len(shapes) + 1  # one kernel per product and one for the three tensors together, nothing else
     for replay in range(3):
         clear()
         assert hip.hipGraphLaunch(gexec, stream) == 0
         assert hip.hipStreamSynchronize(stream) == 0
         for (_, r, m), y, w_ in zip(shapes, Y, want):
             assert np.array_equal(y.to_numpy(np.float32, (m, r)), w_), replay
+        for r, y, w_ in zip(qkv_rows, qkv_Y, qkv_want):
+            assert np.array_equal(y.to_numpy(np.float32, (n_tok, r)), w_), (replay, r)
         qlinear.gemm_bf16_any_dev(Q5K, W[1], dX, Y[1], 640, K, 100, K, 640, None)  # eager work between replays
         qlinear.sync()
     assert hip.hipGraphExecDestroy(gexec) == 0 and hip.hipGraphDestroy(graph) == 0
     assert hip.hipStreamDestroy(stream) == 0
-    for b in W + Y + [dX]:
+    for b in W + Y + [dX] + qkv_W + qkv_Y:
         b.free()
